@@ -1,0 +1,166 @@
+/*
+ * tfjs_hip.h -- C ABI of the MI355X (gfx950) native half of tfjs-backend-hip.
+ *
+ * One process, one GPU, one HIP stream. Every entry point returns 0 on success
+ * and a non-zero status on failure; tfhip_last_error() then describes the
+ * failure (the N-API shim turns it into a thrown JS Error, the convention of
+ * tfjs-node/binding/utils.h:46-94). Kernel entry points only enqueue work on
+ * the library's stream; tfhip_download() and tfhip_sync() are the sync points.
+ *
+ * Device memory is owned by the library: tfhip_alloc() hands out device
+ * pointers from a size-bucketed pool and records every live block, and every
+ * kernel entry point checks that each operand range lies inside a live block
+ * before launching, so a wrong shape is an error return and never a GPU fault.
+ *
+ * All tensors are dense, row-major float32 unless stated. "Reference" citations
+ * are file:line in the tensorflow/tfjs source tree and name the interface each
+ * entry point stands in for.
+ */
+#ifndef TFJS_HIP_H_
+#define TFJS_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Fused activation codes. Numbering of FusableActivation,
+ * tfjs-backend-wasm/src/cc/backend.h:32-40 and
+ * tfjs-backend-wasm/src/kernels/types.ts:28-36. */
+enum tfhip_activation {
+  TFHIP_LINEAR = 0,
+  TFHIP_RELU = 1,
+  TFHIP_RELU6 = 2,
+  TFHIP_PRELU = 3,
+  TFHIP_LEAKYRELU = 4,
+  TFHIP_SIGMOID = 5,
+  TFHIP_ELU = 6
+};
+
+/* ---- library lifetime ---------------------------------------------------
+ * Stands in for the wasm backend's init()/dispose()
+ * (tfjs-backend-wasm/src/cc/backend.h:97-120) and for the constructor of
+ * TFJSBackend in the Node addon (tfjs-node/binding/tfjs_backend.cc). */
+int tfhip_init(int device);
+int tfhip_shutdown(void);
+const char *tfhip_last_error(void);
+/* name: device name; arch: gcnArchName; cus: compute units; hbm_bytes: total
+ * device memory. Any out pointer may be NULL. */
+int tfhip_device_info(char *name, size_t name_len, char *arch, size_t arch_len,
+                      int *cus, int *clock_khz, size_t *hbm_bytes);
+
+/* ---- buffers ------------------------------------------------------------
+ * The id -> buffer bookkeeping of register_tensor()/dispose_data()
+ * (tfjs-backend-wasm/src/cc/backend.h:107-115) and of createTensor /
+ * deleteTensor / tensorDataSync in the Node addon
+ * (tfjs-node/binding/tfjs_binding.cc:303-327). Here the handle is the device
+ * pointer itself. */
+int tfhip_alloc(size_t bytes, void **dptr);
+int tfhip_free(void *dptr);
+/* Asynchronous host->device copy of `bytes` bytes to dst (+dst_offset bytes)
+ * through pinned staging; the host range may be reused on return. */
+int tfhip_upload(void *dst, size_t dst_offset, const void *host, size_t bytes);
+/* Waits for the stream, then copies device->host. */
+int tfhip_download(void *host, const void *src, size_t src_offset, size_t bytes);
+int tfhip_sync(void);
+/* live: blocks handed out and not freed; live_bytes: their total size;
+ * pooled_bytes: freed blocks kept for reuse. */
+int tfhip_memory_info(size_t *live, size_t *live_bytes, size_t *pooled_bytes);
+/* Lets kernels accept device memory the caller allocated elsewhere. */
+int tfhip_register_external(void *dptr, size_t bytes);
+int tfhip_unregister_external(void *dptr);
+
+/* ---- timing (KernelBackend.time(), tfjs-core/src/backends/backend.ts:88-92)
+ * Events are recorded on the library's stream. tfhip_event_record(slot) marks
+ * slot (0..TFHIP_MAX_EVENTS-1); tfhip_event_elapsed(a, b, &ms) waits for b and
+ * returns the milliseconds between the two marks. */
+#define TFHIP_MAX_EVENTS 4096
+int tfhip_event_record(int slot);
+int tfhip_event_elapsed(int start_slot, int end_slot, float *ms);
+
+/* ---- _FusedMatMul / BatchMatMul ------------------------------------------
+ * Replaces _FusedMatMul(a_id, a_shape, ..., out_id)
+ * (tfjs-backend-wasm/src/cc/kernels/_FusedMatMul.cc:30-43) and BatchMatMul
+ * (tfjs-backend-wasm/src/cc/kernels/BatchMatMul.cc); semantics of
+ * tfjs-backend-cpu/src/kernels/_FusedMatMul.ts:26-62 and BatchMatMul.ts:25-133.
+ *
+ * a is [batch_a, M, K] (or [batch_a, K, M] if transpose_a), b is
+ * [batch_b, K, N] (or [batch_b, N, K] if transpose_b); out is
+ * [max(batch_a,batch_b), M, N], batch index of each operand taken modulo its
+ * own batch count. bias / prelu_weights may be NULL. When present they are
+ * addressed as base[bi*strides[0] + i*strides[1] + j*strides[2]] for output
+ * element (bi, i, j): a stride of 0 broadcasts along that axis. */
+int tfhip_fused_matmul(const float *a, const float *b, float *out,
+                       int64_t batch_a, int64_t batch_b, int64_t M, int64_t N,
+                       int64_t K, int transpose_a, int transpose_b,
+                       const float *bias, const int64_t bias_strides[3],
+                       int activation, const float *prelu_weights,
+                       const int64_t prelu_strides[3], double leakyrelu_alpha);
+
+/* ---- FusedConv2D -----------------------------------------------------------
+ * Replaces FusedConv2D(x_id, batch_size, input_height, ..., out_id)
+ * (tfjs-backend-wasm/src/cc/kernels/FusedConv2D.cc:33-54); semantics of
+ * tfjs-backend-cpu/src/kernels/FusedConv2D.ts:26-95 over Conv2D.ts:23-103.
+ * The caller has already run computeConv2DInfo
+ * (tfjs-core/src/ops/conv_util.ts:177-236) and passes its numbers.
+ *
+ * x is NHWC [batch,in_h,in_w,in_c] (nchw == 0) or NCHW; filter is HWIO
+ * [f_h,f_w,in_c,out_c]; y has the same data format as x. bias / prelu_weights
+ * are addressed as base[n*s[0] + h*s[1] + w*s[2] + c*s[3]] for output element
+ * (n, h, w, c) whatever the data format. */
+int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
+                       int64_t batch, int64_t in_h, int64_t in_w, int64_t in_c,
+                       int64_t f_h, int64_t f_w, int64_t out_c,
+                       int64_t stride_h, int64_t stride_w, int64_t dilation_h,
+                       int64_t dilation_w, int64_t pad_top, int64_t pad_left,
+                       int64_t out_h, int64_t out_w, int nchw,
+                       const float *bias, const int64_t bias_strides[4],
+                       int activation, const float *prelu_weights,
+                       const int64_t prelu_strides[4], double leakyrelu_alpha);
+
+/* ---- FusedDepthwiseConv2D ----------------------------------------------------
+ * Replaces FusedDepthwiseConv2D(...)
+ * (tfjs-backend-wasm/src/cc/kernels/FusedDepthwiseConv2D.cc); semantics of
+ * tfjs-backend-cpu/src/kernels/FusedDepthwiseConv2D.ts:25-61 over
+ * DepthwiseConv2dNative.ts:23-102. NHWC only; filter is
+ * [f_h,f_w,in_c,ch_mul]; y is [batch,out_h,out_w,in_c*ch_mul]. */
+int tfhip_fused_depthwise_conv2d(
+    const float *x, const float *filter, float *y, int64_t batch, int64_t in_h,
+    int64_t in_w, int64_t in_c, int64_t f_h, int64_t f_w, int64_t ch_mul,
+    int64_t stride_h, int64_t stride_w, int64_t dilation_h, int64_t dilation_w,
+    int64_t pad_top, int64_t pad_left, int64_t out_h, int64_t out_w,
+    const float *bias, const int64_t bias_strides[4], int activation,
+    const float *prelu_weights, const int64_t prelu_strides[4],
+    double leakyrelu_alpha);
+
+/* ---- weight dequantisation on load -----------------------------------------
+ * The quantization branch of decodeWeight, tfjs-core/src/io/io_utils.ts:196-251,
+ * which the reference runs in JavaScript before backend.write(). `q` points at
+ * the quantized bytes on the device (any byte alignment).
+ *   affine (:223-227, :243-247): bits is 8 or 16 (little-endian codes);
+ *     out[i] = fround(double(q[i]) * scale + min), or, when to_int32 != 0,
+ *     Int32Array-store(Math.round(double(q[i]) * scale + min)).
+ *   f16 (:229-231, getFloat16Decoder :720-741): exact binary16 -> binary32. */
+int tfhip_dequant_affine(const void *q, int bits, int64_t n, double scale,
+                         double min, void *out, int to_int32);
+int tfhip_dequant_f16(const void *q, int64_t n, float *out);
+
+/* ---- glue kernels of a MobileNetV2 graph -------------------------------------
+ * tfhip_add: broadcasting Add (tfjs-backend-cpu/src/kernels/Add.ts:23-30,
+ *   utils/binary_impl.ts:25-68). out has `rank` (<= 6) dims out_shape; a and b
+ *   are addressed with element strides per output dim (0 = broadcast).
+ * tfhip_mean_hw: Mean over axes [1,2] of an NHWC tensor
+ *   (tfjs-backend-cpu/src/kernels/Mean.ts:26-56, Sum.ts:30-92):
+ *   y[n,c] = fround(sum_hw double(fround(x / fround(H*W)))). */
+int tfhip_add(const float *a, const int64_t *a_strides, const float *b,
+              const int64_t *b_strides, float *out, const int64_t *out_shape,
+              int rank);
+int tfhip_mean_hw(const float *x, float *y, int64_t batch, int64_t h, int64_t w,
+                  int64_t c);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TFJS_HIP_H_ */

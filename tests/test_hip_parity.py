@@ -1,0 +1,357 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle.
+
+Bar (the acceptance bound of the build): dequantized weights bit-exact; float32
+outputs within max|d| <= 1e-3 * max(1, |ref|), tfjs's own float32 test epsilon
+(tfjs-core/src/test_util.ts:23) made relative for large magnitudes.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from golden_util import assert_close, conv_args, ids, load_cases, tensor  # noqa: E402
+import synth  # noqa: E402
+
+FMM = load_cases("fused_mat_mul.json")
+MM = load_cases("mat_mul.json")
+FCONV = load_cases("fused_conv2d.json")
+CONV = load_cases("conv2d.json")
+FDW = load_cases("fused_depthwise_conv2d.json")
+DW = load_cases("depthwise_conv2d.json")
+
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from tfjs_amd import pyhost
+    pyhost.init(0)
+    yield pyhost
+    info = pyhost.memory_info()
+    assert info["live"] == 0, "device buffers leaked: %s" % info
+
+
+@pytest.fixture(scope="module")
+def orc():
+    from oracle import pyoracle
+    return pyoracle
+
+
+def assert_parity(got, want, tol=TOL):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    assert got.shape == want.shape, "%s vs %s" % (got.shape, want.shape)
+    nan_g, nan_w = np.isnan(got), np.isnan(want)
+    assert np.array_equal(nan_g, nan_w), "NaN pattern differs"
+    err = np.abs(np.where(nan_w, 0, got - want)) / np.maximum(1.0, np.abs(np.where(nan_w, 0, want)))
+    worst = err.max() if err.size else 0.0
+    assert worst <= tol, "max scaled error %.3e at %s (got %r want %r)" % (
+        worst, np.unravel_index(err.argmax(), err.shape), got.flat[err.argmax()], want.flat[err.argmax()])
+    return worst
+
+
+# ---------------------------------------------------------------- golden vectors
+
+@pytest.mark.parametrize("c", FMM + MM, ids=ids(FMM + MM))
+def test_matmul_golden(hip, c):
+    out = hip.fused_matmul(
+        tensor(c["a"]), tensor(c["b"]), bias=tensor(c.get("bias")),
+        activation=c.get("activation") or "linear", prelu=tensor(c.get("preluActivationWeights")),
+        leakyrelu_alpha=c.get("leakyreluAlpha") if c.get("leakyreluAlpha") is not None else 0.2,
+        transpose_a=bool(c.get("transposeA")), transpose_b=bool(c.get("transposeB")))
+    assert_close(out, c["expected"])
+
+
+def _run_conv(mod, c, depthwise):
+    x, w, kw, squeeze = conv_args(c)
+    if depthwise:
+        y = mod.fused_depthwise_conv2d(x, w, **kw)
+    else:
+        y = mod.fused_conv2d(x, w, data_format=c.get("dataFormat") or "NHWC", **kw)
+    return y[0] if squeeze else y
+
+
+@pytest.mark.parametrize("c", FCONV + CONV, ids=ids(FCONV + CONV))
+def test_conv2d_golden(hip, orc, c):
+    got = _run_conv(hip, c, False)
+    assert_close(got, c["expected"])
+    assert_parity(got, _run_conv(orc, c, False))
+
+
+@pytest.mark.parametrize("c", FDW + DW, ids=ids(FDW + DW))
+def test_depthwise_golden(hip, orc, c):
+    got = _run_conv(hip, c, True)
+    assert_close(got, c["expected"])
+    assert_parity(got, _run_conv(orc, c, True))
+
+
+# ------------------------------------------------------- benchmark configurations
+
+def test_config1_fused_matmul(hip, orc):
+    c = synth.config1()
+    assert_parity(hip.fused_matmul(**c), orc.fused_matmul(**c))
+
+
+def test_config2a_stem_conv(hip, orc):
+    c = synth.config2a()
+    x, w = c.pop("x"), c.pop("w")
+    assert_parity(hip.fused_conv2d(x, w, **c), orc.fused_conv2d(x, w, **c))
+
+
+def test_config2b_pointwise_conv(hip, orc):
+    c = synth.config2b()
+    x, w = c.pop("x"), c.pop("w")
+    assert_parity(hip.fused_conv2d(x, w, **c), orc.fused_conv2d(x, w, **c))
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+def test_config3_depthwise(hip, orc, stride):
+    c = synth.config3(stride)
+    x, w = c.pop("x"), c.pop("w")
+    got, want = hip.fused_depthwise_conv2d(x, w, **c), orc.fused_depthwise_conv2d(x, w, **c)
+    assert_parity(got, want)
+    # same tap order and one fused multiply-add per tap: differences can only come
+    # from the reference rounding through double first
+    assert np.mean(got != want) < 1e-3
+
+
+@pytest.mark.parametrize("name", [m[0] for m in synth.BERT_MATMULS])
+def test_config5_bert_matmuls(hip, orc, name):
+    c = synth.config5(name)
+    assert_parity(hip.fused_matmul(**c), orc.fused_matmul(**c))
+
+
+# ------------------------------------------------------------------ shape sweeps
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (5, 3, 7), (47, 49, 48), (64, 64, 16), (65, 63, 17), (130, 100, 36),
+                                   (256, 16, 64), (300, 24, 144), (128, 128, 128), (129, 97, 260), (33, 1000, 1280)])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_matmul_shapes_and_transposes(hip, orc, m, n, k, ta, tb):
+    rng = np.random.default_rng(m * 7919 + n * 31 + k + ta * 2 + tb)
+    a = rng.uniform(-1, 1, (2, k, m) if ta else (2, m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (2, n, k) if tb else (2, k, n)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (n,)).astype(np.float32)
+    kw = dict(bias=bias, activation="relu", transpose_a=bool(ta), transpose_b=bool(tb))
+    assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
+
+
+# (outer dims like [3,1] x [1,4] are left out: the reference sizes its result
+# buffer with max(batchA, batchB) and indexes by modulo, BatchMatMul.ts:74,96-97,
+# which is only meaningful when one batch count divides the other)
+@pytest.mark.parametrize("sa,sb", [((6, 20, 12), (1, 12, 8)), ((20, 12), (5, 12, 8)),
+                                   ((2, 2, 9, 4), (2, 4, 6))])
+def test_matmul_batch_broadcast(hip, orc, sa, sb):
+    rng = np.random.default_rng(5)
+    a = rng.uniform(-1, 1, sa).astype(np.float32)
+    b = rng.uniform(-1, 1, sb).astype(np.float32)
+    got = hip.batch_matmul(a, b)
+    assert_parity(got, orc.batch_matmul(a, b))
+    assert_parity(got, np.matmul(a.astype(np.float64), b.astype(np.float64)), 1e-4)
+
+
+@pytest.mark.parametrize("act", ["linear", "relu", "relu6", "elu", "sigmoid", "leakyrelu", "prelu"])
+@pytest.mark.parametrize("bias_shape", [None, (40,), (1, 40), (24, 40), (24, 1), (3, 1, 1), (3, 24, 40), ()])
+def test_matmul_epilogue_forms(hip, orc, act, bias_shape):
+    rng = np.random.default_rng(17)
+    a = rng.uniform(-2, 2, (3, 24, 16)).astype(np.float32)
+    b = rng.uniform(-2, 2, (3, 16, 40)).astype(np.float32)
+    bias = None if bias_shape is None else rng.uniform(-1, 1, bias_shape).astype(np.float32)
+    prelu = rng.uniform(0, 1, (1, 40)).astype(np.float32) if act == "prelu" else None
+    kw = dict(bias=bias, activation=act, prelu=prelu, leakyrelu_alpha=0.3)
+    assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
+
+
+def test_matmul_nan_and_signed_zero_through_relu(hip, orc):
+    a = np.array([[[np.nan, 1.0], [-1.0, 0.0], [0.0, 0.0]]], np.float32)
+    b = np.array([[[1.0, 2.0], [0.0, 1.0]]], np.float32)
+    for act in ("relu", "relu6", "linear"):
+        got, want = hip.fused_matmul(a, b, activation=act), orc.fused_matmul(a, b, activation=act)
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        np.testing.assert_array_equal(got[~np.isnan(want)], want[~np.isnan(want)])
+
+
+CONV_SWEEP = [
+    # x shape, filter shape, strides, dilations, pad
+    ((2, 9, 7, 3), (3, 3, 3, 5), (2, 2), 1, "same"),
+    ((1, 8, 8, 4), (3, 2, 4, 8), (1, 1), (2, 1), "same"),
+    ((1, 10, 9, 2), (5, 3, 2, 4), (3, 2), 1, "valid"),
+    ((2, 6, 6, 8), (1, 1, 8, 6), (1, 1), 1, "valid"),
+    ((1, 7, 5, 3), (3, 3, 3, 2), (1, 1), 1, [[0, 0], [2, 1], [0, 3], [0, 0]]),
+    ((3, 14, 14, 64), (1, 1, 64, 384), 1, 1, "same"),
+    ((3, 14, 14, 32), (3, 3, 32, 48), 1, 1, "same"),
+    ((2, 15, 15, 16), (3, 3, 16, 20), 2, 1, "same"),
+    ((2, 16, 16, 12), (1, 1, 12, 8), 2, 1, "same"),
+    ((1, 12, 12, 8), (3, 3, 8, 16), 1, 2, 1),
+]
+
+
+@pytest.mark.parametrize("xs,fs,stride,dil,pad", CONV_SWEEP)
+@pytest.mark.parametrize("fmt", ["NHWC", "NCHW"])
+def test_conv2d_shapes(hip, orc, xs, fs, stride, dil, pad, fmt):
+    rng = np.random.default_rng(sum(xs) * 13 + sum(fs))
+    x = rng.uniform(-1, 1, xs).astype(np.float32)
+    w = rng.normal(0, 0.3, fs).astype(np.float32)
+    bias = rng.uniform(-1, 1, (fs[3],)).astype(np.float32)
+    if fmt == "NCHW":
+        x = np.ascontiguousarray(x.transpose(0, 3, 1, 2))
+        if isinstance(pad, list):
+            pad = [pad[0], pad[3], pad[1], pad[2]]
+    kw = dict(strides=stride, pad=pad, dilations=dil, data_format=fmt, bias=bias, activation="relu6")
+    assert_parity(hip.fused_conv2d(x, w, **kw), orc.fused_conv2d(x, w, **kw))
+
+
+@pytest.mark.parametrize("act", ["elu", "sigmoid", "leakyrelu", "prelu"])
+@pytest.mark.parametrize("bias_shape,prelu_shape", [((12,), (12,)), ((), (1, 1, 12)), ((5, 12), (6, 5, 1)), ((2, 6, 5, 12), (1,))])
+def test_conv2d_epilogue_forms(hip, orc, act, bias_shape, prelu_shape):
+    rng = np.random.default_rng(23)
+    x = rng.uniform(-1, 1, (2, 6, 5, 8)).astype(np.float32)
+    w = rng.normal(0, 0.5, (3, 3, 8, 12)).astype(np.float32)
+    kw = dict(pad="same", bias=rng.uniform(-1, 1, bias_shape).astype(np.float32), activation=act,
+              prelu=rng.uniform(0, 1, prelu_shape).astype(np.float32) if act == "prelu" else None,
+              leakyrelu_alpha=0.1)
+    assert_parity(hip.fused_conv2d(x, w, **kw), orc.fused_conv2d(x, w, **kw))
+
+
+@pytest.mark.parametrize("xs,fs,stride,dil,pad", [
+    ((2, 9, 8, 4), (3, 3, 4, 1), 1, 1, "same"), ((2, 9, 8, 4), (3, 3, 4, 1), 2, 1, "same"),
+    ((1, 20, 33, 36), (3, 3, 36, 1), 1, 1, "same"), ((1, 21, 33, 36), (3, 3, 36, 1), 2, 1, "same"),
+    ((3, 7, 7, 960), (3, 3, 960, 1), 1, 1, "same"), ((2, 14, 14, 576), (3, 3, 576, 1), 2, 1, "same"),
+    ((2, 9, 8, 4), (3, 3, 4, 2), 1, 1, "same"), ((2, 9, 8, 3), (3, 3, 3, 1), 1, 1, "valid"),
+    ((1, 11, 10, 6), (5, 3, 6, 3), (2, 1), 1, "same"), ((1, 11, 10, 8), (3, 3, 8, 1), 1, 2, "same"),
+    ((1, 8, 8, 8), (3, 3, 8, 1), 1, 1, 1), ((1, 6, 6, 8), (3, 3, 8, 1), 1, 1, [[0, 0], [2, 0], [1, 3], [0, 0]]),
+])
+def test_depthwise_shapes(hip, orc, xs, fs, stride, dil, pad):
+    rng = np.random.default_rng(sum(xs) + sum(fs) * 3)
+    x = rng.uniform(0, 1, xs).astype(np.float32)
+    w = rng.normal(0, 0.5, fs).astype(np.float32)
+    bias = rng.uniform(-0.1, 0.1, (fs[2] * fs[3],)).astype(np.float32)
+    kw = dict(strides=stride, pad=pad, dilations=dil, bias=bias, activation="relu6")
+    assert_parity(hip.fused_depthwise_conv2d(x, w, **kw), orc.fused_depthwise_conv2d(x, w, **kw))
+
+
+def test_depthwise_linearity_full_size(hip):
+    # size-independent property at the benchmark shape: conv(x1 + x2) = conv(x1) + conv(x2)
+    c = synth.config3(1)
+    x, w = c["x"], c["w"]
+    x2 = np.roll(x, 1, axis=2)
+    y = hip.fused_depthwise_conv2d(x + x2, w, pad="same")
+    y12 = hip.fused_depthwise_conv2d(x, w, pad="same") + hip.fused_depthwise_conv2d(x2, w, pad="same")
+    assert np.abs(y - y12).max() <= 1e-4
+
+
+# ---------------------------------------------------------------------- dequant
+
+@pytest.mark.parametrize("bits", [8, 16])
+@pytest.mark.parametrize("scale,min_", [(0.1, -1.0), (2 / 255, -3.0), (3.3e-5, -1.07), (1e30, -1e30), (7.0, 1e9)])
+def test_dequant_affine_exhaustive_bit_exact(hip, orc, bits, scale, min_):
+    codes = np.arange(1 << bits, dtype=np.uint8 if bits == 8 else np.uint16)
+    for dtype in ("float32", "int32"):
+        spec = [{"name": "w", "dtype": dtype, "shape": [codes.size],
+                 "quantization": {"dtype": "uint%d" % bits, "scale": scale, "min": min_}}]
+        got = hip.decode_weights(codes.tobytes(), spec)["w"]
+        want = orc.decode_weights(codes.tobytes(), spec)["w"]
+        np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_dequant_f16_exhaustive_bit_exact(hip, orc):
+    h = np.arange(65536, dtype=np.uint16)
+    spec = [{"name": "w", "dtype": "float32", "shape": [65536], "quantization": {"dtype": "float16"}}]
+    got = hip.decode_weights(h.tobytes(), spec)["w"]
+    want = orc.decode_weights(h.tobytes(), spec)["w"]
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_decode_weights_mixed_manifest_bit_exact(hip, orc):
+    """A shard with ragged sizes: every tensor after the first starts at an odd
+    or otherwise unaligned byte offset."""
+    from oracle import quantization as oq
+    rng = np.random.default_rng(3)
+    specs, chunks = [], []
+    for i, (shape, kind) in enumerate([((3, 3, 3, 5), np.uint8), ((7,), np.uint16), ((1, 1, 33, 9), np.float16),
+                                       ((13,), None), ((2, 5), np.uint8), ((1001,), np.uint16), ((4099,), np.uint8),
+                                       ((5,), "int32q")]):
+        data = rng.normal(0, 0.3, shape).astype(np.float32)
+        entry = {"name": "t%d" % i, "shape": list(shape), "dtype": "float32"}
+        if kind is None:
+            chunks.append(data.tobytes())
+        elif kind == "int32q":
+            ints = rng.integers(-50, 50, shape).astype(np.int32)
+            q, meta = oq.quantize_weights(ints, np.uint8)
+            entry["dtype"] = "int32"
+            entry["quantization"] = {"dtype": "uint8", "scale": meta["scale"], "min": meta["min"]}
+            chunks.append(q.tobytes())
+        else:
+            q, meta = oq.quantize_weights(data, kind)
+            entry["quantization"] = dict({"dtype": np.dtype(kind).name}, **({} if kind == np.float16 else
+                                                                            {"scale": meta["scale"], "min": meta["min"]}))
+            chunks.append(q.tobytes())
+        specs.append(entry)
+    buf = b"".join(chunks)
+    got, want = hip.decode_weights(buf, specs), orc.decode_weights(buf, specs)
+    for s in specs:
+        assert got[s["name"]].dtype == want[s["name"]].dtype and got[s["name"]].shape == want[s["name"]].shape
+        np.testing.assert_array_equal(got[s["name"]].view(np.uint32), want[s["name"]].view(np.uint32))
+
+
+@pytest.mark.parametrize("kind", [np.uint8, np.uint16, np.float16])
+def test_dequant_large_bit_exact(hip, orc, kind):
+    from oracle import quantization as oq
+    rng = np.random.default_rng(8)
+    data = rng.normal(0, 0.05, (3469760,)).astype(np.float32)     # MobileNetV2 weight count
+    q, meta = oq.quantize_weights(data, kind)
+    quant = {"dtype": np.dtype(kind).name}
+    if kind != np.float16:
+        quant.update(scale=meta["scale"], min=meta["min"])
+    spec = [{"name": "w", "dtype": "float32", "shape": [data.size], "quantization": quant}]
+    got, want = hip.decode_weights(q.tobytes(), spec)["w"], orc.decode_weights(q.tobytes(), spec)["w"]
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    if kind != np.float16:
+        # round trip of the producer's own quantizer: within half a quantization step
+        assert np.abs(got - data).max() <= meta["scale"] * 0.5001
+
+
+def test_decode_weights_errors(hip):
+    with pytest.raises(ValueError, match="doesn't have corresponding metadata min and scale"):
+        hip.decode_weights(b"\0", [{"name": "w", "dtype": "float32", "shape": [1],
+                                    "quantization": {"dtype": "uint8", "scale": 1}}])
+    with pytest.raises(ValueError, match="which only supports weights of type float32 not int32"):
+        hip.decode_weights(b"\0\0", [{"name": "w", "dtype": "int32", "shape": [1],
+                                      "quantization": {"dtype": "float16"}}])
+    with pytest.raises(ValueError, match="unknown quantization dtype int8"):
+        hip.decode_weights(b"\0", [{"name": "w", "dtype": "float32", "shape": [1],
+                                    "quantization": {"dtype": "int8", "scale": 1, "min": 0}}])
+
+
+# ------------------------------------------------------------------------- glue
+
+def test_add_and_mean(hip, orc):
+    rng = np.random.default_rng(4)
+    a = rng.uniform(-1, 1, (2, 7, 7, 20)).astype(np.float32)
+    for bshape in [(2, 7, 7, 20), (20,), (7, 1, 20), (2, 1, 1, 1), ()]:
+        b = rng.uniform(-1, 1, bshape).astype(np.float32)
+        np.testing.assert_array_equal(hip.add(a, b), orc.add(a, b))
+    np.testing.assert_array_equal(hip.mean_hw(a), orc.mean_hw(a))
+    big = rng.uniform(0, 6, (4, 7, 7, 1280)).astype(np.float32)
+    np.testing.assert_array_equal(hip.mean_hw(big), orc.mean_hw(big))
+
+
+# ------------------------------------------------------------------ error paths
+
+def test_bad_operands_are_errors_not_faults(hip):
+    from tfjs_amd import capi
+    lib = capi.load_library()
+    with capi.DeviceBuffer(64) as small:
+        # 'a' claims 1024 x 1024 floats but the buffer holds 16
+        rc = lib.tfhip_fused_matmul(small.ptr, small.ptr, small.ptr, 1, 1, 1024, 1024, 1024, 0, 0, None,
+                                    capi.i64_array([0, 0, 0]), 0, None, capi.i64_array([0, 0, 0]), 0.2)
+        assert rc != 0 and b"not inside a live device buffer" in lib.tfhip_last_error()
+        rc = lib.tfhip_fused_matmul(small.ptr, small.ptr, small.ptr, 1, 1, 2, 2, 2, 0, 0, None,
+                                    capi.i64_array([0, 0, 0]), 9, None, capi.i64_array([0, 0, 0]), 0.2)
+        assert rc != 0 and b"unknown activation" in lib.tfhip_last_error()
+        rc = lib.tfhip_dequant_affine(small.ptr, 12, 4, 1.0, 0.0, small.ptr, 0)
+        assert rc != 0 and b"bits must be 8 or 16" in lib.tfhip_last_error()
+    rc = lib.tfhip_free(ctypes.c_void_p(0x1000))
+    assert rc != 0
+    with pytest.raises(ValueError, match="inner shapes"):
+        hip.fused_matmul(np.zeros((2, 3), np.float32), np.zeros((4, 2), np.float32))

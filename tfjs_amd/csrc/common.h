@@ -1,0 +1,76 @@
+// Internal declarations shared by the translation units of libtfjs_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/tfjs_hip.h"
+
+namespace tfhip {
+
+// Records the message returned by tfhip_last_error() and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+enum Status {
+  kOk = 0,
+  kNotInitialised = 1,
+  kHipError = 2,
+  kBadArgument = 3,
+  kOutOfRange = 4,
+  kOutOfMemory = 5
+};
+
+bool initialised();
+hipStream_t stream();
+int num_cus();
+
+// True when [p, p + bytes) lies inside one live block (own or external).
+bool range_is_live(const void *p, size_t bytes);
+
+#define TFHIP_REQUIRE_INIT()                                              \
+  do {                                                                    \
+    if (!::tfhip::initialised())                                          \
+      return ::tfhip::fail(::tfhip::kNotInitialised,                      \
+                           "%s: tfhip_init has not been called", __func__); \
+  } while (0)
+
+#define TFHIP_CHECK_HIP(expr)                                               \
+  do {                                                                      \
+    hipError_t e_ = (expr);                                                 \
+    if (e_ != hipSuccess)                                                   \
+      return ::tfhip::fail(::tfhip::kHipError, "%s: %s failed: %s", __func__, \
+                           #expr, hipGetErrorString(e_));                   \
+  } while (0)
+
+#define TFHIP_CHECK_ARG(cond, ...)                                \
+  do {                                                            \
+    if (!(cond)) return ::tfhip::fail(::tfhip::kBadArgument, __VA_ARGS__); \
+  } while (0)
+
+// Operand `name` of `elems` float-sized (`esize` bytes) elements must be live.
+#define TFHIP_CHECK_RANGE(ptr, elems, esize, name)                             \
+  do {                                                                         \
+    if ((ptr) == nullptr || !::tfhip::range_is_live((ptr), (size_t)(elems) * (esize))) \
+      return ::tfhip::fail(::tfhip::kOutOfRange,                               \
+                           "%s: operand '%s' (%lld elements of %d bytes at %p) " \
+                           "is not inside a live device buffer",               \
+                           __func__, name, (long long)(elems), (int)(esize),   \
+                           (const void *)(ptr));                               \
+  } while (0)
+
+// Checks the launch that was just enqueued.
+#define TFHIP_CHECK_LAUNCH()  TFHIP_CHECK_HIP(hipGetLastError())
+
+// Largest element offset reached by a strided broadcast operand, plus one.
+inline int64_t strided_extent(const int64_t *dims, const int64_t *strides, int rank) {
+  int64_t last = 0;
+  for (int i = 0; i < rank; ++i) {
+    if (dims[i] <= 0) return 0;
+    last += (dims[i] - 1) * strides[i];
+  }
+  return last + 1;
+}
+
+}  // namespace tfhip

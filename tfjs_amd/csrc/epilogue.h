@@ -1,0 +1,92 @@
+// Fused bias + activation tail shared by the matmul, conv and depthwise kernels.
+//
+// The reference runs three float32-rounded passes (kernel, broadcasting Add of
+// the bias, activation: tfjs-backend-cpu/src/kernels/_FusedMatMul.ts:41-55,
+// FusedConv2D.ts:43-92); here the same three roundings happen in registers
+// before the single store.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tfhip {
+
+// How bias / prelu weights are addressed for an output element.
+//  kChannel: base[col * s_col] only (rank-1 bias over the last axis, or scalar)
+//  kMatmul:  base[batch*s[0] + row*s[1] + col*s[2]]
+//  kConv:    row is split into (n, oh, ow): base[n*s[0] + oh*s[1] + ow*s[2] + col*s[3]]
+enum EpilogueAddressing { kChannel = 0, kMatmul = 1, kConv = 2 };
+
+struct Epilogue {
+  const float *bias;
+  const float *prelu;
+  long long bias_s[4];
+  long long prelu_s[4];
+  double leaky_alpha;
+  int activation;
+  int addressing;
+  // kConv only: spatial extent of the output for the row split, and the output
+  // strides for (n, oh, ow, c) so NCHW outputs can be written in place.
+  int out_h, out_w;
+  long long y_s[4];
+};
+
+__device__ __forceinline__ float activate(float v, int act, float alpha, double leaky) {
+  switch (act) {
+    case TFHIP_RELU:
+      // Math.max(0, x): NaN stays NaN, -0 becomes +0 (Relu.ts:22)
+      return (v > 0.f || v != v) ? v : 0.f;
+    case TFHIP_RELU6: {
+      // Math.min(Math.max(0, x), 6) (Relu6.ts:22-23)
+      const float t = (v > 0.f || v != v) ? v : 0.f;
+      return t > 6.f ? 6.f : t;
+    }
+    case TFHIP_PRELU:
+      // x < 0 ? alpha * x : x (Prelu.ts:24-25)
+      return v < 0.f ? alpha * v : v;
+    case TFHIP_LEAKYRELU:
+      // the reference keeps alpha as a double attribute (LeakyRelu.ts:38-40)
+      return v < 0.f ? (float)(leaky * (double)v) : v;
+    case TFHIP_SIGMOID:
+      // 1 / (1 + exp(-x)) (Sigmoid.ts:25-26)
+      return 1.f / (1.f + expf(-v));
+    case TFHIP_ELU:
+      // x >= 0 ? x : exp(x) - 1 (Elu.ts:22-23)
+      return v >= 0.f ? v : expm1f(v);
+    default:
+      return v;
+  }
+}
+
+// Applies bias and activation to `v`, the raw contraction result of output
+// element (batch, row, col). For kConv, (n, oh, ow) is the split of `row`.
+__device__ __forceinline__ float finish(const Epilogue &e, float v, long long batch,
+                                        long long row, long long col, long long n,
+                                        long long oh, long long ow) {
+  if (e.bias) {
+    long long idx;
+    if (e.addressing == kChannel) {
+      idx = col * e.bias_s[3];
+    } else if (e.addressing == kMatmul) {
+      idx = batch * e.bias_s[0] + row * e.bias_s[1] + col * e.bias_s[2];
+    } else {
+      idx = n * e.bias_s[0] + oh * e.bias_s[1] + ow * e.bias_s[2] + col * e.bias_s[3];
+    }
+    v = v + e.bias[idx];
+  }
+  float alpha = 0.f;
+  if (e.activation == TFHIP_PRELU) {
+    long long idx;
+    if (e.addressing == kChannel) {
+      idx = col * e.prelu_s[3];
+    } else if (e.addressing == kMatmul) {
+      idx = batch * e.prelu_s[0] + row * e.prelu_s[1] + col * e.prelu_s[2];
+    } else {
+      idx = n * e.prelu_s[0] + oh * e.prelu_s[1] + ow * e.prelu_s[2] + col * e.prelu_s[3];
+    }
+    alpha = e.prelu[idx];
+  }
+  return activate(v, e.activation, alpha, e.leaky_alpha);
+}
+
+}  // namespace tfhip

@@ -1,0 +1,121 @@
+// The few non-contraction kernels a MobileNetV2 graph needs between the fused
+// ops, so that no tensor leaves the device mid-graph: the residual Add and the
+// global average pool (Mean over H and W).
+#include "common.h"
+
+namespace tfhip {
+namespace {
+
+constexpr int kMaxRank = 6;
+
+struct AddParams {
+  const float *a;
+  const float *b;
+  float *out;
+  long long total;
+  int rank;
+  long long shape[kMaxRank];
+  long long a_s[kMaxRank];
+  long long b_s[kMaxRank];
+};
+
+__global__ __launch_bounds__(256) void add_same_shape(const float4 *__restrict__ a, const float4 *__restrict__ b,
+                                                      float4 *__restrict__ out, long long groups) {
+  const long long stride = (long long)gridDim.x * 256;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < groups; i += stride) {
+    const float4 u = a[i], v = b[i];
+    out[i] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+  }
+}
+
+__global__ __launch_bounds__(256) void add_broadcast(AddParams p) {
+  const long long stride = (long long)gridDim.x * 256;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < p.total; i += stride) {
+    long long rem = i, ia = 0, ib = 0;
+#pragma unroll
+    for (int d = kMaxRank - 1; d >= 0; --d) {
+      if (d < p.rank) {
+        const long long loc = rem % p.shape[d];
+        rem /= p.shape[d];
+        ia += loc * p.a_s[d];
+        ib += loc * p.b_s[d];
+      }
+    }
+    p.out[i] = p.a[ia] + p.b[ib];
+  }
+}
+
+// One lane per (n, c): consecutive lanes read consecutive channels.
+__global__ __launch_bounds__(256) void mean_hw(const float *__restrict__ x, float *__restrict__ y, long long batch,
+                                               long long hw, long long c) {
+  const float denom = (float)hw;
+  const long long total = batch * c;
+  const long long stride = (long long)gridDim.x * 256;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+    const long long n = i / c, ch = i - n * c;
+    const float *px = x + n * hw * c + ch;
+    double sum = 0.0;
+    for (long long j = 0; j < hw; ++j) sum += (double)__fdiv_rn(px[j * c], denom);
+    y[i] = (float)sum;
+  }
+}
+
+int grid_for(long long items) {
+  long long blocks = (items + 255) / 256;
+  const long long cap = (long long)num_cus() * 32;
+  if (blocks > cap) blocks = cap;
+  return blocks < 1 ? 1 : (int)blocks;
+}
+
+}  // namespace
+}  // namespace tfhip
+
+using namespace tfhip;
+
+extern "C" {
+
+int tfhip_add(const float *a, const int64_t *a_strides, const float *b, const int64_t *b_strides, float *out,
+              const int64_t *out_shape, int rank) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_ARG(rank >= 0 && rank <= kMaxRank, "tfhip_add: rank %d not in 0..%d", rank, kMaxRank);
+  TFHIP_CHECK_ARG(rank == 0 || (a_strides && b_strides && out_shape), "tfhip_add: missing shape or strides");
+  AddParams p = {};
+  p.a = a; p.b = b; p.out = out; p.rank = rank;
+  long long total = 1;
+  bool dense = true;
+  for (int d = rank - 1; d >= 0; --d) {
+    TFHIP_CHECK_ARG(out_shape[d] >= 0 && a_strides[d] >= 0 && b_strides[d] >= 0, "tfhip_add: negative extent or stride");
+    if (out_shape[d] > 1 && (a_strides[d] != total || b_strides[d] != total)) dense = false;
+    p.shape[d] = out_shape[d];
+    p.a_s[d] = a_strides[d];
+    p.b_s[d] = b_strides[d];
+    total *= out_shape[d];
+  }
+  p.total = total;
+  if (total == 0) return kOk;
+  TFHIP_CHECK_RANGE(a, strided_extent(out_shape, a_strides, rank), 4, "a");
+  TFHIP_CHECK_RANGE(b, strided_extent(out_shape, b_strides, rank), 4, "b");
+  TFHIP_CHECK_RANGE(out, total, 4, "out");
+  const bool aligned = reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  if (dense && aligned && total % 4 == 0) {
+    add_same_shape<<<grid_for(total / 4), 256, 0, stream()>>>((const float4 *)a, (const float4 *)b, (float4 *)out, total / 4);
+  } else {
+    add_broadcast<<<grid_for(total), 256, 0, stream()>>>(p);
+  }
+  TFHIP_CHECK_LAUNCH();
+  return kOk;
+}
+
+int tfhip_mean_hw(const float *x, float *y, int64_t batch, int64_t h, int64_t w, int64_t c) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_ARG(batch >= 0 && h > 0 && w > 0 && c >= 0, "tfhip_mean_hw: bad dimensions");
+  if (batch * c == 0) return kOk;
+  TFHIP_CHECK_RANGE(x, batch * h * w * c, 4, "x");
+  TFHIP_CHECK_RANGE(y, batch * c, 4, "y");
+  mean_hw<<<grid_for(batch * c), 256, 0, stream()>>>(x, y, batch, h * w, c);
+  TFHIP_CHECK_LAUNCH();
+  return kOk;
+}
+
+}  // extern "C"

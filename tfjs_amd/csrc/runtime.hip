@@ -1,0 +1,316 @@
+// Library lifetime, the single stream, the pooled device allocator with its
+// live-block registry, host<->device copies through pinned staging, and event
+// timing.
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "common.h"
+
+namespace tfhip {
+namespace {
+
+constexpr size_t kStagingBytes = size_t(32) << 20;  // per pinned staging buffer
+constexpr int kStagingBuffers = 2;
+
+struct Runtime {
+  bool ready = false;
+  int device = 0;
+  hipStream_t stream = nullptr;
+  hipDeviceProp_t prop;
+  // live blocks: base address -> usable size. `owned` blocks came from the pool.
+  std::map<uintptr_t, size_t> live;
+  std::map<uintptr_t, bool> owned;
+  std::unordered_map<size_t, std::vector<void *>> free_lists;  // by class size
+  size_t live_bytes = 0, pooled_bytes = 0;
+  void *staging[kStagingBuffers] = {nullptr, nullptr};
+  hipEvent_t staging_done[kStagingBuffers] = {nullptr, nullptr};
+  bool staging_busy[kStagingBuffers] = {false, false};
+  int next_staging = 0;
+  hipEvent_t events[TFHIP_MAX_EVENTS] = {};
+  bool event_recorded[TFHIP_MAX_EVENTS] = {};
+};
+
+Runtime g;
+std::mutex g_mutex;
+thread_local char g_error[1024] = "";
+
+// Size classes: eight per power of two, at least 256 bytes.
+size_t class_size(size_t bytes) {
+  if (bytes <= 256) return 256;
+  size_t p = 256;
+  while (p < bytes) p <<= 1;
+  const size_t step = p >> 4;  // p/2 .. p in eight steps of p/16
+  const size_t lo = p >> 1;
+  size_t c = lo + ((bytes - lo + step - 1) / step) * step;
+  return c < 256 ? 256 : c;
+}
+
+void release_pool_locked() {
+  for (auto &kv : g.free_lists) {
+    for (void *p : kv.second) (void)hipFree(p);
+    kv.second.clear();
+  }
+  g.pooled_bytes = 0;
+}
+
+}  // namespace
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof g_error, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool initialised() { return g.ready; }
+hipStream_t stream() { return g.stream; }
+int num_cus() { return g.prop.multiProcessorCount; }
+
+bool range_is_live(const void *p, size_t bytes) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+  auto it = g.live.upper_bound(a);
+  if (it == g.live.begin()) return false;
+  --it;
+  return a >= it->first && a + bytes <= it->first + it->second && a + bytes >= a;
+}
+
+}  // namespace tfhip
+
+using namespace tfhip;
+
+extern "C" {
+
+const char *tfhip_last_error(void) { return g_error; }
+
+int tfhip_init(int device) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (g.ready) {
+    if (device == g.device) return kOk;
+    return fail(kBadArgument, "tfhip_init: already initialised on device %d", g.device);
+  }
+  int count = 0;
+  TFHIP_CHECK_HIP(hipGetDeviceCount(&count));
+  TFHIP_CHECK_ARG(device >= 0 && device < count,
+                  "tfhip_init: device %d not present (%d visible)", device, count);
+  TFHIP_CHECK_HIP(hipSetDevice(device));
+  TFHIP_CHECK_HIP(hipGetDeviceProperties(&g.prop, device));
+  if (strncmp(g.prop.gcnArchName, "gfx950", 6) != 0) {
+    return fail(kBadArgument,
+                "tfhip_init: device %d is %s; this library carries gfx950 code only",
+                device, g.prop.gcnArchName);
+  }
+  TFHIP_CHECK_HIP(hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking));
+  for (int i = 0; i < kStagingBuffers; ++i) {
+    TFHIP_CHECK_HIP(hipHostMalloc(&g.staging[i], kStagingBytes, hipHostMallocDefault));
+    TFHIP_CHECK_HIP(hipEventCreateWithFlags(&g.staging_done[i], hipEventDisableTiming));
+    g.staging_busy[i] = false;
+  }
+  g.device = device;
+  g.ready = true;
+  return kOk;
+}
+
+int tfhip_shutdown(void) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (!g.ready) return kOk;
+  (void)hipStreamSynchronize(g.stream);
+  for (auto &kv : g.live) {
+    if (g.owned[kv.first]) (void)hipFree(reinterpret_cast<void *>(kv.first));
+  }
+  g.live.clear();
+  g.owned.clear();
+  g.live_bytes = 0;
+  release_pool_locked();
+  for (int i = 0; i < kStagingBuffers; ++i) {
+    if (g.staging[i]) (void)hipHostFree(g.staging[i]);
+    if (g.staging_done[i]) (void)hipEventDestroy(g.staging_done[i]);
+    g.staging[i] = nullptr;
+    g.staging_done[i] = nullptr;
+  }
+  for (int i = 0; i < TFHIP_MAX_EVENTS; ++i) {
+    if (g.events[i]) (void)hipEventDestroy(g.events[i]);
+    g.events[i] = nullptr;
+    g.event_recorded[i] = false;
+  }
+  (void)hipStreamDestroy(g.stream);
+  g.stream = nullptr;
+  g.ready = false;
+  return kOk;
+}
+
+int tfhip_device_info(char *name, size_t name_len, char *arch, size_t arch_len,
+                      int *cus, int *clock_khz, size_t *hbm_bytes) {
+  TFHIP_REQUIRE_INIT();
+  if (name && name_len) snprintf(name, name_len, "%s", g.prop.name);
+  if (arch && arch_len) snprintf(arch, arch_len, "%s", g.prop.gcnArchName);
+  if (cus) *cus = g.prop.multiProcessorCount;
+  if (clock_khz) *clock_khz = g.prop.clockRate;
+  if (hbm_bytes) *hbm_bytes = g.prop.totalGlobalMem;
+  return kOk;
+}
+
+int tfhip_alloc(size_t bytes, void **dptr) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_ARG(dptr != nullptr, "tfhip_alloc: dptr is NULL");
+  const size_t cls = class_size(bytes);
+  std::lock_guard<std::mutex> lock(g_mutex);
+  void *p = nullptr;
+  auto &fl = g.free_lists[cls];
+  if (!fl.empty()) {
+    p = fl.back();
+    fl.pop_back();
+    g.pooled_bytes -= cls;
+  } else {
+    hipError_t e = hipMalloc(&p, cls);
+    if (e == hipErrorOutOfMemory) {
+      (void)hipGetLastError();
+      (void)hipStreamSynchronize(g.stream);
+      release_pool_locked();
+      e = hipMalloc(&p, cls);
+    }
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(kOutOfMemory, "tfhip_alloc: hipMalloc(%zu) failed: %s", cls,
+                  hipGetErrorString(e));
+    }
+  }
+  g.live[reinterpret_cast<uintptr_t>(p)] = cls;
+  g.owned[reinterpret_cast<uintptr_t>(p)] = true;
+  g.live_bytes += cls;
+  *dptr = p;
+  return kOk;
+}
+
+int tfhip_free(void *dptr) {
+  TFHIP_REQUIRE_INIT();
+  std::lock_guard<std::mutex> lock(g_mutex);
+  const uintptr_t a = reinterpret_cast<uintptr_t>(dptr);
+  auto it = g.live.find(a);
+  if (it == g.live.end() || !g.owned[a]) {
+    return fail(kBadArgument, "tfhip_free: %p is not a live block of this library", dptr);
+  }
+  // Work already enqueued on the single stream runs before any later kernel
+  // that is handed this block again, so the block can be reused at once.
+  const size_t cls = it->second;
+  g.live.erase(it);
+  g.owned.erase(a);
+  g.live_bytes -= cls;
+  g.free_lists[cls].push_back(dptr);
+  g.pooled_bytes += cls;
+  return kOk;
+}
+
+int tfhip_register_external(void *dptr, size_t bytes) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_ARG(dptr != nullptr && bytes > 0, "tfhip_register_external: empty range");
+  std::lock_guard<std::mutex> lock(g_mutex);
+  g.live[reinterpret_cast<uintptr_t>(dptr)] = bytes;
+  g.owned[reinterpret_cast<uintptr_t>(dptr)] = false;
+  return kOk;
+}
+
+int tfhip_unregister_external(void *dptr) {
+  TFHIP_REQUIRE_INIT();
+  std::lock_guard<std::mutex> lock(g_mutex);
+  const uintptr_t a = reinterpret_cast<uintptr_t>(dptr);
+  auto it = g.live.find(a);
+  if (it == g.live.end() || g.owned[a]) {
+    return fail(kBadArgument, "tfhip_unregister_external: %p was not registered", dptr);
+  }
+  g.live.erase(it);
+  g.owned.erase(a);
+  return kOk;
+}
+
+int tfhip_memory_info(size_t *live, size_t *live_bytes, size_t *pooled_bytes) {
+  TFHIP_REQUIRE_INIT();
+  std::lock_guard<std::mutex> lock(g_mutex);
+  size_t n = 0;
+  for (auto &kv : g.owned) n += kv.second ? 1 : 0;
+  if (live) *live = n;
+  if (live_bytes) *live_bytes = g.live_bytes;
+  if (pooled_bytes) *pooled_bytes = g.pooled_bytes;
+  return kOk;
+}
+
+int tfhip_upload(void *dst, size_t dst_offset, const void *host, size_t bytes) {
+  TFHIP_REQUIRE_INIT();
+  if (bytes == 0) return kOk;
+  TFHIP_CHECK_ARG(host != nullptr, "tfhip_upload: host pointer is NULL");
+  char *d = static_cast<char *>(dst) + dst_offset;
+  TFHIP_CHECK_RANGE(d, bytes, 1, "dst");
+  const char *h = static_cast<const char *>(host);
+  size_t done = 0;
+  while (done < bytes) {
+    const size_t chunk = bytes - done < kStagingBytes ? bytes - done : kStagingBytes;
+    const int s = g.next_staging;
+    g.next_staging = (s + 1) % kStagingBuffers;
+    if (g.staging_busy[s]) TFHIP_CHECK_HIP(hipEventSynchronize(g.staging_done[s]));
+    memcpy(g.staging[s], h + done, chunk);
+    TFHIP_CHECK_HIP(hipMemcpyAsync(d + done, g.staging[s], chunk, hipMemcpyHostToDevice, g.stream));
+    TFHIP_CHECK_HIP(hipEventRecord(g.staging_done[s], g.stream));
+    g.staging_busy[s] = true;
+    done += chunk;
+  }
+  return kOk;
+}
+
+int tfhip_download(void *host, const void *src, size_t src_offset, size_t bytes) {
+  TFHIP_REQUIRE_INIT();
+  if (bytes == 0) {
+    TFHIP_CHECK_HIP(hipStreamSynchronize(g.stream));
+    return kOk;
+  }
+  TFHIP_CHECK_ARG(host != nullptr, "tfhip_download: host pointer is NULL");
+  const char *s = static_cast<const char *>(src) + src_offset;
+  TFHIP_CHECK_RANGE(s, bytes, 1, "src");
+  char *h = static_cast<char *>(host);
+  size_t done = 0;
+  while (done < bytes) {
+    const size_t chunk = bytes - done < kStagingBytes ? bytes - done : kStagingBytes;
+    const int b = g.next_staging;
+    g.next_staging = (b + 1) % kStagingBuffers;
+    if (g.staging_busy[b]) TFHIP_CHECK_HIP(hipEventSynchronize(g.staging_done[b]));
+    g.staging_busy[b] = false;
+    TFHIP_CHECK_HIP(hipMemcpyAsync(g.staging[b], s + done, chunk, hipMemcpyDeviceToHost, g.stream));
+    TFHIP_CHECK_HIP(hipStreamSynchronize(g.stream));
+    memcpy(h + done, g.staging[b], chunk);
+    done += chunk;
+  }
+  return kOk;
+}
+
+int tfhip_sync(void) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_HIP(hipStreamSynchronize(g.stream));
+  return kOk;
+}
+
+int tfhip_event_record(int slot) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_ARG(slot >= 0 && slot < TFHIP_MAX_EVENTS, "tfhip_event_record: slot %d out of range", slot);
+  if (!g.events[slot]) TFHIP_CHECK_HIP(hipEventCreate(&g.events[slot]));
+  TFHIP_CHECK_HIP(hipEventRecord(g.events[slot], g.stream));
+  g.event_recorded[slot] = true;
+  return kOk;
+}
+
+int tfhip_event_elapsed(int start_slot, int end_slot, float *ms) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_ARG(start_slot >= 0 && start_slot < TFHIP_MAX_EVENTS && end_slot >= 0 &&
+                      end_slot < TFHIP_MAX_EVENTS && ms != nullptr,
+                  "tfhip_event_elapsed: bad arguments");
+  TFHIP_CHECK_ARG(g.event_recorded[start_slot] && g.event_recorded[end_slot],
+                  "tfhip_event_elapsed: slot %d or %d was never recorded", start_slot, end_slot);
+  TFHIP_CHECK_HIP(hipEventSynchronize(g.events[end_slot]));
+  TFHIP_CHECK_HIP(hipEventElapsedTime(ms, g.events[start_slot], g.events[end_slot]));
+  return kOk;
+}
+
+}  // extern "C"

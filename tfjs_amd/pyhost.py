@@ -1,0 +1,262 @@
+"""numpy-in / numpy-out host mirror of the four fused kernels and the weight
+decoder, over the C ABI. It exists so the parity tests and the Python benchmark
+can drive the HIP kernels with the same call shapes as the reference's kernels
+(tfjs-backend-cpu/src/kernels/{_FusedMatMul,BatchMatMul,FusedConv2D,
+FusedDepthwiseConv2D}.ts, tfjs-core/src/io/io_utils.ts decodeWeights); the
+JavaScript backend in tfjs_amd/js is the product-side host.
+
+Each call uploads its operands, launches, downloads the result and frees its
+buffers; `device_*` variants keep data resident for benchmarking.
+"""
+import ctypes
+
+import numpy as np
+
+from . import capi
+from .capi import ACTIVATIONS, DeviceBuffer, check, i64_array, load_library
+from .conv_util import broadcast_shape, broadcast_strides, compute_conv2d_info
+
+_initialised = False
+
+
+def init(device=0):
+    global _initialised
+    if not _initialised:
+        check(load_library().tfhip_init(device))
+        _initialised = True
+
+
+def shutdown():
+    global _initialised
+    if _initialised:
+        check(load_library().tfhip_shutdown())
+        _initialised = False
+
+
+def device_info():
+    init()
+    name = ctypes.create_string_buffer(256)
+    arch = ctypes.create_string_buffer(256)
+    cus, clk, mem = ctypes.c_int(), ctypes.c_int(), ctypes.c_size_t()
+    check(load_library().tfhip_device_info(name, 256, arch, 256, ctypes.byref(cus), ctypes.byref(clk),
+                                           ctypes.byref(mem)))
+    return dict(name=name.value.decode(), arch=arch.value.decode(), cus=cus.value, clock_khz=clk.value,
+                hbm_bytes=mem.value)
+
+
+def memory_info():
+    live, live_bytes, pooled = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    check(load_library().tfhip_memory_info(ctypes.byref(live), ctypes.byref(live_bytes), ctypes.byref(pooled)))
+    return dict(live=live.value, live_bytes=live_bytes.value, pooled_bytes=pooled.value)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _opt(a):
+    return None if a is None else _f32(a)
+
+
+def matmul_dims(a_shape, b_shape, transpose_a, transpose_b):
+    """Shape bookkeeping of BatchMatMul.ts:36-74 (error text included)."""
+    a_shape, b_shape = list(a_shape), list(b_shape)
+    inner_a = a_shape[-2] if transpose_a else a_shape[-1]
+    inner_b = b_shape[-1] if transpose_b else b_shape[-2]
+    outer_a = a_shape[-1] if transpose_a else a_shape[-2]
+    outer_b = b_shape[-2] if transpose_b else b_shape[-1]
+    batch_a = int(np.prod(a_shape[:-2], dtype=np.int64))
+    batch_b = int(np.prod(b_shape[:-2], dtype=np.int64))
+    outer = broadcast_shape(a_shape[:-2], b_shape[:-2])
+    if inner_a != inner_b:
+        raise ValueError(
+            "Error in matMul: inner shapes (%d) and (%d) of Tensors with shapes %s and %s and "
+            "transposeA=%s and transposeB=%s must match." %
+            (inner_a, inner_b, ",".join(map(str, a_shape)), ",".join(map(str, b_shape)),
+             str(bool(transpose_a)).lower(), str(bool(transpose_b)).lower()))
+    return batch_a, batch_b, outer_a, outer_b, inner_a, outer + [outer_a, outer_b]
+
+
+def device_fused_matmul(a, b, out, batch_a, batch_b, m, n, k, transpose_a=False, transpose_b=False,
+                        bias=None, bias_strides=None, activation="linear", prelu=None,
+                        prelu_strides=None, leakyrelu_alpha=0.2):
+    """Launch on DeviceBuffers already resident (no copies, no sync)."""
+    check(load_library().tfhip_fused_matmul(
+        a.ptr, b.ptr, out.ptr, batch_a, batch_b, m, n, k, int(bool(transpose_a)), int(bool(transpose_b)),
+        bias.ptr if bias is not None else None, i64_array(bias_strides or [0, 0, 0]),
+        ACTIVATIONS[activation], prelu.ptr if prelu is not None else None,
+        i64_array(prelu_strides or [0, 0, 0]), float(leakyrelu_alpha)))
+
+
+def fused_matmul(a, b, bias=None, activation="linear", prelu=None, leakyrelu_alpha=0.2,
+                 transpose_a=False, transpose_b=False):
+    """_FusedMatMul / BatchMatMul: a and b of rank >= 2, batch dims broadcast."""
+    init()
+    a, b, bias, prelu = _f32(a), _f32(b), _opt(bias), _opt(prelu)
+    batch_a, batch_b, m, n, k, out_shape = matmul_dims(a.shape, b.shape, transpose_a, transpose_b)
+    batch = max(batch_a, batch_b)
+    view = [batch, m, n]
+    bias_strides = broadcast_strides(list(bias.shape), view) if bias is not None else None
+    prelu_strides = broadcast_strides(list(prelu.shape), view) if prelu is not None else None
+    bufs = []
+    try:
+        da, db = DeviceBuffer.from_numpy(a), DeviceBuffer.from_numpy(b)
+        dout = DeviceBuffer(batch * m * n * 4)
+        bufs += [da, db, dout]
+        dbias = DeviceBuffer.from_numpy(bias) if bias is not None else None
+        dprelu = DeviceBuffer.from_numpy(prelu) if prelu is not None else None
+        bufs += [x for x in (dbias, dprelu) if x is not None]
+        device_fused_matmul(da, db, dout, batch_a, batch_b, m, n, k, transpose_a, transpose_b, dbias,
+                            bias_strides, activation, dprelu, prelu_strides, leakyrelu_alpha)
+        return dout.download(np.float32, batch * m * n).reshape(out_shape)
+    finally:
+        for buf in bufs:
+            buf.free()
+
+
+def batch_matmul(a, b, transpose_a=False, transpose_b=False):
+    return fused_matmul(a, b, transpose_a=transpose_a, transpose_b=transpose_b)
+
+
+def _conv_call(depthwise, x, w, strides, pad, data_format, dilations, dim_rounding_mode, bias, activation,
+               prelu, leakyrelu_alpha):
+    init()
+    x, w, bias, prelu = _f32(x), _f32(w), _opt(bias), _opt(prelu)
+    fmt = "channelsLast" if data_format == "NHWC" else "channelsFirst"
+    ci = compute_conv2d_info(x.shape, w.shape, strides, dilations, pad, dim_rounding_mode, depthwise, fmt)
+    nchw = fmt == "channelsFirst"
+    out_shape = ci["outShape"]
+    nhwc_view = [ci["batchSize"], ci["outHeight"], ci["outWidth"], ci["outChannels"]]
+
+    def strides_for(t):
+        if t is None:
+            return None
+        shape = list(t.shape)
+        if nchw and len(shape) == 1 and shape[0] != 1:
+            shape = [shape[0], 1, 1]          # FusedConv2D.ts:55-61, :76-86
+        s = broadcast_strides(shape, out_shape)
+        # the C ABI takes strides in (n, h, w, c) order whatever the data format
+        return [s[0], s[2], s[3], s[1]] if nchw else s
+
+    bias_strides, prelu_strides = strides_for(bias), strides_for(prelu)
+    bufs = []
+    try:
+        dx, dw = DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(w)
+        total = int(np.prod(out_shape, dtype=np.int64))
+        dy = DeviceBuffer(total * 4)
+        bufs += [dx, dw, dy]
+        dbias = DeviceBuffer.from_numpy(bias) if bias is not None else None
+        dprelu = DeviceBuffer.from_numpy(prelu) if prelu is not None else None
+        bufs += [b for b in (dbias, dprelu) if b is not None]
+        common = [ci["batchSize"], ci["inHeight"], ci["inWidth"], ci["inChannels"], ci["filterHeight"],
+                  ci["filterWidth"]]
+        tail = [ci["strideHeight"], ci["strideWidth"], ci["dilationHeight"], ci["dilationWidth"],
+                ci["padInfo"]["top"], ci["padInfo"]["left"], ci["outHeight"], ci["outWidth"]]
+        epi = [dbias.ptr if dbias else None, i64_array(bias_strides or [0] * 4), ACTIVATIONS[activation],
+               dprelu.ptr if dprelu else None, i64_array(prelu_strides or [0] * 4), float(leakyrelu_alpha)]
+        if depthwise:
+            check(load_library().tfhip_fused_depthwise_conv2d(
+                dx.ptr, dw.ptr, dy.ptr, *common, w.shape[3], *tail, *epi))
+        else:
+            check(load_library().tfhip_fused_conv2d(
+                dx.ptr, dw.ptr, dy.ptr, *common, ci["outChannels"], *tail, int(nchw), *epi))
+        del nhwc_view
+        return dy.download(np.float32, total).reshape(out_shape)
+    finally:
+        for buf in bufs:
+            buf.free()
+
+
+def fused_conv2d(x, w, strides=1, pad="valid", data_format="NHWC", dilations=1, dim_rounding_mode=None,
+                 bias=None, activation="linear", prelu=None, leakyrelu_alpha=0.2):
+    return _conv_call(False, x, w, strides, pad, data_format, dilations, dim_rounding_mode, bias, activation,
+                      prelu, leakyrelu_alpha)
+
+
+def fused_depthwise_conv2d(x, w, strides=1, pad="valid", dilations=1, dim_rounding_mode=None, bias=None,
+                           activation="linear", prelu=None, leakyrelu_alpha=0.2):
+    return _conv_call(True, x, w, strides, pad, "NHWC", dilations, dim_rounding_mode, bias, activation, prelu,
+                      leakyrelu_alpha)
+
+
+def add(a, b):
+    init()
+    a, b = _f32(a), _f32(b)
+    shape = broadcast_shape(list(a.shape), list(b.shape))
+    total = int(np.prod(shape, dtype=np.int64))
+    with DeviceBuffer.from_numpy(a) as da, DeviceBuffer.from_numpy(b) as db, DeviceBuffer(total * 4) as do:
+        check(load_library().tfhip_add(da.ptr, i64_array(broadcast_strides(list(a.shape), shape)), db.ptr,
+                                       i64_array(broadcast_strides(list(b.shape), shape)), do.ptr,
+                                       i64_array(shape), len(shape)))
+        return do.download(np.float32, total).reshape(shape)
+
+
+def mean_hw(x):
+    init()
+    x = _f32(x)
+    n, h, w, c = x.shape
+    with DeviceBuffer.from_numpy(x) as dx, DeviceBuffer(n * c * 4) as dy:
+        check(load_library().tfhip_mean_hw(dx.ptr, dy.ptr, n, h, w, c))
+        return dy.download(np.float32, n * c).reshape(n, c)
+
+
+# tfjs-core/src/io/types.ts:23-31
+DTYPE_VALUE_SIZE_MAP = {"float32": 4, "float16": 2, "int32": 4, "uint16": 2, "uint8": 1, "bool": 1,
+                        "complex64": 8}
+
+
+def decode_weights(buffer, specs):
+    """decodeWeights (tfjs-core/src/io/io_utils.ts:119-292) with the dequantize
+    step on the GPU: the whole weight buffer is uploaded once, each quantized
+    entry is expanded by a kernel reading at its byte offset, and plain float32 /
+    int32 / bool entries are returned from the host bytes. Returns
+    {name: ndarray}; error messages follow the reference's."""
+    init()
+    raw = np.frombuffer(bytes(buffer), dtype=np.uint8)
+    plan, offset = [], 0
+    for spec in specs:
+        name, dtype, shape = spec["name"], spec["dtype"], list(spec["shape"])
+        size = int(np.prod(shape, dtype=np.int64)) if shape else 1
+        if "quantization" in spec:
+            q = spec["quantization"]
+            qd = q["dtype"]
+            if qd in ("uint8", "uint16"):
+                if not ("min" in q and "scale" in q):
+                    raise ValueError("Weight %s with quantization %s doesn't have corresponding metadata "
+                                     "min and scale." % (name, qd))
+            elif qd == "float16":
+                if dtype != "float32":
+                    raise ValueError("Weight %s is quantized with %s which only supports weights of type "
+                                     "float32 not %s." % (name, qd, dtype))
+            else:
+                raise ValueError("Weight %s has unknown quantization dtype %s. Supported quantization "
+                                 "dtypes are: 'uint8', 'uint16', and 'float16'." % (name, qd))
+            if dtype not in ("float32", "int32"):
+                raise ValueError("Unsupported dtype in weight '%s': %s" % (name, dtype))
+            nbytes = size * DTYPE_VALUE_SIZE_MAP[qd]
+            plan.append((name, dtype, shape, size, offset, q))
+        else:
+            if dtype not in ("float32", "int32", "bool"):
+                raise ValueError("Unsupported dtype in weight '%s': %s" % (name, dtype))
+            nbytes = size * DTYPE_VALUE_SIZE_MAP[dtype]
+            plan.append((name, dtype, shape, size, offset, None))
+        offset += nbytes
+    out = {}
+    lib = load_library()
+    with DeviceBuffer.from_numpy(raw) as dq:
+        for name, dtype, shape, size, off, q in plan:
+            if q is None:
+                np_dtype = {"float32": np.float32, "int32": np.int32, "bool": np.uint8}[dtype]
+                out[name] = np.frombuffer(raw[off:off + size * np.dtype(np_dtype).itemsize].tobytes(),
+                                          dtype=np_dtype).reshape(shape).copy()
+                continue
+            with DeviceBuffer(size * 4) as dout:
+                src = ctypes.c_void_p(dq.ptr + off)
+                if q["dtype"] == "float16":
+                    check(lib.tfhip_dequant_f16(src, size, dout.ptr))
+                else:
+                    check(lib.tfhip_dequant_affine(src, 8 if q["dtype"] == "uint8" else 16, size,
+                                                   float(q["scale"]), float(q["min"]), dout.ptr,
+                                                   int(dtype == "int32")))
+                out[name] = dout.download(np.float32 if dtype == "float32" else np.int32, size).reshape(shape)
+    return out
