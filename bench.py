@@ -1,0 +1,344 @@
+#!/usr/bin/env python3
+"""Benchmark of the tfjs-backend-hip hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one MobileNetV2 1.0/224 inference at batch 32 through the backend:
+synthetic input resident in HBM, random-init weights stored uint8-quantized in
+the converter's shard format and dequantized on the GPU at load, every kernel on
+the library's single stream, and the logits downloaded at the end of the step
+(the reference's own definition of one timed inference,
+e2e/benchmarks/benchmark_util.js:246-286). Prints ONE JSON line.
+
+Besides `value` (images/s) the line carries
+  roofline      the kernel symbol with the largest share of the step, measured
+                with HIP events on the library's stream: algorithmic bytes (or
+                flops) of its launches in one step / their summed duration
+  kernels       the same figure for each benchmark configuration's own kernel
+                (fused matmul, stem and pointwise conv, depthwise, BERT matmuls,
+                dequant), each launched back to back between two events
+  cpu_baseline  the same graph at batch 1 on one host thread, timed beside it
+
+Other modes:  --kernels-only (skip the model), --no-cpu-baseline.
+"""
+import argparse
+import ctypes
+import json
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
+RIDGE = MFMA_FP32_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+BATCH = 32
+
+
+def roofline_entry(flops, nbytes, seconds):
+    """Prices `seconds` against the roof that bounds a kernel of this intensity."""
+    if nbytes > 0 and flops / nbytes > RIDGE:
+        achieved = flops / seconds / 1e12
+        return dict(bound="mfma", achieved=round(achieved, 3), peak=MFMA_FP32_PEAK_TFLOPS, unit="TFLOP/s",
+                    frac=round(achieved / MFMA_FP32_PEAK_TFLOPS, 4))
+    achieved = nbytes / seconds / 1e9
+    return dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                frac=round(achieved / HBM_PEAK_GBS, 4))
+
+
+class Events:
+    """Pairs of HIP events on the library's stream."""
+
+    def __init__(self, lib, check):
+        self.lib, self.check = lib, check
+
+    def record(self, slot):
+        self.check(self.lib.tfhip_event_record(slot))
+
+    def elapsed_ms(self, a, b):
+        ms = ctypes.c_float()
+        self.check(self.lib.tfhip_event_elapsed(a, b, ctypes.byref(ms)))
+        return ms.value
+
+
+def last_kernel(lib):
+    buf = ctypes.create_string_buffer(256)
+    lib.tfhip_last_kernel(buf, 256)
+    return buf.value.decode()
+
+
+def time_launches(lib, check, ev, fn, repeat=50, rounds=3):
+    """Average duration in seconds of one launch of the kernel `fn` enqueues:
+    `repeat` launches back to back between two events, best of `rounds`."""
+    fn()
+    check(lib.tfhip_sync())
+    check(lib.tfhip_set_launch_repeat(repeat))
+    best = None
+    try:
+        for _ in range(rounds):
+            ev.record(0)
+            fn()
+            ev.record(1)
+            ms = ev.elapsed_ms(0, 1) / repeat
+            best = ms if best is None else min(best, ms)
+    finally:
+        check(lib.tfhip_set_launch_repeat(1))
+    return best * 1e-3
+
+
+def bench_model(model_dir, steps, warmup):
+    from tfjs_amd import pyhost, workloads
+    from tfjs_amd.capi import check, load_library
+    lib = load_library()
+    model = workloads.DeviceMobileNetV2(model_dir, BATCH)
+    try:
+        model.set_input(workloads.mobilenet_v2_input(BATCH))
+        for _ in range(warmup):
+            model.predict()
+        check(lib.tfhip_sync())
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            model.predict()
+        check(lib.tfhip_sync())
+        seconds = time.perf_counter() - t0
+
+        # per-op durations on the stream: each op's kernel enqueued `repeat` times
+        # between two events, after the timed region
+        ev = Events(lib, check)
+        repeat = 20
+        names = {}
+        check(lib.tfhip_set_launch_repeat(repeat))
+        try:
+            def before(i, op):
+                ev.record(2 * i)
+
+            def after(i, op):
+                ev.record(2 * i + 1)
+                names[i] = last_kernel(lib)
+            per_op = np.zeros(len(model.plan))
+            rounds = 3
+            for r in range(rounds):
+                out = model.forward(before, after)
+                check(lib.tfhip_sync())
+                out.free()
+                d = np.array([ev.elapsed_ms(2 * i, 2 * i + 1) / repeat * 1e-3 for i in range(len(model.plan))])
+                per_op = d if r == 0 else np.minimum(per_op, d)
+        finally:
+            check(lib.tfhip_set_launch_repeat(1))
+        by_symbol = {}
+        for i in range(len(model.plan)):
+            flops, nbytes = model.op_work(i)
+            s = by_symbol.setdefault(names[i], dict(seconds=0.0, flops=0, bytes=0, launches=0))
+            s["seconds"] += per_op[i]
+            s["flops"] += flops
+            s["bytes"] += nbytes
+            s["launches"] += 1
+        kernel_seconds = float(per_op.sum())
+    finally:
+        model.close()
+    dominant = max(by_symbol, key=lambda k: by_symbol[k]["seconds"])
+    d = by_symbol[dominant]
+    roof = roofline_entry(d["flops"], d["bytes"], d["seconds"])
+    roof.update(kernel=dominant, launches_per_step=d["launches"],
+                avg_launch_us=round(d["seconds"] / d["launches"] * 1e6, 2),
+                share_of_kernel_time=round(d["seconds"] / kernel_seconds, 3), traffic=None)
+    symbols = {k: dict(us_per_step=round(v["seconds"] * 1e6, 1), launches=v["launches"],
+                       **roofline_entry(v["flops"], v["bytes"], v["seconds"])) for k, v in by_symbol.items()}
+    return dict(ms_per_step=seconds / steps * 1e3, kernel_ms_per_step=kernel_seconds * 1e3, roofline=roof,
+                symbols=symbols)
+
+
+def bench_kernels():
+    """One line per benchmark configuration: its kernel at its shape."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import synth
+    from tfjs_amd import pyhost, workloads
+    from tfjs_amd.capi import ACTIVATIONS, DeviceBuffer, check, i64_array, load_library
+    from tfjs_amd.conv_util import compute_conv2d_info
+    lib = load_library()
+    pyhost.init()
+    ev = Events(lib, check)
+    out = []
+
+    def matmul(name, a, b, bias, activation, transpose_b=False, **_):
+        bA, bB, m, n, k, _shape = pyhost.matmul_dims(a.shape, b.shape, False, transpose_b)
+        bufs = [DeviceBuffer.from_numpy(a), DeviceBuffer.from_numpy(b), DeviceBuffer(max(bA, bB) * m * n * 4)]
+        if bias is not None:
+            bufs.append(DeviceBuffer.from_numpy(bias))
+        fn = lambda: pyhost.device_fused_matmul(bufs[0], bufs[1], bufs[2], bA, bB, m, n, k, False, transpose_b,
+                                                bufs[3] if bias is not None else None, [0, 0, 1], activation)
+        sec = time_launches(lib, check, ev, fn)
+        flops = 2.0 * max(bA, bB) * m * n * k
+        nbytes = 4.0 * (a.size + b.size + max(bA, bB) * m * n + (bias.size if bias is not None else 0))
+        out.append(dict(config=name, kernel=last_kernel(lib), us=round(sec * 1e6, 2), flops=flops, bytes=nbytes,
+                        **roofline_entry(flops, nbytes, sec)))
+        for buf in bufs:
+            buf.free()
+
+    def conv(name, x, w, bias, strides, pad, activation, depthwise=False):
+        ci = compute_conv2d_info(x.shape, w.shape, strides, 1, pad, None, depthwise)
+        n_out = int(np.prod(ci["outShape"]))
+        bufs = [DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(w), DeviceBuffer(n_out * 4),
+                DeviceBuffer.from_numpy(bias)]
+        geom = [ci["batchSize"], ci["inHeight"], ci["inWidth"], ci["inChannels"], ci["filterHeight"],
+                ci["filterWidth"], w.shape[3], ci["strideHeight"], ci["strideWidth"], 1, 1, ci["padInfo"]["top"],
+                ci["padInfo"]["left"], ci["outHeight"], ci["outWidth"]]
+        epi = [bufs[3].ptr, i64_array([0, 0, 0, 1]), ACTIVATIONS[activation], None, i64_array([0] * 4), 0.2]
+        if depthwise:
+            fn = lambda: check(lib.tfhip_fused_depthwise_conv2d(bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, *geom, *epi))
+            flops = 2.0 * n_out * w.shape[0] * w.shape[1]
+        else:
+            fn = lambda: check(lib.tfhip_fused_conv2d(bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, *geom, 0, *epi))
+            flops = 2.0 * n_out * w.shape[0] * w.shape[1] * w.shape[2]
+        sec = time_launches(lib, check, ev, fn)
+        nbytes = 4.0 * (x.size + w.size + bias.size + n_out)
+        out.append(dict(config=name, kernel=last_kernel(lib), us=round(sec * 1e6, 2), flops=flops, bytes=nbytes,
+                        **roofline_entry(flops, nbytes, sec)))
+        for buf in bufs:
+            buf.free()
+
+    def dequant(name, n, kind):
+        item = 1 if kind == "uint8" else 2
+        q = DeviceBuffer.from_numpy(np.random.default_rng(0).integers(0, 255, n * item, dtype=np.uint8))
+        o = DeviceBuffer(n * 4)
+        if kind == "float16":
+            fn = lambda: check(lib.tfhip_dequant_f16(q.ptr, n, o.ptr))
+        else:
+            fn = lambda: check(lib.tfhip_dequant_affine(q.ptr, item * 8, n, 0.0123, -1.5, o.ptr, 0))
+        sec = time_launches(lib, check, ev, fn)
+        nbytes = float(n * (item + 4))
+        out.append(dict(config=name, kernel=last_kernel(lib), us=round(sec * 1e6, 2), flops=0.0, bytes=nbytes,
+                        **roofline_entry(0.0, nbytes, sec)))
+        q.free()
+        o.free()
+
+    c = synth.config1()
+    matmul("cfg1 _FusedMatMul 256x512x512 +bias relu", **c)
+    c = synth.config2a()
+    conv("cfg2a FusedConv2D stem [1,224,224,3] 3x3/2 ->32 relu6", c["x"], c["w"], c["bias"], 2, "same", "relu6")
+    c = synth.config2b()
+    conv("cfg2b FusedConv2D 1x1 [8,56,56,144]->24", c["x"], c["w"], c["bias"], 1, "same", "linear")
+    for s in (1, 2):
+        c = synth.config3(s)
+        conv("cfg3 FusedDepthwiseConv2D [8,112,112,96] 3x3 s%d relu6" % s, c["x"], c["w"], c["bias"], s, "same",
+             "relu6", depthwise=True)
+    for name, *_ in synth.BERT_MATMULS:
+        matmul("cfg5 %s" % name, **synth.config5(name))
+    dequant("cfg4 dequant uint8 3469760 weights", 3469760, "uint8")
+    dequant("cfg5 dequant float16 7077888 weights", 7077888, "float16")
+    dequant("dequant uint8 268435456 weights", 1 << 28, "uint8")
+    dequant("dequant float16 134217728 weights", 1 << 27, "float16")
+    return out
+
+
+def cpu_baseline_child(model_dir):
+    """Runs in a child process with one OpenMP thread: the CPU oracle's
+    MobileNetV2 at batch 1, three inferences, best time."""
+    from oracle import pyoracle as orc
+    from tfjs_amd import workloads
+    buf, specs = workloads.read_model(model_dir)
+    t0 = time.perf_counter()
+    weights = orc.decode_weights(buf, specs)
+    decode_s = time.perf_counter() - t0
+    ops, _ = workloads.mobilenet_v2_graph()
+    x = workloads.mobilenet_v2_input(1)
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        workloads.run_graph(orc, ops, weights, x)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    print(json.dumps(dict(seconds_per_image=best, decode_seconds=decode_s)))
+
+
+def cpu_baseline(model_dir):
+    node = shutil.which("node")
+    script = os.path.join(ROOT, "oracle", "js", "bench_cpu.js")
+    if node and os.path.exists(script):
+        proc = subprocess.run([node, script, model_dir], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                              timeout=600)
+        if proc.returncode == 0:
+            r = json.loads(proc.stdout.strip().splitlines()[-1])
+            return dict(value=round(1.0 / r["seconds_per_image"], 4), unit="images/s", cores=1, kind="port",
+                        sample="MobileNetV2 1.0/224 batch 1, %d inferences after 1 warm-up, median; JavaScript "
+                               "restatement of tfjs-backend-cpu in Node %s, one thread" % (r["runs"], r["node"]),
+                        host_cpus=os.cpu_count())
+        sys.stderr.write("node cpu baseline failed, falling back to the C oracle:\n%s\n" % proc.stderr[-2000:])
+    env = dict(os.environ, OMP_NUM_THREADS="1")
+    proc = subprocess.run([sys.executable, os.path.abspath(__file__), "--cpu-baseline-child", model_dir],
+                          stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=env, timeout=600)
+    if proc.returncode != 0:
+        raise RuntimeError("cpu baseline failed: %s" % proc.stderr[-2000:])
+    r = json.loads(proc.stdout.strip().splitlines()[-1])
+    return dict(value=round(1.0 / r["seconds_per_image"], 4), unit="images/s", cores=1, kind="port",
+                sample="MobileNetV2 1.0/224 batch 1, best of 3 inferences; C restatement of tfjs-backend-cpu, "
+                       "one thread", host_cpus=os.cpu_count())
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--kernels-only", action="store_true")
+    ap.add_argument("--no-kernels", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-baseline-child", metavar="MODEL_DIR")
+    args = ap.parse_args()
+    if args.cpu_baseline_child:
+        cpu_baseline_child(args.cpu_baseline_child)
+        return
+    if args.gpus != 1:
+        sys.stderr.write("bench.py: this build runs on one GPU; --gpus %d is not supported "
+                         "(the path shards by batch with no exchange step, see DESIGN.md)\n" % args.gpus)
+        sys.exit(2)
+    if args.kernels_only:
+        print(json.dumps(dict(kernels=bench_kernels())))
+        return
+
+    from tfjs_amd import pyhost, workloads
+    pyhost.init(0)
+    info = pyhost.device_info()
+    model_dir = tempfile.mkdtemp(prefix="tfjs_hip_mobilenet_")
+    try:
+        workloads.write_model(model_dir, workloads.mobilenet_v2_weights(seed=3), np.uint8)
+        m = bench_model(model_dir, args.steps, args.warmup)
+        cpu = None if args.no_cpu_baseline else cpu_baseline(model_dir)
+    finally:
+        shutil.rmtree(model_dir, ignore_errors=True)
+    kernels = None if args.no_kernels else bench_kernels()
+    line = {
+        "metric": "MobileNetV2 b32 images/s + fused-op TFLOP/s & % of roofline, 1 MI355X",
+        "value": round(BATCH / (m["ms_per_step"] * 1e-3), 1),
+        "unit": "images/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(m["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "MobileNetV2 1.0/224, batch 32, NHWC fp32, uint8-quantized random-init weights "
+                               "dequantized on load (benchmark configuration 4)", "batch": BATCH,
+                   "host": "python/ctypes over the C ABI", "device": info["arch"], "cus": info["cus"]},
+        "kernel_ms_per_step": round(m["kernel_ms_per_step"], 4),
+        "tflops_model": round(BATCH * workloads.mobilenet_v2_flops_per_image() / (m["ms_per_step"] * 1e-3) / 1e12, 3),
+        "roofline": m["roofline"],
+        "cpu_baseline": cpu,
+        "symbols": m["symbols"],
+        "kernels": kernels,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

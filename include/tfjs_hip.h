@@ -80,6 +80,16 @@ int tfhip_unregister_external(void *dptr);
 int tfhip_event_record(int slot);
 int tfhip_event_elapsed(int start_slot, int end_slot, float *ms);
 
+/* ---- measurement aids (no counterpart in the reference) ----------------------
+ * tfhip_set_launch_repeat(n): every kernel entry point enqueues its kernel n
+ *   times back to back (the kernels are idempotent), so that a pair of events
+ *   around one call times n launches without n trips through the caller's
+ *   language. n = 1 is normal operation.
+ * tfhip_last_kernel: symbol of the kernel the last entry point chose, spelled as
+ *   a profiler demangles it, e.g. "gemm_kernel<128, 128, 16, 2, 2, 0, 1>". */
+int tfhip_set_launch_repeat(int n);
+int tfhip_last_kernel(char *name, size_t name_len);
+
 /* ---- _FusedMatMul / BatchMatMul ------------------------------------------
  * Replaces _FusedMatMul(a_id, a_shape, ..., out_id)
  * (tfjs-backend-wasm/src/cc/kernels/_FusedMatMul.cc:30-43) and BatchMatMul

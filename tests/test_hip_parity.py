@@ -265,7 +265,7 @@ def test_dequant_f16_exhaustive_bit_exact(hip, orc):
 def test_decode_weights_mixed_manifest_bit_exact(hip, orc):
     """A shard with ragged sizes: every tensor after the first starts at an odd
     or otherwise unaligned byte offset."""
-    from oracle import quantization as oq
+    from tfjs_amd import quantization as oq
     rng = np.random.default_rng(3)
     specs, chunks = [], []
     for i, (shape, kind) in enumerate([((3, 3, 3, 5), np.uint8), ((7,), np.uint16), ((1, 1, 33, 9), np.float16),
@@ -296,7 +296,7 @@ def test_decode_weights_mixed_manifest_bit_exact(hip, orc):
 
 @pytest.mark.parametrize("kind", [np.uint8, np.uint16, np.float16])
 def test_dequant_large_bit_exact(hip, orc, kind):
-    from oracle import quantization as oq
+    from tfjs_amd import quantization as oq
     rng = np.random.default_rng(8)
     data = rng.normal(0, 0.05, (3469760,)).astype(np.float32)     # MobileNetV2 weight count
     q, meta = oq.quantize_weights(data, kind)
@@ -355,3 +355,32 @@ def test_bad_operands_are_errors_not_faults(hip):
     assert rc != 0
     with pytest.raises(ValueError, match="inner shapes"):
         hip.fused_matmul(np.zeros((2, 3), np.float32), np.zeros((4, 2), np.float32))
+
+
+# ------------------------------------------------------------- MobileNetV2 graph
+
+def test_config4_mobilenet_v2_batch1_vs_oracle(hip, orc, tmp_path):
+    """The whole graph, uint8-quantized weights dequantized on load, device
+    resident, against the oracle run layer by layer on the same decoded weights."""
+    from tfjs_amd import workloads
+    weights = workloads.mobilenet_v2_weights(seed=3)
+    workloads.write_model(str(tmp_path), weights, np.uint8)
+    buf, specs = workloads.read_model(str(tmp_path))
+    decoded = orc.decode_weights(buf, specs)
+    x = workloads.mobilenet_v2_input(2)
+    ops, _ = workloads.mobilenet_v2_graph()
+    want = workloads.run_graph(orc, ops, decoded, x)
+    model = workloads.DeviceMobileNetV2(str(tmp_path), 2)
+    try:
+        for name, (dbuf, shape) in model.weights.items():
+            got_w = dbuf.download(np.float32, int(np.prod(shape)))
+            np.testing.assert_array_equal(got_w.view(np.uint32), decoded[name].reshape(-1).view(np.uint32))
+        model.set_input(x)
+        got = model.predict()
+        assert_parity(got, want)
+        again = model.predict()
+        np.testing.assert_array_equal(got, again)
+    finally:
+        model.close()
+    # the kernel-by-kernel host mirror agrees too
+    assert_parity(workloads.run_graph(hip, ops, decoded, x[:1]), want[:1])

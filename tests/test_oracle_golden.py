@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from oracle import pyoracle as orc
-from oracle import quantization as oq
+from tfjs_amd import quantization as oq
 from golden_util import assert_close, conv_args, ids, load_cases, tensor
 
 import json

@@ -35,6 +35,8 @@ SIGNATURES = {
     "tfhip_unregister_external": [ctypes.c_void_p],
     "tfhip_event_record": [ctypes.c_int],
     "tfhip_event_elapsed": [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float)],
+    "tfhip_set_launch_repeat": [ctypes.c_int],
+    "tfhip_last_kernel": [ctypes.c_char_p, ctypes.c_size_t],
     "tfhip_fused_matmul": [c_f32p, c_f32p, c_f32p, c_i64, c_i64, c_i64, c_i64, c_i64, ctypes.c_int,
                            ctypes.c_int, c_f32p, c_i64p, ctypes.c_int, c_f32p, c_i64p, ctypes.c_double],
     "tfhip_fused_conv2d": [c_f32p, c_f32p, c_f32p] + [c_i64] * 15 + [ctypes.c_int, c_f32p, c_i64p,

@@ -63,6 +63,21 @@ bool range_is_live(const void *p, size_t bytes);
 // Checks the launch that was just enqueued.
 #define TFHIP_CHECK_LAUNCH()  TFHIP_CHECK_HIP(hipGetLastError())
 
+// Launch bookkeeping for measurement: the label of the kernel an entry point
+// chose (as a profiler prints the symbol), and how many times each entry point
+// enqueues its kernel (see tfhip_set_launch_repeat).
+void note_kernel(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+int launch_repeat();
+
+// Enqueues `launch_expr` launch_repeat() times and checks the launch.
+#define TFHIP_LAUNCH(launch_expr)                                  \
+  do {                                                             \
+    for (int r_ = ::tfhip::launch_repeat(); r_ > 0; --r_) {        \
+      launch_expr;                                                 \
+    }                                                              \
+    TFHIP_CHECK_LAUNCH();                                          \
+  } while (0)
+
 // Largest element offset reached by a strided broadcast operand, plus one.
 inline int64_t strided_extent(const int64_t *dims, const int64_t *strides, int rank) {
   int64_t last = 0;

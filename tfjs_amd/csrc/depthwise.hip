@@ -151,8 +151,6 @@ extern "C" int tfhip_fused_depthwise_conv2d(
   const int64_t lim = 0x7fffffff;
   TFHIP_CHECK_ARG(batch < lim && in_h < lim && in_w < lim && in_c * ch_mul < lim && out_h < lim && out_w < lim,
                   "tfhip_fused_depthwise_conv2d: dimension exceeds 2^31-1");
-  // The last tap of the last output must not lie before the input: a layout that
-  // computeConv2DInfo (tfjs-core/src/ops/conv_util.ts:429-481) cannot produce.
   TFHIP_CHECK_ARG(pad_top >= 0 && pad_left >= 0, "tfhip_fused_depthwise_conv2d: negative padding");
   const int64_t out_c = in_c * ch_mul;
   const int64_t total = batch * out_h * out_w * out_c;
@@ -221,18 +219,18 @@ extern "C" int tfhip_fused_depthwise_conv2d(
     const int tiles_h = ((int)out_h + tile_h - 1) / tile_h, tiles_w = ((int)out_w + tile_w - 1) / tile_w;
     if (lds <= 64 * 1024) {
       dim3 grid(tiles_h * tiles_w, (c4_total + kCQ - 1) / kCQ, (unsigned)batch);
+      note_kernel("depthwise_3x3_halo<%d>", S);
       if (S == 1)
-        depthwise_3x3_halo<1><<<grid, 256, lds, stream()>>>(p, e, tile_h, tile_w, tiles_w, c4_total);
+        TFHIP_LAUNCH((depthwise_3x3_halo<1><<<grid, 256, lds, stream()>>>(p, e, tile_h, tile_w, tiles_w, c4_total)));
       else
-        depthwise_3x3_halo<2><<<grid, 256, lds, stream()>>>(p, e, tile_h, tile_w, tiles_w, c4_total);
-      TFHIP_CHECK_LAUNCH();
+        TFHIP_LAUNCH((depthwise_3x3_halo<2><<<grid, 256, lds, stream()>>>(p, e, tile_h, tile_w, tiles_w, c4_total)));
       return kOk;
     }
   }
   long long blocks = (total + 255) / 256;
   const long long cap = (long long)num_cus() * 64;
   if (blocks > cap) blocks = cap;
-  depthwise_generic<<<(int)blocks, 256, 0, stream()>>>(p, e, total);
-  TFHIP_CHECK_LAUNCH();
+  note_kernel("depthwise_generic");
+  TFHIP_LAUNCH((depthwise_generic<<<(int)blocks, 256, 0, stream()>>>(p, e, total)));
   return kOk;
 }

@@ -146,32 +146,32 @@ int launch(const void *q, int bytes_per, long long n, double scale, double min, 
   long long groups = aligned ? n / 4 : 0;
   hipStream_t s = stream();
   if (groups > 0) {
+    note_kernel(bytes_per == 1 ? "dequant_u8_vec" : "dequant_u16_vec");
     const int grid = grid_for(groups);
     if (bytes_per == 1) {
       if (mode == 1)
-        dequant_u8_vec<true><<<grid, kThreads, 0, s>>>((const unsigned *)q, (float4 *)out, groups, scale, min);
+        TFHIP_LAUNCH((dequant_u8_vec<true><<<grid, kThreads, 0, s>>>((const unsigned *)q, (float4 *)out, groups, scale, min)));
       else
-        dequant_u8_vec<false><<<grid, kThreads, 0, s>>>((const unsigned *)q, (float4 *)out, groups, scale, min);
+        TFHIP_LAUNCH((dequant_u8_vec<false><<<grid, kThreads, 0, s>>>((const unsigned *)q, (float4 *)out, groups, scale, min)));
     } else {
       if (mode == 2)
-        dequant_u16_vec<2><<<grid, kThreads, 0, s>>>((const uint2 *)q, (float4 *)out, groups, scale, min);
+        TFHIP_LAUNCH((dequant_u16_vec<2><<<grid, kThreads, 0, s>>>((const uint2 *)q, (float4 *)out, groups, scale, min)));
       else if (mode == 1)
-        dequant_u16_vec<1><<<grid, kThreads, 0, s>>>((const uint2 *)q, (float4 *)out, groups, scale, min);
+        TFHIP_LAUNCH((dequant_u16_vec<1><<<grid, kThreads, 0, s>>>((const uint2 *)q, (float4 *)out, groups, scale, min)));
       else
-        dequant_u16_vec<0><<<grid, kThreads, 0, s>>>((const uint2 *)q, (float4 *)out, groups, scale, min);
+        TFHIP_LAUNCH((dequant_u16_vec<0><<<grid, kThreads, 0, s>>>((const uint2 *)q, (float4 *)out, groups, scale, min)));
     }
-    TFHIP_CHECK_LAUNCH();
   }
   const long long first = groups * 4;
   if (first < n) {
+    if (groups == 0) note_kernel("dequant_bytes");
     const int grid = grid_for(n - first);
     if (mode == 2)
-      dequant_bytes<2><<<grid, kThreads, 0, s>>>((const unsigned char *)q, (unsigned *)out, first, n, bytes_per, scale, min);
+        TFHIP_LAUNCH((dequant_bytes<2><<<grid, kThreads, 0, s>>>((const unsigned char *)q, (unsigned *)out, first, n, bytes_per, scale, min)));
     else if (mode == 1)
-      dequant_bytes<1><<<grid, kThreads, 0, s>>>((const unsigned char *)q, (unsigned *)out, first, n, bytes_per, scale, min);
+        TFHIP_LAUNCH((dequant_bytes<1><<<grid, kThreads, 0, s>>>((const unsigned char *)q, (unsigned *)out, first, n, bytes_per, scale, min)));
     else
-      dequant_bytes<0><<<grid, kThreads, 0, s>>>((const unsigned char *)q, (unsigned *)out, first, n, bytes_per, scale, min);
-    TFHIP_CHECK_LAUNCH();
+        TFHIP_LAUNCH((dequant_bytes<0><<<grid, kThreads, 0, s>>>((const unsigned char *)q, (unsigned *)out, first, n, bytes_per, scale, min)));
   }
   return kOk;
 }

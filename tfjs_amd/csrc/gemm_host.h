@@ -49,9 +49,9 @@ inline int launch_gemm(GemmParams &p) {
   const long long grid = (long long)p.tiles_m * p.tiles_n * p.batch;
   if (grid <= 0) return kOk;
   if (grid > 0x7fffffffLL) return fail(kBadArgument, "gemm: %lld tiles exceed the grid limit", grid);
-  gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>
-      <<<dim3((unsigned)grid), dim3(256), T::LDS_FLOATS * sizeof(float), stream()>>>(p);
-  TFHIP_CHECK_LAUNCH();
+  note_kernel("gemm_kernel<%d, %d, %d, %d, %d, %d, %d>", BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND);
+  TFHIP_LAUNCH((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>
+                <<<dim3((unsigned)grid), dim3(256), T::LDS_FLOATS * sizeof(float), stream()>>>(p)));
   return kOk;
 }
 

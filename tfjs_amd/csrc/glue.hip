@@ -99,11 +99,13 @@ int tfhip_add(const float *a, const int64_t *a_strides, const float *b, const in
   const bool aligned = reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(out) % 16 == 0;
   if (dense && aligned && total % 4 == 0) {
-    add_same_shape<<<grid_for(total / 4), 256, 0, stream()>>>((const float4 *)a, (const float4 *)b, (float4 *)out, total / 4);
+    note_kernel("add_same_shape");
+    TFHIP_LAUNCH((add_same_shape<<<grid_for(total / 4), 256, 0, stream()>>>((const float4 *)a, (const float4 *)b,
+                                                                          (float4 *)out, total / 4)));
   } else {
-    add_broadcast<<<grid_for(total), 256, 0, stream()>>>(p);
+    note_kernel("add_broadcast");
+    TFHIP_LAUNCH((add_broadcast<<<grid_for(total), 256, 0, stream()>>>(p)));
   }
-  TFHIP_CHECK_LAUNCH();
   return kOk;
 }
 
@@ -113,8 +115,8 @@ int tfhip_mean_hw(const float *x, float *y, int64_t batch, int64_t h, int64_t w,
   if (batch * c == 0) return kOk;
   TFHIP_CHECK_RANGE(x, batch * h * w * c, 4, "x");
   TFHIP_CHECK_RANGE(y, batch * c, 4, "y");
-  mean_hw<<<grid_for(batch * c), 256, 0, stream()>>>(x, y, batch, h * w, c);
-  TFHIP_CHECK_LAUNCH();
+  note_kernel("mean_hw");
+  TFHIP_LAUNCH((mean_hw<<<grid_for(batch * c), 256, 0, stream()>>>(x, y, batch, h * w, c)));
   return kOk;
 }
 

@@ -37,6 +37,8 @@ struct Runtime {
 Runtime g;
 std::mutex g_mutex;
 thread_local char g_error[1024] = "";
+char g_kernel[256] = "";
+int g_repeat = 1;
 
 // Size classes: eight per power of two, at least 256 bytes.
 size_t class_size(size_t bytes) {
@@ -66,6 +68,15 @@ int fail(int code, const char *fmt, ...) {
   va_end(ap);
   return code;
 }
+
+void note_kernel(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_kernel, sizeof g_kernel, fmt, ap);
+  va_end(ap);
+}
+
+int launch_repeat() { return g_repeat; }
 
 bool initialised() { return g.ready; }
 hipStream_t stream() { return g.stream; }
@@ -283,6 +294,17 @@ int tfhip_download(void *host, const void *src, size_t src_offset, size_t bytes)
     memcpy(h + done, g.staging[b], chunk);
     done += chunk;
   }
+  return kOk;
+}
+
+int tfhip_set_launch_repeat(int n) {
+  if (n < 1 || n > 100000) return fail(kBadArgument, "tfhip_set_launch_repeat: %d not in 1..100000", n);
+  g_repeat = n;
+  return kOk;
+}
+
+int tfhip_last_kernel(char *name, size_t name_len) {
+  if (name && name_len) snprintf(name, name_len, "%s", g_kernel);
   return kOk;
 }
 

@@ -205,14 +205,10 @@ DTYPE_VALUE_SIZE_MAP = {"float32": 4, "float16": 2, "int32": 4, "uint16": 2, "ui
                         "complex64": 8}
 
 
-def decode_weights(buffer, specs):
-    """decodeWeights (tfjs-core/src/io/io_utils.ts:119-292) with the dequantize
-    step on the GPU: the whole weight buffer is uploaded once, each quantized
-    entry is expanded by a kernel reading at its byte offset, and plain float32 /
-    int32 / bool entries are returned from the host bytes. Returns
-    {name: ndarray}; error messages follow the reference's."""
-    init()
-    raw = np.frombuffer(bytes(buffer), dtype=np.uint8)
+def _decode_plan(specs):
+    """Validates the manifest entries as decodeWeight does
+    (tfjs-core/src/io/io_utils.ts:196-216, :248-250, :288-290) and returns
+    [(name, dtype, shape, size, byte offset, quantization or None)], total bytes."""
     plan, offset = [], 0
     for spec in specs:
         name, dtype, shape = spec["name"], spec["dtype"], list(spec["shape"])
@@ -241,22 +237,54 @@ def decode_weights(buffer, specs):
             nbytes = size * DTYPE_VALUE_SIZE_MAP[dtype]
             plan.append((name, dtype, shape, size, offset, None))
         offset += nbytes
-    out = {}
+    return plan, offset
+
+
+def decode_weights_to_device(buffer, specs):
+    """The dequantize-on-load path with everything staying on the GPU: the whole
+    weight buffer is uploaded once, each quantized entry is expanded by one
+    kernel reading at its byte offset inside that upload, plain entries are
+    copied from the host bytes. Returns {name: (DeviceBuffer, shape)} holding
+    float32 / int32 values (bool entries as bytes)."""
+    init()
+    raw = np.frombuffer(bytes(buffer), dtype=np.uint8)
+    plan, total = _decode_plan(specs)
+    if total > raw.size:
+        raise ValueError("weight buffer holds %d bytes, the manifest needs %d" % (raw.size, total))
     lib = load_library()
-    with DeviceBuffer.from_numpy(raw) as dq:
+    out = {}
+    dq = DeviceBuffer.from_numpy(raw) if any(q is not None for *_, q in plan) else None
+    try:
         for name, dtype, shape, size, off, q in plan:
             if q is None:
-                np_dtype = {"float32": np.float32, "int32": np.int32, "bool": np.uint8}[dtype]
-                out[name] = np.frombuffer(raw[off:off + size * np.dtype(np_dtype).itemsize].tobytes(),
-                                          dtype=np_dtype).reshape(shape).copy()
-                continue
-            with DeviceBuffer(size * 4) as dout:
+                item = 1 if dtype == "bool" else 4
+                dst = DeviceBuffer(size * item)
+                dst.upload(raw[off:off + size * item])
+            else:
+                dst = DeviceBuffer(size * 4)
                 src = ctypes.c_void_p(dq.ptr + off)
                 if q["dtype"] == "float16":
-                    check(lib.tfhip_dequant_f16(src, size, dout.ptr))
+                    check(lib.tfhip_dequant_f16(src, size, dst.ptr))
                 else:
                     check(lib.tfhip_dequant_affine(src, 8 if q["dtype"] == "uint8" else 16, size,
-                                                   float(q["scale"]), float(q["min"]), dout.ptr,
+                                                   float(q["scale"]), float(q["min"]), dst.ptr,
                                                    int(dtype == "int32")))
-                out[name] = dout.download(np.float32 if dtype == "float32" else np.int32, size).reshape(shape)
+            out[name] = (dst, shape)
+    finally:
+        if dq is not None:
+            dq.free()
+    return out
+
+
+def decode_weights(buffer, specs):
+    """decodeWeights (tfjs-core/src/io/io_utils.ts:119-292) with the dequantize
+    step on the GPU; returns {name: ndarray}. Error messages follow the
+    reference's."""
+    dtypes = {s["name"]: s["dtype"] for s in specs}
+    np_dtype = {"float32": np.float32, "int32": np.int32, "bool": np.uint8}
+    out = {}
+    for name, (buf, shape) in decode_weights_to_device(buffer, specs).items():
+        size = int(np.prod(shape, dtype=np.int64)) if shape else 1
+        out[name] = buf.download(np_dtype[dtypes[name]], size).reshape(shape)
+        buf.free()
     return out

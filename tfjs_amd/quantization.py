@@ -1,14 +1,20 @@
-"""Producer side of the quantized weight format (TEST INFRASTRUCTURE ONLY).
+"""Producer side of the quantized weight format: what the converter writes and the
+dequantize-on-load path consumes.
 
-numpy restatement of tfjs-converter/python/tensorflowjs/quantization.py:
-quantize_weights :93-147, dequantize_weights :151-173 and
-_get_affine_quantization_range :175-216. The tests and the benchmark use it to
-make the uint8 / uint16 / float16 fixtures that the dequantize-on-load path
-consumes; the product never imports it.
+quantize_weights / dequantize_weights / get_affine_quantization_range follow
+tfjs-converter/python/tensorflowjs/quantization.py (:93-147, :151-173, :175-216);
+write_weights follows the byte layout and manifest of
+tfjs-converter/python/tensorflowjs/write_weights.py (:241-337): the entries of a
+group are concatenated in manifest order, quantized entries as their uint8 /
+uint16 / float16 bytes, and the stream is cut into shards of shard_size_bytes.
 
 All range arithmetic is float64, as in the reference (min/max are cast with
-astype(np.float64) at :123-124).
+astype(np.float64) at quantization.py:123-124).
 """
+import json
+import math
+import os
+
 import numpy as np
 
 
@@ -71,3 +77,39 @@ def dequantize_weights(data, metadata, original_dtype=np.float32):
     raise ValueError(
         "Invalid dtype %s for dequantization\nSupported dtypes are uint8, "
         "uint16, float16" % dtype.name)
+
+
+def write_weights(write_dir, weight_groups, quantization_dtype=None, shard_size_bytes=4 * 1024 * 1024):
+    """Writes `weight_groups` (a list of groups, each a list of
+    {'name': str, 'data': ndarray}) as .bin shards plus weights_manifest.json
+    under write_dir and returns the manifest. quantization_dtype (np.uint8,
+    np.uint16, np.float16 or None) is applied to every float32 / int32 entry it
+    supports, one (scale, min) pair per tensor."""
+    os.makedirs(write_dir, exist_ok=True)
+    manifest = []
+    for group_index, group in enumerate(weight_groups):
+        chunks, entries = [], []
+        for entry in group:
+            data = np.ascontiguousarray(entry["data"])
+            spec = {"name": entry["name"], "shape": list(data.shape), "dtype": data.dtype.name}
+            quantizable = quantization_dtype is not None and (
+                data.dtype == np.float32 or (data.dtype == np.int32 and quantization_dtype != np.float16))
+            if quantizable:
+                q, meta = quantize_weights(data, quantization_dtype)
+                spec["quantization"] = dict({"dtype": np.dtype(quantization_dtype).name}, **meta)
+                data = q
+            chunks.append(data.tobytes())
+            entries.append(spec)
+        stream = b"".join(chunks)
+        shard = shard_size_bytes or max(1, len(stream))
+        num_shards = max(1, int(math.ceil(len(stream) / float(shard))))
+        paths = []
+        for i in range(num_shards):
+            name = "group%d-shard%dof%d.bin" % (group_index + 1, i + 1, num_shards)
+            with open(os.path.join(write_dir, name), "wb") as f:
+                f.write(stream[i * shard:(i + 1) * shard])
+            paths.append(name)
+        manifest.append({"paths": paths, "weights": entries})
+    with open(os.path.join(write_dir, "weights_manifest.json"), "w") as f:
+        json.dump(manifest, f)
+    return manifest
