@@ -155,6 +155,22 @@ def bench_model(model_dir, steps, warmup):
                 symbols=symbols)
 
 
+def bench_model_node(model_dir, steps, warmup):
+    """The headline measurement: MobileNetV2 through the tfjs API in Node on the
+    hip backend (KernelBackend + kernel configs + N-API addon). Returns the
+    script's JSON, or None when Node or the addon is not available."""
+    node = shutil.which("node")
+    script = os.path.join(ROOT, "tfjs_amd", "js", "bench", "mobilenet_bench.js")
+    addon = os.path.join(ROOT, "tfjs_amd", "lib", "tfjs_hip.node")
+    if not (node and os.path.exists(addon)):
+        return None
+    proc = subprocess.run([node, script, model_dir, str(BATCH), str(steps), str(warmup)], stdout=subprocess.PIPE,
+                          stderr=subprocess.PIPE, text=True, timeout=900)
+    if proc.returncode != 0:
+        raise RuntimeError("node benchmark failed:\n%s" % proc.stderr[-3000:])
+    return json.loads(proc.stdout.strip().splitlines()[-1])
+
+
 def bench_kernels():
     """One line per benchmark configuration: its kernel at its shape."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
@@ -309,19 +325,23 @@ def main():
     model_dir = tempfile.mkdtemp(prefix="tfjs_hip_mobilenet_")
     try:
         workloads.write_model(model_dir, workloads.mobilenet_v2_weights(seed=3), np.uint8)
+        js = bench_model_node(model_dir, args.steps, args.warmup)
         m = bench_model(model_dir, args.steps, args.warmup)
         cpu = None if args.no_cpu_baseline else cpu_baseline(model_dir)
     finally:
         shutil.rmtree(model_dir, ignore_errors=True)
     kernels = None if args.no_kernels else bench_kernels()
+    ms_per_step = js["ms_per_step"] if js else m["ms_per_step"]
+    host = ("node %s, tfjs API -> KernelBackend 'hip' -> N-API addon -> C ABI (tfjs-core: %s)" % (js["node"], js["core"])
+            if js else "python/ctypes over the C ABI (node or the addon not found)")
     line = {
         "metric": "MobileNetV2 b32 images/s + fused-op TFLOP/s & % of roofline, 1 MI355X",
-        "value": round(BATCH / (m["ms_per_step"] * 1e-3), 1),
+        "value": round(BATCH / (ms_per_step * 1e-3), 1),
         "unit": "images/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(m["ms_per_step"], 4),
+        "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -329,9 +349,11 @@ def main():
         "data": "synthetic",
         "config": {"workload": "MobileNetV2 1.0/224, batch 32, NHWC fp32, uint8-quantized random-init weights "
                                "dequantized on load (benchmark configuration 4)", "batch": BATCH,
-                   "host": "python/ctypes over the C ABI", "device": info["arch"], "cus": info["cus"]},
+                   "host": host, "device": info["arch"], "cus": info["cus"]},
+        "weights_load_ms": round(js["load_ms"], 2) if js else None,
+        "python_host_ms_per_step": round(m["ms_per_step"], 4),
         "kernel_ms_per_step": round(m["kernel_ms_per_step"], 4),
-        "tflops_model": round(BATCH * workloads.mobilenet_v2_flops_per_image() / (m["ms_per_step"] * 1e-3) / 1e12, 3),
+        "tflops_model": round(BATCH * workloads.mobilenet_v2_flops_per_image() / (ms_per_step * 1e-3) / 1e12, 3),
         "roofline": m["roofline"],
         "cpu_baseline": cpu,
         "symbols": m["symbols"],

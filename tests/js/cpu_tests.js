@@ -1,0 +1,243 @@
+'use strict';
+/**
+ * CPU-tier Node tests (no GPU): the JavaScript oracle against the reference's
+ * golden vectors, the offline tfjs-core stand-in's engine semantics, and the
+ * storage logic of HipBackend over a fake addon.
+ */
+process.env.TFJS_HIP_ADDON = require('path').join(__dirname, 'fake_addon.js');
+process.env.TFJS_HIP_FORCE_STANDIN = '1';
+const h = require('./harness');
+const golden = require('./golden_cases');
+const cpu = require('../../oracle/js/backend_cpu');
+const oracleDecode = require('../../oracle/js/decode_weights');
+const hip = require('../../tfjs_amd/js/index');
+
+const tf = cpu.tf;
+cpu.register();
+h.assert(tf === hip.tf, 'one tfjs-core instance');
+
+function useBackend(name) {
+  h.assert(tf.engine().setBackend(name) === true, `setBackend(${name})`);
+}
+
+// ---- oracle vs golden vectors ---------------------------------------------------
+golden.FILES.forEach(file => {
+  h.loadGolden(file).cases.forEach(c => {
+    h.test(`oracle ${file} :: ${c.name} @${c.source.split(':').pop()}`, () => {
+      useBackend('cpu');
+      tf.tidy(() => {
+        const out = golden.runCase(tf, c);
+        if (c.expected.shape != null) {
+          h.assertEqual(out.shape, c.expected.shape, 'shape');
+        }
+        h.assertClose(out.dataSync(), c.expected.values);
+      });
+    });
+  });
+});
+
+h.loadGolden('conv_util.json').cases.forEach(c => {
+  h.test(`standin computeConv2DInfo :: ${c.name} @${c.source.split(':').pop()}`, () => {
+    const a = c.args;
+    const info = tf.backend_util.computeConv2DInfo(
+        a.inShape, a.filterShape, a.strides, a.dilations, a.pad, a.roundingMode == null ? undefined : a.roundingMode,
+        !!a.depthwise, a.dataFormat || 'channelsLast');
+    Object.keys(c.expected).forEach(k => {
+      let got = info;
+      k.split('.').forEach(part => got = got[part]);
+      h.assertEqual(got, c.expected[k], k);
+    });
+  });
+});
+
+const wd = JSON.parse(require('fs').readFileSync(require('path').join(__dirname, '..', 'golden', 'weights_decode.json')));
+wd.decode_cases.forEach(c => {
+  h.test(`oracle decodeWeights :: ${c.name}`, () => {
+    const out = oracleDecode.decodeWeightsToArrays(new Uint8Array(c.bytes).buffer, c.specs);
+    Object.keys(c.expected).forEach(name => {
+      const e = c.expected[name];
+      h.assert((e.dtype === 'int32') === (out[name] instanceof Int32Array), 'dtype');
+      if (e.close) {
+        h.assertClose(out[name], e.close);
+      } else {
+        h.assertEqual(Array.from(out[name]), e.equal);
+      }
+    });
+  });
+});
+wd.float16_cases.forEach(c => {
+  h.test(`oracle float16 :: ${c.name}`, () => {
+    const f32 = oracleDecode.getFloat16Decoder()(new Uint16Array(c.half_bits));
+    if (c.expected) {
+      const special = {NaN: NaN, Infinity: Infinity, '-Infinity': -Infinity, '0': 0, '-0': -0};
+      c.expected.forEach((s, i) => h.assert(Object.is(f32[i], special[s]), `${f32[i]} vs ${s}`));
+    } else {
+      c.expected_close_2_digits.forEach((v, i) => h.assert(Math.abs(f32[i] - v) < 0.005));
+    }
+  });
+});
+
+// ---- engine stand-in semantics (tfjs-core/src/engine_test.ts) ---------------------
+h.test('engine: unknown backend and unknown kernel throw the reference errors', () => {
+  h.assertThrows(() => tf.engine().setBackend('nope'), /Backend name 'nope' not found in registry/);
+  useBackend('cpu');
+  h.assertThrows(() => tf.engine().runKernel('NoSuchKernel', {}, {}),
+                 /Kernel 'NoSuchKernel' not registered for backend 'cpu'/);
+});
+
+h.test('engine: registerBackend twice returns false; failing factory is skipped by priority order', () => {
+  h.assert(tf.registerBackend('cpu', () => null) === false);
+  tf.registerBackend('broken', () => { throw new Error('boom'); }, 100);
+  const warn = console.warn;
+  console.warn = () => {};
+  try {
+    h.assert(tf.engine().setBackend('broken') === false, 'failing factory -> false');
+    tf.engine().backendInstance = null;
+    tf.engine().backendName = null;
+    h.assert(tf.engine().backend != null, 'next factory by priority is used');
+    h.assert(tf.getBackend() !== 'broken');
+  } finally {
+    console.warn = warn;
+    tf.removeBackend('broken');
+  }
+});
+
+h.test('engine: async backend factory resolves through setBackend', async () => {
+  tf.registerBackend('asynccpu', () => Promise.resolve(new cpu.OracleBackendCPU()), 0);
+  const ok = await tf.setBackend('asynccpu');
+  h.assert(ok === true);
+  tf.removeBackend('asynccpu');
+  useBackend('cpu');
+});
+
+h.test('engine: IS_TEST leak check flags a kernel that leaks a data id', () => {
+  useBackend('cpu');
+  tf.env().set('IS_TEST', true);
+  tf.registerKernel({
+    kernelName: 'Leaky', backendName: 'cpu',
+    kernelFunc: ({backend}) => {
+      backend.makeTensorInfo([1], 'float32', new Float32Array(1));   // never disposed
+      return backend.makeTensorInfo([1], 'float32', new Float32Array(1));
+    }
+  });
+  try {
+    h.assertThrows(() => tf.engine().runKernel('Leaky', {}, {}),
+                   /Backend 'cpu' has an internal memory leak \(1 data ids\) after running 'Leaky'/);
+    // the oracle's own fused kernels dispose their intermediates
+    tf.tidy(() => tf.fused.matMul({a: tf.tensor([[1, 2]]), b: tf.tensor([[1], [1]]), bias: tf.tensor([1]), activation: 'relu'}).dataSync());
+  } finally {
+    tf.env().set('IS_TEST', false);
+    tf.unregisterKernel('Leaky', 'cpu');
+  }
+});
+
+h.test('engine: tidy disposes intermediates, keeps the result; reshape aliases the buffer', () => {
+  useBackend('cpu');
+  const before = tf.memory().numTensors, ids = tf.backend().numDataIds();
+  const y = tf.tidy(() => {
+    const a = tf.tensor([1, 2, 3, 4], [2, 2]);
+    const r = tf.reshape(a, [4]);
+    h.assert(r.dataId === a.dataId, 'Reshape returns the same dataId');
+    h.assertEqual(tf.backend().refCount(a.dataId), 2);
+    return tf.add(r, r);
+  });
+  h.assertEqual(tf.memory().numTensors, before + 1);
+  h.assertEqual(tf.backend().numDataIds(), ids + 1);
+  h.assertEqual(Array.from(y.dataSync()), [2, 4, 6, 8]);
+  y.dispose();
+  h.assertEqual(tf.backend().numDataIds(), ids);
+});
+
+// ---- HipBackend storage over the fake addon ---------------------------------------
+h.test('hip storage: write/read round trip, refCounts, disposeData', () => {
+  useBackend('hip');
+  const backend = tf.backend();
+  h.assert(backend instanceof hip.HipBackend);
+  const ids0 = backend.numDataIds(), live0 = backend.memory().numDeviceBuffers;
+  const t = tf.tensor([1.5, -2, 3], [3]);
+  h.assertEqual(backend.numDataIds(), ids0 + 1);
+  h.assertEqual(Array.from(t.dataSync()), [1.5, -2, 3]);
+  const i = tf.tensor([1, 2, 3], [3], 'int32');
+  h.assert(i.dataSync() instanceof Int32Array);
+  const r = tf.reshape(t, [3, 1]);
+  h.assertEqual(backend.refCount(t.dataId), 2);
+  t.dispose();
+  h.assertEqual(backend.numDataIds(), ids0 + 2, 'buffer survives while the alias lives');
+  h.assertEqual(Array.from(r.dataSync()), [1.5, -2, 3]);
+  r.dispose();
+  i.dispose();
+  h.assertEqual(backend.numDataIds(), ids0);
+  h.assertEqual(backend.memory().numDeviceBuffers, live0);
+  h.assertEqual(backend.disposeData({}), true, 'unknown dataId is reported as released');
+});
+
+h.test('hip storage: tensors move between backends with their refCount (engine.moveData)', () => {
+  useBackend('cpu');
+  const cpuBackend = tf.backend();
+  const a = tf.tensor([1, 2, 3, 4], [2, 2]);
+  const alias = tf.reshape(a, [4]);
+  const cpuIds = cpuBackend.numDataIds();
+  useBackend('hip');
+  const hipBackend = tf.backend();
+  const hipIds = hipBackend.numDataIds();
+  tf.env().set('IS_TEST', true);
+  try {
+    // touching the cpu-resident tensor from a hip kernel migrates it
+    const out = tf.add(alias, alias);
+    h.assertEqual(cpuBackend.numDataIds(), cpuIds - 1);
+    h.assertEqual(hipBackend.numDataIds(), hipIds + 2);
+    h.assertEqual(hipBackend.refCount(a.dataId), 2, 'refCount carried over');
+    h.assertEqual(Array.from(a.dataSync()), [1, 2, 3, 4], 'values uploaded on move');
+    out.dispose();
+  } finally {
+    tf.env().set('IS_TEST', false);
+  }
+  a.dispose();
+  alias.dispose();
+  h.assertEqual(hipBackend.numDataIds(), hipIds);
+});
+
+h.test('hip kernels: argument checks happen on the host before any launch', () => {
+  useBackend('hip');
+  const x = tf.tensor(new Float32Array(2 * 4 * 4 * 3), [2, 4, 4, 3]);
+  const w = tf.tensor(new Float32Array(3 * 3 * 3 * 8), [3, 3, 3, 8]);
+  h.assertThrows(() => tf.fused.conv2d({x, filter: w, strides: 1, pad: 'same', bias: tf.tensor([1, 2, 3])}),
+                 /Operands could not be broadcast together/);
+  h.assertThrows(() => tf.fused.conv2d({x, filter: w, strides: 1, pad: 'same', dimRoundingMode: 'floor'}),
+                 /pad must be an integer when using dimRoundingMode floor but got pad same/);
+  h.assertThrows(() => tf.fused.matMul({a: tf.tensor([[1, 2, 3]]), b: tf.tensor([[1, 2]])}),
+                 /inner shapes \(3\) and \(1\)/);
+  h.assertThrows(() => tf.fused.matMul({a: tf.tensor([[1, 2]]), b: tf.tensor([[1], [2]]), activation: 'swish'}),
+                 /Activation swish has not been implemented for the hip backend/);
+  h.assertThrows(() => tf.mean(x, [0]), /global average pool only/);
+  const xi = tf.tensor([1, 2, 3, 4], [1, 2, 2, 1], 'int32');
+  h.assertThrows(() => tf.engine().runKernel('FusedConv2D', {x: xi, filter: tf.tensor([1], [1, 1, 1, 1])},
+                                             {strides: 1, pad: 'valid', dataFormat: 'NHWC', dilations: [1, 1]}),
+                 /non-float32 tensors is not supported/);
+  const calls = require('./fake_addon').calls.length;
+  const y = tf.fused.conv2d({x, filter: w, strides: 2, pad: 'same', bias: tf.tensor(new Float32Array(8)), activation: 'relu6'});
+  h.assertEqual(y.shape, [2, 2, 2, 8]);
+  h.assertEqual(require('./fake_addon').calls.length, calls + 1);
+});
+
+h.test('hip decodeWeights: reference error messages, plain entries pass through', () => {
+  useBackend('hip');
+  h.assertThrows(() => hip.decodeWeights(new ArrayBuffer(1), [{name: 'w', dtype: 'float32', shape: [1], quantization: {dtype: 'uint8', scale: 1}}]),
+                 /doesn't have corresponding metadata min and scale/);
+  h.assertThrows(() => hip.decodeWeights(new ArrayBuffer(2), [{name: 'w', dtype: 'int32', shape: [1], quantization: {dtype: 'float16'}}]),
+                 /which only supports weights of type float32 not int32/);
+  h.assertThrows(() => hip.decodeWeights(new ArrayBuffer(1), [{name: 'w', dtype: 'float32', shape: [1], quantization: {dtype: 'int8', scale: 1, min: 0}}]),
+                 /unknown quantization dtype int8/);
+  h.assertThrows(() => hip.decodeWeights(new ArrayBuffer(2), [{name: 'x', dtype: 'int16', shape: [1]}]),
+                 /Unsupported dtype in weight 'x': int16/);
+  const bytes = new Uint8Array(1 + 8);
+  new Uint8Array(bytes.buffer).set([7], 0);
+  new Uint8Array(bytes.buffer).set(new Uint8Array(new Float32Array([1.5, -2]).buffer), 1);
+  const out = hip.decodeWeights(bytes.buffer, [{name: 'b', dtype: 'bool', shape: [1]}, {name: 'f', dtype: 'float32', shape: [2]}]);
+  h.assertEqual(Array.from(out.f.dataSync()), [1.5, -2]);
+  h.assertEqual(Array.from(out.b.dataSync()), [7]);
+  useBackend('cpu');
+  h.assertThrows(() => hip.decodeWeights(new ArrayBuffer(0), []), /needs the 'hip' backend to be active/);
+});
+
+h.run('node cpu tests');

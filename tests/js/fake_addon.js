@@ -1,0 +1,60 @@
+'use strict';
+/**
+ * Test double for the N-API addon (selected with TFJS_HIP_ADDON): "device"
+ * buffers are host ArrayBuffers keyed by made-up addresses, and the kernel
+ * entry points only record that they were called. It lets the storage logic of
+ * HipBackend (dataIds, refCounts, moves, disposal, leak accounting) run in the
+ * CPU-only test tier. It computes nothing.
+ */
+let next = 0x1000;
+const blocks = new Map();
+const calls = [];
+let inited = false;
+
+function need(ptr) {
+  if (!blocks.has(ptr)) {
+    throw new Error(`fake addon: ${ptr} is not a live block`);
+  }
+  return blocks.get(ptr);
+}
+
+module.exports = {
+  calls,
+  init() { inited = true; },
+  shutdown() { inited = false; blocks.clear(); },
+  deviceInfo() { return {name: 'fake', arch: 'gfx950:fake', cus: 256, clockKhz: 2400000, hbmBytes: 1 << 30}; },
+  alloc(bytes) {
+    if (!inited) {
+      throw new Error('fake addon: init has not been called');
+    }
+    const ptr = next;
+    next += Math.max(256, Math.ceil(bytes / 256) * 256);
+    blocks.set(ptr, new Uint8Array(bytes));
+    return ptr;
+  },
+  free(ptr) { need(ptr); blocks.delete(ptr); },
+  upload(ptr, offset, data) {
+    need(ptr).set(new Uint8Array(data.buffer, data.byteOffset, data.byteLength), offset);
+  },
+  download(ptr, offset, out) {
+    new Uint8Array(out.buffer, out.byteOffset, out.byteLength).set(need(ptr).subarray(offset, offset + out.byteLength));
+    return out;
+  },
+  sync() {},
+  memoryInfo() {
+    let bytes = 0;
+    blocks.forEach(b => bytes += b.byteLength);
+    return {live: blocks.size, liveBytes: bytes, pooledBytes: 0};
+  },
+  eventRecord() {},
+  eventElapsed() { return 0; },
+  setLaunchRepeat() {},
+  lastKernel() { return 'fake'; },
+  fusedMatMul() { calls.push('fusedMatMul'); },
+  fusedConv2D() { calls.push('fusedConv2D'); },
+  fusedDepthwiseConv2D() { calls.push('fusedDepthwiseConv2D'); },
+  dequantAffine() { calls.push('dequantAffine'); },
+  dequantF16() { calls.push('dequantF16'); },
+  add() { calls.push('add'); },
+  meanHW() { calls.push('meanHW'); }
+};

@@ -1,0 +1,200 @@
+'use strict';
+/**
+ * GPU-tier Node tests: the hip backend driven through the tfjs API, compared
+ * with the JavaScript oracle (backend 'cpu') on the same typed arrays.
+ * Bar: dequantized weights bit-exact; float32 outputs within
+ * max|d| <= 1e-3 * max(1, |ref|).
+ */
+const fs = require('fs');
+const os = require('os');
+const path = require('path');
+const h = require('./harness');
+const golden = require('./golden_cases');
+const cpu = require('../../oracle/js/backend_cpu');
+const oracleDecode = require('../../oracle/js/decode_weights');
+const hip = require('../../tfjs_amd/js/index');
+const mobilenet = require('../../tfjs_amd/js/models/mobilenet_v2');
+
+const tf = cpu.tf;
+cpu.register();
+
+function on(name, fn) {
+  h.assert(tf.engine().setBackend(name) === true, `setBackend(${name})`);
+  return tf.tidy(fn);
+}
+
+/** Runs fn(tf) on both backends from the same host arrays; returns [hipData, cpuData, shape]. */
+function both(fn) {
+  const a = on('hip', () => {
+    const y = fn();
+    return {data: y.dataSync(), shape: y.shape};
+  });
+  const b = on('cpu', () => {
+    const y = fn();
+    return {data: y.dataSync(), shape: y.shape};
+  });
+  h.assertEqual(a.shape, b.shape, 'shape');
+  return [a.data, b.data];
+}
+
+golden.FILES.forEach(file => {
+  h.loadGolden(file).cases.forEach(c => {
+    h.test(`hip ${file} :: ${c.name} @${c.source.split(':').pop()}`, () => {
+      on('hip', () => {
+        tf.env().set('IS_TEST', true);
+        try {
+          const out = golden.runCase(tf, c);
+          if (c.expected.shape != null) {
+            h.assertEqual(out.shape, c.expected.shape, 'shape');
+          }
+          h.assertClose(out.dataSync(), c.expected.values);
+        } finally {
+          tf.env().set('IS_TEST', false);
+        }
+      });
+    });
+  });
+});
+
+h.test('config 1: _FusedMatMul [1,256,512] x [1,512,512] + bias, relu', () => {
+  const r = h.rng(11);
+  const a = r.uniform(256 * 512, -1, 1), b = r.uniform(512 * 512, -1, 1), bias = r.uniform(512, -1, 1);
+  const [got, want] = both(() => tf.fused.matMul({a: tf.tensor(a, [1, 256, 512]), b: tf.tensor(b, [1, 512, 512]),
+                                                   bias: tf.tensor(bias, [512]), activation: 'relu'}));
+  h.assertParity(got, want);
+});
+
+h.test('config 2: stem conv 3x3/2 and 1x1 pointwise conv', () => {
+  const r = h.rng(12);
+  const x = r.uniform(224 * 224 * 3, 0, 1), w = r.uniform(3 * 3 * 3 * 32, -0.4, 0.4), bias = r.uniform(32, -0.1, 0.1);
+  let [got, want] = both(() => tf.fused.conv2d({x: tf.tensor(x, [1, 224, 224, 3]), filter: tf.tensor(w, [3, 3, 3, 32]),
+                                                 strides: 2, pad: 'same', bias: tf.tensor(bias, [32]), activation: 'relu6'}));
+  h.assertParity(got, want);
+  const x2 = r.uniform(2 * 56 * 56 * 144, 0, 1), w2 = r.uniform(144 * 24, -0.2, 0.2), b2 = r.uniform(24, -0.1, 0.1);
+  [got, want] = both(() => tf.fused.conv2d({x: tf.tensor(x2, [2, 56, 56, 144]), filter: tf.tensor(w2, [1, 1, 144, 24]),
+                                             strides: 1, pad: 'same', bias: tf.tensor(b2, [24])}));
+  h.assertParity(got, want);
+});
+
+h.test('config 3: depthwise 3x3 stride 1 and 2, relu6', () => {
+  const r = h.rng(13);
+  const x = r.uniform(2 * 112 * 112 * 96, 0, 1), w = r.uniform(9 * 96, -0.7, 0.7), bias = r.uniform(96, -0.1, 0.1);
+  [1, 2].forEach(stride => {
+    const [got, want] = both(() => tf.fused.depthwiseConv2d({
+      x: tf.tensor(x, [2, 112, 112, 96]), filter: tf.tensor(w, [3, 3, 96, 1]), strides: stride, pad: 'same',
+      bias: tf.tensor(bias, [96]), activation: 'relu6'}));
+    h.assertParity(got, want);
+  });
+});
+
+h.test('config 5: batched matmuls with transposeB and rank-4 operands', () => {
+  const r = h.rng(15);
+  const q = r.uniform(2 * 3 * 32 * 16, -1, 1), k = r.uniform(2 * 3 * 32 * 16, -1, 1);
+  let [got, want] = both(() => tf.matMul(tf.tensor(q, [2, 3, 32, 16]), tf.tensor(k, [2, 3, 32, 16]), false, true));
+  h.assertParity(got, want);
+  const a = r.uniform(64 * 96, -1, 1), w = r.uniform(96 * 40, -0.05, 0.05), bias = r.uniform(40, -0.05, 0.05);
+  [got, want] = both(() => tf.fused.matMul({a: tf.tensor(a, [64, 96]), b: tf.tensor(w, [96, 40]), bias: tf.tensor(bias, [40]), activation: 'relu'}));
+  h.assertParity(got, want);
+});
+
+h.test('decodeWeights on the GPU is bit-identical to the JavaScript decoder (uint8, uint16, float16, int32, unaligned)', () => {
+  const r = h.rng(21);
+  const n8 = 1001, n16 = 777, nh = 4099, ni = 13, nf = 5;
+  const bytes = new Uint8Array(n8 + 2 * n16 + 2 * nh + ni + 4 * nf);
+  for (let i = 0; i < bytes.length; i++) {
+    bytes[i] = (Math.imul(i + 7, 2654435761) >>> 24) & 0xff;
+  }
+  const plain = r.uniform(nf, -1, 1);
+  bytes.set(new Uint8Array(plain.buffer), n8 + 2 * n16 + 2 * nh + ni);
+  const specs = [
+    {name: 'a', dtype: 'float32', shape: [n8], quantization: {dtype: 'uint8', scale: 0.00123, min: -0.157}},
+    {name: 'b', dtype: 'float32', shape: [n16], quantization: {dtype: 'uint16', scale: 3.3e-5, min: -1.07}},
+    {name: 'c', dtype: 'float32', shape: [nh], quantization: {dtype: 'float16'}},
+    {name: 'd', dtype: 'int32', shape: [ni], quantization: {dtype: 'uint8', scale: 0.5, min: -20.25}},
+    {name: 'e', dtype: 'float32', shape: [nf]}
+  ];
+  const want = oracleDecode.decodeWeightsToArrays(bytes.buffer, specs);
+  on('hip', () => {
+    const got = hip.decodeWeights(bytes.buffer, specs);
+    specs.forEach(s => {
+      h.assertEqual(got[s.name].shape, s.shape);
+      h.assertEqual(got[s.name].dtype, s.dtype);
+      h.assertBitsEqual(got[s.name].dataSync(), want[s.name]);
+    });
+    // the same bytes split into shards decode identically
+    const parts = [bytes.slice(0, 500).buffer, bytes.slice(500, 3000).buffer, bytes.slice(3000).buffer];
+    const again = hip.decodeWeights(parts, specs);
+    specs.forEach(s => h.assertBitsEqual(again[s.name].dataSync(), want[s.name]));
+  });
+});
+
+h.test('float16 decode: all 65536 bit patterns', () => {
+  const all = new Uint16Array(65536);
+  for (let i = 0; i < 65536; i++) {
+    all[i] = i;
+  }
+  const specs = [{name: 'w', dtype: 'float32', shape: [65536], quantization: {dtype: 'float16'}}];
+  const want = oracleDecode.decodeWeightsToArrays(all.buffer, specs).w;
+  on('hip', () => h.assertBitsEqual(hip.decodeWeights(all.buffer, specs).w.dataSync(), want));
+});
+
+h.test('config 4: MobileNetV2 batch 2 through the tfjs API, uint8 weights dequantized on the GPU', () => {
+  const dir = process.env.TFJS_HIP_TEST_MODEL_DIR;
+  h.assert(dir && fs.existsSync(path.join(dir, 'weights_manifest.json')),
+           'TFJS_HIP_TEST_MODEL_DIR must hold a model written by tfjs_amd.workloads.write_model');
+  const m = mobilenet.readModel(dir);
+  const x = mobilenet.syntheticInput(2, 3);
+  const wantW = oracleDecode.decodeWeightsToArrays(m.buffer, m.specs);
+  h.assert(tf.engine().setBackend('hip') === true);
+  const wHip = hip.decodeWeights(m.buffer, m.specs);
+  m.specs.forEach(s => h.assertBitsEqual(wHip[s.name].dataSync(), wantW[s.name]));
+  const before = tf.backend().numDataIds();
+  tf.env().set('IS_TEST', true);
+  let got;
+  try {
+    got = tf.tidy(() => mobilenet.buildPredict(tf, wHip)(tf.tensor(x, [2, 224, 224, 3])).dataSync());
+  } finally {
+    tf.env().set('IS_TEST', false);
+  }
+  h.assertEqual(tf.backend().numDataIds(), before, 'no device buffers leaked by predict');
+  tf.dispose(wHip);
+  h.assert(tf.engine().setBackend('cpu') === true);
+  const wCpu = oracleDecode.decodeWeights(m.buffer, m.specs);
+  const want = tf.tidy(() => mobilenet.buildPredict(tf, wCpu)(tf.tensor(x, [2, 224, 224, 3])).dataSync());
+  tf.dispose(wCpu);
+  h.assertEqual(got.length, 2000);
+  h.assertParity(got, want);
+});
+
+h.test('backend: tensors migrate cpu <-> hip with values and refCounts; tf.time reports device ms', async () => {
+  h.assert(tf.engine().setBackend('cpu') === true);
+  const a = tf.tensor([1, 2, 3, 4], [2, 2]);
+  h.assert(tf.engine().setBackend('hip') === true);
+  const ids = tf.backend().numDataIds();
+  const y = tf.add(a, a);
+  h.assertEqual(tf.backend().numDataIds(), ids + 2);
+  h.assertEqual(Array.from(y.dataSync()), [2, 4, 6, 8]);
+  h.assertEqual(Array.from(await y.data()), [2, 4, 6, 8]);
+  const t = await tf.time(() => tf.add(y, y).dispose());
+  h.assert(t.kernelMs >= 0 && t.wallMs >= 0);
+  h.assert(tf.engine().setBackend('cpu') === true);
+  const z = tf.add(y, a);   // both now migrate back to cpu
+  h.assertEqual(Array.from(z.dataSync()), [3, 6, 9, 12]);
+  tf.dispose([a, y, z]);
+  h.assert(tf.engine().setBackend('hip') === true);
+  h.assertEqual(tf.backend().numDataIds(), ids);
+  const info = tf.backend().deviceInfo;
+  h.assert(/^gfx950/.test(info.arch), `arch ${info.arch}`);
+});
+
+h.test('native errors surface as thrown Errors, not faults', () => {
+  const addon = require('../../tfjs_amd/js/binding').addon;
+  h.assertThrows(() => addon.free(4096), /not a live block/);
+  const p = addon.alloc(64);
+  h.assertThrows(() => addon.fusedMatMul(p, p, p, 1, 1, 1024, 1024, 1024, 0, 0, null, null, 0, null, null, 0.2),
+                 /not inside a live device buffer/);
+  h.assertThrows(() => addon.dequantAffine(p, 0, 12, 4, 1, 0, p, 0), /bits must be 8 or 16/);
+  addon.free(p);
+});
+
+h.run('node gpu tests');

@@ -1,0 +1,195 @@
+'use strict';
+/**
+ * HipBackend: the KernelBackend of tfjs-backend-hip
+ * (contract: tfjs-core/src/backends/backend.ts:100-156).
+ *
+ * Storage follows MathBackendCPU (tfjs-backend-cpu/src/backend_cpu.ts:52-193)
+ * and BackendWasm (tfjs-backend-wasm/src/backend_wasm.ts:50-236): a
+ * DataStorage keyed by dataId objects holding {ptr, bytes, dtype, shape,
+ * refCount}, where ptr is a device buffer from the native library's pool.
+ *   write      new dataId, refCount 1, host values uploaded asynchronously
+ *   move       adopt a dataId that lived on another backend (upload, keep refCount)
+ *   read       Promise of readSync
+ *   readSync   stream sync + device->host copy into a fresh typed array
+ *   disposeData decrement; free the device buffer at 0 or when forced
+ * Kernels only enqueue work on the library's single stream; read / readSync
+ * are the sync points.
+ */
+const tf = require('./core');
+const {addon} = require('./binding');
+
+const BYTES = {float32: 4, int32: 4, bool: 1};
+
+function typedArrayFor(dtype, size) {
+  if (dtype === 'float32') {
+    return new Float32Array(size);
+  } else if (dtype === 'int32') {
+    return new Int32Array(size);
+  } else if (dtype === 'bool') {
+    return new Uint8Array(size);
+  }
+  throw new Error(`tfjs-backend-hip does not support dtype ${dtype}`);
+}
+
+class HipBackend extends tf.KernelBackend {
+  constructor(device) {
+    super();
+    addon.init(device == null ? 0 : device);
+    this.deviceInfo = addon.deviceInfo();
+    this.data = new tf.DataStorage(this, tf.engine());
+    this.nextEventSlot = 0;
+  }
+
+  nextDataId() {
+    return {id: HipBackend.nextId++};
+  }
+
+  /** Device buffer of `size` elements of `dtype`; registers a new dataId. */
+  allocate(shape, dtype, dataId) {
+    const size = tf.util.sizeFromShape(shape);
+    if (!(dtype in BYTES)) {
+      throw new Error(`tfjs-backend-hip does not support dtype ${dtype}`);
+    }
+    const bytes = size * BYTES[dtype];
+    const ptr = addon.alloc(Math.max(bytes, 1));
+    dataId = dataId || this.nextDataId();
+    this.data.set(dataId, {ptr, bytes, dtype, shape: shape.slice(), refCount: 1});
+    return dataId;
+  }
+
+  write(values, shape, dtype) {
+    const dataId = this.allocate(shape, dtype);
+    if (values != null) {
+      this.uploadValues(dataId, values);
+    }
+    return dataId;
+  }
+
+  uploadValues(dataId, values) {
+    const info = this.data.get(dataId);
+    let typed = values;
+    if (!ArrayBuffer.isView(values) ||
+        values.BYTES_PER_ELEMENT !== BYTES[info.dtype] ||
+        (info.dtype === 'float32' && !(values instanceof Float32Array)) ||
+        (info.dtype === 'int32' && !(values instanceof Int32Array))) {
+      typed = typedArrayFor(info.dtype, values.length);
+      typed.set(values);
+    }
+    if (typed.byteLength !== info.bytes) {
+      throw new Error(
+          `tfjs-backend-hip: ${typed.byteLength} bytes given for a tensor of ` +
+          `${info.bytes} bytes`);
+    }
+    if (info.bytes > 0) {
+      addon.upload(info.ptr, 0, typed);
+    }
+  }
+
+  move(dataId, values, shape, dtype, refCount) {
+    this.allocate(shape, dtype, dataId);
+    this.data.get(dataId).refCount = refCount;
+    if (values != null) {
+      this.uploadValues(dataId, values);
+    }
+  }
+
+  /** Registers a result buffer for a kernel: TensorInfo with a fresh dataId. */
+  makeOutput(shape, dtype) {
+    const dataId = this.allocate(shape, dtype || 'float32');
+    return {dataId, shape, dtype: dtype || 'float32'};
+  }
+
+  ptr(dataId) {
+    return this.data.get(dataId).ptr;
+  }
+
+  refCount(dataId) {
+    if (this.data.has(dataId)) {
+      return this.data.get(dataId).refCount;
+    }
+    return 0;
+  }
+
+  incRef(dataId) {
+    this.data.get(dataId).refCount++;
+  }
+
+  decRef(dataId) {
+    if (this.data.has(dataId)) {
+      this.data.get(dataId).refCount--;
+    }
+  }
+
+  numDataIds() {
+    return this.data.numDataIds();
+  }
+
+  readSync(dataId) {
+    const info = this.data.get(dataId);
+    const out = typedArrayFor(info.dtype, info.bytes / BYTES[info.dtype]);
+    if (info.bytes > 0) {
+      addon.download(info.ptr, 0, out);
+    }
+    return out;
+  }
+
+  read(dataId) {
+    return new Promise(resolve => resolve(this.readSync(dataId)));
+  }
+
+  disposeData(dataId, force) {
+    if (this.data.has(dataId)) {
+      const info = this.data.get(dataId);
+      info.refCount--;
+      if (!force && info.refCount > 0) {
+        return false;
+      }
+      addon.free(info.ptr);
+      this.data.delete(dataId);
+    }
+    return true;
+  }
+
+  disposeIntermediateTensorInfo(tensorInfo) {
+    this.disposeData(tensorInfo.dataId);
+  }
+
+  /** Device time of f() between two events on the library's stream. */
+  time(f) {
+    const a = this.nextEventSlot, b = this.nextEventSlot + 1;
+    this.nextEventSlot = (this.nextEventSlot + 2) % 4096;
+    addon.eventRecord(a);
+    f();
+    addon.eventRecord(b);
+    return Promise.resolve({kernelMs: addon.eventElapsed(a, b)});
+  }
+
+  timerAvailable() {
+    return true;
+  }
+
+  memory() {
+    const m = addon.memoryInfo();
+    return {
+      unreliable: false,
+      numDeviceBuffers: m.live,
+      numBytesInGPU: m.liveBytes,
+      numBytesInGPUPool: m.pooledBytes
+    };
+  }
+
+  floatPrecision() {
+    return 32;
+  }
+
+  epsilon() {
+    return 1e-7;
+  }
+
+  dispose() {
+    addon.shutdown();
+  }
+}
+HipBackend.nextId = 0;
+
+module.exports = {HipBackend, typedArrayFor, BYTES};

@@ -1,0 +1,69 @@
+'use strict';
+/**
+ * MobileNetV2 through the tfjs API on the hip backend, timed the reference's way
+ * (predict plus download of the result, e2e/benchmarks/benchmark_util.js:246-286).
+ *   node tfjs_amd/js/bench/mobilenet_bench.js MODEL_DIR BATCH STEPS WARMUP
+ * Prints one JSON line: ms_per_step (wall clock around STEPS steps, stream
+ * drained on both sides), load_ms (read + upload + GPU dequant of the weights),
+ * kernel_ms_per_step (device time between two events around the same steps).
+ */
+const hip = require('../index');
+const model = require('../models/mobilenet_v2');
+const {addon} = require('../binding');
+
+const tf = hip.tf;
+
+async function main() {
+  const modelDir = process.argv[2];
+  const batch = parseInt(process.argv[3] || '32', 10);
+  const steps = parseInt(process.argv[4] || '50', 10);
+  const warmup = parseInt(process.argv[5] || '5', 10);
+  await tf.setBackend('hip');
+  const t0 = tf.util.now();
+  const m = model.readModel(modelDir);
+  const weights = hip.decodeWeights(m.buffer, m.specs);
+  addon.sync();
+  const loadMs = tf.util.now() - t0;
+  const predict = model.buildPredict(tf, weights);
+  const x = tf.tensor(model.syntheticInput(batch, 3), [batch, 224, 224, 3]);
+  let checksum = 0;
+  const step = () => {
+    const y = predict(x);
+    const data = y.dataSync();
+    checksum = data[0];
+    y.dispose();
+  };
+  for (let i = 0; i < warmup; i++) {
+    step();
+  }
+  addon.sync();
+  addon.eventRecord(0);
+  const start = tf.util.now();
+  for (let i = 0; i < steps; i++) {
+    step();
+  }
+  addon.sync();
+  const wallMs = tf.util.now() - start;
+  addon.eventRecord(1);
+  const deviceMs = addon.eventElapsed(0, 1);
+  const mem = tf.memory();
+  console.log(JSON.stringify({
+    ms_per_step: wallMs / steps,
+    device_ms_per_step: deviceMs / steps,
+    load_ms: loadMs,
+    batch,
+    steps,
+    warmup,
+    checksum,
+    node: process.version,
+    core: tf.usingStandin ? 'standin' : '@tensorflow/tfjs-core',
+    device: tf.backend().deviceInfo,
+    num_tensors: mem.numTensors,
+    num_device_buffers: mem.numDeviceBuffers
+  }));
+}
+
+main().catch(e => {
+  console.error(e.stack || e.message);
+  process.exit(1);
+});

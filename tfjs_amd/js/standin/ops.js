@@ -1,0 +1,297 @@
+'use strict';
+/**
+ * Offline stand-in for the op wrappers that call the hot path
+ * (tfjs-core/src/ops/fused/{mat_mul,conv2d,depthwise_conv2d}.ts,
+ * ops/{mat_mul,conv2d,depthwise_conv2d,add,mean,reshape}.ts): argument
+ * defaults, the reshapes to the rank the kernels are handed, the validation
+ * that throws before any backend is reached, and ENGINE.runKernel with the
+ * kernel names and attribute objects of tfjs-core/src/kernel_names.ts.
+ * No gradients: every call takes the fused path.
+ */
+const {ENGINE, Tensor} = require('./engine');
+const {util, backend_util, broadcast_util} = require('./util');
+
+function inferShape(values) {
+  const shape = [];
+  let v = values;
+  while (Array.isArray(v) || ArrayBuffer.isView(v)) {
+    shape.push(v.length);
+    v = v[0];
+    if (ArrayBuffer.isView(values)) {
+      break;
+    }
+  }
+  return shape;
+}
+
+function flatten(values, out) {
+  if (Array.isArray(values)) {
+    for (let i = 0; i < values.length; i++) {
+      flatten(values[i], out);
+    }
+  } else {
+    out.push(values);
+  }
+  return out;
+}
+
+function toTypedArray(values, dtype) {
+  if (ArrayBuffer.isView(values)) {
+    if ((dtype === 'float32' && values instanceof Float32Array) ||
+        (dtype === 'int32' && values instanceof Int32Array) ||
+        (dtype === 'bool' && values instanceof Uint8Array)) {
+      return values;
+    }
+    values = Array.prototype.slice.call(values);
+  }
+  const flat = Array.isArray(values) ? flatten(values, []) : [values];
+  const out = util.getTypedArrayFromDType(dtype, flat.length);
+  for (let i = 0; i < flat.length; i++) {
+    out[i] = dtype === 'bool' ? (flat[i] ? 1 : 0) : flat[i];
+  }
+  return out;
+}
+
+function tensor(values, shape, dtype) {
+  dtype = dtype || 'float32';
+  const inferred = inferShape(values);
+  shape = shape || inferred;
+  const data = toTypedArray(values, dtype);
+  util.assert(
+      data.length === util.sizeFromShape(shape),
+      () => `Based on the provided shape, [${shape}], the tensor should have ` +
+          `${util.sizeFromShape(shape)} values but has ${data.length}`);
+  return ENGINE.makeTensor(data, shape, dtype);
+}
+
+function convertToTensor(x, argName, opName, dtype) {
+  if (x instanceof Tensor) {
+    return x;
+  }
+  if (x == null) {
+    throw new Error(
+        `Argument '${argName}' passed to '${opName}' must be a Tensor ` +
+        `or TensorLike, but got 'null'`);
+  }
+  return tensor(x, null, dtype || 'float32');
+}
+
+function assertFloat32(t, argName, opName) {
+  if (t.dtype !== 'float32') {
+    throw new Error(
+        `Argument '${argName}' passed to '${opName}' must be float32 ` +
+        `tensor, but got ${t.dtype} tensor`);
+  }
+}
+
+function reshape(x, shape) {
+  const $x = convertToTensor(x, 'x', 'reshape');
+  return ENGINE.runKernel('Reshape', {x: $x}, {shape});
+}
+
+function add(a, b) {
+  const $a = convertToTensor(a, 'a', 'add');
+  const $b = convertToTensor(b, 'b', 'add');
+  return ENGINE.runKernel('Add', {a: $a, b: $b});
+}
+
+function mean(x, axis, keepDims) {
+  const $x = convertToTensor(x, 'x', 'mean');
+  return ENGINE.runKernel(
+      'Mean', {x: $x}, {axis: axis == null ? null : axis, keepDims: !!keepDims});
+}
+
+/** tfjs-core/src/ops/mat_mul.ts:44-57 */
+function matMul(a, b, transposeA, transposeB) {
+  const $a = convertToTensor(a, 'a', 'matMul');
+  const $b = convertToTensor(b, 'b', 'matMul');
+  return ENGINE.runKernel(
+      'BatchMatMul', {a: $a, b: $b},
+      {transposeA: !!transposeA, transposeB: !!transposeB});
+}
+
+/** tfjs-core/src/ops/fused/mat_mul.ts:58-211 */
+function fusedMatMul(args) {
+  const transposeA = !!args.transposeA, transposeB = !!args.transposeB;
+  const activation = args.activation || 'linear';
+  const leakyreluAlpha = args.leakyreluAlpha == null ? 0.2 : args.leakyreluAlpha;
+  const $a = convertToTensor(args.a, 'a', 'fused matMul');
+  const $b = convertToTensor(args.b, 'b', 'fused matMul');
+  const aRank = $a.shape.length, bRank = $b.shape.length;
+  const innerShapeA = transposeA ? $a.shape[aRank - 2] : $a.shape[aRank - 1];
+  const innerShapeB = transposeB ? $b.shape[bRank - 1] : $b.shape[bRank - 2];
+  const outerShapeA = transposeA ? $a.shape[aRank - 1] : $a.shape[aRank - 2];
+  const outerShapeB = transposeB ? $b.shape[bRank - 2] : $b.shape[bRank - 1];
+  const batchDimA = util.sizeFromShape($a.shape.slice(0, -2));
+  const batchDimB = util.sizeFromShape($b.shape.slice(0, -2));
+  util.assert(
+      innerShapeA === innerShapeB,
+      () => `Error in fused matMul: inner shapes (${innerShapeA}) and (` +
+          `${innerShapeB}) of Tensors with shapes ${$a.shape} and ` +
+          `${$b.shape} and transposeA=${transposeA}` +
+          ` and transposeB=${transposeB} must match.`);
+  const outShapeOuterDims = broadcast_util.assertAndGetBroadcastShape(
+      $a.shape.slice(0, -2), $b.shape.slice(0, -2));
+  const outShape = outShapeOuterDims.concat([outerShapeA, outerShapeB]);
+  return ENGINE.tidy(() => {
+    const a3D = transposeA ? reshape($a, [batchDimA, innerShapeA, outerShapeA]) :
+                             reshape($a, [batchDimA, outerShapeA, innerShapeA]);
+    const b3D = transposeB ? reshape($b, [batchDimB, outerShapeB, innerShapeB]) :
+                             reshape($b, [batchDimB, innerShapeB, outerShapeB]);
+    let $bias;
+    if (args.bias != null) {
+      $bias = convertToTensor(args.bias, 'bias', 'fused matMul');
+      broadcast_util.assertAndGetBroadcastShape(outShape, $bias.shape);
+    }
+    let $prelu;
+    if (args.preluActivationWeights != null) {
+      $prelu = convertToTensor(
+          args.preluActivationWeights, 'prelu weights', 'fused matMul');
+    }
+    const res = ENGINE.runKernel(
+        '_FusedMatMul',
+        {a: a3D, b: b3D, bias: $bias, preluActivationWeights: $prelu},
+        {transposeA, transposeB, activation, leakyreluAlpha});
+    return reshape(res, outShape);
+  });
+}
+
+function convCommon(opDesc, kernelName, args, depthwise) {
+  const dataFormat = args.dataFormat || 'NHWC';
+  const dilations = args.dilations == null ? [1, 1] : args.dilations;
+  const activation = args.activation || 'linear';
+  const $x = convertToTensor(args.x, 'x', opDesc, 'float32');
+  const $filter = convertToTensor(args.filter, 'filter', opDesc, 'float32');
+  assertFloat32($x, 'x', opDesc);
+  assertFloat32($filter, 'filter', opDesc);
+  return ENGINE.tidy(() => {
+    let x4D = $x;
+    let reshapedTo4D = false;
+    if ($x.rank === 3) {
+      reshapedTo4D = true;
+      x4D = reshape($x, [1, $x.shape[0], $x.shape[1], $x.shape[2]]);
+    }
+    util.assert(
+        x4D.rank === 4,
+        () => `Error in fused ${opDesc}: input must be rank 4, but got rank ` +
+            `${x4D.rank}.`);
+    util.assert(
+        $filter.rank === 4,
+        () => `Error in fused ${opDesc}: filter must be rank 4, but got rank ` +
+            `${$filter.rank}.`);
+    backend_util.checkPadOnDimRoundingMode(
+        `fused ${opDesc}`, args.pad, args.dimRoundingMode);
+    const inputChannels = dataFormat === 'NHWC' ? x4D.shape[3] : x4D.shape[1];
+    util.assert(
+        $filter.shape[2] === inputChannels,
+        () => depthwise ?
+            `Error in fused depthwiseConv2d: number of input channels ` +
+                `(${inputChannels}) must match the inChannels dimension in ` +
+                `filter ${$filter.shape[2]}.` :
+            `Error in conv2d: depth of input (${inputChannels}) must match ` +
+                `input depth for filter ${$filter.shape[2]}.`);
+    util.assert(
+        backend_util.eitherStridesOrDilationsAreOne(args.strides, dilations),
+        () => `Error in ${depthwise ? 'fused depthwiseConv2d' : 'conv2D'}: ` +
+            `Either strides or dilations must be 1. ` +
+            `Got strides ${args.strides} and dilations '${dilations}'`);
+    const convInfo = backend_util.computeConv2DInfo(
+        x4D.shape, $filter.shape, args.strides, dilations, args.pad,
+        args.dimRoundingMode, depthwise);
+    let $bias;
+    if (args.bias != null) {
+      $bias = convertToTensor(args.bias, 'bias', `fused ${opDesc}`);
+      if (dataFormat === 'NHWC') {
+        broadcast_util.assertAndGetBroadcastShape(convInfo.outShape, $bias.shape);
+      } else {
+        util.assert(
+            $bias.shape.length <= 1,
+            () => `Error in fused conv2d: only supports scalar or 1-D Tensor ` +
+                `bias for NCHW format but got the bias of ` +
+                `rank-${$bias.shape.length}.`);
+      }
+    }
+    let $prelu;
+    if (args.preluActivationWeights != null) {
+      $prelu = convertToTensor(
+          args.preluActivationWeights, 'prelu weights', `fused ${opDesc}`);
+    }
+    const res = ENGINE.runKernel(
+        kernelName,
+        {x: x4D, filter: $filter, bias: $bias, preluActivationWeights: $prelu}, {
+          strides: args.strides,
+          pad: args.pad,
+          dataFormat,
+          dilations,
+          dimRoundingMode: args.dimRoundingMode,
+          activation,
+          leakyreluAlpha: args.leakyreluAlpha
+        });
+    if (reshapedTo4D) {
+      return reshape(res, [res.shape[1], res.shape[2], res.shape[3]]);
+    }
+    return res;
+  });
+}
+
+/** tfjs-core/src/ops/fused/conv2d.ts:96-331 */
+function fusedConv2d(args) {
+  return convCommon('conv2d', 'FusedConv2D', args, false);
+}
+
+/** tfjs-core/src/ops/fused/depthwise_conv2d.ts:90-259 */
+function fusedDepthwiseConv2d(args) {
+  return convCommon('depthwiseConv2d', 'FusedDepthwiseConv2D', args, true);
+}
+
+/** tfjs-core/src/ops/conv2d.ts (unfused) */
+function conv2d(x, filter, strides, pad, dataFormat, dilations, dimRoundingMode) {
+  const $x = convertToTensor(x, 'x', 'conv2d', 'float32');
+  const $filter = convertToTensor(filter, 'filter', 'conv2d', 'float32');
+  return ENGINE.tidy(() => {
+    const x4D = $x.rank === 3 ?
+        reshape($x, [1, $x.shape[0], $x.shape[1], $x.shape[2]]) : $x;
+    const res = ENGINE.runKernel('Conv2D', {x: x4D, filter: $filter}, {
+      strides,
+      pad,
+      dataFormat: dataFormat || 'NHWC',
+      dilations: dilations == null ? [1, 1] : dilations,
+      dimRoundingMode
+    });
+    return $x.rank === 3 ? reshape(res, res.shape.slice(1)) : res;
+  });
+}
+
+/** tfjs-core/src/ops/depthwise_conv2d.ts (unfused) */
+function depthwiseConv2d(x, filter, strides, pad, dataFormat, dilations, dimRoundingMode) {
+  const $x = convertToTensor(x, 'x', 'depthwiseConv2d', 'float32');
+  const $filter = convertToTensor(filter, 'filter', 'depthwiseConv2d', 'float32');
+  return ENGINE.tidy(() => {
+    const x4D = $x.rank === 3 ?
+        reshape($x, [1, $x.shape[0], $x.shape[1], $x.shape[2]]) : $x;
+    const res = ENGINE.runKernel('DepthwiseConv2dNative', {x: x4D, filter: $filter}, {
+      strides,
+      pad,
+      dataFormat: dataFormat || 'NHWC',
+      dilations: dilations == null ? [1, 1] : dilations,
+      dimRoundingMode
+    });
+    return $x.rank === 3 ? reshape(res, res.shape.slice(1)) : res;
+  });
+}
+
+module.exports = {
+  tensor,
+  scalar: (v, dtype) => tensor([v], [], dtype),
+  tensor1d: (v, dtype) => tensor(v, null, dtype),
+  tensor2d: (v, shape, dtype) => tensor(v, shape, dtype),
+  tensor3d: (v, shape, dtype) => tensor(v, shape, dtype),
+  tensor4d: (v, shape, dtype) => tensor(v, shape, dtype),
+  reshape,
+  add,
+  mean,
+  matMul,
+  conv2d,
+  depthwiseConv2d,
+  fused: {matMul: fusedMatMul, conv2d: fusedConv2d, depthwiseConv2d: fusedDepthwiseConv2d}
+};
