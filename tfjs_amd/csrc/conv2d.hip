@@ -28,6 +28,8 @@ extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
   const int64_t M = batch * out_h * out_w, K = f_h * f_w * in_c;
   TFHIP_CHECK_ARG(M < lim && K < lim && out_c < lim && in_h < lim && in_w < lim && batch * in_h * in_w * in_c < (lim << 8),
                   "tfhip_fused_conv2d: dimension exceeds the supported range");
+  TFHIP_CHECK_ARG(batch * in_h * in_w * in_c * 4 <= 0xfffffffeLL,
+                  "tfhip_fused_conv2d: an input above 4 GiB is not supported");
   if (M == 0) return kOk;
   TFHIP_CHECK_RANGE(x, batch * in_h * in_w * in_c, 4, "x");
   TFHIP_CHECK_RANGE(filter, K * out_c, 4, "filter");
@@ -67,7 +69,13 @@ extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
     p.epi.y_s[0] = out_h * out_w * out_c; p.epi.y_s[1] = out_w * out_c; p.epi.y_s[2] = out_c; p.epi.y_s[3] = 1;
   }
 
-  const bool x16 = reinterpret_cast<uintptr_t>(x) % 16 == 0, w16 = reinterpret_cast<uintptr_t>(filter) % 16 == 0;
+  const int64_t kMaxBufferBytes = 0xfffffffeLL;   // one buffer descriptor addresses at most this much
+  const int64_t x_bytes = batch * in_h * in_w * in_c * 4, w_bytes = K * out_c * 4;
+  p.a_bytes = (unsigned)(x_bytes <= kMaxBufferBytes ? x_bytes : 0);
+  p.b_bytes = (unsigned)(w_bytes <= kMaxBufferBytes ? w_bytes : 0);
+  p.vec_store = !nchw && out_c % 4 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+  const bool x16 = reinterpret_cast<uintptr_t>(x) % 16 == 0 && p.a_bytes != 0,
+             w16 = reinterpret_cast<uintptr_t>(filter) % 16 == 0 && p.b_bytes != 0;
   const bool vec = !nchw && x16 && w16 && in_c % 4 == 0 && out_c % 4 == 0;
   const bool pointwise = !nchw && f_h == 1 && f_w == 1 && stride_h == 1 && stride_w == 1 && pad_top == 0 &&
                          pad_left == 0 && out_h == in_h && out_w == in_w;

@@ -47,7 +47,12 @@ extern "C" int tfhip_fused_matmul(const float *a, const float *b, float *out, in
                          prelu_strides, leakyrelu_alpha, kMatmul);
   if (rc) return rc;
 
-  const bool a16 = reinterpret_cast<uintptr_t>(a) % 16 == 0, b16 = reinterpret_cast<uintptr_t>(b) % 16 == 0;
+  const int64_t kMaxBufferBytes = 0xfffffffeLL;   // one buffer descriptor addresses at most this much
+  p.a_bytes = (unsigned)(M * K * 4 <= kMaxBufferBytes ? M * K * 4 : 0);
+  p.b_bytes = (unsigned)(K * N * 4 <= kMaxBufferBytes ? K * N * 4 : 0);
+  p.vec_store = N % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const bool a16 = reinterpret_cast<uintptr_t>(a) % 16 == 0 && p.a_bytes != 0,
+             b16 = reinterpret_cast<uintptr_t>(b) % 16 == 0 && p.b_bytes != 0;
   // float4 loads need the contiguous extent (and with it every row start and
   // batch start) to be a multiple of four elements
   const bool a_vec = a16 && K > 0 && (transpose_a ? M % 4 == 0 : K % 4 == 0) && (M * K) % 4 == 0;

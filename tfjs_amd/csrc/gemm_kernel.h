@@ -8,16 +8,25 @@
 //   block over 4 values of k). Lane l feeds A[row l%16][k l/16] and
 //   B[k l/16][col l%16] and receives C[rows 4*(l/16)..+3][col l%16].
 // * Both operands are staged in LDS k-major ("[k][x]", x = row of A or column
-//   of B), so the 16 lanes that share k read 16 consecutive words: no bank
-//   conflicts whichever way the operand lies in global memory.
-// * Global -> register -> LDS double buffering: while the matrix cores work on
-//   LDS buffer t, the loads of tile t+1 are in flight into registers; they are
-//   written to the other LDS buffer after the compute, one barrier per step.
+//   of B) with a row pitch congruent to 16 modulo the 32 banks, so the 16 lanes
+//   that share k read 16 consecutive words and the two k rows of a half
+//   wavefront fall in different bank halves: fragment reads never conflict.
+//   Operands that arrive k-contiguous are transposed on the way into LDS; an
+//   XOR swizzle of the x index by the k group keeps those scattered writes
+//   conflict-free too.
+// * Software pipeline: global loads of tile t+1 are issued (as buffer loads,
+//   out-of-range lanes read zero, no branches) before the matrix work on tile t
+//   starts and are written to the other LDS buffer just before its last k step;
+//   LDS fragments of k step s+1 are fetched while the MFMAs of step s issue.
+//   One barrier per tile.
+// * Epilogue: the accumulators are laid out through LDS so that every lane
+//   applies bias + activation to four consecutive columns and writes one
+//   float4: output rows leave as whole contiguous spans.
 // * Loaders (template parameter) decide how a tile is fetched:
 //     kLoadKVec   operand is k-contiguous in memory (A row-major, or B given
-//                 transposed): float4 loads along k, transposed into LDS
+//                 transposed): 16-byte loads along k, transposed into LDS
 //     kLoadXVec   operand is x-contiguous (B row-major, or A given transposed):
-//                 float4 loads along x, float4 LDS stores
+//                 16-byte loads along x, 16-byte LDS stores
 //     kLoadScalar any strides, element loads with bounds checks
 //     kLoadIm2colVec / kLoadIm2colScalar (A only): the rows of A are the
 //                 receptive fields of an NHWC (or, scalar only, any-stride)
@@ -54,89 +63,164 @@ struct GemmParams {
   // element (i, k) of A at a[i*a_sx + k*a_sk]; element (k, j) of B at b[j*b_sx + k*b_sk]
   long long a_sx, a_sk, b_sx, b_sk;
   long long ldc;
+  // bytes addressable from the (per-batch) base of each operand, for the buffer descriptors
+  unsigned a_bytes, b_bytes;
   int tiles_m, tiles_n;
+  int vec_store;  // rows of C are 16-byte aligned and N % 4 == 0
   ConvGeom conv;
   Epilogue epi;
 };
 
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
+
+constexpr unsigned kNoOffset = 0xffffffffu;  // a buffer offset no descriptor covers: loads return 0
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int A_KIND, int B_KIND>
 struct GemmTile {
   static constexpr int kThreads = 256;
   static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per workgroup");
+  static_assert(BK == 16 || BK == 32, "k step of the tile");
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   static constexpr int TM = WM / 16, TN = WN / 16;
-  static_assert(WM % 16 == 0 && WN % 16 == 0 && BK % 4 == 0, "tile shape");
-  // Row pitch of the k-major LDS tiles: congruent to 16 modulo the 32 banks, so
-  // the two k rows a half-wavefront reads never collide.
+  static_assert(WM % 16 == 0 && WN % 16 == 0, "tile shape");
+  // x index swizzle for operands whose LDS writes are transposing
+  static constexpr bool A_SWZ = A_KIND != kLoadXVec && BM % 32 == 0 && WM % 32 == 0;
+  static constexpr bool B_SWZ = B_KIND != kLoadXVec && BN % 32 == 0 && WN % 32 == 0;
   static constexpr int LDA = BM % 32 == 0 ? BM + 16 : BM + 32;
   static constexpr int LDB = BN % 32 == 0 ? BN + 16 : BN + 32;
-  // float4 fetches per thread per tile (the last round may be partly idle)
+  // 16-byte fetches per thread per tile (the last round may be partly idle)
   static constexpr int A_VECS = (BM * BK / 4 + kThreads - 1) / kThreads;
   static constexpr int B_VECS = (BN * BK / 4 + kThreads - 1) / kThreads;
-  static constexpr int LDS_FLOATS = 2 * BK * (LDA + LDB);
+  static constexpr int A_BUF = BK * LDA, B_BUF = BK * LDB;
+  static constexpr int OPERAND_FLOATS = 2 * (A_BUF + B_BUF);
+  static constexpr int LDC = BN + 4;   // rows 4 apart land 16 banks apart
+  // the C tile goes through LDS in EPI_PASSES horizontal bands of whole wavefront rows
+  static constexpr int EPI_PASSES = (BM * LDC * 4 > 60 * 1024) ? 2 : 1;
+  static_assert(WAVES_M % EPI_PASSES == 0, "a band holds whole wavefront tiles");
+  static constexpr int EPI_ROWS = BM / EPI_PASSES;
+  static constexpr int C_FLOATS = EPI_ROWS * LDC;
+  static constexpr int LDS_FLOATS = OPERAND_FLOATS > C_FLOATS ? OPERAND_FLOATS : C_FLOATS;
 };
 
-// Fetches this thread's share of a BX x BK operand tile into registers.
-// `x0`/`k0` are the tile origin; the operand has X rows (M or N) and K columns.
+// XOR applied to the x index of LDS row k: the k group (k / 4) spread over the
+// bank bits the rows of one half wavefront leave free.
+template <int BK>
+__device__ __forceinline__ constexpr int swizzle_of(int k) {
+  return BK == 32 ? (((k >> 2) & 7) << 2) : (((k >> 2) & 3) << 3);
+}
+
+__device__ __forceinline__ float4 as_float4(uint4_t v) {
+  return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+}
+
+// Per-thread addressing state of one operand loader, fixed across k tiles.
+template <int VECS>
+struct LoaderState {
+  unsigned row_off[VECS];   // byte offset of this thread's row (or kNoOffset)
+  int row_ih[VECS];         // im2col: top-left input coordinate of the row's window
+  int row_iw[VECS];
+};
+
 template <int BX, int BK, int KIND, int VECS>
-__device__ __forceinline__ void load_tile(float4 (&reg)[VECS], const float *__restrict__ base, long long sx,
-                                          long long sk, int X, int K, int x0, int k0, int tid,
-                                          const ConvGeom &g, const long long (&row_base)[VECS],
-                                          const int (&row_ih)[VECS], const int (&row_iw)[VECS]) {
-  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+__device__ __forceinline__ void init_loader(LoaderState<VECS> &st, long long sx, long long sk, int X, int x0, int tid,
+                                            const ConvGeom &g) {
 #pragma unroll
   for (int i = 0; i < VECS; ++i) {
     const int f = tid + i * 256;
+    st.row_ih[i] = st.row_iw[i] = 0;
     if ((BX * BK / 4) % 256 != 0 && f >= BX * BK / 4) {
-      reg[i] = zero;
+      st.row_off[i] = kNoOffset;
       continue;
     }
     if (KIND == kLoadKVec) {
-      // BK/4 float4 per row; K % 4 == 0 so a float4 is wholly inside or outside
-      const int row = f / (BK / 4), kq = f % (BK / 4);
-      const int x = x0 + row, k = k0 + kq * 4;
-      reg[i] = (x < X && k < K) ? *reinterpret_cast<const float4 *>(base + (long long)x * sx + k) : zero;
+      const int x = x0 + f / (BK / 4);
+      st.row_off[i] = x < X ? (unsigned)((long long)x * sx * 4) : kNoOffset;
     } else if (KIND == kLoadXVec) {
-      // BX/4 float4 per k row; X % 4 == 0
-      const int kr = f / (BX / 4), xq = f % (BX / 4);
-      const int x = x0 + xq * 4, k = k0 + kr;
-      reg[i] = (x < X && k < K) ? *reinterpret_cast<const float4 *>(base + (long long)k * sk + x) : zero;
-    } else if (KIND == kLoadScalar) {
-      // four elements along k (stride sk) of one row
-      const int row = f / (BK / 4), kq = f % (BK / 4);
-      const int x = x0 + row, k = k0 + kq * 4;
-      float v[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) v[j] = (x < X && k + j < K) ? base[(long long)x * sx + (long long)(k + j) * sk] : 0.f;
-      reg[i] = make_float4(v[0], v[1], v[2], v[3]);
-    } else if (KIND == kLoadIm2colVec) {
-      // in_c % 4 == 0: the four k values share one filter tap (r, s)
-      const int kq = f % (BK / 4);
-      const int k = k0 + kq * 4;
-      float4 v = zero;
-      if (row_base[i] >= 0 && k < K) {
-        const int tap = k / g.in_c, c = k - tap * g.in_c;
-        const int r = tap / g.f_w, s = tap - r * g.f_w;
-        const int ih = row_ih[i] + r * g.dil_h, iw = row_iw[i] + s * g.dil_w;
-        if (ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w)
-          v = *reinterpret_cast<const float4 *>(base + row_base[i] + ih * g.xs_h + iw * g.xs_w + c);
+      const int x = x0 + (f % (BX / 4)) * 4;
+      st.row_off[i] = x < X ? (unsigned)(x * 4) : kNoOffset;
+    } else if (KIND == kLoadIm2colVec || KIND == kLoadIm2colScalar) {
+      const int m = x0 + f / (BK / 4);
+      if (m < X) {
+        const int ow = m % g.out_w;
+        const int t2 = m / g.out_w;
+        const int oh = t2 % g.out_h, n = t2 / g.out_h;
+        st.row_off[i] = (unsigned)((long long)n * g.xs_n * 4);
+        st.row_ih[i] = oh * g.stride_h - g.pad_top;
+        st.row_iw[i] = ow * g.stride_w - g.pad_left;
+      } else {
+        st.row_off[i] = kNoOffset;
       }
-      reg[i] = v;
-    } else {  // kLoadIm2colScalar
-      const int kq = f % (BK / 4);
+    } else {
+      st.row_off[i] = 0;
+    }
+  }
+}
+
+// Issues this thread's share of the loads of the BX x BK tile at (x0, k0).
+template <int BX, int BK, int KIND, int VECS>
+__device__ __forceinline__ void load_tile(float4 (&reg)[VECS], const LoaderState<VECS> &st,
+                                          __amdgpu_buffer_rsrc_t rsrc, const float *__restrict__ base, long long sx,
+                                          long long sk, int X, int K, int x0, int k0, int tid, const ConvGeom &g) {
+  if (KIND == kLoadKVec) {
+    // the k offset of a thread is the same for all its rows (256 % (BK/4) == 0)
+    const int k = k0 + (tid % (BK / 4)) * 4;
+    const bool k_ok = k < K;
+#pragma unroll
+    for (int i = 0; i < VECS; ++i) {
+      const unsigned off = (k_ok && st.row_off[i] != kNoOffset) ? st.row_off[i] + (unsigned)(k * 4) : kNoOffset;
+      reg[i] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
+    }
+  } else if (KIND == kLoadXVec) {
+#pragma unroll
+    for (int i = 0; i < VECS; ++i) {
+      const int k = k0 + (tid + i * 256) / (BX / 4);
+      const unsigned off =
+          (k < K && st.row_off[i] != kNoOffset) ? st.row_off[i] + (unsigned)((long long)k * sk * 4) : kNoOffset;
+      reg[i] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
+    }
+  } else if (KIND == kLoadIm2colVec) {
+    // in_c % 4 == 0: the four k values of a fetch share one filter tap (r, s)
+    const int k = k0 + (tid % (BK / 4)) * 4;
+    const int tap = k / g.in_c, c = k - tap * g.in_c;
+    const int r = tap / g.f_w, s = tap - r * g.f_w;
+    const int dh = r * g.dil_h, dw = s * g.dil_w;
+    const bool k_ok = k < K;
+#pragma unroll
+    for (int i = 0; i < VECS; ++i) {
+      const int ih = st.row_ih[i] + dh, iw = st.row_iw[i] + dw;
+      const bool ok = k_ok && st.row_off[i] != kNoOffset && ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
+      const unsigned off = ok ? st.row_off[i] + (unsigned)((ih * g.xs_h + iw * g.xs_w + c) * 4) : kNoOffset;
+      reg[i] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
+    }
+  } else if (KIND == kLoadScalar) {
+#pragma unroll
+    for (int i = 0; i < VECS; ++i) {
+      const int f = tid + i * 256;
+      const int x = x0 + f / (BK / 4), k = k0 + (f % (BK / 4)) * 4;
       float v[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int k = k0 + kq * 4 + j;
+        const bool ok = st.row_off[i] != kNoOffset && x < X && k + j < K;
+        v[j] = ok ? base[(long long)x * sx + (long long)(k + j) * sk] : 0.f;
+      }
+      reg[i] = make_float4(v[0], v[1], v[2], v[3]);
+    }
+  } else {  // kLoadIm2colScalar
+#pragma unroll
+    for (int i = 0; i < VECS; ++i) {
+      const int f = tid + i * 256;
+      float v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int k = k0 + (f % (BK / 4)) * 4 + j;
         v[j] = 0.f;
-        if (row_base[i] >= 0 && k < K) {
+        if (st.row_off[i] != kNoOffset && k < K) {
           const int tap = k / g.in_c, c = k - tap * g.in_c;
           const int r = tap / g.f_w, s = tap - r * g.f_w;
-          const int ih = row_ih[i] + r * g.dil_h, iw = row_iw[i] + s * g.dil_w;
+          const int ih = st.row_ih[i] + r * g.dil_h, iw = st.row_iw[i] + s * g.dil_w;
           if (ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w)
-            v[j] = base[row_base[i] + ih * g.xs_h + iw * g.xs_w + c * g.xs_c];
+            v[j] = base[(long long)(st.row_off[i] >> 2) + ih * g.xs_h + iw * g.xs_w + c * g.xs_c];
         }
       }
       reg[i] = make_float4(v[0], v[1], v[2], v[3]);
@@ -145,7 +229,7 @@ __device__ __forceinline__ void load_tile(float4 (&reg)[VECS], const float *__re
 }
 
 // Writes the registers fetched by load_tile into a k-major LDS tile [BK][LD].
-template <int BX, int BK, int LD, int KIND, int VECS>
+template <int BX, int BK, int LD, int KIND, bool SWZ, int VECS>
 __device__ __forceinline__ void store_tile(float *__restrict__ lds, const float4 (&reg)[VECS], int tid) {
 #pragma unroll
   for (int i = 0; i < VECS; ++i) {
@@ -156,7 +240,8 @@ __device__ __forceinline__ void store_tile(float *__restrict__ lds, const float4
       *reinterpret_cast<float4 *>(lds + kr * LD + xq * 4) = reg[i];
     } else {
       const int row = f / (BK / 4), kq = f % (BK / 4);
-      float *d = lds + (kq * 4) * LD + row;
+      const int col = SWZ ? (row ^ swizzle_of<BK>(kq * 4)) : row;   // the swizzle is the same for k .. k+3
+      float *d = lds + (kq * 4) * LD + col;
       d[0] = reg[i].x;
       d[LD] = reg[i].y;
       d[2 * LD] = reg[i].z;
@@ -165,19 +250,29 @@ __device__ __forceinline__ void store_tile(float *__restrict__ lds, const float4
   }
 }
 
+// Fragment of k step `kk` (a multiple of 4) for NT 16-wide blocks starting at
+// lane_base[.] (the lane's position, pre-XORed for each low swizzle value).
+template <int BK, int LD, int NT, bool SWZ>
+__device__ __forceinline__ void load_fragment(float (&frag)[NT], const float *const (&lane_base)[4], int buf_off,
+                                              int kk) {
+  const int sw = SWZ ? swizzle_of<BK>(kk) : 0;
+  const float *p = lane_base[(sw & 12) >> 2] + buf_off + kk * LD;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) frag[t] = p[(t * 16) ^ (sw & 16)];
+}
+
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int A_KIND, int B_KIND>
 __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   using T = GemmTile<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>;
   extern __shared__ float lds[];
-  float *lds_a = lds;                      // [2][BK][LDA]
-  float *lds_b = lds + 2 * BK * T::LDA;    // [2][BK][LDB]
+  float *lds_a = lds;                   // [2][BK][LDA]
+  float *lds_b = lds + 2 * T::A_BUF;    // [2][BK][LDB]
 
   // Workgroup id -> (batch, tile_m, tile_n). Ids i, i+8, i+16, ... share an XCD;
   // give each XCD one contiguous band of the tile sequence.
-  const int total = gridDim.x;
   int id = blockIdx.x;
   {
-    const int per_xcd = total / 8;
+    const int per_xcd = gridDim.x / 8;
     if (per_xcd > 0 && id < per_xcd * 8) id = (id % 8) * per_xcd + id / 8;
   }
   const int tiles_per_batch = p.tiles_m * p.tiles_n;
@@ -189,41 +284,26 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   const float *A = p.a + (long long)(bz % p.batch_a) * p.a_batch_stride;
   const float *B = p.b + (long long)(bz % p.batch_b) * p.b_batch_stride;
   float *C = p.c + (long long)bz * p.c_batch_stride;
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)A, 0, (int)p.a_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void *)B, 0, (int)p.b_bytes, 0x00020000);
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave / WAVES_N) * T::WM, wn0 = (wave % WAVES_N) * T::WN;
 
-  // im2col: the output pixel behind each A row this thread fetches is fixed
-  // across k, so split it once. row_base < 0 marks a row beyond M.
-  long long row_base[T::A_VECS];
-  int row_ih[T::A_VECS], row_iw[T::A_VECS];
-  if (A_KIND == kLoadIm2colVec || A_KIND == kLoadIm2colScalar) {
+  LoaderState<T::A_VECS> sa;
+  LoaderState<T::B_VECS> sb;
+  init_loader<BM, BK, A_KIND, T::A_VECS>(sa, p.a_sx, p.a_sk, p.M, m0, tid, p.conv);
+  init_loader<BN, BK, B_KIND, T::B_VECS>(sb, p.b_sx, p.b_sk, p.N, n0, tid, p.conv);
+
+  // lane position inside the k-major tiles, once per low-bits swizzle value
+  const float *a_lane[4], *b_lane[4];
 #pragma unroll
-    for (int i = 0; i < T::A_VECS; ++i) {
-      const int row = (tid + i * 256) / (BK / 4);
-      const int m = m0 + row;
-      if (row < BM && m < p.M) {
-        const int ow = m % p.conv.out_w;
-        const int t2 = m / p.conv.out_w;
-        const int oh = t2 % p.conv.out_h, n = t2 / p.conv.out_h;
-        row_base[i] = (long long)n * p.conv.xs_n;
-        row_ih[i] = oh * p.conv.stride_h - p.conv.pad_top;
-        row_iw[i] = ow * p.conv.stride_w - p.conv.pad_left;
-      } else {
-        row_base[i] = -1;
-        row_ih[i] = row_iw[i] = 0;
-      }
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < T::A_VECS; ++i) {
-      row_base[i] = 0;
-      row_ih[i] = row_iw[i] = 0;
-    }
+  for (int c = 0; c < 4; ++c) {
+    a_lane[c] = lds_a + (lane >> 4) * T::LDA + wm0 + ((lane & 15) ^ (T::A_SWZ ? c * 4 : 0));
+    b_lane[c] = lds_b + (lane >> 4) * T::LDB + wn0 + ((lane & 15) ^ (T::B_SWZ ? c * 4 : 0));
   }
-  const long long no_base[T::B_VECS] = {};
-  const int no_pos[T::B_VECS] = {};
 
   float4_t acc[T::TM][T::TN];
 #pragma unroll
@@ -234,67 +314,87 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   float4 ra[T::A_VECS], rb[T::B_VECS];
   const int k_tiles = (p.K + BK - 1) / BK;
 
-  load_tile<BM, BK, A_KIND, T::A_VECS>(ra, A, p.a_sx, p.a_sk, p.M, p.K, m0, 0, tid, p.conv, row_base, row_ih, row_iw);
-  load_tile<BN, BK, B_KIND, T::B_VECS>(rb, B, p.b_sx, p.b_sk, p.N, p.K, n0, 0, tid, p.conv, no_base, no_pos, no_pos);
-  store_tile<BM, BK, T::LDA, A_KIND, T::A_VECS>(lds_a, ra, tid);
-  store_tile<BN, BK, T::LDB, B_KIND, T::B_VECS>(lds_b, rb, tid);
+  load_tile<BM, BK, A_KIND, T::A_VECS>(ra, sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, 0, tid, p.conv);
+  load_tile<BN, BK, B_KIND, T::B_VECS>(rb, sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, 0, tid, p.conv);
+  store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a, ra, tid);
+  store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b, rb, tid);
   __syncthreads();
 
   for (int kt = 0; kt < k_tiles; ++kt) {
     const int cur = kt & 1;
     const bool more = kt + 1 < k_tiles;
     if (more) {
-      load_tile<BM, BK, A_KIND, T::A_VECS>(ra, A, p.a_sx, p.a_sk, p.M, p.K, m0, (kt + 1) * BK, tid, p.conv, row_base, row_ih, row_iw);
-      load_tile<BN, BK, B_KIND, T::B_VECS>(rb, B, p.b_sx, p.b_sk, p.N, p.K, n0, (kt + 1) * BK, tid, p.conv, no_base, no_pos, no_pos);
+      load_tile<BM, BK, A_KIND, T::A_VECS>(ra, sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, (kt + 1) * BK, tid, p.conv);
+      load_tile<BN, BK, B_KIND, T::B_VECS>(rb, sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, (kt + 1) * BK, tid, p.conv);
     }
-    const float *ta = lds_a + cur * BK * T::LDA + (lane >> 4) * T::LDA + wm0 + (lane & 15);
-    const float *tb = lds_b + cur * BK * T::LDB + (lane >> 4) * T::LDB + wn0 + (lane & 15);
+    const int a_off = cur * T::A_BUF, b_off = cur * T::B_BUF;
+    float fa[2][T::TM], fb[2][T::TN];
+    load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[0], a_lane, a_off, 0);
+    load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[0], b_lane, b_off, 0);
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 4) {
-      float fa[T::TM], fb[T::TN];
-#pragma unroll
-      for (int i = 0; i < T::TM; ++i) fa[i] = ta[kk * T::LDA + i * 16];
-#pragma unroll
-      for (int j = 0; j < T::TN; ++j) fb[j] = tb[kk * T::LDB + j * 16];
+    for (int s = 0; s < BK / 4; ++s) {
+      if (s + 1 < BK / 4) {
+        load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[(s + 1) & 1], a_lane, a_off, (s + 1) * 4);
+        load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[(s + 1) & 1], b_lane, b_off, (s + 1) * 4);
+      } else if (more) {
+        // the next tile goes to the other buffer while the last k step computes
+        store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a + (cur ^ 1) * T::A_BUF, ra, tid);
+        store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b + (cur ^ 1) * T::B_BUF, rb, tid);
+      }
 #pragma unroll
       for (int i = 0; i < T::TM; ++i)
 #pragma unroll
         for (int j = 0; j < T::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
-    }
-    if (more) {
-      store_tile<BM, BK, T::LDA, A_KIND, T::A_VECS>(lds_a + (cur ^ 1) * BK * T::LDA, ra, tid);
-      store_tile<BN, BK, T::LDB, B_KIND, T::B_VECS>(lds_b + (cur ^ 1) * BK * T::LDB, rb, tid);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
     }
     __syncthreads();
   }
 
-  // Epilogue: lane l holds rows 4*(l/16)..+3 of column l%16 of each 16x16 block.
+  // ---- epilogue: accumulators -> LDS [EPI_ROWS][LDC] -> float4 per lane -> global ----
+  float *lds_c = lds;
   const Epilogue &e = p.epi;
+  constexpr int kColGroups = BN / 4;
 #pragma unroll
-  for (int i = 0; i < T::TM; ++i) {
+  for (int pass = 0; pass < T::EPI_PASSES; ++pass) {
+    const int band0 = pass * T::EPI_ROWS;
+    if (pass > 0) __syncthreads();
+    if (wm0 >= band0 && wm0 < band0 + T::EPI_ROWS) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int row = m0 + wm0 + i * 16 + (lane >> 4) * 4 + r;
-      if (row >= p.M) continue;
+      for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            lds_c[(wm0 - band0 + i * 16 + (lane >> 4) * 4 + r) * T::LDC + wn0 + j * 16 + (lane & 15)] = acc[i][j][r];
+    }
+    __syncthreads();
+    for (int idx = tid; idx < T::EPI_ROWS * kColGroups; idx += 256) {
+      const int lr = idx / kColGroups, lc = (idx - lr * kColGroups) * 4;
+      const int row = m0 + band0 + lr, col = n0 + lc;
+      if (row >= p.M || col >= p.N) continue;
+      const float4 v = *reinterpret_cast<const float4 *>(lds_c + lr * T::LDC + lc);
       long long n = 0, oh = 0, ow = 0;
-      long long out_row;
       if (e.addressing == kConv) {
         ow = row % e.out_w;
         const int t2 = row / e.out_w;
         oh = t2 % e.out_h;
         n = t2 / e.out_h;
-        out_row = n * e.y_s[0] + oh * e.y_s[1] + ow * e.y_s[2];
-      } else {
-        out_row = (long long)row * p.ldc;
       }
+      const float in[4] = {v.x, v.y, v.z, v.w};
+      float out[4];
 #pragma unroll
-      for (int j = 0; j < T::TN; ++j) {
-        const int col = n0 + wn0 + j * 16 + (lane & 15);
-        if (col >= p.N) continue;
-        const float v = finish(e, acc[i][j][r], bz, row, col, n, oh, ow);
-        const long long off = (e.addressing == kConv) ? out_row + col * e.y_s[3] : out_row + col;
-        C[off] = v;
+      for (int q = 0; q < 4; ++q) out[q] = (col + q < p.N) ? finish(e, in[q], bz, row, col + q, n, oh, ow) : 0.f;
+      if (p.vec_store) {
+        *reinterpret_cast<float4 *>(C + (long long)row * p.ldc + col) = make_float4(out[0], out[1], out[2], out[3]);
+      } else if (e.addressing == kConv) {
+        const long long base = n * e.y_s[0] + oh * e.y_s[1] + ow * e.y_s[2];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (col + q < p.N) C[base + (col + q) * e.y_s[3]] = out[q];
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (col + q < p.N) C[(long long)row * p.ldc + col + q] = out[q];
       }
     }
   }
