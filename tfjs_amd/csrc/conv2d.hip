@@ -84,7 +84,7 @@ extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
     return launch_plain_gemm(p, false, false, vec);
   }
   if (vec) {
-    const int shape = choose_tile_shape(M, out_c, 1, num_cus());
+    const int shape = choose_tile_shape(M, out_c, K, 1, num_cus());
     return launch_gemm_shape<kLoadIm2colVec, kLoadXVec>(shape, p);
   }
   if (out_c <= 32) return launch_gemm<256, 32, 16, 4, 1, kLoadIm2colScalar, kLoadScalar>(p);

@@ -58,6 +58,16 @@ __device__ __forceinline__ float activate(float v, int act, float alpha, double 
   }
 }
 
+// Index of the bias (which == 0) or PReLU weight (which == 1) that goes with
+// output element (batch, row, col); for kConv (n, oh, ow) is the split of row.
+__device__ __forceinline__ long long operand_index(const Epilogue &e, int which, long long batch, long long row,
+                                                   long long col, long long n, long long oh, long long ow) {
+  const long long *s = which == 0 ? e.bias_s : e.prelu_s;
+  if (e.addressing == kChannel) return col * s[3];
+  if (e.addressing == kMatmul) return batch * s[0] + row * s[1] + col * s[2];
+  return n * s[0] + oh * s[1] + ow * s[2] + col * s[3];
+}
+
 // Applies bias and activation to `v`, the raw contraction result of output
 // element (batch, row, col). For kConv, (n, oh, ow) is the split of `row`.
 __device__ __forceinline__ float finish(const Epilogue &e, float v, long long batch,

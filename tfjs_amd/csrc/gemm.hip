@@ -6,7 +6,7 @@ using namespace tfhip;
 
 int tfhip::launch_plain_gemm(GemmParams &p, bool transpose_a, bool transpose_b, bool vec) {
   if (vec) {
-    const int shape = choose_tile_shape(p.M, p.N, p.batch, num_cus());
+    const int shape = choose_tile_shape(p.M, p.N, p.K, p.batch, num_cus());
     if (!transpose_a && !transpose_b) return launch_gemm_shape<kLoadKVec, kLoadXVec>(shape, p);
     if (!transpose_a && transpose_b) return launch_gemm_shape<kLoadKVec, kLoadKVec>(shape, p);
     if (transpose_a && !transpose_b) return launch_gemm_shape<kLoadXVec, kLoadXVec>(shape, p);

@@ -2,33 +2,42 @@
 // choice and the launch of one gemm_kernel instantiation.
 #pragma once
 
+#include <stdlib.h>
+
 #include "common.h"
 #include "gemm_kernel.h"
 
 namespace tfhip {
 
 struct TileShape {
-  int bm, bn;
+  int bm, bn, bk;
   double quality;  // relative speed of a full tile of this shape
 };
 
-// Shapes instantiated for every loader combination, best first.
+// Shapes instantiated for every loader combination.
 static const TileShape kTileShapes[] = {
-    {128, 128, 1.00}, {128, 96, 0.97}, {128, 64, 0.90}, {64, 64, 0.78}, {256, 32, 0.80}, {256, 16, 0.60},
+    {128, 128, 16, 1.00}, {128, 96, 16, 0.97}, {128, 64, 16, 0.90}, {64, 64, 16, 0.78},  {256, 32, 16, 0.80},
+    {256, 16, 16, 0.60},  {64, 96, 16, 0.85},  {128, 128, 32, 1.02}, {128, 96, 32, 0.99}, {64, 64, 32, 0.80},
 };
-constexpr int kNumTileShapes = 6;
+constexpr int kNumTileShapes = 10;
 
 // Picks the shape with the best estimated throughput for an M x N output
 // repeated `batch` times on `cus` compute units: useful fraction of the padded
 // tiles, times the fill of the last round of workgroups, times tile quality.
-inline int choose_tile_shape(long long M, long long N, long long batch, int cus, int only = -1) {
-  if (only >= 0) return only;
+// TFHIP_TILE=<index> in the environment overrides the choice (tuning aid).
+inline int choose_tile_shape(long long M, long long N, long long K, long long batch, int cus) {
+  static const int forced = [] {
+    const char *e = getenv("TFHIP_TILE");
+    return e ? atoi(e) : -1;
+  }();
+  if (forced >= 0 && forced < kNumTileShapes) return forced;
   int best = 0;
   double best_score = -1.0;
   for (int i = 0; i < kNumTileShapes; ++i) {
     const TileShape &t = kTileShapes[i];
     const long long tm = (M + t.bm - 1) / t.bm, tn = (N + t.bn - 1) / t.bn;
-    const double useful = (double)(M * N) / (double)(tm * t.bm * tn * t.bn);
+    const long long kp = (K + t.bk - 1) / t.bk * t.bk;
+    const double useful = (double)(M * N) / (double)(tm * t.bm * tn * t.bn) * ((double)(K > 0 ? K : 1) / (double)(kp > 0 ? kp : 1));
     const long long tiles = tm * tn * batch;
     const long long rounds = (tiles + cus - 1) / cus;
     const double fill = (double)tiles / (double)(rounds * cus);
@@ -64,7 +73,11 @@ inline int launch_gemm_shape(int shape, GemmParams &p) {
     case 2: return launch_gemm<128, 64, 16, 2, 2, A_KIND, B_KIND>(p);
     case 3: return launch_gemm<64, 64, 16, 2, 2, A_KIND, B_KIND>(p);
     case 4: return launch_gemm<256, 32, 16, 4, 1, A_KIND, B_KIND>(p);
-    default: return launch_gemm<256, 16, 16, 4, 1, A_KIND, B_KIND>(p);
+    case 5: return launch_gemm<256, 16, 16, 4, 1, A_KIND, B_KIND>(p);
+    case 6: return launch_gemm<64, 96, 16, 2, 2, A_KIND, B_KIND>(p);
+    case 7: return launch_gemm<128, 128, 32, 2, 2, A_KIND, B_KIND>(p);
+    case 8: return launch_gemm<128, 96, 32, 2, 2, A_KIND, B_KIND>(p);
+    default: return launch_gemm<64, 64, 32, 2, 2, A_KIND, B_KIND>(p);
   }
 }
 

@@ -14,11 +14,11 @@
 //   Operands that arrive k-contiguous are transposed on the way into LDS; an
 //   XOR swizzle of the x index by the k group keeps those scattered writes
 //   conflict-free too.
-// * Software pipeline: global loads of tile t+1 are issued (as buffer loads,
-//   out-of-range lanes read zero, no branches) before the matrix work on tile t
-//   starts and are written to the other LDS buffer just before its last k step;
-//   LDS fragments of k step s+1 are fetched while the MFMAs of step s issue.
-//   One barrier per tile.
+// * Software pipeline: a ring of registers keeps the global loads of the next
+//   2 or 4 tiles in flight (buffer loads: out-of-range lanes read zero, no
+//   branches); tile t+1 moves from its ring slot to the other LDS buffer just
+//   before the last k step of tile t; LDS fragments of k step s+1 are fetched
+//   while the MFMAs of step s issue. One barrier per tile.
 // * Epilogue: the accumulators are laid out through LDS so that every lane
 //   applies bias + activation to four consecutive columns and writes one
 //   float4: output rows leave as whole contiguous spans.
@@ -39,6 +39,10 @@
 #include <hip/hip_runtime.h>
 
 #include "epilogue.h"
+
+#ifndef TFHIP_EXP
+#define TFHIP_EXP 0
+#endif
 
 namespace tfhip {
 
@@ -93,6 +97,8 @@ struct GemmTile {
   static constexpr int A_VECS = (BM * BK / 4 + kThreads - 1) / kThreads;
   static constexpr int B_VECS = (BN * BK / 4 + kThreads - 1) / kThreads;
   static constexpr int A_BUF = BK * LDA, B_BUF = BK * LDB;
+  // tiles in flight between global memory and LDS (even, see the main loop)
+  static constexpr int PREFETCH = (A_VECS + B_VECS) * 4 * 4 <= 96 ? 4 : 2;
   static constexpr int OPERAND_FLOATS = 2 * (A_BUF + B_BUF);
   static constexpr int LDC = BN + 4;   // rows 4 apart land 16 banks apart
   // the C tile goes through LDS in EPI_PASSES horizontal bands of whole wavefront rows
@@ -100,7 +106,9 @@ struct GemmTile {
   static_assert(WAVES_M % EPI_PASSES == 0, "a band holds whole wavefront tiles");
   static constexpr int EPI_ROWS = BM / EPI_PASSES;
   static constexpr int C_FLOATS = EPI_ROWS * LDC;
-  static constexpr int LDS_FLOATS = OPERAND_FLOATS > C_FLOATS ? OPERAND_FLOATS : C_FLOATS;
+  // the epilogue also keeps BN bias values and BN PReLU weights behind the C band
+  static constexpr int EPI_FLOATS = C_FLOATS + 2 * BN;
+  static constexpr int LDS_FLOATS = OPERAND_FLOATS > EPI_FLOATS ? OPERAND_FLOATS : EPI_FLOATS;
 };
 
 // XOR applied to the x index of LDS row k: the k group (k / 4) spread over the
@@ -311,49 +319,83 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 #pragma unroll
     for (int j = 0; j < T::TN; ++j) acc[i][j] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-  float4 ra[T::A_VECS], rb[T::B_VECS];
+  // Register ring of D tiles in flight: tile t is fetched D iterations before it
+  // is needed, so the loop tolerates D tile-times of memory latency.
+  constexpr int D = T::PREFETCH;
+  float4 ra[D][T::A_VECS], rb[D][T::B_VECS];
   const int k_tiles = (p.K + BK - 1) / BK;
 
-  load_tile<BM, BK, A_KIND, T::A_VECS>(ra, sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, 0, tid, p.conv);
-  load_tile<BN, BK, B_KIND, T::B_VECS>(rb, sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, 0, tid, p.conv);
-  store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a, ra, tid);
-  store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b, rb, tid);
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    if (d == 0 || d < k_tiles) {
+      load_tile<BM, BK, A_KIND, T::A_VECS>(ra[d], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, d * BK, tid, p.conv);
+      load_tile<BN, BK, B_KIND, T::B_VECS>(rb[d], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, d * BK, tid, p.conv);
+    }
+  }
+  store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a, ra[0], tid);
+  store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b, rb[0], tid);
+  if (D < k_tiles) {
+    load_tile<BM, BK, A_KIND, T::A_VECS>(ra[0], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, D * BK, tid, p.conv);
+    load_tile<BN, BK, B_KIND, T::B_VECS>(rb[0], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, D * BK, tid, p.conv);
+  }
   __syncthreads();
 
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    const int cur = kt & 1;
-    const bool more = kt + 1 < k_tiles;
-    if (more) {
-      load_tile<BM, BK, A_KIND, T::A_VECS>(ra, sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, (kt + 1) * BK, tid, p.conv);
-      load_tile<BN, BK, B_KIND, T::B_VECS>(rb, sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, (kt + 1) * BK, tid, p.conv);
-    }
-    const int a_off = cur * T::A_BUF, b_off = cur * T::B_BUF;
-    float fa[2][T::TM], fb[2][T::TN];
-    load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[0], a_lane, a_off, 0);
-    load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[0], b_lane, b_off, 0);
+  for (int kt0 = 0; kt0 < k_tiles; kt0 += D) {
 #pragma unroll
-    for (int s = 0; s < BK / 4; ++s) {
-      if (s + 1 < BK / 4) {
-        load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[(s + 1) & 1], a_lane, a_off, (s + 1) * 4);
-        load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[(s + 1) & 1], b_lane, b_off, (s + 1) * 4);
-      } else if (more) {
-        // the next tile goes to the other buffer while the last k step computes
-        store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a + (cur ^ 1) * T::A_BUF, ra, tid);
-        store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b + (cur ^ 1) * T::B_BUF, rb, tid);
+    for (int u = 0; u < D; ++u) {
+      const int kt = kt0 + u;
+      if (kt < k_tiles) {
+        const int cur = u & 1;            // D is even, so the LDS buffer of tile kt is u & 1
+        const int nxt = (u + 1) % D;      // ring slot of tile kt + 1
+        const bool more = kt + 1 < k_tiles;
+        const int a_off = cur * T::A_BUF, b_off = cur * T::B_BUF;
+        float fa[2][T::TM], fb[2][T::TN];
+        load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[0], a_lane, a_off, 0);
+        load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[0], b_lane, b_off, 0);
+#pragma unroll
+        for (int s = 0; s < BK / 4; ++s) {
+          if (!(TFHIP_EXP & 8) && s + 1 < BK / 4) {
+            load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[(s + 1) & 1], a_lane, a_off, (s + 1) * 4);
+            load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[(s + 1) & 1], b_lane, b_off, (s + 1) * 4);
+          } else if (!(TFHIP_EXP & 2) && more) {
+            // tile kt+1 goes to the other LDS buffer while the last k step computes;
+            // its ring slot is refilled with tile kt+1+D at once
+            store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a + (cur ^ 1) * T::A_BUF, ra[nxt], tid);
+            store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b + (cur ^ 1) * T::B_BUF, rb[nxt], tid);
+            if (!(TFHIP_EXP & 1) && kt + 1 + D < k_tiles) {
+              load_tile<BM, BK, A_KIND, T::A_VECS>(ra[nxt], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0,
+                                                   (kt + 1 + D) * BK, tid, p.conv);
+              load_tile<BN, BK, B_KIND, T::B_VECS>(rb[nxt], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0,
+                                                   (kt + 1 + D) * BK, tid, p.conv);
+            }
+          }
+          // keep the fetches above ahead of the matrix work below: the compiler
+          // would otherwise sink each LDS read next to its first use
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+            for (int j = 0; j < T::TN; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (!(TFHIP_EXP & 4)) __syncthreads();
       }
-#pragma unroll
-      for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-        for (int j = 0; j < T::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
     }
-    __syncthreads();
   }
 
   // ---- epilogue: accumulators -> LDS [EPI_ROWS][LDC] -> float4 per lane -> global ----
   float *lds_c = lds;
+  float *lds_bias = lds + T::C_FLOATS, *lds_prelu = lds_bias + BN;
   const Epilogue &e = p.epi;
   constexpr int kColGroups = BN / 4;
+  if (e.addressing == kChannel && tid < BN) {
+    // bias and PReLU weights of this tile's columns, fetched once per workgroup
+    // (the loop's last barrier has passed: the operand buffers are free)
+    const int col = n0 + tid;
+    lds_bias[tid] = (e.bias && col < p.N) ? e.bias[(long long)col * e.bias_s[3]] : 0.f;
+    lds_prelu[tid] = (e.activation == TFHIP_PRELU && col < p.N) ? e.prelu[(long long)col * e.prelu_s[3]] : 0.f;
+  }
 #pragma unroll
   for (int pass = 0; pass < T::EPI_PASSES; ++pass) {
     const int band0 = pass * T::EPI_ROWS;
@@ -368,26 +410,47 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
             lds_c[(wm0 - band0 + i * 16 + (lane >> 4) * 4 + r) * T::LDC + wn0 + j * 16 + (lane & 15)] = acc[i][j][r];
     }
     __syncthreads();
+    // One float4 of the band per lane and trip. The trip loop stays rolled: the
+    // activation code is large and an unrolled epilogue would not fit the
+    // instruction cache.
+    const bool staged = e.addressing == kChannel;   // bias / PReLU weights sit in LDS, indexed by tile column
     for (int idx = tid; idx < T::EPI_ROWS * kColGroups; idx += 256) {
       const int lr = idx / kColGroups, lc = (idx - lr * kColGroups) * 4;
       const int row = m0 + band0 + lr, col = n0 + lc;
       if (row >= p.M || col >= p.N) continue;
       const float4 v = *reinterpret_cast<const float4 *>(lds_c + lr * T::LDC + lc);
-      long long n = 0, oh = 0, ow = 0;
-      if (e.addressing == kConv) {
-        ow = row % e.out_w;
-        const int t2 = row / e.out_w;
-        oh = t2 % e.out_h;
-        n = t2 / e.out_h;
-      }
       const float in[4] = {v.x, v.y, v.z, v.w};
+      float bq[4] = {0.f, 0.f, 0.f, 0.f}, pq[4] = {0.f, 0.f, 0.f, 0.f};
+      if (staged) {
+        const float4 b4 = *reinterpret_cast<const float4 *>(lds_bias + lc);
+        const float4 p4 = *reinterpret_cast<const float4 *>(lds_prelu + lc);
+        bq[0] = b4.x; bq[1] = b4.y; bq[2] = b4.z; bq[3] = b4.w;
+        pq[0] = p4.x; pq[1] = p4.y; pq[2] = p4.z; pq[3] = p4.w;
+      } else {
+        long long n = 0, oh = 0, ow = 0;
+        if (e.addressing == kConv) {
+          ow = row % e.out_w;
+          const int t2 = row / e.out_w;
+          oh = t2 % e.out_h;
+          n = t2 / e.out_h;
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (col + q < p.N) {
+            if (e.bias) bq[q] = e.bias[operand_index(e, 0, bz, row, col + q, n, oh, ow)];
+            if (e.activation == TFHIP_PRELU) pq[q] = e.prelu[operand_index(e, 1, bz, row, col + q, n, oh, ow)];
+          }
+        }
+      }
       float out[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) out[q] = (col + q < p.N) ? finish(e, in[q], bz, row, col + q, n, oh, ow) : 0.f;
+      for (int q = 0; q < 4; ++q) out[q] = activate(in[q] + bq[q], e.activation, pq[q], e.leaky_alpha);
       if (p.vec_store) {
         *reinterpret_cast<float4 *>(C + (long long)row * p.ldc + col) = make_float4(out[0], out[1], out[2], out[3]);
       } else if (e.addressing == kConv) {
-        const long long base = n * e.y_s[0] + oh * e.y_s[1] + ow * e.y_s[2];
+        const int ow = row % e.out_w;
+        const int t2 = row / e.out_w;
+        const long long base = (long long)(t2 / e.out_h) * e.y_s[0] + (long long)(t2 % e.out_h) * e.y_s[1] + ow * e.y_s[2];
 #pragma unroll
         for (int q = 0; q < 4; ++q)
           if (col + q < p.N) C[base + (col + q) * e.y_s[3]] = out[q];
