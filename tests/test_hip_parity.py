@@ -230,6 +230,33 @@ def test_depthwise_shapes(hip, orc, xs, fs, stride, dil, pad):
     assert_parity(hip.fused_depthwise_conv2d(x, w, **kw), orc.fused_depthwise_conv2d(x, w, **kw))
 
 
+@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("act", ["linear", "relu", "elu", "sigmoid", "leakyrelu", "prelu"])
+@pytest.mark.parametrize("bias_shape,prelu_shape", [((8,), (8,)), ((), (1, 1, 8)), ((5, 8), (6, 5, 1)), ((2, 6, 5, 8), (1,))])
+def test_depthwise_epilogue_forms(hip, orc, act, bias_shape, prelu_shape, stride):
+    # 3x3 with four-channel groups: the row-pipeline kernel, both epilogue variants
+    rng = np.random.default_rng(29)
+    x = rng.uniform(-1, 1, (2, 6 * stride, 5 * stride, 8)).astype(np.float32)
+    w = rng.normal(0, 0.5, (3, 3, 8, 1)).astype(np.float32)
+    kw = dict(pad="same", strides=stride, bias=rng.uniform(-1, 1, bias_shape).astype(np.float32), activation=act,
+              prelu=rng.uniform(0, 1, prelu_shape).astype(np.float32) if act == "prelu" else None,
+              leakyrelu_alpha=0.1)
+    assert_parity(hip.fused_depthwise_conv2d(x, w, **kw), orc.fused_depthwise_conv2d(x, w, **kw))
+
+
+@pytest.mark.parametrize("rows", [1, 2, 3, 5, 7, 16])
+@pytest.mark.parametrize("stride,pad", [(1, "same"), (2, "same"), (1, "valid"), (2, "valid")])
+def test_depthwise_row_chunks(hip, orc, monkeypatch, rows, stride, pad):
+    # every chunk length of the row pipeline, ragged last chunk and ragged last column strip
+    monkeypatch.setenv("TFHIP_DW_ROWS", str(rows))
+    rng = np.random.default_rng(31 + rows)
+    x = rng.uniform(-1, 1, (2, 23, 13, 12)).astype(np.float32)
+    w = rng.normal(0, 0.5, (3, 3, 12, 1)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (12,)).astype(np.float32)
+    kw = dict(pad=pad, strides=stride, bias=bias, activation="relu6")
+    assert_parity(hip.fused_depthwise_conv2d(x, w, **kw), orc.fused_depthwise_conv2d(x, w, **kw))
+
+
 def test_depthwise_linearity_full_size(hip):
     # size-independent property at the benchmark shape: conv(x1 + x2) = conv(x1) + conv(x2)
     c = synth.config3(1)

@@ -1,13 +1,19 @@
 // FusedDepthwiseConv2D, NHWC float32.
 //
-// Bandwidth-bound (about 2 flops per byte), so no matrix cores: the 3x3 kernel
-// stages an input halo tile of 32 channels in LDS once per workgroup, so each
-// input element is fetched from memory once per tile instead of up to nine
-// times, and every global access is a float4 over the contiguous channel axis.
+// Bandwidth-bound (about 2 flops per byte), so no matrix cores. Three kernels:
+//  * depthwise_3x3_rows: 3x3, stride 1 or 2, channel multiplier 1 (every
+//    MobileNet layer). A register row pipeline: each input row is fetched once
+//    per lane as float4 over the contiguous channel axis and scattered into
+//    rotating accumulators; no LDS, no barriers.
+//  * depthwise_3x3_halo: the same shapes when a tensor is too large for 32-bit
+//    buffer offsets; stages an input halo tile of 32 channels in LDS.
+//  * depthwise_generic: any filter, stride, dilation, channel multiplier.
 // Each output accumulates its taps in the reference's own order (filter row,
 // then filter column: tfjs-backend-cpu/src/kernels/DepthwiseConv2dNative.ts:62-95)
 // with one fused multiply-add per tap, which is the reference's
 // "fround(y + x*w)" per tap up to double rounding.
+#include <stdlib.h>
+
 #include "common.h"
 #include "epilogue.h"
 
@@ -123,9 +129,269 @@ __global__ __launch_bounds__(256) void depthwise_3x3_halo(DwParams p, Epilogue e
   }
 }
 
+
+// ---- 3x3, channel multiplier 1, dilation 1, stride S: register row pipeline ----
+// Each lane owns four channels (one float4) of a strip of 4 output columns and
+// walks down `rows` output rows. Every input row it needs is fetched exactly
+// once by that lane (4*S + 2 float4 loads: the 8 lanes that share a pixel read
+// one contiguous 128-byte line, the column overlap with the neighbouring strip
+// is served by the vector cache) and is scattered at once into the accumulators
+// of the up to three output rows it contributes to, which live in registers and
+// rotate as rows complete. The loads of input row i+1 are issued before the
+// arithmetic of row i. No barriers, no LDS: the only traffic besides the
+// compulsory reads and writes is the halo rows of vertically adjacent chunks.
+//
+// All accesses are buffer loads/stores over the whole tensor with 32-bit byte
+// offsets: padding taps and ragged edges use an offset outside the descriptor,
+// which reads as zero and drops stores, so the row pipeline has no branches.
+constexpr int kRowsPW = 4;   // output columns per lane
+#ifndef DW_WAVES
+#define DW_WAVES 1
+#endif
+constexpr unsigned kDwNoOffset = 0xffffffffu;
+typedef unsigned int dw_uint4 __attribute__((ext_vector_type(4)));
+
+struct DwRowsArgs {
+  int strips_w;      // column strips per output row
+  int chunks_h;      // row chunks per image
+  int rows;          // output rows per chunk
+  int c4_total;
+  long long strips;  // batch * chunks_h * strips_w
+  unsigned x_bytes, y_bytes;
+};
+
+template <int S>
+struct DwRowsState {
+  static constexpr int NIN = (kRowsPW - 1) * S + 3;   // input columns a strip needs
+  static constexpr int NSLOT = S == 1 ? 3 : 2;          // output rows in flight
+  float4 acc[NSLOT][kRowsPW];
+  float4 w[9];
+  float4 bias4;               // per-channel bias of this lane (channel addressing)
+  unsigned x_col[NIN];        // byte offset of input column j (+ channel group) within a row, or kDwNoOffset
+  unsigned y_col[kRowsPW];    // same for the output columns
+  unsigned x_img, y_img;      // byte offset of the image
+  unsigned x_row, y_row;      // bytes per row
+  int in_h, out_h, ih0, oh0, ow0, rows, rows_in, c, n;
+};
+
+__device__ __forceinline__ float4 dw_load4(__amdgpu_buffer_rsrc_t r, unsigned off) {
+  const dw_uint4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+  return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+}
+
+__device__ __forceinline__ void dw_store4(__amdgpu_buffer_rsrc_t r, unsigned off, float4 v) {
+  dw_uint4 u;
+  u.x = __float_as_uint(v.x); u.y = __float_as_uint(v.y); u.z = __float_as_uint(v.z); u.w = __float_as_uint(v.w);
+  __builtin_amdgcn_raw_buffer_store_b128(u, r, (int)off, 0, 0);
+}
+
+// Bias + activation of four channels. The common case (per-channel operands,
+// relu-family activation) is a handful of instructions inline; anything else
+// takes one out-of-line call so that the row pipeline stays small.
+__device__ __noinline__ float4 dw_finish4_general(const Epilogue &e, float4 a, int c, int n, int oh, int ow) {
+  float4 r;
+  r.x = finish(e, a.x, 0, 0, c + 0, n, oh, ow);
+  r.y = finish(e, a.y, 0, 0, c + 1, n, oh, ow);
+  r.z = finish(e, a.z, 0, 0, c + 2, n, oh, ow);
+  r.w = finish(e, a.w, 0, 0, c + 3, n, oh, ow);
+  return r;
+}
+
+__device__ __forceinline__ float relu_family(float v, int act) {
+  if (act == TFHIP_LINEAR) return v;
+  const float t = (v > 0.f || v != v) ? v : 0.f;     // Math.max(0, x): NaN stays, -0 becomes +0
+  return (act == TFHIP_RELU6 && t > 6.f) ? 6.f : t;
+}
+
+template <bool GENERAL>
+__device__ __forceinline__ float4 dw_finish4(const Epilogue &e, float4 a, float4 bias4, int c, int n, int oh, int ow) {
+  if (!GENERAL) {
+    float4 r;
+    r.x = relu_family(a.x + bias4.x, e.activation);
+    r.y = relu_family(a.y + bias4.y, e.activation);
+    r.z = relu_family(a.z + bias4.z, e.activation);
+    r.w = relu_family(a.w + bias4.w, e.activation);
+    return r;
+  }
+  return dw_finish4_general(e, a, c, n, oh, ow);
+}
+
+// Issues the loads of input row i of the chunk (relative to its first input row).
+template <int S>
+__device__ __forceinline__ void dw_load_row(const DwRowsState<S> &st, __amdgpu_buffer_rsrc_t rx, int i,
+                                            float4 (&in)[DwRowsState<S>::NIN]) {
+  const int ih = st.ih0 + i;
+  const bool row_ok = ih >= 0 && ih < st.in_h && i < st.rows_in;
+  const unsigned row_off = st.x_img + (unsigned)ih * st.x_row;
+#pragma unroll
+  for (int j = 0; j < DwRowsState<S>::NIN; ++j) {
+    const unsigned off = (row_ok && st.x_col[j] != kDwNoOffset) ? row_off + st.x_col[j] : kDwNoOffset;
+    in[j] = dw_load4(rx, off);
+  }
+}
+
+// Scatters input row i into the output rows it is a tap row of; PHASE is i
+// modulo the rotation period of the accumulators, so slots are compile-time.
+template <int S, int PHASE, bool GENERAL>
+__device__ __forceinline__ void dw_compute_row(DwRowsState<S> &st, const Epilogue &e, __amdgpu_buffer_rsrc_t ry,
+                                               int i, const float4 (&in)[DwRowsState<S>::NIN]) {
+  using St = DwRowsState<S>;
+  constexpr int PERIOD = S * St::NSLOT;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int wr = 0; wr < 3; ++wr) {
+    constexpr int kBig = 4 * PERIOD;
+    if ((PHASE - wr + kBig) % S != 0) continue;          // this input row is not tap row `wr` of any output row
+    const int o = (i - wr) / S;                            // output row (relative to the chunk) it feeds
+    if (i - wr < 0 || o >= st.rows) continue;
+    const int slot = ((PHASE - wr + kBig) / S) % St::NSLOT;
+#pragma unroll
+    for (int x = 0; x < kRowsPW; ++x) {
+      float4 a = wr == 0 ? zero : st.acc[slot][x];
+#pragma unroll
+      for (int wc = 0; wc < 3; ++wc) {
+        const float4 xv = in[x * S + wc];
+        const float4 wv = st.w[wr * 3 + wc];
+        a.x = fmaf(xv.x, wv.x, a.x);
+        a.y = fmaf(xv.y, wv.y, a.y);
+        a.z = fmaf(xv.z, wv.z, a.z);
+        a.w = fmaf(xv.w, wv.w, a.w);
+      }
+      st.acc[slot][x] = a;
+    }
+    if (wr == 2) {
+      // the row is complete: bias + activation, one float4 store per column
+      const int oh = st.oh0 + o;
+      const bool row_ok = oh < st.out_h;
+      const unsigned row_off = st.y_img + (unsigned)oh * st.y_row;
+#pragma unroll
+      for (int x = 0; x < kRowsPW; ++x) {
+        const unsigned off = (row_ok && st.y_col[x] != kDwNoOffset) ? row_off + st.y_col[x] : kDwNoOffset;
+        dw_store4(ry, off, dw_finish4<GENERAL>(e, st.acc[slot][x], st.bias4, st.c, st.n, oh, st.ow0 + x));
+      }
+    }
+  }
+}
+
+// One pipeline step: `a` holds input row i0+K, `b` receives row i0+K+1.
+template <int S, int K, bool GENERAL>
+__device__ __forceinline__ void dw_step(DwRowsState<S> &st, const Epilogue &e, __amdgpu_buffer_rsrc_t rx,
+                                        __amdgpu_buffer_rsrc_t ry, int i0, const float4 (&a)[DwRowsState<S>::NIN],
+                                        float4 (&b)[DwRowsState<S>::NIN]) {
+  constexpr int PERIOD = S * DwRowsState<S>::NSLOT;
+  if (i0 + K >= st.rows_in) return;
+  dw_load_row<S>(st, rx, i0 + K + 1, b);
+  dw_compute_row<S, K % PERIOD, GENERAL>(st, e, ry, i0 + K, a);
+}
+
+// GENERAL = false: per-channel bias and a relu-family activation, all inline.
+template <int S, bool GENERAL>
+__global__ __launch_bounds__(256, DW_WAVES) void depthwise_3x3_rows(DwParams p, Epilogue e, DwRowsArgs g) {
+  using St = DwRowsState<S>;
+  const int c4 = blockIdx.y * kCQ + (threadIdx.x % kCQ);
+  const long long strip = (long long)blockIdx.x * kSlots + threadIdx.x / kCQ;
+  if (c4 >= g.c4_total || strip >= g.strips) return;
+  const int sw = (int)(strip % g.strips_w);
+  const long long t = strip / g.strips_w;
+  const int ch = (int)(t % g.chunks_h);
+  const int n = (int)(t / g.chunks_h);
+  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, (int)g.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc((void *)p.y, 0, (int)g.y_bytes, 0x00020000);
+
+  St st;
+  st.in_h = p.in_h; st.out_h = p.out_h;
+  st.oh0 = ch * g.rows;
+  st.ow0 = sw * kRowsPW;
+  st.ih0 = st.oh0 * S - p.pad_top;
+  st.rows = g.rows;
+  st.rows_in = (g.rows - 1) * S + 3;
+  st.c = c4 * 4;
+  st.n = n;
+  const unsigned pix = (unsigned)g.c4_total * 16u;   // bytes per pixel
+  st.x_row = (unsigned)p.in_w * pix;
+  st.y_row = (unsigned)p.out_w * pix;
+  st.x_img = (unsigned)n * (unsigned)p.in_h * st.x_row;
+  st.y_img = (unsigned)n * (unsigned)p.out_h * st.y_row;
+  const int iw0 = st.ow0 * S - p.pad_left;
+#pragma unroll
+  for (int j = 0; j < St::NIN; ++j) {
+    const int iw = iw0 + j;
+    st.x_col[j] = (iw >= 0 && iw < p.in_w) ? (unsigned)iw * pix + (unsigned)c4 * 16u : kDwNoOffset;
+  }
+#pragma unroll
+  for (int x = 0; x < kRowsPW; ++x) {
+    const int ow = st.ow0 + x;
+    st.y_col[x] = ow < p.out_w ? (unsigned)ow * pix + (unsigned)c4 * 16u : kDwNoOffset;
+  }
+  const float4 *w4 = reinterpret_cast<const float4 *>(p.w) + c4;
+#pragma unroll
+  for (int k = 0; k < 9; ++k) st.w[k] = w4[(long long)k * g.c4_total];
+  st.bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (!GENERAL && e.bias) {
+    const long long bs = e.bias_s[3];
+    st.bias4 = make_float4(e.bias[(st.c + 0) * bs], e.bias[(st.c + 1) * bs], e.bias[(st.c + 2) * bs],
+                           e.bias[(st.c + 3) * bs]);
+  }
+
+  // The two row buffers swap roles every step, so the loop is unrolled by an
+  // even multiple of the accumulator rotation period.
+  constexpr int PERIOD = S * St::NSLOT;
+  constexpr int UNROLL = PERIOD % 2 == 0 ? PERIOD : 2 * PERIOD;
+  float4 cur[St::NIN], nxt[St::NIN];
+  dw_load_row<S>(st, rx, 0, cur);
+  for (int i0 = 0; i0 < st.rows_in; i0 += UNROLL) {
+    dw_step<S, 0, GENERAL>(st, e, rx, ry, i0, cur, nxt);
+    dw_step<S, 1, GENERAL>(st, e, rx, ry, i0, nxt, cur);
+    dw_step<S, 2, GENERAL>(st, e, rx, ry, i0, cur, nxt);
+    dw_step<S, 3, GENERAL>(st, e, rx, ry, i0, nxt, cur);
+    if (UNROLL > 4) {
+      dw_step<S, 4, GENERAL>(st, e, rx, ry, i0, cur, nxt);
+      dw_step<S, 5, GENERAL>(st, e, rx, ry, i0, nxt, cur);
+    }
+  }
+}
+
 int balanced_tile(int extent, int max_tile) {
   const int tiles = (extent + max_tile - 1) / max_tile;
   return (extent + tiles - 1) / tiles;
+}
+
+// Output rows per lane for the row pipeline. A lane that walks more rows
+// re-reads fewer halo rows (each chunk of r output rows fetches (r-1)*S+3 input
+// rows) but is a longer serial chain of row fetches, and fewer, longer chains
+// may not keep enough loads in flight. The estimate below is
+// max(latency chain, traffic / bandwidth) with constants fitted to sweeps over
+// r on MI355X (one row fetch per lane is about 0.8 us of memory latency, one
+// wavefront sustains about 7.5 GB/s, the chip about 6.5 TB/s; halo rows of a
+// working set that fits the 256 MB memory-side cache mostly hit it).
+int choose_rows(int batch, int in_h, int in_w, int in_c, int out_h, int out_w, int S, int cus) {
+  const double in_bytes = 4.0 * batch * in_h * in_w * in_c;
+  const double out_bytes = 4.0 * batch * out_h * out_w * in_c;
+  const int strips_w = (out_w + kRowsPW - 1) / kRowsPW;
+  const int c_blocks = (in_c / 4 + kCQ - 1) / kCQ;
+  const long long slots = (long long)cus * 8;   // resident wavefronts: two per SIMD at this kernel's register count
+  const bool cached = in_bytes + out_bytes <= 250e6;
+  int best = 1;
+  double best_t = 1e30;
+  for (int r = 1; r <= 24 && r <= out_h; ++r) {
+    const int chunks = (out_h + r - 1) / r;
+    const int rb = (out_h + chunks - 1) / chunks;
+    if (rb != r) continue;   // the balanced tile is what runs: only score those
+    const int rows_in = (rb - 1) * S + 3;
+    const long long wgs = (((long long)batch * chunks * strips_w + kSlots - 1) / kSlots) * c_blocks;
+    const long long waves = wgs * 4;
+    const long long rounds = (waves + slots - 1) / slots;
+    const double halo = (double)chunks * rows_in / in_h;
+    const double traffic = in_bytes * (cached ? 1.0 + (halo - 1.0) * 0.3 : halo) + out_bytes;
+    const double wave_bw = 7500.0 * (S == 2 ? 1.5 : 1.0);   // bytes per us
+    const double conc = (double)(waves < slots ? waves : slots);
+    const double bw = conc * wave_bw < 6.5e6 ? conc * wave_bw : 6.5e6;
+    const double t_bw = traffic / bw;
+    const double t_lat = rounds * (1.5 + rows_in * 0.8);
+    const double t = t_lat > t_bw ? t_lat : t_bw;
+    if (t < best_t) { best_t = t; best = r; }
+  }
+  return best;
 }
 
 }  // namespace
@@ -201,6 +467,38 @@ extern "C" int tfhip_fused_depthwise_conv2d(
   const bool fast = f_h == 3 && f_w == 3 && ch_mul == 1 && dilation_h == 1 && dilation_w == 1 &&
                     stride_h == stride_w && (stride_h == 1 || stride_h == 2) && in_c % 4 == 0 && aligned16 &&
                     batch <= 65535;
+  // the row pipeline addresses both tensors with 32-bit byte offsets
+  const bool fits32 = batch * in_h * in_w * in_c * 4 <= 0xfffffff0LL && total * 4 <= 0xfffffff0LL;
+  if (fast && fits32 && !getenv("TFHIP_DW_HALO")) {
+    const int S = (int)stride_h;
+    DwRowsArgs g;
+    g.c4_total = (int)(in_c / 4);
+    g.strips_w = ((int)out_w + kRowsPW - 1) / kRowsPW;
+    int rows = choose_rows((int)batch, (int)in_h, (int)in_w, (int)in_c, (int)out_h, (int)out_w, S, num_cus());
+    if (const char *env = getenv("TFHIP_DW_ROWS")) rows = atoi(env);   // tuning override
+    rows = rows < 1 ? 1 : (rows > 32 ? 32 : rows);
+    if (rows > out_h) rows = (int)out_h;
+    g.rows = balanced_tile((int)out_h, rows);
+    g.chunks_h = ((int)out_h + g.rows - 1) / g.rows;
+    g.strips = (long long)batch * g.chunks_h * g.strips_w;
+    g.x_bytes = (unsigned)(batch * in_h * in_w * in_c * 4);
+    g.y_bytes = (unsigned)(total * 4);
+    const long long blocks_x = (g.strips + kSlots - 1) / kSlots;
+    if (blocks_x <= 0x7fffffffLL) {
+      dim3 grid((unsigned)blocks_x, (g.c4_total + kCQ - 1) / kCQ, 1);
+      const bool general = !(e.addressing == kChannel && activation <= TFHIP_RELU6);
+      note_kernel("depthwise_3x3_rows<%d,%d>", S, (int)general);
+      if (S == 1 && !general)
+        TFHIP_LAUNCH((depthwise_3x3_rows<1, false><<<grid, 256, 0, stream()>>>(p, e, g)));
+      else if (S == 1)
+        TFHIP_LAUNCH((depthwise_3x3_rows<1, true><<<grid, 256, 0, stream()>>>(p, e, g)));
+      else if (!general)
+        TFHIP_LAUNCH((depthwise_3x3_rows<2, false><<<grid, 256, 0, stream()>>>(p, e, g)));
+      else
+        TFHIP_LAUNCH((depthwise_3x3_rows<2, true><<<grid, 256, 0, stream()>>>(p, e, g)));
+      return kOk;
+    }
+  }
   if (fast) {
     const int S = (int)stride_h;
     const int c4_total = (int)(in_c / 4);
