@@ -19,7 +19,8 @@ Besides `value` (images/s) the line carries
                 dequant), each launched back to back between two events
   cpu_baseline  the same graph at batch 1 on one host thread, timed beside it
 
-Other modes:  --kernels-only (skip the model), --no-cpu-baseline.
+Other modes:  --kernels-only (skip the model), --no-kernels, --no-cpu-baseline,
+--copy-yardstick MIB (adds copies of known size for hardware-counter runs).
 """
 import argparse
 import ctypes
@@ -40,6 +41,25 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 RIDGE = MFMA_FP32_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
 BATCH = 32
+
+# HBM bytes per launch (reads + writes), averaged over a symbol's launches in one
+# MobileNetV2 b32 inference: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each
+# scaled by its reading for a 256 MiB copy kernel
+# (profiles/mobilenet_v2_b32_hbm_traffic.md holds the runs). Hardware counters
+# cannot be read from inside this script, so the table is refreshed by hand when a
+# kernel changes; a symbol that is not listed reports null.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
+    "gemm_kernel<256, 32, 16, 4, 1, 4, 2>": 71218476,
+    "depthwise_3x3_rows<1,0>": 38791876,
+    "gemm_kernel<256, 16, 16, 4, 1, 0, 1>": 46572946,
+    "gemm_kernel<64, 96, 16, 2, 2, 0, 1>": 180058853,
+    "depthwise_3x3_rows<2,0>": 89025911,
+    "gemm_kernel<256, 32, 16, 4, 1, 0, 1>": 73976888,
+    "add_same_shape": 8326066,
+    "gemm_kernel<64, 64, 16, 2, 2, 0, 1>": 16900669,
+    "gemm_kernel<64, 64, 32, 2, 2, 0, 1>": 12874294,
+    "mean_hw": 8230159,
+}
 
 
 def roofline_entry(flops, nbytes, seconds):
@@ -148,7 +168,9 @@ def bench_model(model_dir, steps, warmup):
     roof = roofline_entry(d["flops"], d["bytes"], d["seconds"])
     roof.update(kernel=dominant, launches_per_step=d["launches"],
                 avg_launch_us=round(d["seconds"] / d["launches"] * 1e6, 2),
-                share_of_kernel_time=round(d["seconds"] / kernel_seconds, 3), traffic=None)
+                share_of_kernel_time=round(d["seconds"] / kernel_seconds, 3),
+                algorithmic_bytes_per_launch=round(d["bytes"] / d["launches"]),
+                traffic=MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(dominant))
     symbols = {k: dict(us_per_step=round(v["seconds"] * 1e6, 1), launches=v["launches"],
                        **roofline_entry(v["flops"], v["bytes"], v["seconds"])) for k, v in by_symbol.items()}
     return dict(ms_per_step=seconds / steps * 1e3, kernel_ms_per_step=kernel_seconds * 1e3, roofline=roof,
@@ -298,6 +320,27 @@ def cpu_baseline(model_dir):
                        "one thread", host_cpus=os.cpu_count())
 
 
+def copy_yardstick(mib):
+    """Three plain device-to-device copies of `mib` MiB (kernel copy_f4); returns GB/s moved (read + write)."""
+    from tfjs_amd.capi import DeviceBuffer, check, load_library
+    lib = load_library()
+    src, dst = DeviceBuffer(mib << 20), DeviceBuffer(mib << 20)
+    ev = Events(lib, check)
+    try:
+        check(lib.tfhip_copy(src.ptr, dst.ptr, mib << 20))    # touch both once
+        best = None
+        for _ in range(3):
+            ev.record(0)
+            check(lib.tfhip_copy(dst.ptr, src.ptr, mib << 20))
+            ev.record(1)
+            ms = ev.elapsed_ms(0, 1)
+            best = ms if best is None else min(best, ms)
+    finally:
+        src.free()
+        dst.free()
+    return round(2.0 * (mib << 20) / (best * 1e-3) / 1e9, 1)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -307,6 +350,9 @@ def main():
     ap.add_argument("--no-kernels", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-baseline-child", metavar="MODEL_DIR")
+    ap.add_argument("--copy-yardstick", type=int, metavar="MIB", default=0,
+                    help="also run three device-to-device copies of this many MiB, so that a hardware-counter run "
+                         "of this command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.cpu_baseline_child:
         cpu_baseline_child(args.cpu_baseline_child)
@@ -331,6 +377,7 @@ def main():
     finally:
         shutil.rmtree(model_dir, ignore_errors=True)
     kernels = None if args.no_kernels else bench_kernels()
+    copy_gbs = copy_yardstick(args.copy_yardstick) if args.copy_yardstick else None
     ms_per_step = js["ms_per_step"] if js else m["ms_per_step"]
     host = ("node %s, tfjs API -> KernelBackend 'hip' -> N-API addon -> C ABI (tfjs-core: %s)" % (js["node"], js["core"])
             if js else "python/ctypes over the C ABI (node or the addon not found)")
@@ -356,6 +403,7 @@ def main():
         "tflops_model": round(BATCH * workloads.mobilenet_v2_flops_per_image() / (ms_per_step * 1e-3) / 1e12, 3),
         "roofline": m["roofline"],
         "cpu_baseline": cpu,
+        "copy_yardstick_gbs": copy_gbs,
         "symbols": m["symbols"],
         "kernels": kernels,
     }

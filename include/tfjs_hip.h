@@ -86,9 +86,14 @@ int tfhip_event_elapsed(int start_slot, int end_slot, float *ms);
  *   around one call times n launches without n trips through the caller's
  *   language. n = 1 is normal operation.
  * tfhip_last_kernel: symbol of the kernel the last entry point chose, spelled as
- *   a profiler demangles it, e.g. "gemm_kernel<128, 128, 16, 2, 2, 0, 1>". */
+ *   a profiler demangles it, e.g. "gemm_kernel<128, 128, 16, 2, 2, 0, 1>".
+ * tfhip_copy: a plain device-to-device copy kernel ("copy_f4": reads `bytes`,
+ *   writes `bytes`; both pointers 16-byte aligned, bytes a multiple of 16): the
+ *   yardstick that a kernel's bandwidth and a profiler's traffic counters are
+ *   scaled by. */
 int tfhip_set_launch_repeat(int n);
 int tfhip_last_kernel(char *name, size_t name_len);
+int tfhip_copy(void *dst, const void *src, size_t bytes);
 
 /* ---- _FusedMatMul / BatchMatMul ------------------------------------------
  * Replaces _FusedMatMul(a_id, a_shape, ..., out_id)

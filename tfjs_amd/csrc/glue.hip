@@ -60,6 +60,11 @@ __global__ __launch_bounds__(256) void mean_hw(const float *__restrict__ x, floa
   }
 }
 
+__global__ __launch_bounds__(256) void copy_f4(const float4 *__restrict__ src, float4 *__restrict__ dst, long long n4) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) dst[i] = src[i];
+}
+
 int grid_for(long long items) {
   long long blocks = (items + 255) / 256;
   const long long cap = (long long)num_cus() * 32;
@@ -117,6 +122,20 @@ int tfhip_mean_hw(const float *x, float *y, int64_t batch, int64_t h, int64_t w,
   TFHIP_CHECK_RANGE(y, batch * c, 4, "y");
   note_kernel("mean_hw");
   TFHIP_LAUNCH((mean_hw<<<grid_for(batch * c), 256, 0, stream()>>>(x, y, batch, h * w, c)));
+  return kOk;
+}
+
+int tfhip_copy(void *dst, const void *src, size_t bytes) {
+  TFHIP_REQUIRE_INIT();
+  if (bytes == 0) return kOk;
+  TFHIP_CHECK_ARG(bytes % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(src) % 16 == 0,
+                  "tfhip_copy: pointers and size must be multiples of 16 bytes");
+  TFHIP_CHECK_RANGE(src, bytes, 1, "src");
+  TFHIP_CHECK_RANGE(dst, bytes, 1, "dst");
+  note_kernel("copy_f4");
+  TFHIP_LAUNCH((copy_f4<<<grid_for(bytes / 16), 256, 0, stream()>>>((const float4 *)src, (float4 *)dst,
+                                                                      (long long)(bytes / 16))));
   return kOk;
 }
 
