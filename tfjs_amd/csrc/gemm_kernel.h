@@ -38,13 +38,24 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "epilogue.h"
 
 #ifndef TFHIP_EXP
 #define TFHIP_EXP 0
 #endif
-
 namespace tfhip {
+
+// Workgroup barrier that orders LDS traffic only. __syncthreads() also fences
+// global memory, which makes every wave wait for all of its outstanding global
+// loads (vmcnt(0)) at each barrier and so drains the prefetch ring once per k
+// tile; the tiles exchanged between waves here live in LDS alone.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 
 enum LoadKind { kLoadKVec = 0, kLoadXVec = 1, kLoadScalar = 2, kLoadIm2colVec = 3, kLoadIm2colScalar = 4 };
 
@@ -325,64 +336,90 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   float4 ra[D][T::A_VECS], rb[D][T::B_VECS];
   const int k_tiles = (p.K + BK - 1) / BK;
 
+  // Every fetch below is unconditional: a tile past K reads as zeros through
+  // the buffer descriptor at no memory cost, and with no branch around a load
+  // the compiler can count exactly how many loads may stay in flight at each use
+  // (a conditional load makes it assume the shortest queue and wait for all).
 #pragma unroll
   for (int d = 0; d < D; ++d) {
-    if (d == 0 || d < k_tiles) {
-      load_tile<BM, BK, A_KIND, T::A_VECS>(ra[d], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, d * BK, tid, p.conv);
-      load_tile<BN, BK, B_KIND, T::B_VECS>(rb[d], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, d * BK, tid, p.conv);
-    }
+    load_tile<BM, BK, A_KIND, T::A_VECS>(ra[d], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, d * BK, tid, p.conv);
+    load_tile<BN, BK, B_KIND, T::B_VECS>(rb[d], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, d * BK, tid, p.conv);
   }
   store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a, ra[0], tid);
   store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b, rb[0], tid);
-  if (D < k_tiles) {
-    load_tile<BM, BK, A_KIND, T::A_VECS>(ra[0], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, D * BK, tid, p.conv);
-    load_tile<BN, BK, B_KIND, T::B_VECS>(rb[0], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, D * BK, tid, p.conv);
-  }
-  __syncthreads();
+  load_tile<BM, BK, A_KIND, T::A_VECS>(ra[0], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, D * BK, tid, p.conv);
+  load_tile<BN, BK, B_KIND, T::B_VECS>(rb[0], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, D * BK, tid, p.conv);
+  lds_barrier();
 
-  for (int kt0 = 0; kt0 < k_tiles; kt0 += D) {
+  // One k tile: tile kt sits in LDS buffer u & 1 (kt and u have the same parity),
+  // tile kt+1 in ring slot (u+1) % D.
+  auto tile_step = [&](int kt, auto u_tag) {
+    constexpr int u = decltype(u_tag)::value;
+    constexpr int cur = u & 1;
+    constexpr int nxt = (u + 1) % D;
+    const int a_off = cur * T::A_BUF, b_off = cur * T::B_BUF;
+    float fa[2][T::TM], fb[2][T::TN];
+    load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[0], a_lane, a_off, 0);
+    load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[0], b_lane, b_off, 0);
 #pragma unroll
-    for (int u = 0; u < D; ++u) {
-      const int kt = kt0 + u;
-      if (kt < k_tiles) {
-        const int cur = u & 1;            // D is even, so the LDS buffer of tile kt is u & 1
-        const int nxt = (u + 1) % D;      // ring slot of tile kt + 1
-        const bool more = kt + 1 < k_tiles;
-        const int a_off = cur * T::A_BUF, b_off = cur * T::B_BUF;
-        float fa[2][T::TM], fb[2][T::TN];
-        load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[0], a_lane, a_off, 0);
-        load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[0], b_lane, b_off, 0);
-#pragma unroll
-        for (int s = 0; s < BK / 4; ++s) {
-          if (!(TFHIP_EXP & 8) && s + 1 < BK / 4) {
-            load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[(s + 1) & 1], a_lane, a_off, (s + 1) * 4);
-            load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[(s + 1) & 1], b_lane, b_off, (s + 1) * 4);
-          } else if (!(TFHIP_EXP & 2) && more) {
-            // tile kt+1 goes to the other LDS buffer while the last k step computes;
-            // its ring slot is refilled with tile kt+1+D at once
-            store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a + (cur ^ 1) * T::A_BUF, ra[nxt], tid);
-            store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b + (cur ^ 1) * T::B_BUF, rb[nxt], tid);
-            if (!(TFHIP_EXP & 1) && kt + 1 + D < k_tiles) {
-              load_tile<BM, BK, A_KIND, T::A_VECS>(ra[nxt], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0,
-                                                   (kt + 1 + D) * BK, tid, p.conv);
-              load_tile<BN, BK, B_KIND, T::B_VECS>(rb[nxt], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0,
-                                                   (kt + 1 + D) * BK, tid, p.conv);
-            }
-          }
-          // keep the fetches above ahead of the matrix work below: the compiler
-          // would otherwise sink each LDS read next to its first use
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-            for (int j = 0; j < T::TN; ++j)
-              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        if (!(TFHIP_EXP & 4)) __syncthreads();
+    for (int s = 0; s < BK / 4; ++s) {
+      if (s + 1 < BK / 4) {
+        load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[(s + 1) & 1], a_lane, a_off, (s + 1) * 4);
+        load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[(s + 1) & 1], b_lane, b_off, (s + 1) * 4);
       }
+      if (s == 0) {
+        // tile kt+1 goes to the other LDS buffer (free since the barrier that
+        // ended tile kt-1) at the start of the tile, so the stores finish under
+        // the matrix work instead of in front of the closing barrier
+        store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a + (cur ^ 1) * T::A_BUF, ra[nxt], tid);
+        store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b + (cur ^ 1) * T::B_BUF, rb[nxt], tid);
+      } else if (s == 1) {
+        // its ring slot is refilled with tile kt+1+D, one operand per k step
+        load_tile<BM, BK, A_KIND, T::A_VECS>(ra[nxt], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, (kt + 1 + D) * BK,
+                                             tid, p.conv);
+      } else if (s == 2) {
+        load_tile<BN, BK, B_KIND, T::B_VECS>(rb[nxt], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, (kt + 1 + D) * BK,
+                                             tid, p.conv);
+      }
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
+    }
+    // Issue order for the whole tile: after every matrix instruction a little of
+    // the side work (next fragments from LDS, the LDS stores of tile kt+1, the
+    // global fetches of tile kt+1+D and their address arithmetic), so that it
+    // issues in the shadow of the matrix pipe instead of in a block in front of
+    // it. A wave issues in order: side work that is not interleaved is exposed
+    // whenever a SIMD holds a single wave.
+#pragma unroll
+    for (int m = 0; m < (BK / 4) * T::TM * T::TN; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // one LDS write
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one global read
+      __builtin_amdgcn_sched_group_barrier(0x006, 3, 0);   // a few vector / scalar ALU
+    }
+    __builtin_amdgcn_sched_barrier(0);   // nothing of this tile moves past its closing barrier
+    lds_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // Full groups of D tiles run without a branch between them; the remainder
+  // (fewer than D tiles) follows with one check per tile.
+  int kt = 0;
+  for (; kt + D <= k_tiles; kt += D) {
+    tile_step(kt, std::integral_constant<int, 0>());
+    tile_step(kt + 1, std::integral_constant<int, 1>());
+    if (D > 2) {
+      tile_step(kt + 2, std::integral_constant<int, 2 % D>());
+      tile_step(kt + 3, std::integral_constant<int, 3 % D>());
     }
   }
+  if (kt < k_tiles) tile_step(kt, std::integral_constant<int, 0>());
+  if (kt + 1 < k_tiles) tile_step(kt + 1, std::integral_constant<int, 1>());
+  if (D > 2 && kt + 2 < k_tiles) tile_step(kt + 2, std::integral_constant<int, 2 % D>());
 
   // ---- epilogue: accumulators -> LDS [EPI_ROWS][LDC] -> float4 per lane -> global ----
   float *lds_c = lds;
@@ -399,7 +436,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 #pragma unroll
   for (int pass = 0; pass < T::EPI_PASSES; ++pass) {
     const int band0 = pass * T::EPI_ROWS;
-    if (pass > 0) __syncthreads();
+    if (pass > 0) lds_barrier();
     if (wm0 >= band0 && wm0 < band0 + T::EPI_ROWS) {
 #pragma unroll
       for (int i = 0; i < T::TM; ++i)
@@ -409,7 +446,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
           for (int r = 0; r < 4; ++r)
             lds_c[(wm0 - band0 + i * 16 + (lane >> 4) * 4 + r) * T::LDC + wn0 + j * 16 + (lane & 15)] = acc[i][j][r];
     }
-    __syncthreads();
+    lds_barrier();
     // One float4 of the band per lane and trip. The trip loop stays rolled: the
     // activation code is large and an unrolled epilogue would not fit the
     // instruction cache.

@@ -1,0 +1,46 @@
+/**
+ * Type declarations of tfjs-backend-hip. The shapes are those of tfjs-core:
+ * KernelBackend (tfjs-core/src/backends/backend.ts:100-156), KernelConfig
+ * (tfjs-core/src/kernel_registry.ts:55-61), decodeWeights
+ * (tfjs-core/src/io/io_utils.ts:119-135).
+ */
+import {DataId, DataType, KernelBackend, KernelConfig, NamedTensorMap, TensorInfo, io} from '@tensorflow/tfjs-core';
+
+export interface HipMemoryInfo {
+  unreliable: boolean;
+  /** device blocks handed out and not freed */
+  numDeviceBuffers: number;
+  numBytesInGPU: number;
+  /** freed blocks kept by the pool for reuse */
+  numBytesInGPUPool: number;
+}
+
+export declare class HipBackend extends KernelBackend {
+  constructor(device?: number);
+  write(values: ArrayBufferView, shape: number[], dtype: DataType): DataId;
+  move(dataId: DataId, values: ArrayBufferView, shape: number[], dtype: DataType, refCount: number): void;
+  read(dataId: DataId): Promise<ArrayBufferView>;
+  readSync(dataId: DataId): ArrayBufferView;
+  disposeData(dataId: DataId, force?: boolean): boolean;
+  refCount(dataId: DataId): number;
+  incRef(dataId: DataId): void;
+  decRef(dataId: DataId): void;
+  numDataIds(): number;
+  memory(): HipMemoryInfo;
+  time(f: () => void): Promise<{kernelMs: number}>;
+  timerAvailable(): boolean;
+  floatPrecision(): 16|32;
+  epsilon(): number;
+  dispose(): void;
+  /** Allocates an uninitialised device tensor (kernel outputs). */
+  makeOutput(shape: number[], dtype: DataType): TensorInfo;
+  /** Device pointer of a tensor's storage, as the addon takes it. */
+  ptr(dataId: DataId): number;
+}
+
+/** decodeWeights with the dequantize step on the GPU; inject as GraphModel's tfio. */
+export declare function decodeWeights(
+    weightData: ArrayBuffer|ArrayBuffer[], specs: io.WeightsManifestEntry[]): NamedTensorMap;
+
+export declare const kernelConfigs: KernelConfig[];
+export declare const version: string;
