@@ -25,6 +25,7 @@ struct Epilogue {
   double leaky_alpha;
   int activation;
   int addressing;
+  int channel_operands;  // bias and PReLU weights (if any) are indexed by column alone
   // kConv only: spatial extent of the output for the row split, and the output
   // strides for (n, oh, ow, c) so NCHW outputs can be written in place.
   int out_h, out_w;

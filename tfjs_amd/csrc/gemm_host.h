@@ -71,8 +71,22 @@ inline int launch_gemm(GemmParams &p) {
   if (grid <= 0) return kOk;
   if (grid > 0x7fffffffLL) return fail(kBadArgument, "gemm: %lld tiles exceed the grid limit", grid);
   note_kernel("gemm_kernel<%d, %d, %d, %d, %d, %d, %d>", BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND);
-  TFHIP_LAUNCH((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>
-                <<<dim3((unsigned)grid), dim3(256), T::LDS_FLOATS * sizeof(float), stream()>>>(p)));
+  // The fused epilogue covers per-column operands with a relu-family activation;
+  // anything else leaves raw sums for gemm_finish.
+  const Epilogue &e = p.epi;
+  p.inline_epilogue = e.channel_operands && (e.activation <= TFHIP_LEAKYRELU);
+  if (p.inline_epilogue) {
+    TFHIP_LAUNCH((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>
+                  <<<dim3((unsigned)grid), dim3(256), T::LDS_FLOATS * sizeof(float), stream()>>>(p)));
+  } else {
+    const long long total = (long long)p.M * p.N * p.batch;
+    long long blocks = (total + 255) / 256;
+    const long long cap = (long long)num_cus() * 16;
+    if (blocks > cap) blocks = cap;
+    TFHIP_LAUNCH((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>
+                  <<<dim3((unsigned)grid), dim3(256), T::LDS_FLOATS * sizeof(float), stream()>>>(p),
+                  gemm_finish<<<dim3((unsigned)blocks), dim3(256), 0, stream()>>>(p)));
+  }
   return kOk;
 }
 
@@ -129,6 +143,7 @@ inline int fill_epilogue(Epilogue &e, const char *who, const int64_t *dims, int 
                   (long long)extent);
     if (which == 0) e.bias = ptr; else e.prelu = ptr;
   }
+  e.channel_operands = channel_only ? 1 : 0;
   if (channel_only) {
     e.addressing = kChannel;
     e.bias_s[3] = bias ? bias_strides[rank - 1] : 0;

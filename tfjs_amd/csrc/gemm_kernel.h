@@ -19,9 +19,14 @@
 //   branches); tile t+1 moves from its ring slot to the other LDS buffer just
 //   before the last k step of tile t; LDS fragments of k step s+1 are fetched
 //   while the MFMAs of step s issue. One barrier per tile.
-// * Epilogue: the accumulators are laid out through LDS so that every lane
-//   applies bias + activation to four consecutive columns and writes one
-//   float4: output rows leave as whole contiguous spans.
+// * The two MFMA operands are passed swapped (the instruction computes the
+//   transposed block), so a lane ends up with four consecutive COLUMNS of one
+//   output row: the epilogue applies bias + activation in registers and writes
+//   one float4 per 16x16 block, with no trip through LDS and no barrier.
+//   Epilogues that are not "per-column operands + relu-family activation"
+//   (sigmoid, elu, bias or PReLU weights that vary along rows or batch) store
+//   the raw sums and are completed in place by gemm_finish, a second kernel
+//   enqueued right behind.
 // * Loaders (template parameter) decide how a tile is fetched:
 //     kLoadKVec   operand is k-contiguous in memory (A row-major, or B given
 //                 transposed): 16-byte loads along k, transposed into LDS
@@ -82,6 +87,7 @@ struct GemmParams {
   unsigned a_bytes, b_bytes;
   int tiles_m, tiles_n;
   int vec_store;  // rows of C are 16-byte aligned and N % 4 == 0
+  int inline_epilogue;  // bias + activation happen in gemm_kernel (else gemm_finish completes the raw sums)
   ConvGeom conv;
   Epilogue epi;
 };
@@ -110,16 +116,7 @@ struct GemmTile {
   static constexpr int A_BUF = BK * LDA, B_BUF = BK * LDB;
   // tiles in flight between global memory and LDS (even, see the main loop)
   static constexpr int PREFETCH = (A_VECS + B_VECS) * 4 * 4 <= 96 ? 4 : 2;
-  static constexpr int OPERAND_FLOATS = 2 * (A_BUF + B_BUF);
-  static constexpr int LDC = BN + 4;   // rows 4 apart land 16 banks apart
-  // the C tile goes through LDS in EPI_PASSES horizontal bands of whole wavefront rows
-  static constexpr int EPI_PASSES = (BM * LDC * 4 > 60 * 1024) ? 2 : 1;
-  static_assert(WAVES_M % EPI_PASSES == 0, "a band holds whole wavefront tiles");
-  static constexpr int EPI_ROWS = BM / EPI_PASSES;
-  static constexpr int C_FLOATS = EPI_ROWS * LDC;
-  // the epilogue also keeps BN bias values and BN PReLU weights behind the C band
-  static constexpr int EPI_FLOATS = C_FLOATS + 2 * BN;
-  static constexpr int LDS_FLOATS = OPERAND_FLOATS > EPI_FLOATS ? OPERAND_FLOATS : EPI_FLOATS;
+  static constexpr int LDS_FLOATS = 2 * (A_BUF + B_BUF);
 };
 
 // XOR applied to the x index of LDS row k: the k group (k / 4) spread over the
@@ -385,7 +382,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
       for (int i = 0; i < T::TM; ++i)
 #pragma unroll
         for (int j = 0; j < T::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[s & 1][i], fb[s & 1][j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb[s & 1][j], fa[s & 1][i], acc[i][j], 0, 0, 0);
     }
     // Issue order for the whole tile: after every matrix instruction a little of
     // the side work (next fragments from LDS, the LDS stores of tile kt+1, the
@@ -421,82 +418,96 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   if (kt + 1 < k_tiles) tile_step(kt + 1, std::integral_constant<int, 1>());
   if (D > 2 && kt + 2 < k_tiles) tile_step(kt + 2, std::integral_constant<int, 2 % D>());
 
-  // ---- epilogue: accumulators -> LDS [EPI_ROWS][LDC] -> float4 per lane -> global ----
-  float *lds_c = lds;
-  float *lds_bias = lds + T::C_FLOATS, *lds_prelu = lds_bias + BN;
+  // ---- epilogue: registers -> global. Lane l of a 16x16 block holds row l % 16,
+  // columns 4 * (l / 16) .. +3 (the operands went into the MFMA swapped).
   const Epilogue &e = p.epi;
-  constexpr int kColGroups = BN / 4;
-  if (e.addressing == kChannel && tid < BN) {
-    // bias and PReLU weights of this tile's columns, fetched once per workgroup
-    // (the loop's last barrier has passed: the operand buffers are free)
-    const int col = n0 + tid;
-    lds_bias[tid] = (e.bias && col < p.N) ? e.bias[(long long)col * e.bias_s[3]] : 0.f;
-    lds_prelu[tid] = (e.activation == TFHIP_PRELU && col < p.N) ? e.prelu[(long long)col * e.prelu_s[3]] : 0.f;
-  }
+  const int lane_m = lane & 15, lane_n = (lane >> 4) * 4;
+  const bool fused = p.inline_epilogue != 0;
+  float bias_q[T::TN][4], alpha_q[T::TN][4];
 #pragma unroll
-  for (int pass = 0; pass < T::EPI_PASSES; ++pass) {
-    const int band0 = pass * T::EPI_ROWS;
-    if (pass > 0) lds_barrier();
-    if (wm0 >= band0 && wm0 < band0 + T::EPI_ROWS) {
+  for (int j = 0; j < T::TN; ++j) {
+    const int col = n0 + wn0 + j * 16 + lane_n;
 #pragma unroll
-      for (int i = 0; i < T::TM; ++i)
-#pragma unroll
-        for (int j = 0; j < T::TN; ++j)
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            lds_c[(wm0 - band0 + i * 16 + (lane >> 4) * 4 + r) * T::LDC + wn0 + j * 16 + (lane & 15)] = acc[i][j][r];
+    for (int q = 0; q < 4; ++q) {
+      const bool ok = fused && col + q < p.N;
+      bias_q[j][q] = (ok && e.bias) ? e.bias[(long long)(col + q) * e.bias_s[3]] : 0.f;
+      alpha_q[j][q] = (ok && e.activation == TFHIP_PRELU) ? e.prelu[(long long)(col + q) * e.prelu_s[3]] : 0.f;
     }
-    lds_barrier();
-    // One float4 of the band per lane and trip. The trip loop stays rolled: the
-    // activation code is large and an unrolled epilogue would not fit the
-    // instruction cache.
-    const bool staged = e.addressing == kChannel;   // bias / PReLU weights sit in LDS, indexed by tile column
-    for (int idx = tid; idx < T::EPI_ROWS * kColGroups; idx += 256) {
-      const int lr = idx / kColGroups, lc = (idx - lr * kColGroups) * 4;
-      const int row = m0 + band0 + lr, col = n0 + lc;
-      if (row >= p.M || col >= p.N) continue;
-      const float4 v = *reinterpret_cast<const float4 *>(lds_c + lr * T::LDC + lc);
-      const float in[4] = {v.x, v.y, v.z, v.w};
-      float bq[4] = {0.f, 0.f, 0.f, 0.f}, pq[4] = {0.f, 0.f, 0.f, 0.f};
-      if (staged) {
-        const float4 b4 = *reinterpret_cast<const float4 *>(lds_bias + lc);
-        const float4 p4 = *reinterpret_cast<const float4 *>(lds_prelu + lc);
-        bq[0] = b4.x; bq[1] = b4.y; bq[2] = b4.z; bq[3] = b4.w;
-        pq[0] = p4.x; pq[1] = p4.y; pq[2] = p4.z; pq[3] = p4.w;
-      } else {
-        long long n = 0, oh = 0, ow = 0;
-        if (e.addressing == kConv) {
-          ow = row % e.out_w;
-          const int t2 = row / e.out_w;
-          oh = t2 % e.out_h;
-          n = t2 / e.out_h;
-        }
+  }
+  auto write_out = [&](auto act_tag) {
+    constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          if (col + q < p.N) {
-            if (e.bias) bq[q] = e.bias[operand_index(e, 0, bz, row, col + q, n, oh, ow)];
-            if (e.activation == TFHIP_PRELU) pq[q] = e.prelu[operand_index(e, 1, bz, row, col + q, n, oh, ow)];
-          }
-        }
-      }
-      float out[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) out[q] = activate(in[q] + bq[q], e.activation, pq[q], e.leaky_alpha);
-      if (p.vec_store) {
-        *reinterpret_cast<float4 *>(C + (long long)row * p.ldc + col) = make_float4(out[0], out[1], out[2], out[3]);
-      } else if (e.addressing == kConv) {
+    for (int i = 0; i < T::TM; ++i) {
+      const int row = m0 + wm0 + i * 16 + lane_m;
+      if (row >= p.M) continue;
+      long long base = (long long)row * p.ldc, col_stride = 1;
+      if (e.addressing == kConv) {
         const int ow = row % e.out_w;
         const int t2 = row / e.out_w;
-        const long long base = (long long)(t2 / e.out_h) * e.y_s[0] + (long long)(t2 % e.out_h) * e.y_s[1] + ow * e.y_s[2];
+        base = (long long)(t2 / e.out_h) * e.y_s[0] + (long long)(t2 % e.out_h) * e.y_s[1] + ow * e.y_s[2];
+        col_stride = e.y_s[3];
+      }
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          if (col + q < p.N) C[base + (col + q) * e.y_s[3]] = out[q];
-      } else {
+      for (int j = 0; j < T::TN; ++j) {
+        const int col = n0 + wn0 + j * 16 + lane_n;
+        if (col >= p.N) continue;
+        float out[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          if (col + q < p.N) C[(long long)row * p.ldc + col + q] = out[q];
+        for (int q = 0; q < 4; ++q) {
+          const float v = acc[i][j][q] + bias_q[j][q];
+          if (ACT == TFHIP_RELU) {
+            out[q] = (v > 0.f || v != v) ? v : 0.f;
+          } else if (ACT == TFHIP_RELU6) {
+            const float t = (v > 0.f || v != v) ? v : 0.f;
+            out[q] = t > 6.f ? 6.f : t;
+          } else if (ACT == TFHIP_PRELU) {
+            out[q] = v < 0.f ? alpha_q[j][q] * v : v;
+          } else if (ACT == TFHIP_LEAKYRELU) {
+            out[q] = v < 0.f ? (float)(e.leaky_alpha * (double)v) : v;
+          } else {
+            out[q] = v;
+          }
+        }
+        if (p.vec_store) {
+          *reinterpret_cast<float4 *>(C + base + col) = make_float4(out[0], out[1], out[2], out[3]);
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (col + q < p.N) C[base + (col + q) * col_stride] = out[q];
+        }
       }
     }
+  };
+  switch (fused ? e.activation : TFHIP_LINEAR) {
+    case TFHIP_RELU: write_out(std::integral_constant<int, TFHIP_RELU>()); break;
+    case TFHIP_RELU6: write_out(std::integral_constant<int, TFHIP_RELU6>()); break;
+    case TFHIP_PRELU: write_out(std::integral_constant<int, TFHIP_PRELU>()); break;
+    case TFHIP_LEAKYRELU: write_out(std::integral_constant<int, TFHIP_LEAKYRELU>()); break;
+    default: write_out(std::integral_constant<int, TFHIP_LINEAR>()); break;
+  }
+}
+
+// Completes in place an output that gemm_kernel stored as raw sums: bias with
+// any broadcast shape and any activation, one element per thread and trip.
+static __global__ __launch_bounds__(256) void gemm_finish(GemmParams p) {
+  const Epilogue &e = p.epi;
+  const long long per_batch = (long long)p.M * p.N;
+  const long long total = per_batch * p.batch;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+    const long long bz = idx / per_batch;
+    const long long rem = idx - bz * per_batch;
+    const long long row = rem / p.N, col = rem - row * p.N;
+    long long n = 0, oh = 0, ow = 0;
+    long long at = bz * p.c_batch_stride + row * p.ldc + col;
+    if (e.addressing == kConv) {
+      ow = row % e.out_w;
+      const long long t2 = row / e.out_w;
+      oh = t2 % e.out_h;
+      n = t2 / e.out_h;
+      at = n * e.y_s[0] + oh * e.y_s[1] + ow * e.y_s[2] + col * e.y_s[3];
+    }
+    p.c[at] = finish(e, p.c[at], bz, row, col, n, oh, ow);
   }
 }
 
