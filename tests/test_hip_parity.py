@@ -267,6 +267,32 @@ def test_depthwise_linearity_full_size(hip):
     assert np.abs(y - y12).max() <= 1e-4
 
 
+@pytest.mark.parametrize("splits", [2, 3, 5])
+@pytest.mark.parametrize("act,bias_shape", [("relu", (70,)), ("sigmoid", (33, 70)), ("linear", None)])
+def test_matmul_split_k(hip, orc, monkeypatch, splits, act, bias_shape):
+    # K cut into slices summed through the workspace; ragged last slice and ragged tiles
+    monkeypatch.setenv("TFHIP_SPLITK", str(splits))
+    rng = np.random.default_rng(41 + splits)
+    a = rng.uniform(-1, 1, (2, 33, 203)).astype(np.float32)
+    b = rng.uniform(-1, 1, (2, 203, 70)).astype(np.float32)
+    bias = None if bias_shape is None else rng.uniform(-1, 1, bias_shape).astype(np.float32)
+    kw = dict(bias=bias, activation=act)
+    assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
+
+
+@pytest.mark.parametrize("fmt", ["NHWC", "NCHW"])
+def test_conv2d_split_k(hip, orc, monkeypatch, fmt):
+    monkeypatch.setenv("TFHIP_SPLITK", "3")
+    rng = np.random.default_rng(43)
+    x = rng.uniform(-1, 1, (2, 9, 7, 16)).astype(np.float32)
+    w = rng.normal(0, 0.3, (3, 3, 16, 12)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (12,)).astype(np.float32)
+    if fmt == "NCHW":
+        x = np.ascontiguousarray(x.transpose(0, 3, 1, 2))
+    kw = dict(pad="same", strides=1, data_format=fmt, bias=bias, activation="relu6")
+    assert_parity(hip.fused_conv2d(x, w, **kw), orc.fused_conv2d(x, w, **kw))
+
+
 # ---------------------------------------------------------------------- dequant
 
 @pytest.mark.parametrize("bits", [8, 16])

@@ -25,6 +25,8 @@ enum Status {
 bool initialised();
 hipStream_t stream();
 int num_cus();
+// Device scratch of at least `bytes` (nullptr if it cannot be allocated); valid until the next call.
+void *workspace(size_t bytes);
 
 // True when [p, p + bytes) lies inside one live block (own or external).
 bool range_is_live(const void *p, size_t bytes);

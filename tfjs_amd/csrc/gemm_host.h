@@ -2,6 +2,7 @@
 // choice and the launch of one gemm_kernel instantiation.
 #pragma once
 
+#include <math.h>
 #include <stdlib.h>
 
 #include "common.h"
@@ -67,14 +68,63 @@ inline int launch_gemm(GemmParams &p) {
   using T = GemmTile<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>;
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
-  const long long grid = (long long)p.tiles_m * p.tiles_n * p.batch;
-  if (grid <= 0) return kOk;
+  const long long tiles = (long long)p.tiles_m * p.tiles_n * p.batch;
+  if (tiles <= 0) return kOk;
+  // Split K when the tiles alone leave compute units idle and K is long: each
+  // copy of the tile set sums a slice of k into the workspace and gemm_finish
+  // adds the slices. Time model (us): fixed + k tiles on the busiest compute unit
+  // x tile time, plus the second kernel.
+  p.splits = 1;
+  p.k_per_split = p.K;
+  p.ws = nullptr;
+  {
+    const int k_tiles = (p.K + BK - 1) / BK;
+    const double tile_us = (BM / 16) * (BN / 16) / 4 * (BK / 4) * 32 / 2400.0 / 0.63;
+    const int cus = num_cus();
+    int best = 1;
+    double best_us = 0;
+    for (int s = 1; s <= 8; ++s) {
+      if (s > 1 && k_tiles / s < 6) break;
+      // the busiest compute unit runs `rounds` workgroups of `kt` k tiles each; a
+      // unit holding several at once gains little (measured about 8%)
+      const long long rounds = (tiles * s + cus - 1) / cus;
+      const int kt = (k_tiles + s - 1) / s;
+      const double us = 5.5 + (double)rounds * kt * tile_us / (rounds > 1 ? 1.08 : 1.0) +
+                        (s > 1 ? 4.0 + 2e-6 * p.M * p.N * p.batch * s : 0);
+      if (s == 1 || us < best_us * 0.93) {   // split further only for a clear gain
+        best_us = us;
+        best = s;
+      }
+    }
+    const char *env = getenv("TFHIP_SPLITK");   // tuning / test override
+    const int forced = env ? atoi(env) : 0;
+    if (forced > 0 && forced <= 64 && forced <= k_tiles) best = forced;
+    if (best > 1) {
+      const size_t bytes = (size_t)best * p.batch * p.M * p.N * sizeof(float);
+      float *ws = bytes <= (size_t(1) << 30) ? static_cast<float *>(workspace(bytes)) : nullptr;
+      if (ws) {
+        p.splits = best;
+        p.k_per_split = ((k_tiles + best - 1) / best) * BK;
+        p.ws = ws;
+      }
+    }
+  }
+  const long long grid = tiles * p.splits;
+  {
+    // ids resident together on one XCD: its share of the grid, at most two
+    // workgroups on each of its 32 compute units
+    const long long per_xcd = grid / 8 < 1 ? 1 : grid / 8;
+    const double together = (double)(per_xcd < 64 ? per_xcd : 64);
+    int g = (int)(sqrt(together * BN / BM) + 0.5);
+    g = g < 1 ? 1 : g;
+    p.group_m = g > p.tiles_m ? p.tiles_m : g;
+  }
   if (grid > 0x7fffffffLL) return fail(kBadArgument, "gemm: %lld tiles exceed the grid limit", grid);
   note_kernel("gemm_kernel<%d, %d, %d, %d, %d, %d, %d>", BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND);
   // The fused epilogue covers per-column operands with a relu-family activation;
   // anything else leaves raw sums for gemm_finish.
   const Epilogue &e = p.epi;
-  p.inline_epilogue = e.channel_operands && (e.activation <= TFHIP_LEAKYRELU);
+  p.inline_epilogue = p.splits == 1 && e.channel_operands && (e.activation <= TFHIP_LEAKYRELU);
   if (p.inline_epilogue) {
     TFHIP_LAUNCH((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>
                   <<<dim3((unsigned)grid), dim3(256), T::LDS_FLOATS * sizeof(float), stream()>>>(p)));

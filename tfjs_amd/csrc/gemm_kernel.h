@@ -86,6 +86,11 @@ struct GemmParams {
   // bytes addressable from the (per-batch) base of each operand, for the buffer descriptors
   unsigned a_bytes, b_bytes;
   int tiles_m, tiles_n;
+  int group_m;    // tile rows per panel of the tile numbering
+  // split K: the grid holds `splits` copies of the tile set, copy s sums
+  // k in [s * k_per_split, (s+1) * k_per_split) into ws[s][batch][M][N]
+  int splits, k_per_split;
+  float *ws;
   int vec_store;  // rows of C are 16-byte aligned and N % 4 == 0
   int inline_epilogue;  // bias + activation happen in gemm_kernel (else gemm_finish completes the raw sums)
   ConvGeom conv;
@@ -124,6 +129,13 @@ struct GemmTile {
 template <int BK>
 __device__ __forceinline__ constexpr int swizzle_of(int k) {
   return BK == 32 ? (((k >> 2) & 7) << 2) : (((k >> 2) & 3) << 3);
+}
+
+__device__ __forceinline__ const float *uniform_pointer(const float *ptr) {
+  const unsigned long long v = reinterpret_cast<unsigned long long>(ptr);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v);
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+  return reinterpret_cast<const float *>(((unsigned long long)hi << 32) | lo);
 }
 
 __device__ __forceinline__ float4 as_float4(uint4_t v) {
@@ -246,9 +258,11 @@ __device__ __forceinline__ void load_tile(float4 (&reg)[VECS], const LoaderState
 
 // Writes the registers fetched by load_tile into a k-major LDS tile [BK][LD].
 template <int BX, int BK, int LD, int KIND, bool SWZ, int VECS>
-__device__ __forceinline__ void store_tile(float *__restrict__ lds, const float4 (&reg)[VECS], int tid) {
+__device__ __forceinline__ void store_tile(float *__restrict__ lds, const float4 (&reg)[VECS], int tid,
+                                           int first = 0, int last = VECS) {
 #pragma unroll
   for (int i = 0; i < VECS; ++i) {
+    if (i < first || i >= last) continue;
     const int f = tid + i * 256;
     if ((BX * BK / 4) % 256 != 0 && f >= BX * BK / 4) continue;
     if (KIND == kLoadXVec) {
@@ -292,14 +306,29 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     if (per_xcd > 0 && id < per_xcd * 8) id = (id % 8) * per_xcd + id / 8;
   }
   const int tiles_per_batch = p.tiles_m * p.tiles_n;
+  const int split = id / (tiles_per_batch * p.batch);
+  id -= split * tiles_per_batch * p.batch;
   const int bz = id / tiles_per_batch;
   const int t = id - bz * tiles_per_batch;
-  const int tile_m = t / p.tiles_n, tile_n = t - tile_m * p.tiles_n;
+  const int k_begin = split * p.k_per_split;
+  const int k_end = k_begin + p.k_per_split < p.K ? k_begin + p.k_per_split : p.K;
+  // Tiles are numbered in panels of group_m tile rows, column by column inside a
+  // panel, so that the run of consecutive ids that is resident on one XCD covers
+  // a near-square block of C: the rows of A and columns of B it needs per k tile
+  // are as few as possible and stay in that XCD's L2.
+  const int width = p.group_m * p.tiles_n;
+  const int first_m = (t / width) * p.group_m;
+  const int gsz = p.tiles_m - first_m < p.group_m ? p.tiles_m - first_m : p.group_m;
+  const int in_group = t % width;
+  const int tile_m = first_m + in_group % gsz, tile_n = in_group / gsz;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-  const float *A = p.a + (long long)(bz % p.batch_a) * p.a_batch_stride;
-  const float *B = p.b + (long long)(bz % p.batch_b) * p.b_batch_stride;
-  float *C = p.c + (long long)bz * p.c_batch_stride;
+  // The operand bases are the same for the whole workgroup; readfirstlane pins
+  // them to scalar registers so that the buffer descriptors built from them are
+  // scalar too (a descriptor the compiler believes to vary per lane makes it
+  // wrap every buffer load in a loop over the distinct values).
+  const float *A = uniform_pointer(p.a + (long long)(bz % p.batch_a) * p.a_batch_stride);
+  const float *B = uniform_pointer(p.b + (long long)(bz % p.batch_b) * p.b_batch_stride);
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)A, 0, (int)p.a_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void *)B, 0, (int)p.b_bytes, 0x00020000);
 
@@ -331,7 +360,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   // is needed, so the loop tolerates D tile-times of memory latency.
   constexpr int D = T::PREFETCH;
   float4 ra[D][T::A_VECS], rb[D][T::B_VECS];
-  const int k_tiles = (p.K + BK - 1) / BK;
+  const int k_tiles = (k_end - k_begin + BK - 1) / BK;
 
   // Every fetch below is unconditional: a tile past K reads as zeros through
   // the buffer descriptor at no memory cost, and with no branch around a load
@@ -339,18 +368,18 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   // (a conditional load makes it assume the shortest queue and wait for all).
 #pragma unroll
   for (int d = 0; d < D; ++d) {
-    load_tile<BM, BK, A_KIND, T::A_VECS>(ra[d], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, d * BK, tid, p.conv);
-    load_tile<BN, BK, B_KIND, T::B_VECS>(rb[d], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, d * BK, tid, p.conv);
+    load_tile<BM, BK, A_KIND, T::A_VECS>(ra[d], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0, k_begin + d * BK, tid, p.conv);
+    load_tile<BN, BK, B_KIND, T::B_VECS>(rb[d], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0, k_begin + d * BK, tid, p.conv);
   }
   store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a, ra[0], tid);
   store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b, rb[0], tid);
-  load_tile<BM, BK, A_KIND, T::A_VECS>(ra[0], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, D * BK, tid, p.conv);
-  load_tile<BN, BK, B_KIND, T::B_VECS>(rb[0], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, D * BK, tid, p.conv);
+  load_tile<BM, BK, A_KIND, T::A_VECS>(ra[0], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0, k_begin + D * BK, tid, p.conv);
+  load_tile<BN, BK, B_KIND, T::B_VECS>(rb[0], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0, k_begin + D * BK, tid, p.conv);
   lds_barrier();
 
   // One k tile: tile kt sits in LDS buffer u & 1 (kt and u have the same parity),
   // tile kt+1 in ring slot (u+1) % D.
-  auto tile_step = [&](int kt, auto u_tag) {
+  auto tile_step = [&](int kt, auto u_tag) __attribute__((always_inline)) {
     constexpr int u = decltype(u_tag)::value;
     constexpr int cur = u & 1;
     constexpr int nxt = (u + 1) % D;
@@ -358,48 +387,67 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     float fa[2][T::TM], fb[2][T::TN];
     load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[0], a_lane, a_off, 0);
     load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[0], b_lane, b_off, 0);
+    // Side work of the tile, cut into pieces that are dealt out over the k steps
+    // (LDS serves the four waves in order: a burst of tile stores in one step
+    // would hold up the fragment reads queued behind it):
+    //   pieces 0 .. A_VECS-1            one 16-byte vector of tile kt+1 -> LDS (A)
+    //   pieces A_VECS .. A_VECS+B_VECS-1  the same for B
+    //   then the global fetches of tile kt+1+D into the ring slot just drained,
+    //   A and B as one piece each.
+    // Tile kt+1 goes to the other LDS buffer, free since the barrier that ended
+    // tile kt-1.
+    constexpr int kSteps = BK / 4;
+    constexpr int kPieces = T::A_VECS + T::B_VECS + 2;
+    constexpr int kPerStep = (kPieces + kSteps - 1) / kSteps;
 #pragma unroll
-    for (int s = 0; s < BK / 4; ++s) {
-      if (s + 1 < BK / 4) {
+    for (int s = 0; s < kSteps; ++s) {
+      if (s + 1 < kSteps) {
         load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[(s + 1) & 1], a_lane, a_off, (s + 1) * 4);
         load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[(s + 1) & 1], b_lane, b_off, (s + 1) * 4);
       }
-      if (s == 0) {
-        // tile kt+1 goes to the other LDS buffer (free since the barrier that
-        // ended tile kt-1) at the start of the tile, so the stores finish under
-        // the matrix work instead of in front of the closing barrier
-        store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a + (cur ^ 1) * T::A_BUF, ra[nxt], tid);
-        store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b + (cur ^ 1) * T::B_BUF, rb[nxt], tid);
-      } else if (s == 1) {
-        // its ring slot is refilled with tile kt+1+D, one operand per k step
-        load_tile<BM, BK, A_KIND, T::A_VECS>(ra[nxt], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, p.K, m0, (kt + 1 + D) * BK,
-                                             tid, p.conv);
-      } else if (s == 2) {
-        load_tile<BN, BK, B_KIND, T::B_VECS>(rb[nxt], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, p.K, n0, (kt + 1 + D) * BK,
-                                             tid, p.conv);
+#pragma unroll
+      for (int piece = s * kPerStep; piece < (s + 1) * kPerStep && piece < kPieces; ++piece) {
+        if (piece < T::A_VECS) {
+          if (!(TFHIP_EXP & 2))
+            store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a + (cur ^ 1) * T::A_BUF, ra[nxt], tid, piece,
+                                                                    piece + 1);
+        } else if (piece < T::A_VECS + T::B_VECS) {
+          if (!(TFHIP_EXP & 2))
+            store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b + (cur ^ 1) * T::B_BUF, rb[nxt], tid,
+                                                                    piece - T::A_VECS, piece - T::A_VECS + 1);
+        } else if (piece == T::A_VECS + T::B_VECS) {
+          if (!(TFHIP_EXP & 1))
+            load_tile<BM, BK, A_KIND, T::A_VECS>(ra[nxt], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0,
+                                                 k_begin + (kt + 1 + D) * BK, tid, p.conv);
+        } else {
+          if (!(TFHIP_EXP & 1))
+            load_tile<BN, BK, B_KIND, T::B_VECS>(rb[nxt], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0,
+                                                 k_begin + (kt + 1 + D) * BK, tid, p.conv);
+        }
       }
 #pragma unroll
       for (int i = 0; i < T::TM; ++i)
 #pragma unroll
         for (int j = 0; j < T::TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb[s & 1][j], fa[s & 1][i], acc[i][j], 0, 0, 0);
-    }
-    // Issue order for the whole tile: after every matrix instruction a little of
-    // the side work (next fragments from LDS, the LDS stores of tile kt+1, the
-    // global fetches of tile kt+1+D and their address arithmetic), so that it
-    // issues in the shadow of the matrix pipe instead of in a block in front of
-    // it. A wave issues in order: side work that is not interleaved is exposed
-    // whenever a SIMD holds a single wave.
+      // Issue order inside the step: after every matrix instruction a little of
+      // the side work, so that it issues in the shadow of the matrix pipe. A wave
+      // issues in order: side work in a block in front of the MFMAs is exposed
+      // whenever a SIMD holds a single wave.
 #pragma unroll
-    for (int m = 0; m < (BK / 4) * T::TM * T::TN; ++m) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
-      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // one LDS write
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one global read
-      __builtin_amdgcn_sched_group_barrier(0x006, 3, 0);   // a few vector / scalar ALU
+      for (int m = 0; m < T::TM * T::TN; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // one LDS write
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one global read
+        __builtin_amdgcn_sched_group_barrier(0x006, 3, 0);   // a few vector / scalar ALU
+      }
+      __builtin_amdgcn_sched_barrier(0);   // steps stay in order
     }
     __builtin_amdgcn_sched_barrier(0);   // nothing of this tile moves past its closing barrier
+#if !(TFHIP_EXP & 4)
     lds_barrier();
+#endif
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -423,6 +471,12 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   const Epilogue &e = p.epi;
   const int lane_m = lane & 15, lane_n = (lane >> 4) * 4;
   const bool fused = p.inline_epilogue != 0;
+  // destination: the output itself, or this split's dense [M][N] slab of the workspace
+  const bool to_ws = p.splits > 1;
+  float *C = to_ws ? p.ws + ((long long)split * p.batch + bz) * p.M * p.N : p.c + (long long)bz * p.c_batch_stride;
+  const long long ldc = to_ws ? p.N : p.ldc;
+  const bool conv_addr = !to_ws && e.addressing == kConv;
+  const bool vec = to_ws ? p.N % 4 == 0 : p.vec_store != 0;
   float bias_q[T::TN][4], alpha_q[T::TN][4];
 #pragma unroll
   for (int j = 0; j < T::TN; ++j) {
@@ -434,14 +488,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
       alpha_q[j][q] = (ok && e.activation == TFHIP_PRELU) ? e.prelu[(long long)(col + q) * e.prelu_s[3]] : 0.f;
     }
   }
-  auto write_out = [&](auto act_tag) {
+  auto write_out = [&](auto act_tag) __attribute__((always_inline)) {
     constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
     for (int i = 0; i < T::TM; ++i) {
       const int row = m0 + wm0 + i * 16 + lane_m;
       if (row >= p.M) continue;
-      long long base = (long long)row * p.ldc, col_stride = 1;
-      if (e.addressing == kConv) {
+      long long base = (long long)row * ldc, col_stride = 1;
+      if (conv_addr) {
         const int ow = row % e.out_w;
         const int t2 = row / e.out_w;
         base = (long long)(t2 / e.out_h) * e.y_s[0] + (long long)(t2 % e.out_h) * e.y_s[1] + ow * e.y_s[2];
@@ -468,7 +522,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
             out[q] = v;
           }
         }
-        if (p.vec_store) {
+        if (vec) {
           *reinterpret_cast<float4 *>(C + base + col) = make_float4(out[0], out[1], out[2], out[3]);
         } else {
 #pragma unroll
@@ -487,8 +541,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   }
 }
 
-// Completes in place an output that gemm_kernel stored as raw sums: bias with
-// any broadcast shape and any activation, one element per thread and trip.
+// Completes an output that gemm_kernel left as raw sums (in place, or as split-K
+// partial slabs in the workspace): bias with any broadcast shape and any
+// activation, one element per thread and trip.
 static __global__ __launch_bounds__(256) void gemm_finish(GemmParams p) {
   const Epilogue &e = p.epi;
   const long long per_batch = (long long)p.M * p.N;
@@ -507,7 +562,15 @@ static __global__ __launch_bounds__(256) void gemm_finish(GemmParams p) {
       n = t2 / e.out_h;
       at = n * e.y_s[0] + oh * e.y_s[1] + ow * e.y_s[2] + col * e.y_s[3];
     }
-    p.c[at] = finish(e, p.c[at], bz, row, col, n, oh, ow);
+    float v;
+    if (p.splits > 1) {
+      // partial sums in ascending k order
+      v = p.ws[idx];
+      for (int sp = 1; sp < p.splits; ++sp) v += p.ws[(long long)sp * total + idx];
+    } else {
+      v = p.c[at];
+    }
+    p.c[at] = finish(e, v, bz, row, col, n, oh, ow);
   }
 }
 

@@ -30,6 +30,8 @@ struct Runtime {
   hipEvent_t staging_done[kStagingBuffers] = {nullptr, nullptr};
   bool staging_busy[kStagingBuffers] = {false, false};
   int next_staging = 0;
+  void *workspace = nullptr;
+  size_t workspace_bytes = 0;
   hipEvent_t events[TFHIP_MAX_EVENTS] = {};
   bool event_recorded[TFHIP_MAX_EVENTS] = {};
 };
@@ -81,6 +83,25 @@ int launch_repeat() { return g_repeat; }
 bool initialised() { return g.ready; }
 hipStream_t stream() { return g.stream; }
 int num_cus() { return g.prop.multiProcessorCount; }
+
+// Scratch for kernels that need device memory beyond their operands (split-K
+// partial sums). One block that only grows; work on the single stream is
+// ordered, so consecutive launches may share it.
+void *workspace(size_t bytes) {
+  if (bytes <= g.workspace_bytes) return g.workspace;
+  (void)hipStreamSynchronize(g.stream);   // a launch in flight may still use the old block
+  if (g.workspace) (void)hipFree(g.workspace);
+  g.workspace = nullptr;
+  g.workspace_bytes = 0;
+  const size_t want = (bytes + (size_t(1) << 24) - 1) & ~((size_t(1) << 24) - 1);
+  if (hipMalloc(&g.workspace, want) != hipSuccess) {
+    (void)hipGetLastError();
+    g.workspace = nullptr;
+    return nullptr;
+  }
+  g.workspace_bytes = want;
+  return g.workspace;
+}
 
 bool range_is_live(const void *p, size_t bytes) {
   std::lock_guard<std::mutex> lock(g_mutex);
@@ -149,6 +170,9 @@ int tfhip_shutdown(void) {
     g.events[i] = nullptr;
     g.event_recorded[i] = false;
   }
+  if (g.workspace) (void)hipFree(g.workspace);
+  g.workspace = nullptr;
+  g.workspace_bytes = 0;
   (void)hipStreamDestroy(g.stream);
   g.stream = nullptr;
   g.ready = false;
