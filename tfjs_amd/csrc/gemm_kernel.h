@@ -15,10 +15,11 @@
 //   XOR swizzle of the x index by the k group keeps those scattered writes
 //   conflict-free too.
 // * Software pipeline: a ring of registers keeps the global loads of the next
-//   2 or 4 tiles in flight (buffer loads: out-of-range lanes read zero, no
-//   branches); tile t+1 moves from its ring slot to the other LDS buffer just
-//   before the last k step of tile t; LDS fragments of k step s+1 are fetched
-//   while the MFMAs of step s issue. One barrier per tile.
+//   three tiles in flight (buffer loads: out-of-range lanes read zero, no
+//   branches); tile t+1 moves from its ring slot to one of three LDS buffers
+//   during the first k steps of tile t; LDS fragments of k step s+1 (also across
+//   the tile boundary) are fetched while the MFMAs of step s issue. One
+//   LDS-only barrier per tile, in the middle of the tile.
 // * The two MFMA operands are passed swapped (the instruction computes the
 //   transposed block), so a lane ends up with four consecutive COLUMNS of one
 //   output row: the epilogue applies bias + activation in registers and writes
@@ -47,9 +48,6 @@
 
 #include "epilogue.h"
 
-#ifndef TFHIP_EXP
-#define TFHIP_EXP 0
-#endif
 namespace tfhip {
 
 // Workgroup barrier that orders LDS traffic only. __syncthreads() also fences
@@ -119,9 +117,13 @@ struct GemmTile {
   static constexpr int A_VECS = (BM * BK / 4 + kThreads - 1) / kThreads;
   static constexpr int B_VECS = (BN * BK / 4 + kThreads - 1) / kThreads;
   static constexpr int A_BUF = BK * LDA, B_BUF = BK * LDB;
-  // tiles in flight between global memory and LDS (even, see the main loop)
-  static constexpr int PREFETCH = (A_VECS + B_VECS) * 4 * 4 <= 96 ? 4 : 2;
-  static constexpr int LDS_FLOATS = 2 * (A_BUF + B_BUF);
+  // three tiles in flight between global memory and LDS, three LDS buffers
+  static constexpr int PREFETCH = 3;
+  // LDS fragments are fetched FRAG_DEPTH-1 k steps ahead of their use. A k step
+  // is TM*TN MFMAs of 32 cycles: a small wave tile needs more steps of distance to
+  // cover the LDS round trip (well over 128 cycles when several waves queue).
+  static constexpr int FRAG_DEPTH = TM * TN >= 12 ? 2 : (TM * TN >= 6 ? 3 : 4);
+  static constexpr int LDS_FLOATS = 3 * (A_BUF + B_BUF);
 };
 
 // XOR applied to the x index of LDS row k: the k group (k / 4) spread over the
@@ -295,8 +297,8 @@ template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int A_KIND, int B_KI
 __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   using T = GemmTile<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>;
   extern __shared__ float lds[];
-  float *lds_a = lds;                   // [2][BK][LDA]
-  float *lds_b = lds + 2 * T::A_BUF;    // [2][BK][LDB]
+  float *lds_a = lds;                   // [3][BK][LDA]
+  float *lds_b = lds + 3 * T::A_BUF;    // [3][BK][LDB]
 
   // Workgroup id -> (batch, tile_m, tile_n). Ids i, i+8, i+16, ... share an XCD;
   // give each XCD one contiguous band of the tile sequence.
@@ -356,80 +358,102 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 #pragma unroll
     for (int j = 0; j < T::TN; ++j) acc[i][j] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-  // Register ring of D tiles in flight: tile t is fetched D iterations before it
-  // is needed, so the loop tolerates D tile-times of memory latency.
+  // Software pipeline over k tiles, three deep at both levels:
+  //  * registers: tile t lives in ring slot t % 3 from its global fetch (issued
+  //    while tile t-4 computes) until it is stored to LDS (while tile t-1 computes)
+  //  * LDS: tile t lives in buffer t % 3. It is written during the first k steps of
+  //    tile t-1, ONE barrier in the middle of tile t-1 publishes it, and the last k
+  //    step of tile t-1 already fetches its first fragments, so no wave ever waits
+  //    for LDS at a tile boundary. The buffer it overwrites held tile t-3, which
+  //    every wave finished before it reached the barrier inside tile t-2.
   constexpr int D = T::PREFETCH;
   float4 ra[D][T::A_VECS], rb[D][T::B_VECS];
   const int k_tiles = (k_end - k_begin + BK - 1) / BK;
 
-  // Every fetch below is unconditional: a tile past K reads as zeros through
-  // the buffer descriptor at no memory cost, and with no branch around a load
-  // the compiler can count exactly how many loads may stay in flight at each use
-  // (a conditional load makes it assume the shortest queue and wait for all).
+  // Every fetch is unconditional: a tile past K reads as zeros through the buffer
+  // descriptor at no memory cost, and with no branch around a load the compiler
+  // can count exactly how many loads may stay in flight at each use (a
+  // conditional load makes it assume the shortest queue and wait for all).
 #pragma unroll
   for (int d = 0; d < D; ++d) {
-    load_tile<BM, BK, A_KIND, T::A_VECS>(ra[d], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0, k_begin + d * BK, tid, p.conv);
-    load_tile<BN, BK, B_KIND, T::B_VECS>(rb[d], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0, k_begin + d * BK, tid, p.conv);
+    load_tile<BM, BK, A_KIND, T::A_VECS>(ra[d], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0, k_begin + d * BK, tid,
+                                         p.conv);
+    load_tile<BN, BK, B_KIND, T::B_VECS>(rb[d], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0, k_begin + d * BK, tid,
+                                         p.conv);
   }
   store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a, ra[0], tid);
   store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b, rb[0], tid);
-  load_tile<BM, BK, A_KIND, T::A_VECS>(ra[0], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0, k_begin + D * BK, tid, p.conv);
-  load_tile<BN, BK, B_KIND, T::B_VECS>(rb[0], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0, k_begin + D * BK, tid, p.conv);
+  load_tile<BM, BK, A_KIND, T::A_VECS>(ra[0], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0, k_begin + D * BK, tid,
+                                       p.conv);
+  load_tile<BN, BK, B_KIND, T::B_VECS>(rb[0], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0, k_begin + D * BK, tid,
+                                       p.conv);
   lds_barrier();
 
-  // One k tile: tile kt sits in LDS buffer u & 1 (kt and u have the same parity),
-  // tile kt+1 in ring slot (u+1) % D.
+  // ring of fragments: k step g (counted through all tiles) uses slot g % F and
+  // was fetched F-1 steps earlier, across tile boundaries too
+  constexpr int F = T::FRAG_DEPTH;
+  float fa[F][T::TM], fb[F][T::TN];
+#pragma unroll
+  for (int f = 0; f < F - 1; ++f) {
+    load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[f], a_lane, 0, f * 4);
+    load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[f], b_lane, 0, f * 4);
+  }
+
+  // Side work of a tile, cut into pieces that are dealt out over its k steps (LDS
+  // serves the four waves in order: a burst of tile stores in one step would hold
+  // up the fragment reads queued behind it):
+  //   pieces 0 .. A_VECS-1              one 16-byte vector of tile kt+1 -> LDS (A)
+  //   pieces A_VECS .. A_VECS+B_VECS-1  the same for B
+  //   then the global fetches of tile kt+4 into the ring slot just drained, A and
+  //   B as one piece each.
+  constexpr int kSteps = BK / 4;
+  constexpr int kStores = T::A_VECS + T::B_VECS;
+  constexpr int kPieces = kStores + 2;
+  // the stores must be over by step kSteps - F: the steps after it already read
+  // the next tile's fragments
+  constexpr int kEven = (kPieces + kSteps - 1) / kSteps;
+  constexpr int kForStores = (kStores + kSteps - F) / (kSteps - F + 1);
+  constexpr int kPerStep = kEven > kForStores ? kEven : kForStores;
+  constexpr int kBarrierStep = (kStores - 1) / kPerStep;   // the step that holds the last store
+  static_assert(F - 1 <= kSteps && kBarrierStep <= kSteps - F, "fragments of the next tile are read after the barrier");
+  static_assert((3 * kSteps) % F == 0, "fragment slots are compile-time over a group of three tiles");
+
+  // One k tile: tile kt sits in LDS buffer u = kt % 3, tile kt+1 in ring slot (u+1) % 3.
   auto tile_step = [&](int kt, auto u_tag) __attribute__((always_inline)) {
     constexpr int u = decltype(u_tag)::value;
-    constexpr int cur = u & 1;
-    constexpr int nxt = (u + 1) % D;
-    const int a_off = cur * T::A_BUF, b_off = cur * T::B_BUF;
-    float fa[2][T::TM], fb[2][T::TN];
-    load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[0], a_lane, a_off, 0);
-    load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[0], b_lane, b_off, 0);
-    // Side work of the tile, cut into pieces that are dealt out over the k steps
-    // (LDS serves the four waves in order: a burst of tile stores in one step
-    // would hold up the fragment reads queued behind it):
-    //   pieces 0 .. A_VECS-1            one 16-byte vector of tile kt+1 -> LDS (A)
-    //   pieces A_VECS .. A_VECS+B_VECS-1  the same for B
-    //   then the global fetches of tile kt+1+D into the ring slot just drained,
-    //   A and B as one piece each.
-    // Tile kt+1 goes to the other LDS buffer, free since the barrier that ended
-    // tile kt-1.
-    constexpr int kSteps = BK / 4;
-    constexpr int kPieces = T::A_VECS + T::B_VECS + 2;
-    constexpr int kPerStep = (kPieces + kSteps - 1) / kSteps;
+    constexpr int nb = (u + 1) % 3;
+    const int a_off = u * T::A_BUF, b_off = u * T::B_BUF;
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
-      if (s + 1 < kSteps) {
-        load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[(s + 1) & 1], a_lane, a_off, (s + 1) * 4);
-        load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[(s + 1) & 1], b_lane, b_off, (s + 1) * 4);
+      constexpr int kAhead = F - 1;
+      const int slot_now = (u * kSteps + s) % F, slot_ahead = (u * kSteps + s + kAhead) % F;
+      if (s + kAhead < kSteps) {
+        load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[slot_ahead], a_lane, a_off, (s + kAhead) * 4);
+        load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[slot_ahead], b_lane, b_off, (s + kAhead) * 4);
+      } else {
+        load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[slot_ahead], a_lane, nb * T::A_BUF, (s + kAhead - kSteps) * 4);
+        load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[slot_ahead], b_lane, nb * T::B_BUF, (s + kAhead - kSteps) * 4);
       }
 #pragma unroll
       for (int piece = s * kPerStep; piece < (s + 1) * kPerStep && piece < kPieces; ++piece) {
         if (piece < T::A_VECS) {
-          if (!(TFHIP_EXP & 2))
-            store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a + (cur ^ 1) * T::A_BUF, ra[nxt], tid, piece,
-                                                                    piece + 1);
-        } else if (piece < T::A_VECS + T::B_VECS) {
-          if (!(TFHIP_EXP & 2))
-            store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b + (cur ^ 1) * T::B_BUF, rb[nxt], tid,
-                                                                    piece - T::A_VECS, piece - T::A_VECS + 1);
-        } else if (piece == T::A_VECS + T::B_VECS) {
-          if (!(TFHIP_EXP & 1))
-            load_tile<BM, BK, A_KIND, T::A_VECS>(ra[nxt], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0,
-                                                 k_begin + (kt + 1 + D) * BK, tid, p.conv);
+          store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a + nb * T::A_BUF, ra[nb], tid, piece, piece + 1);
+        } else if (piece < kStores) {
+          store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b + nb * T::B_BUF, rb[nb], tid,
+                                                                  piece - T::A_VECS, piece - T::A_VECS + 1);
+        } else if (piece == kStores) {
+          load_tile<BM, BK, A_KIND, T::A_VECS>(ra[nb], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0,
+                                               k_begin + (kt + 1 + D) * BK, tid, p.conv);
         } else {
-          if (!(TFHIP_EXP & 1))
-            load_tile<BN, BK, B_KIND, T::B_VECS>(rb[nxt], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0,
-                                                 k_begin + (kt + 1 + D) * BK, tid, p.conv);
+          load_tile<BN, BK, B_KIND, T::B_VECS>(rb[nb], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0,
+                                               k_begin + (kt + 1 + D) * BK, tid, p.conv);
         }
       }
 #pragma unroll
       for (int i = 0; i < T::TM; ++i)
 #pragma unroll
         for (int j = 0; j < T::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb[s & 1][j], fa[s & 1][i], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb[slot_now][j], fa[slot_now][i], acc[i][j], 0, 0, 0);
       // Issue order inside the step: after every matrix instruction a little of
       // the side work, so that it issues in the shadow of the matrix pipe. A wave
       // issues in order: side work in a block in front of the MFMAs is exposed
@@ -443,28 +467,23 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
         __builtin_amdgcn_sched_group_barrier(0x006, 3, 0);   // a few vector / scalar ALU
       }
       __builtin_amdgcn_sched_barrier(0);   // steps stay in order
+      if (s == kBarrierStep) {
+        lds_barrier();                     // tile kt+1 is complete in LDS
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
-    __builtin_amdgcn_sched_barrier(0);   // nothing of this tile moves past its closing barrier
-#if !(TFHIP_EXP & 4)
-    lds_barrier();
-#endif
-    __builtin_amdgcn_sched_barrier(0);
   };
 
-  // Full groups of D tiles run without a branch between them; the remainder
-  // (fewer than D tiles) follows with one check per tile.
+  // Full groups of three tiles run without a branch between them; the remainder
+  // (one or two tiles) follows with one check per tile.
   int kt = 0;
-  for (; kt + D <= k_tiles; kt += D) {
+  for (; kt + 3 <= k_tiles; kt += 3) {
     tile_step(kt, std::integral_constant<int, 0>());
     tile_step(kt + 1, std::integral_constant<int, 1>());
-    if (D > 2) {
-      tile_step(kt + 2, std::integral_constant<int, 2 % D>());
-      tile_step(kt + 3, std::integral_constant<int, 3 % D>());
-    }
+    tile_step(kt + 2, std::integral_constant<int, 2>());
   }
   if (kt < k_tiles) tile_step(kt, std::integral_constant<int, 0>());
   if (kt + 1 < k_tiles) tile_step(kt + 1, std::integral_constant<int, 1>());
-  if (D > 2 && kt + 2 < k_tiles) tile_step(kt + 2, std::integral_constant<int, 2 % D>());
 
   // ---- epilogue: registers -> global. Lane l of a 16x16 block holds row l % 16,
   // columns 4 * (l / 16) .. +3 (the operands went into the MFMA swapped).
