@@ -280,6 +280,26 @@ def test_matmul_split_k(hip, orc, monkeypatch, splits, act, bias_shape):
     assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
 
 
+@pytest.mark.parametrize("act,bias_shape", [("relu6", (16,)), ("linear", None), ("sigmoid", (16,)), ("prelu", "per_column"),
+                                            ("relu", ())])
+@pytest.mark.parametrize("xs,fs,stride,dil,pad", [
+    ((2, 13, 11, 3), (3, 3, 3, 16), 2, 1, "same"), ((1, 9, 10, 1), (5, 3, 1, 16), 1, 2, "same"),
+    ((2, 8, 8, 4), (3, 3, 4, 16), (1, 2), 1, "valid"), ((1, 7, 6, 2), (2, 2, 2, 16), 1, 1, [[0, 0], [1, 0], [0, 2], [0, 0]]),
+])
+def test_conv2d_few_input_channels(hip, orc, xs, fs, stride, dil, pad, act, bias_shape):
+    # the direct stem kernel: one to four input channels, every epilogue form
+    rng = np.random.default_rng(47)
+    x = rng.uniform(-1, 1, xs).astype(np.float32)
+    w = rng.normal(0, 0.4, fs).astype(np.float32)
+    if bias_shape == "per_column":   # a bias that varies along the output width as well
+        out_w = orc.fused_conv2d(x, w, strides=stride, dilations=dil, pad=pad).shape[2]
+        bias_shape = (out_w, 16)
+    kw = dict(strides=stride, dilations=dil, pad=pad, activation=act,
+              bias=None if bias_shape is None else rng.uniform(-1, 1, bias_shape).astype(np.float32),
+              prelu=rng.uniform(0, 1, (16,)).astype(np.float32) if act == "prelu" else None)
+    assert_parity(hip.fused_conv2d(x, w, **kw), orc.fused_conv2d(x, w, **kw))
+
+
 @pytest.mark.parametrize("fmt", ["NHWC", "NCHW"])
 def test_conv2d_split_k(hip, orc, monkeypatch, fmt):
     monkeypatch.setenv("TFHIP_SPLITK", "3")

@@ -12,6 +12,94 @@
 
 using namespace tfhip;
 
+namespace {
+
+// Direct convolution for images with very few input channels (a network stem:
+// 3 channels, K = 27). The implicit GEMM wastes most of a k tile on such a
+// short contraction and gathers the image element by element; here one lane
+// owns one output pixel and OC output channels in registers, the image values
+// are fetched once per tap, and the filter values are the same for every lane,
+// so they come through the scalar cache as instruction operands. Taps
+// accumulate in the reference's order (filter row, column, input channel:
+// tfjs-backend-cpu/src/kernels/Conv2D.ts:64-96), out-of-range taps are skipped
+// like there. NHWC, per-channel bias and relu-family activations only; other
+// forms take the implicit GEMM.
+struct FewChannelsArgs {
+  const float *x, *w, *bias;
+  float *y;
+  long long xs_n, xs_h, xs_w, bias_stride;
+  int M, out_c, in_h, in_w, in_c, f_h, f_w, stride_h, stride_w, dil_h, dil_w, pad_top, pad_left, out_h, out_w;
+  int activation;   // linear, relu or relu6
+};
+
+template <int OC>
+__global__ __launch_bounds__(256) void conv_few_channels(FewChannelsArgs g) {
+  const int m = blockIdx.x * 256 + threadIdx.x;
+  if (m >= g.M) return;
+  const int oc0 = blockIdx.y * OC;
+  const int ow = m % g.out_w;
+  const int t2 = m / g.out_w;
+  const int oh = t2 % g.out_h, n = t2 / g.out_h;
+  const float *__restrict__ x = g.x + (long long)n * g.xs_n;
+  const float *__restrict__ w = g.w + oc0;
+  float acc[OC], bias[OC];
+#pragma unroll
+  for (int o = 0; o < OC; ++o) acc[o] = bias[o] = 0.f;
+  if (g.bias) {   // the same values in every lane; fetched ahead of the taps
+#pragma unroll
+    for (int o = 0; o < OC; ++o) bias[o] = g.bias[(long long)(oc0 + o) * g.bias_stride];
+  }
+  for (int r = 0; r < g.f_h; ++r) {
+    const int ih = oh * g.stride_h - g.pad_top + r * g.dil_h;
+    for (int s = 0; s < g.f_w; ++s) {
+      const int iw = ow * g.stride_w - g.pad_left + s * g.dil_w;
+      const bool inside = ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
+      const float *xp = x + (inside ? (long long)ih * g.xs_h + (long long)iw * g.xs_w : 0);
+      for (int c = 0; c < g.in_c; ++c) {
+        const float xv = xp[c];
+        const float *wk = w + (long long)((r * g.f_w + s) * g.in_c + c) * g.out_c;   // the same address in every lane
+        if (inside) {
+#pragma unroll
+          for (int o = 0; o < OC; ++o) acc[o] = fmaf(xv, wk[o], acc[o]);
+        }
+      }
+    }
+  }
+  float *y = g.y + (long long)m * g.out_c + oc0;
+#pragma unroll
+  for (int o = 0; o < OC; o += 4) {
+    float q[4] = {acc[o], acc[o + 1], acc[o + 2], acc[o + 3]};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      q[k] += bias[o + k];
+      if (g.activation != TFHIP_LINEAR) {
+        q[k] = (q[k] > 0.f || q[k] != q[k]) ? q[k] : 0.f;   // Math.max(0, x): NaN stays, -0 becomes +0
+        if (g.activation == TFHIP_RELU6 && q[k] > 6.f) q[k] = 6.f;
+      }
+    }
+    *reinterpret_cast<float4 *>(y + o) = make_float4(q[0], q[1], q[2], q[3]);
+  }
+}
+
+template <int OC>
+int launch_few_channels(const GemmParams &p, int f_h) {
+  const ConvGeom &c = p.conv;
+  FewChannelsArgs g;
+  g.x = p.a; g.w = p.b; g.y = p.c;
+  g.bias = p.epi.bias; g.bias_stride = p.epi.bias ? p.epi.bias_s[3] : 0;
+  g.xs_n = c.xs_n; g.xs_h = c.xs_h; g.xs_w = c.xs_w;
+  g.M = p.M; g.out_c = p.N; g.in_h = c.in_h; g.in_w = c.in_w; g.in_c = c.in_c; g.f_h = f_h; g.f_w = c.f_w;
+  g.stride_h = c.stride_h; g.stride_w = c.stride_w; g.dil_h = c.dil_h; g.dil_w = c.dil_w;
+  g.pad_top = c.pad_top; g.pad_left = c.pad_left; g.out_h = c.out_h; g.out_w = c.out_w;
+  g.activation = p.epi.activation;
+  dim3 grid((unsigned)((p.M + 255) / 256), (unsigned)(p.N / OC), 1);
+  note_kernel("conv_few_channels<%d>", OC);
+  TFHIP_LAUNCH((conv_few_channels<OC><<<grid, 256, 0, stream()>>>(g)));
+  return kOk;
+}
+
+}  // namespace
+
 extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y, int64_t batch, int64_t in_h,
                                   int64_t in_w, int64_t in_c, int64_t f_h, int64_t f_w, int64_t out_c,
                                   int64_t stride_h, int64_t stride_w, int64_t dilation_h, int64_t dilation_w,
@@ -82,6 +170,12 @@ extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
   if (pointwise) {
     p.a_sx = in_c; p.a_sk = 1;
     return launch_plain_gemm(p, false, false, vec);
+  }
+  if (!nchw && in_c <= 4 && out_c % 8 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+      p.epi.channel_operands && activation <= TFHIP_RELU6) {
+    if (out_c % 32 == 0) return launch_few_channels<32>(p, (int)f_h);
+    if (out_c % 16 == 0) return launch_few_channels<16>(p, (int)f_h);
+    return launch_few_channels<8>(p, (int)f_h);
   }
   if (vec) {
     const int shape = choose_tile_shape(M, out_c, K, 1, num_cus());
