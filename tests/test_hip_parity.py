@@ -267,6 +267,27 @@ def test_depthwise_linearity_full_size(hip):
     assert np.abs(y - y12).max() <= 1e-4
 
 
+@pytest.mark.parametrize("m,n,k,act", [(24600, 24, 144, "linear"), (30001, 96, 16, "relu6"), (98309, 192, 32, "relu"),
+                                        (25000, 64, 196, "prelu"), (24576, 16, 36, "leakyrelu"), (98500, 144, 24, "relu6"),
+                                        (24600, 80, 100, "linear"), (24600, 24, 144, "sigmoid")])
+def test_matmul_tall_small_b(hip, orc, m, n, k, act):
+    # tall products with a small B take the streaming kernel (sigmoid: falls back to the tiled one)
+    rng = np.random.default_rng(m + n + k)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 0.3, (k, n)).astype(np.float32)
+    kw = dict(bias=rng.uniform(-1, 1, (n,)).astype(np.float32), activation=act,
+              prelu=rng.uniform(0, 1, (n,)).astype(np.float32) if act == "prelu" else None, leakyrelu_alpha=0.1)
+    assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
+
+
+def test_pointwise_conv_tall(hip, orc):
+    rng = np.random.default_rng(53)
+    x = rng.uniform(0, 1, (14, 87, 86, 24)).astype(np.float32)
+    w = rng.normal(0, 0.3, (1, 1, 24, 144)).astype(np.float32)
+    kw = dict(pad="same", bias=rng.uniform(-1, 1, (144,)).astype(np.float32), activation="relu6")
+    assert_parity(hip.fused_conv2d(x, w, **kw), orc.fused_conv2d(x, w, **kw))
+
+
 @pytest.mark.parametrize("splits", [2, 3, 5])
 @pytest.mark.parametrize("act,bias_shape", [("relu", (70,)), ("sigmoid", (33, 70)), ("linear", None)])
 def test_matmul_split_k(hip, orc, monkeypatch, splits, act, bias_shape):

@@ -1,0 +1,239 @@
+// Streaming GEMM for tall products with a small B: C[M x N] = A[M x K] * B[K x N]
+// with M in the tens of thousands and K * N small enough for B to sit in LDS
+// (the pointwise convolutions of a mobile network: N = 16 .. 192, K = 16 .. 576).
+//
+// Such a product is bound by reading A and writing C once. The tiled kernel
+// spends its time in per-tile set-up instead (a two- or three-step k loop never
+// fills its pipeline), so this kernel turns the loop around:
+//  * B is transposed into LDS once per workgroup and stays there.
+//  * Each wavefront walks over blocks of 16 rows of A. A lane fetches its part of
+//    A straight from global memory as float4 along k, no LDS in between: the
+//    matrix instruction only needs both operands of a lane to belong to the same
+//    k, so lane (g, r) (g = lane / 16, r = lane % 16) takes k = 16t + 4g + j for
+//    the j-th of four consecutive instructions, which is exactly the float4 it
+//    loaded, and reads the matching B[k][.] from LDS, also as one float4.
+//  * The loads of the next 64 k (or of the next row block) are in flight while
+//    the current ones are consumed.
+//  * Operands are passed swapped, as in gemm_kernel.h, so a lane ends with four
+//    consecutive columns of one row and writes float4s after bias + activation.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <type_traits>
+
+#include "common.h"
+#include "gemm_kernel.h"
+
+namespace tfhip {
+
+struct SkinnyArgs {
+  const float *a, *b, *bias;
+  float *c;
+  long long bias_stride;
+  double leaky_alpha;
+  int M, N, K, k_pad;   // k_pad: K rounded up to 64
+  unsigned a_bytes;
+  int activation;
+};
+
+constexpr int kSkinnyChunk = 64;   // k per pipeline step: four float4 per lane
+
+// WAVES wavefronts per workgroup share one copy of B.
+template <int TN, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
+  constexpr int kThreads = WAVES * 64;
+  extern __shared__ float lds_bt[];          // [16 * TN][k_pad + 16]: B transposed, zero padded
+  const int pitch = g.k_pad + 16;            // rows 16 banks apart: float4 reads of a wave spread over all banks
+  const int tid = threadIdx.x;
+  // B -> LDS, transposed. Columns >= N and rows >= K read as zero; rows beyond
+  // the last 16-row group that holds real data are never read. Consecutive lanes
+  // take consecutive k (conflict-free LDS stores; B itself is small and cached),
+  // and eight fetches are issued before the first is stored, so the fill costs
+  // one or two memory round trips instead of one per element.
+  {
+    const int kk = ((g.K + 15) / 16) * 16;
+    const int items = kk * (16 * TN / 4);
+    for (int i0 = tid; i0 < items; i0 += kThreads * 8) {
+      float4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * kThreads;
+        const int c = (i / kk) * 4, k = i - (i / kk) * kk;
+        v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i < items && k < g.K && c < g.N) v[u] = *reinterpret_cast<const float4 *>(g.b + (long long)k * g.N + c);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * kThreads;
+        if (i >= items) continue;
+        const int c = (i / kk) * 4, k = i - (i / kk) * kk;
+        lds_bt[(c + 0) * pitch + k] = v[u].x;
+        lds_bt[(c + 1) * pitch + k] = v[u].y;
+        lds_bt[(c + 2) * pitch + k] = v[u].z;
+        lds_bt[(c + 3) * pitch + k] = v[u].w;
+      }
+    }
+  }
+  __syncthreads();
+
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = lane >> 4, r = lane & 15;
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)uniform_pointer(g.a), 0, (int)g.a_bytes, 0x00020000);
+
+  const int blocks = (g.M + 15) / 16;
+  const int first = blockIdx.x * WAVES + wave, step = gridDim.x * WAVES;
+  const int chunks = g.k_pad / kSkinnyChunk;
+  const int my_blocks = first < blocks ? (blocks - first + step - 1) / step : 0;
+  const int total = my_blocks * chunks;
+
+  // per-lane epilogue operands: four consecutive columns of each 16-column group
+  float bias_q[TN][4];
+#pragma unroll
+  for (int n = 0; n < TN; ++n)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int col = n * 16 + grp * 4 + q;
+      bias_q[n][q] = (g.bias && col < g.N) ? g.bias[(long long)col * g.bias_stride] : 0.f;
+    }
+
+  // loads of one step: k = c * 64 + 16 t + 4 grp .. +3 of row b * 16 + r
+  auto issue = [&](float4 (&dst)[4], int b, int c) __attribute__((always_inline)) {
+    const int row = b * 16 + r;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int k = c * kSkinnyChunk + 16 * t + 4 * grp;
+      const unsigned off = (row < g.M && k < g.K) ? (unsigned)(((long long)row * g.K + k) * 4) : kNoOffset;
+      dst[t] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
+    }
+  };
+
+  // Two accumulators per column group when there are few groups: consecutive
+  // matrix instructions then never wait for each other's result.
+  constexpr int NA = TN <= 2 ? 2 : 1;
+  float4_t acc[NA][TN];
+#pragma unroll
+  for (int h = 0; h < NA; ++h)
+#pragma unroll
+    for (int n = 0; n < TN; ++n) acc[h][n] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+  float4 cur[4], nxt[4];
+  if (total > 0) issue(cur, first, 0);
+  int b = first, c = 0;
+  for (int q = 0; q < total; ++q) {
+    int nb = b, nc = c + 1;
+    if (nc == chunks) {
+      nc = 0;
+      nb = b + step;
+    }
+    issue(nxt, q + 1 < total ? nb : blocks, nc);   // past the end: every offset is out of range, nothing is read
+
+    const float *bt = lds_bt + r * pitch + c * kSkinnyChunk + 4 * grp;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (c * kSkinnyChunk + 16 * t >= g.K) continue;   // nothing but padding (the same for all lanes)
+      const float a4[4] = {cur[t].x, cur[t].y, cur[t].z, cur[t].w};
+      float4 b4[TN];
+#pragma unroll
+      for (int n = 0; n < TN; ++n) b4[n] = *reinterpret_cast<const float4 *>(bt + n * 16 * pitch + 16 * t);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int n = 0; n < TN; ++n) {
+          const float bv = j == 0 ? b4[n].x : (j == 1 ? b4[n].y : (j == 2 ? b4[n].z : b4[n].w));
+          acc[j % NA][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(bv, a4[j], acc[j % NA][n], 0, 0, 0);
+        }
+      }
+    }
+
+    if (c == chunks - 1) {
+      // the row block is complete: lane holds row b*16 + r, columns n*16 + 4*grp .. +3
+      const int row = b * 16 + r;
+#pragma unroll
+      for (int n = 0; n < TN; ++n) {
+        const int col = n * 16 + grp * 4;
+        float out[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          float v = (NA == 2 ? acc[0][n][k] + acc[NA - 1][n][k] : acc[0][n][k]) + bias_q[n][k];
+          switch (g.activation) {
+            case TFHIP_RELU: v = (v > 0.f || v != v) ? v : 0.f; break;
+            case TFHIP_RELU6: v = (v > 0.f || v != v) ? v : 0.f; v = v > 6.f ? 6.f : v; break;
+            case TFHIP_LEAKYRELU: v = v < 0.f ? (float)(g.leaky_alpha * (double)v) : v; break;
+            default: break;
+          }
+          out[k] = v;
+        }
+        if (row < g.M && col < g.N)
+          *reinterpret_cast<float4 *>(g.c + (long long)row * g.N + col) = make_float4(out[0], out[1], out[2], out[3]);
+#pragma unroll
+        for (int h = 0; h < NA; ++h) acc[h][n] = (float4_t){0.f, 0.f, 0.f, 0.f};
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) cur[t] = nxt[t];
+    b = nb;
+    c = nc;
+  }
+}
+
+// Instantiated widths in groups of 16 columns (0: too wide).
+inline int skinny_groups(int n) {
+  const int tn = (n + 15) / 16;
+  return tn <= 4 ? tn : (tn <= 6 ? 6 : (tn <= 9 ? 9 : (tn <= 12 ? 12 : 0)));
+}
+
+// True when the product fits this kernel: row-major operands, float4-aligned,
+// per-column bias with linear / relu / relu6 / leakyrelu, B small enough
+// for LDS and enough rows to keep every wavefront streaming.
+inline bool skinny_applies(const GemmParams &p, bool transpose_a, bool transpose_b, bool vec) {
+  if (transpose_a || transpose_b || !vec || p.batch != 1) return false;
+  if (p.K % 4 != 0 || p.N % 4 != 0 || !p.vec_store || p.ldc != p.N) return false;
+  if (p.epi.addressing == kConv && !p.vec_store) return false;
+  if (!p.epi.channel_operands || p.epi.activation > TFHIP_LEAKYRELU || p.epi.activation == TFHIP_PRELU) return false;
+  const int tn = skinny_groups(p.N);
+  if (tn == 0 || p.a_bytes == 0) return false;
+  // enough 16-row blocks per wavefront to pay for the B fill (a wide B costs more)
+  if (p.M < (tn >= 9 ? 98304 : 24576)) return false;
+  const long long k_pad = (p.K + kSkinnyChunk - 1) / kSkinnyChunk * kSkinnyChunk;
+  return 16LL * tn * (k_pad + 16) * 4 <= 64 * 1024;
+}
+
+template <int TN>
+inline int launch_skinny_tn(const SkinnyArgs &g) {
+  // Workgroups of four wavefronts, three per compute unit, measured best: fatter
+  // workgroups fill B fewer times but start later and pipeline less.
+  constexpr int WAVES = 4;
+  const int blocks = (g.M + 15) / 16;
+  const size_t lds = (size_t)16 * TN * (g.k_pad + 16) * sizeof(float);
+  long long grid = (blocks + WAVES - 1) / WAVES;
+  const long long cap = (long long)num_cus() * 3;
+  if (grid > cap) grid = cap;
+  note_kernel("skinny_gemm<%d>", TN);
+  TFHIP_LAUNCH((skinny_gemm<TN, WAVES><<<dim3((unsigned)grid), dim3(WAVES * 64), lds, stream()>>>(g)));
+  return kOk;
+}
+
+inline int launch_skinny(const GemmParams &p) {
+  SkinnyArgs g;
+  g.a = p.a; g.b = p.b; g.c = p.c;
+  g.bias = p.epi.bias; g.bias_stride = p.epi.bias ? p.epi.bias_s[3] : 0;
+  g.leaky_alpha = p.epi.leaky_alpha;
+  g.M = p.M; g.N = p.N; g.K = p.K;
+  g.k_pad = (p.K + kSkinnyChunk - 1) / kSkinnyChunk * kSkinnyChunk;
+  g.a_bytes = p.a_bytes;
+  g.activation = p.epi.activation;
+  switch (skinny_groups(p.N)) {
+    case 1: return launch_skinny_tn<1>(g);
+    case 2: return launch_skinny_tn<2>(g);
+    case 3: return launch_skinny_tn<3>(g);
+    case 4: return launch_skinny_tn<4>(g);
+    case 6: return launch_skinny_tn<6>(g);
+    case 9: return launch_skinny_tn<9>(g);
+    default: return launch_skinny_tn<12>(g);
+  }
+}
+
+}  // namespace tfhip
