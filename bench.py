@@ -49,16 +49,18 @@ BATCH = 32
 # cannot be read from inside this script, so the table is refreshed by hand when a
 # kernel changes; a symbol that is not listed reports null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "gemm_kernel<256, 32, 16, 4, 1, 4, 2>": 71218476,
-    "depthwise_3x3_rows<1,0>": 38791876,
-    "gemm_kernel<256, 16, 16, 4, 1, 0, 1>": 46572946,
-    "gemm_kernel<64, 96, 16, 2, 2, 0, 1>": 180058853,
-    "depthwise_3x3_rows<2,0>": 89025911,
-    "gemm_kernel<256, 32, 16, 4, 1, 0, 1>": 73976888,
-    "add_same_shape": 8326066,
-    "gemm_kernel<64, 64, 16, 2, 2, 0, 1>": 16900669,
-    "gemm_kernel<64, 64, 32, 2, 2, 0, 1>": 12874294,
-    "mean_hw": 8230159,
+    "conv_few_channels<32>": 77618041,
+    "depthwise_3x3_rows<1, false>": 38797745,
+    "skinny_gemm<1, 4>": 77197966,
+    "skinny_gemm<6, 4>": 180156082,
+    "depthwise_3x3_rows<2, false>": 89027371,
+    "skinny_gemm<2, 4>": 36045454,
+    "skinny_gemm<9, 4>": 70617637,
+    "add_same_shape": 8326073,
+    "gemm_kernel<64, 64, 16, 2, 2, 0, 1>": 17208388,
+    "gemm_kernel<64, 64, 32, 2, 2, 0, 1>": 13545318,
+    "gemm_finish": 3865670,
+    "mean_hw": 8230203,
 }
 
 

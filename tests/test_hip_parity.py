@@ -39,6 +39,20 @@ def orc():
     return pyoracle
 
 
+@pytest.fixture
+def tuning(hip):
+    """Sets kernel-selection overrides for one test and restores the heuristics after it."""
+    from tfjs_amd.capi import check, load_library
+    lib, used = load_library(), []
+
+    def set_knob(name, value):
+        check(lib.tfhip_set_tuning(name.encode(), value))
+        used.append(name)
+    yield set_knob
+    for name in used:
+        check(lib.tfhip_set_tuning(name.encode(), -1))
+
+
 def assert_parity(got, want, tol=TOL):
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     assert got.shape == want.shape, "%s vs %s" % (got.shape, want.shape)
@@ -246,9 +260,9 @@ def test_depthwise_epilogue_forms(hip, orc, act, bias_shape, prelu_shape, stride
 
 @pytest.mark.parametrize("rows", [1, 2, 3, 5, 7, 16])
 @pytest.mark.parametrize("stride,pad", [(1, "same"), (2, "same"), (1, "valid"), (2, "valid")])
-def test_depthwise_row_chunks(hip, orc, monkeypatch, rows, stride, pad):
+def test_depthwise_row_chunks(hip, orc, tuning, rows, stride, pad):
     # every chunk length of the row pipeline, ragged last chunk and ragged last column strip
-    monkeypatch.setenv("TFHIP_DW_ROWS", str(rows))
+    tuning("dw_rows", rows)
     rng = np.random.default_rng(31 + rows)
     x = rng.uniform(-1, 1, (2, 23, 13, 12)).astype(np.float32)
     w = rng.normal(0, 0.5, (3, 3, 12, 1)).astype(np.float32)
@@ -290,9 +304,9 @@ def test_pointwise_conv_tall(hip, orc):
 
 @pytest.mark.parametrize("splits", [2, 3, 5])
 @pytest.mark.parametrize("act,bias_shape", [("relu", (70,)), ("sigmoid", (33, 70)), ("linear", None)])
-def test_matmul_split_k(hip, orc, monkeypatch, splits, act, bias_shape):
+def test_matmul_split_k(hip, orc, tuning, splits, act, bias_shape):
     # K cut into slices summed through the workspace; ragged last slice and ragged tiles
-    monkeypatch.setenv("TFHIP_SPLITK", str(splits))
+    tuning("splitk", splits)
     rng = np.random.default_rng(41 + splits)
     a = rng.uniform(-1, 1, (2, 33, 203)).astype(np.float32)
     b = rng.uniform(-1, 1, (2, 203, 70)).astype(np.float32)
@@ -322,8 +336,8 @@ def test_conv2d_few_input_channels(hip, orc, xs, fs, stride, dil, pad, act, bias
 
 
 @pytest.mark.parametrize("fmt", ["NHWC", "NCHW"])
-def test_conv2d_split_k(hip, orc, monkeypatch, fmt):
-    monkeypatch.setenv("TFHIP_SPLITK", "3")
+def test_conv2d_split_k(hip, orc, tuning, fmt):
+    tuning("splitk", 3)
     rng = np.random.default_rng(43)
     x = rng.uniform(-1, 1, (2, 9, 7, 16)).astype(np.float32)
     w = rng.normal(0, 0.3, (3, 3, 16, 12)).astype(np.float32)

@@ -71,6 +71,11 @@ bool range_is_live(const void *p, size_t bytes);
 void note_kernel(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 int launch_repeat();
 
+// Tuning overrides (tfhip_set_tuning, or TFHIP_<NAME> in the environment at
+// tfhip_init): -1 when unset.
+enum TuningKey { kTuneTile = 0, kTuneSplitK, kTuneDwRows, kTuneDwHalo, kTuneNoSkinny, kTuneCount };
+int tuning(int key);
+
 // Enqueues `launch_expr` launch_repeat() times and checks the launch.
 #define TFHIP_LAUNCH(launch_expr)                                  \
   do {                                                             \

@@ -469,13 +469,13 @@ extern "C" int tfhip_fused_depthwise_conv2d(
                     batch <= 65535;
   // the row pipeline addresses both tensors with 32-bit byte offsets
   const bool fits32 = batch * in_h * in_w * in_c * 4 <= 0xfffffff0LL && total * 4 <= 0xfffffff0LL;
-  if (fast && fits32 && !getenv("TFHIP_DW_HALO")) {
+  if (fast && fits32 && tuning(kTuneDwHalo) <= 0) {
     const int S = (int)stride_h;
     DwRowsArgs g;
     g.c4_total = (int)(in_c / 4);
     g.strips_w = ((int)out_w + kRowsPW - 1) / kRowsPW;
     int rows = choose_rows((int)batch, (int)in_h, (int)in_w, (int)in_c, (int)out_h, (int)out_w, S, num_cus());
-    if (const char *env = getenv("TFHIP_DW_ROWS")) rows = atoi(env);   // tuning override
+    if (tuning(kTuneDwRows) > 0) rows = tuning(kTuneDwRows);   // tuning override
     rows = rows < 1 ? 1 : (rows > 32 ? 32 : rows);
     if (rows > out_h) rows = (int)out_h;
     g.rows = balanced_tile((int)out_h, rows);
@@ -487,7 +487,7 @@ extern "C" int tfhip_fused_depthwise_conv2d(
     if (blocks_x <= 0x7fffffffLL) {
       dim3 grid((unsigned)blocks_x, (g.c4_total + kCQ - 1) / kCQ, 1);
       const bool general = !(e.addressing == kChannel && activation <= TFHIP_RELU6);
-      note_kernel("depthwise_3x3_rows<%d,%d>", S, (int)general);
+      note_kernel("depthwise_3x3_rows<%d, %s>", S, general ? "true" : "false");
       if (S == 1 && !general)
         TFHIP_LAUNCH((depthwise_3x3_rows<1, false><<<grid, 256, 0, stream()>>>(p, e, g)));
       else if (S == 1)

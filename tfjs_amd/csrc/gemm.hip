@@ -6,7 +6,7 @@
 using namespace tfhip;
 
 int tfhip::launch_plain_gemm(GemmParams &p, bool transpose_a, bool transpose_b, bool vec) {
-  if (skinny_applies(p, transpose_a, transpose_b, vec) && !getenv("TFHIP_NO_SKINNY")) return launch_skinny(p);
+  if (skinny_applies(p, transpose_a, transpose_b, vec) && tuning(kTuneNoSkinny) <= 0) return launch_skinny(p);
   if (vec) {
     const int shape = choose_tile_shape(p.M, p.N, p.K, p.batch, num_cus());
     if (!transpose_a && !transpose_b) return launch_gemm_shape<kLoadKVec, kLoadXVec>(shape, p);

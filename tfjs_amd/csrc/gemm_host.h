@@ -44,12 +44,9 @@ inline double estimate_us(const TileShape &t, long long M, long long N, long lon
 }
 
 // Picks the tile shape with the lowest estimated run time.
-// TFHIP_TILE=<index> in the environment overrides the choice (tuning aid).
+// The "tile" tuning knob overrides the choice.
 inline int choose_tile_shape(long long M, long long N, long long K, long long batch, int cus) {
-  static const int forced = [] {
-    const char *e = getenv("TFHIP_TILE");
-    return e ? atoi(e) : -1;
-  }();
+  const int forced = tuning(kTuneTile);
   if (forced >= 0 && forced < kNumTileShapes) return forced;
   int best = 0;
   double best_us = 0;
@@ -96,8 +93,7 @@ inline int launch_gemm(GemmParams &p) {
         best = s;
       }
     }
-    const char *env = getenv("TFHIP_SPLITK");   // tuning / test override
-    const int forced = env ? atoi(env) : 0;
+    const int forced = tuning(kTuneSplitK);   // tuning / test override
     if (forced > 0 && forced <= 64 && forced <= k_tiles) best = forced;
     if (best > 1) {
       const size_t bytes = (size_t)best * p.batch * p.M * p.N * sizeof(float);

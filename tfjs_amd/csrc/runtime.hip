@@ -80,6 +80,19 @@ void note_kernel(const char *fmt, ...) {
 
 int launch_repeat() { return g_repeat; }
 
+int g_tuning[kTuneCount] = {-1, -1, -1, -1, -1};
+const char *const kTuningNames[kTuneCount] = {"tile", "splitk", "dw_rows", "dw_halo", "no_skinny"};
+int tuning(int key) { return g_tuning[key]; }
+
+void read_tuning_from_environment() {
+  static const char *const env_names[kTuneCount] = {"TFHIP_TILE", "TFHIP_SPLITK", "TFHIP_DW_ROWS", "TFHIP_DW_HALO",
+                                                    "TFHIP_NO_SKINNY"};
+  for (int i = 0; i < kTuneCount; ++i) {
+    const char *e = getenv(env_names[i]);
+    g_tuning[i] = e ? atoi(e) : -1;
+  }
+}
+
 bool initialised() { return g.ready; }
 hipStream_t stream() { return g.stream; }
 int num_cus() { return g.prop.multiProcessorCount; }
@@ -144,6 +157,7 @@ int tfhip_init(int device) {
     g.staging_busy[i] = false;
   }
   g.device = device;
+  read_tuning_from_environment();
   g.ready = true;
   return kOk;
 }
@@ -319,6 +333,16 @@ int tfhip_download(void *host, const void *src, size_t src_offset, size_t bytes)
     done += chunk;
   }
   return kOk;
+}
+
+int tfhip_set_tuning(const char *name, int value) {
+  for (int i = 0; name && i < kTuneCount; ++i) {
+    if (strcmp(name, kTuningNames[i]) == 0) {
+      g_tuning[i] = value < 0 ? -1 : value;
+      return kOk;
+    }
+  }
+  return fail(kBadArgument, "tfhip_set_tuning: unknown knob '%s'", name ? name : "(null)");
 }
 
 int tfhip_set_launch_repeat(int n) {

@@ -211,7 +211,7 @@ inline int launch_skinny_tn(const SkinnyArgs &g) {
   long long grid = (blocks + WAVES - 1) / WAVES;
   const long long cap = (long long)num_cus() * 3;
   if (grid > cap) grid = cap;
-  note_kernel("skinny_gemm<%d>", TN);
+  note_kernel("skinny_gemm<%d, %d>", TN, WAVES);
   TFHIP_LAUNCH((skinny_gemm<TN, WAVES><<<dim3((unsigned)grid), dim3(WAVES * 64), lds, stream()>>>(g)));
   return kOk;
 }
