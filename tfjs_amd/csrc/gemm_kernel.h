@@ -7,13 +7,16 @@
 // * Matrix core instruction: v_mfma_f32_16x16x4_f32 (64 lanes compute a 16x16
 //   block over 4 values of k). Lane l feeds A[row l%16][k l/16] and
 //   B[k l/16][col l%16] and receives C[rows 4*(l/16)..+3][col l%16].
-// * Both operands are staged in LDS k-major ("[k][x]", x = row of A or column
-//   of B) with a row pitch congruent to 16 modulo the 32 banks, so the 16 lanes
-//   that share k read 16 consecutive words and the two k rows of a half
-//   wavefront fall in different bank halves: fragment reads never conflict.
-//   Operands that arrive k-contiguous are transposed on the way into LDS; an
-//   XOR swizzle of the x index by the k group keeps those scattered writes
-//   conflict-free too.
+// * Both operands are staged in LDS x-major ("[x][k]", x = row of A or column
+//   of B, k contiguous, row pitch BK + 8 floats). The matrix instruction only
+//   needs the two operands of a lane to belong to the same k, not any particular
+//   k, so lane (g, r) (g = lane / 16, r = lane % 16) takes k = 16T + 4g + j for
+//   the j-th of four consecutive instructions: one 16-byte LDS read per operand
+//   block feeds four MFMAs. (Element-wise fragment reads run at half the LDS
+//   rate of 16-byte reads on this chip and were the bottleneck of the k loop.)
+//   An operand that is k-contiguous in memory goes into LDS with 16-byte stores;
+//   an x-contiguous one is transposed with element stores, consecutive lanes
+//   taking consecutive k so that the stores of a wave cover consecutive banks.
 // * Software pipeline: a ring of registers keeps the global loads of the next
 //   three tiles in flight (buffer loads: out-of-range lanes read zero, no
 //   branches); tile t+1 moves from its ring slot to one of three LDS buffers
@@ -108,30 +111,16 @@ struct GemmTile {
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   static constexpr int TM = WM / 16, TN = WN / 16;
   static_assert(WM % 16 == 0 && WN % 16 == 0, "tile shape");
-  // x index swizzle for operands whose LDS writes are transposing
-  static constexpr bool A_SWZ = A_KIND != kLoadXVec && BM % 32 == 0 && WM % 32 == 0;
-  static constexpr bool B_SWZ = B_KIND != kLoadXVec && BN % 32 == 0 && WN % 32 == 0;
-  static constexpr int LDA = BM % 32 == 0 ? BM + 16 : BM + 32;
-  static constexpr int LDB = BN % 32 == 0 ? BN + 16 : BN + 32;
+  static constexpr int PITCH = BK + 8;   // floats per LDS row: 16-byte fragment reads of a wave spread over all banks
+  static constexpr int QUADS = BK / 16;  // groups of four MFMA k steps fed by one 16-byte read
   // 16-byte fetches per thread per tile (the last round may be partly idle)
   static constexpr int A_VECS = (BM * BK / 4 + kThreads - 1) / kThreads;
   static constexpr int B_VECS = (BN * BK / 4 + kThreads - 1) / kThreads;
-  static constexpr int A_BUF = BK * LDA, B_BUF = BK * LDB;
+  static constexpr int A_BUF = BM * PITCH, B_BUF = BN * PITCH;
   // three tiles in flight between global memory and LDS, three LDS buffers
   static constexpr int PREFETCH = 3;
-  // LDS fragments are fetched FRAG_DEPTH-1 k steps ahead of their use. A k step
-  // is TM*TN MFMAs of 32 cycles: a small wave tile needs more steps of distance to
-  // cover the LDS round trip (well over 128 cycles when several waves queue).
-  static constexpr int FRAG_DEPTH = TM * TN >= 12 ? 2 : (TM * TN >= 6 ? 3 : 4);
   static constexpr int LDS_FLOATS = 3 * (A_BUF + B_BUF);
 };
-
-// XOR applied to the x index of LDS row k: the k group (k / 4) spread over the
-// bank bits the rows of one half wavefront leave free.
-template <int BK>
-__device__ __forceinline__ constexpr int swizzle_of(int k) {
-  return BK == 32 ? (((k >> 2) & 7) << 2) : (((k >> 2) & 3) << 3);
-}
 
 __device__ __forceinline__ const float *uniform_pointer(const float *ptr) {
   const unsigned long long v = reinterpret_cast<unsigned long long>(ptr);
@@ -167,7 +156,7 @@ __device__ __forceinline__ void init_loader(LoaderState<VECS> &st, long long sx,
       const int x = x0 + f / (BK / 4);
       st.row_off[i] = x < X ? (unsigned)((long long)x * sx * 4) : kNoOffset;
     } else if (KIND == kLoadXVec) {
-      const int x = x0 + (f % (BX / 4)) * 4;
+      const int x = x0 + (f / BK) * 4;   // consecutive lanes: consecutive k
       st.row_off[i] = x < X ? (unsigned)(x * 4) : kNoOffset;
     } else if (KIND == kLoadIm2colVec || KIND == kLoadIm2colScalar) {
       const int m = x0 + f / (BK / 4);
@@ -204,7 +193,7 @@ __device__ __forceinline__ void load_tile(float4 (&reg)[VECS], const LoaderState
   } else if (KIND == kLoadXVec) {
 #pragma unroll
     for (int i = 0; i < VECS; ++i) {
-      const int k = k0 + (tid + i * 256) / (BX / 4);
+      const int k = k0 + (tid + i * 256) % BK;
       const unsigned off =
           (k < K && st.row_off[i] != kNoOffset) ? st.row_off[i] + (unsigned)((long long)k * sk * 4) : kNoOffset;
       reg[i] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
@@ -258,8 +247,9 @@ __device__ __forceinline__ void load_tile(float4 (&reg)[VECS], const LoaderState
   }
 }
 
-// Writes the registers fetched by load_tile into a k-major LDS tile [BK][LD].
-template <int BX, int BK, int LD, int KIND, bool SWZ, int VECS>
+// Writes vectors [first, last) of the registers fetched by load_tile into an
+// x-major LDS tile [BX][PITCH].
+template <int BX, int BK, int PITCH, int KIND, int VECS>
 __device__ __forceinline__ void store_tile(float *__restrict__ lds, const float4 (&reg)[VECS], int tid,
                                            int first = 0, int last = VECS) {
 #pragma unroll
@@ -268,37 +258,41 @@ __device__ __forceinline__ void store_tile(float *__restrict__ lds, const float4
     const int f = tid + i * 256;
     if ((BX * BK / 4) % 256 != 0 && f >= BX * BK / 4) continue;
     if (KIND == kLoadXVec) {
-      const int kr = f / (BX / 4), xq = f % (BX / 4);
-      *reinterpret_cast<float4 *>(lds + kr * LD + xq * 4) = reg[i];
-    } else {
-      const int row = f / (BK / 4), kq = f % (BK / 4);
-      const int col = SWZ ? (row ^ swizzle_of<BK>(kq * 4)) : row;   // the swizzle is the same for k .. k+3
-      float *d = lds + (kq * 4) * LD + col;
+      // four consecutive x at one k: transposed, element by element
+      const int k = f % BK, xq = f / BK;
+      float *d = lds + (xq * 4) * PITCH + k;
       d[0] = reg[i].x;
-      d[LD] = reg[i].y;
-      d[2 * LD] = reg[i].z;
-      d[3 * LD] = reg[i].w;
+      d[PITCH] = reg[i].y;
+      d[2 * PITCH] = reg[i].z;
+      d[3 * PITCH] = reg[i].w;
+    } else {
+      // four consecutive k of one row
+      const int row = f / (BK / 4), kq = f % (BK / 4);
+      *reinterpret_cast<float4 *>(lds + row * PITCH + kq * 4) = reg[i];
     }
   }
 }
 
-// Fragment of k step `kk` (a multiple of 4) for NT 16-wide blocks starting at
-// lane_base[.] (the lane's position, pre-XORed for each low swizzle value).
-template <int BK, int LD, int NT, bool SWZ>
-__device__ __forceinline__ void load_fragment(float (&frag)[NT], const float *const (&lane_base)[4], int buf_off,
-                                              int kk) {
-  const int sw = SWZ ? swizzle_of<BK>(kk) : 0;
-  const float *p = lane_base[(sw & 12) >> 2] + buf_off + kk * LD;
+// Fragments of quad `quad` (16 k) for NT blocks of 16 rows: lane (g, r) reads
+// k = 16 quad + 4 g .. +3 of row r of each block. `lane_base` points at the
+// lane's (r, g) position in block 0 of buffer 0.
+template <int PITCH, int NT>
+__device__ __forceinline__ void load_fragment(float4 (&frag)[NT], const float *lane_base, int buf_off, int quad) {
 #pragma unroll
-  for (int t = 0; t < NT; ++t) frag[t] = p[(t * 16) ^ (sw & 16)];
+  for (int t = 0; t < NT; ++t)
+    frag[t] = *reinterpret_cast<const float4 *>(lane_base + buf_off + t * 16 * PITCH + quad * 16);
+}
+
+__device__ __forceinline__ float quad_element(const float4 &v, int j) {
+  return j == 0 ? v.x : (j == 1 ? v.y : (j == 2 ? v.z : v.w));
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int A_KIND, int B_KIND>
 __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   using T = GemmTile<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>;
   extern __shared__ float lds[];
-  float *lds_a = lds;                   // [3][BK][LDA]
-  float *lds_b = lds + 3 * T::A_BUF;    // [3][BK][LDB]
+  float *lds_a = lds;                   // [3][BM][PITCH]
+  float *lds_b = lds + 3 * T::A_BUF;    // [3][BN][PITCH]
 
   // Workgroup id -> (batch, tile_m, tile_n). Ids i, i+8, i+16, ... share an XCD;
   // give each XCD one contiguous band of the tile sequence.
@@ -344,13 +338,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   init_loader<BM, BK, A_KIND, T::A_VECS>(sa, p.a_sx, p.a_sk, p.M, m0, tid, p.conv);
   init_loader<BN, BK, B_KIND, T::B_VECS>(sb, p.b_sx, p.b_sk, p.N, n0, tid, p.conv);
 
-  // lane position inside the k-major tiles, once per low-bits swizzle value
-  const float *a_lane[4], *b_lane[4];
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    a_lane[c] = lds_a + (lane >> 4) * T::LDA + wm0 + ((lane & 15) ^ (T::A_SWZ ? c * 4 : 0));
-    b_lane[c] = lds_b + (lane >> 4) * T::LDB + wn0 + ((lane & 15) ^ (T::B_SWZ ? c * 4 : 0));
-  }
+  // lane position inside the x-major tiles: row (lane % 16) of the wave's first
+  // block, k group (lane / 16)
+  const float *a_lane = lds_a + (wm0 + (lane & 15)) * T::PITCH + (lane >> 4) * 4;
+  const float *b_lane = lds_b + (wn0 + (lane & 15)) * T::PITCH + (lane >> 4) * 4;
 
   float4_t acc[T::TM][T::TN];
 #pragma unroll
@@ -381,42 +372,41 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     load_tile<BN, BK, B_KIND, T::B_VECS>(rb[d], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0, k_begin + d * BK, tid,
                                          p.conv);
   }
-  store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a, ra[0], tid);
-  store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b, rb[0], tid);
+  store_tile<BM, BK, T::PITCH, A_KIND, T::A_VECS>(lds_a, ra[0], tid);
+  store_tile<BN, BK, T::PITCH, B_KIND, T::B_VECS>(lds_b, rb[0], tid);
   load_tile<BM, BK, A_KIND, T::A_VECS>(ra[0], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0, k_begin + D * BK, tid,
                                        p.conv);
   load_tile<BN, BK, B_KIND, T::B_VECS>(rb[0], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0, k_begin + D * BK, tid,
                                        p.conv);
   lds_barrier();
 
-  // ring of fragments: k step g (counted through all tiles) uses slot g % F and
-  // was fetched F-1 steps earlier, across tile boundaries too
-  constexpr int F = T::FRAG_DEPTH;
-  float fa[F][T::TM], fb[F][T::TN];
-#pragma unroll
-  for (int f = 0; f < F - 1; ++f) {
-    load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[f], a_lane, 0, f * 4);
-    load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[f], b_lane, 0, f * 4);
-  }
+  // fragments of the quad being multiplied and of the one after it (also across
+  // the tile boundary)
+  float4 fa[T::TM], fb[T::TN], na[T::TM], nb4[T::TN];
+  load_fragment<T::PITCH, T::TM>(fa, a_lane, 0, 0);
+  load_fragment<T::PITCH, T::TN>(fb, b_lane, 0, 0);
 
-  // Side work of a tile, cut into pieces that are dealt out over its k steps (LDS
-  // serves the four waves in order: a burst of tile stores in one step would hold
-  // up the fragment reads queued behind it):
+  // A tile is QUADS quads of four MFMA groups (one group = all TM x TN blocks at
+  // one k position of the quad). Side work of the tile is cut into pieces dealt
+  // out over the groups (LDS serves the four waves in order: a burst of tile
+  // stores would hold up the fragment reads queued behind it):
   //   pieces 0 .. A_VECS-1              one 16-byte vector of tile kt+1 -> LDS (A)
   //   pieces A_VECS .. A_VECS+B_VECS-1  the same for B
   //   then the global fetches of tile kt+4 into the ring slot just drained, A and
   //   B as one piece each.
-  constexpr int kSteps = BK / 4;
+  // The next quad's fragments are fetched in group 2 of each quad; for the last
+  // quad of a tile they come from tile kt+1, so its stores and the barrier must
+  // be over by group 1 of that quad.
+  constexpr int Q = T::QUADS;
+  constexpr int kGroups = 4 * Q;
   constexpr int kStores = T::A_VECS + T::B_VECS;
   constexpr int kPieces = kStores + 2;
-  // the stores must be over by step kSteps - F: the steps after it already read
-  // the next tile's fragments
-  constexpr int kEven = (kPieces + kSteps - 1) / kSteps;
-  constexpr int kForStores = (kStores + kSteps - F) / (kSteps - F + 1);
-  constexpr int kPerStep = kEven > kForStores ? kEven : kForStores;
-  constexpr int kBarrierStep = (kStores - 1) / kPerStep;   // the step that holds the last store
-  static_assert(F - 1 <= kSteps && kBarrierStep <= kSteps - F, "fragments of the next tile are read after the barrier");
-  static_assert((3 * kSteps) % F == 0, "fragment slots are compile-time over a group of three tiles");
+  constexpr int kEven = (kPieces + kGroups - 1) / kGroups;
+  constexpr int kStoreGroups = 4 * (Q - 1) + 2;
+  constexpr int kForStores = (kStores + kStoreGroups - 1) / kStoreGroups;
+  constexpr int kPerGroup = kEven > kForStores ? kEven : kForStores;
+  constexpr int kBarrierGroup = (kStores - 1) / kPerGroup;   // the group that holds the last store
+  static_assert(kBarrierGroup <= 4 * (Q - 1) + 1, "fragments of the next tile are read after the barrier");
 
   // One k tile: tile kt sits in LDS buffer u = kt % 3, tile kt+1 in ring slot (u+1) % 3.
   auto tile_step = [&](int kt, auto u_tag) __attribute__((always_inline)) {
@@ -424,53 +414,64 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     constexpr int nb = (u + 1) % 3;
     const int a_off = u * T::A_BUF, b_off = u * T::B_BUF;
 #pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
-      constexpr int kAhead = F - 1;
-      const int slot_now = (u * kSteps + s) % F, slot_ahead = (u * kSteps + s + kAhead) % F;
-      if (s + kAhead < kSteps) {
-        load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[slot_ahead], a_lane, a_off, (s + kAhead) * 4);
-        load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[slot_ahead], b_lane, b_off, (s + kAhead) * 4);
-      } else {
-        load_fragment<BK, T::LDA, T::TM, T::A_SWZ>(fa[slot_ahead], a_lane, nb * T::A_BUF, (s + kAhead - kSteps) * 4);
-        load_fragment<BK, T::LDB, T::TN, T::B_SWZ>(fb[slot_ahead], b_lane, nb * T::B_BUF, (s + kAhead - kSteps) * 4);
-      }
+    for (int quad = 0; quad < Q; ++quad) {
 #pragma unroll
-      for (int piece = s * kPerStep; piece < (s + 1) * kPerStep && piece < kPieces; ++piece) {
-        if (piece < T::A_VECS) {
-          store_tile<BM, BK, T::LDA, A_KIND, T::A_SWZ, T::A_VECS>(lds_a + nb * T::A_BUF, ra[nb], tid, piece, piece + 1);
-        } else if (piece < kStores) {
-          store_tile<BN, BK, T::LDB, B_KIND, T::B_SWZ, T::B_VECS>(lds_b + nb * T::B_BUF, rb[nb], tid,
-                                                                  piece - T::A_VECS, piece - T::A_VECS + 1);
-        } else if (piece == kStores) {
-          load_tile<BM, BK, A_KIND, T::A_VECS>(ra[nb], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0,
-                                               k_begin + (kt + 1 + D) * BK, tid, p.conv);
-        } else {
-          load_tile<BN, BK, B_KIND, T::B_VECS>(rb[nb], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0,
-                                               k_begin + (kt + 1 + D) * BK, tid, p.conv);
+      for (int j = 0; j < 4; ++j) {
+        constexpr int kDummy = 0;
+        (void)kDummy;
+        const int group = quad * 4 + j;
+        if (j == 2) {
+          if (quad + 1 < Q) {
+            load_fragment<T::PITCH, T::TM>(na, a_lane, a_off, quad + 1);
+            load_fragment<T::PITCH, T::TN>(nb4, b_lane, b_off, quad + 1);
+          } else {
+            load_fragment<T::PITCH, T::TM>(na, a_lane, nb * T::A_BUF, 0);
+            load_fragment<T::PITCH, T::TN>(nb4, b_lane, nb * T::B_BUF, 0);
+          }
+        }
+#pragma unroll
+        for (int piece = group * kPerGroup; piece < (group + 1) * kPerGroup && piece < kPieces; ++piece) {
+          if (piece < T::A_VECS) {
+            store_tile<BM, BK, T::PITCH, A_KIND, T::A_VECS>(lds_a + nb * T::A_BUF, ra[nb], tid, piece, piece + 1);
+          } else if (piece < kStores) {
+            store_tile<BN, BK, T::PITCH, B_KIND, T::B_VECS>(lds_b + nb * T::B_BUF, rb[nb], tid, piece - T::A_VECS,
+                                                            piece - T::A_VECS + 1);
+          } else if (piece == kStores) {
+            load_tile<BM, BK, A_KIND, T::A_VECS>(ra[nb], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0,
+                                                 k_begin + (kt + 1 + D) * BK, tid, p.conv);
+          } else {
+            load_tile<BN, BK, B_KIND, T::B_VECS>(rb[nb], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0,
+                                                 k_begin + (kt + 1 + D) * BK, tid, p.conv);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+          for (int jn = 0; jn < T::TN; ++jn)
+            acc[i][jn] = __builtin_amdgcn_mfma_f32_16x16x4f32(quad_element(fb[jn], j), quad_element(fa[i], j),
+                                                              acc[i][jn], 0, 0, 0);
+        // Issue order inside the group: after every matrix instruction a little of
+        // the side work, so that it issues in the shadow of the matrix pipe. A wave
+        // issues in order: side work in a block in front of the MFMAs is exposed
+        // whenever a SIMD holds a single wave.
+#pragma unroll
+        for (int m = 0; m < T::TM * T::TN; ++m) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+          __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // one LDS write
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one global read
+          __builtin_amdgcn_sched_group_barrier(0x006, 3, 0);   // a few vector / scalar ALU
+        }
+        __builtin_amdgcn_sched_barrier(0);   // groups stay in order
+        if (group == kBarrierGroup) {
+          lds_barrier();                     // tile kt+1 is complete in LDS
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
 #pragma unroll
-      for (int i = 0; i < T::TM; ++i)
+      for (int i = 0; i < T::TM; ++i) fa[i] = na[i];
 #pragma unroll
-        for (int j = 0; j < T::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb[slot_now][j], fa[slot_now][i], acc[i][j], 0, 0, 0);
-      // Issue order inside the step: after every matrix instruction a little of
-      // the side work, so that it issues in the shadow of the matrix pipe. A wave
-      // issues in order: side work in a block in front of the MFMAs is exposed
-      // whenever a SIMD holds a single wave.
-#pragma unroll
-      for (int m = 0; m < T::TM * T::TN; ++m) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
-        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // one LDS write
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // one global read
-        __builtin_amdgcn_sched_group_barrier(0x006, 3, 0);   // a few vector / scalar ALU
-      }
-      __builtin_amdgcn_sched_barrier(0);   // steps stay in order
-      if (s == kBarrierStep) {
-        lds_barrier();                     // tile kt+1 is complete in LDS
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      for (int jn = 0; jn < T::TN; ++jn) fb[jn] = nb4[jn];
     }
   };
 
