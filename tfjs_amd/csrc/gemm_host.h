@@ -18,8 +18,9 @@ struct TileShape {
 static const TileShape kTileShapes[] = {
     {128, 128, 16, 2, 2}, {128, 96, 16, 2, 2}, {128, 64, 16, 2, 2}, {64, 64, 16, 2, 2},  {256, 32, 16, 4, 1},
     {256, 16, 16, 4, 1},  {64, 96, 16, 2, 2},  {128, 128, 32, 2, 2}, {128, 96, 32, 2, 2}, {64, 64, 32, 2, 2},
+    {64, 48, 32, 4, 1},   {32, 64, 32, 2, 2},  {32, 32, 32, 2, 2},
 };
-constexpr int kNumTileShapes = 10;
+constexpr int kNumTileShapes = 13;
 
 // Estimated run time in microseconds of an M x N x K product, `batch` times,
 // with tile shape t on `cus` compute units. Per workgroup and K tile the matrix
@@ -32,15 +33,15 @@ inline double estimate_us(const TileShape &t, long long M, long long N, long lon
   const long long k_tiles = (K + t.bk - 1) / t.bk;
   const int tm = t.bm / t.waves_m / 16, tn = t.bn / t.waves_n / 16;
   const double mfma_us = tm * tn * (t.bk / 4) * 32 / 2400.0;
-  const double lat_us = 1.25 * mfma_us + 0.15;
+  const double lat_us = 1.15 * mfma_us + 0.184 * (t.bk / 16.0);
   const long long per_cu = (tiles + cus - 1) / cus;
-  const int resident_max = t.bm * t.bn <= 64 * 96 ? 4 : 2;
+  const int resident_max = t.bm * t.bn <= 64 * 96 ? 3 : 2;
   const double resident = per_cu < resident_max ? (double)per_cu : (double)resident_max;
   const double trip = mfma_us * resident / 0.85 > lat_us ? mfma_us * resident / 0.85 : lat_us;
-  double compute = (double)k_tiles * trip + (1.0 + t.bm * t.bn * 0.37e-3) * (resident > 1 ? 1.41 : 1.0);
+  double compute = (double)k_tiles * trip + 2.0 + t.bm * t.bn * 0.37e-3;
   if (per_cu > resident_max) compute *= (double)per_cu / resident_max;
-  const double hbm = 4.0 * ((double)M * K + (double)K * N + (double)M * N) * batch / 4.5e6;
-  return (compute > hbm ? compute : hbm) + 2.0;
+  const double hbm = 4.0 * ((double)M * K + (double)K * N + (double)M * N) * batch / 4.94e6;
+  return (compute > hbm ? compute : hbm) + 1.9;
 }
 
 // Picks the tile shape with the lowest estimated run time.
@@ -152,7 +153,10 @@ inline int launch_gemm_shape(int shape, GemmParams &p) {
     case 6: return launch_gemm<64, 96, 16, 2, 2, A_KIND, B_KIND>(p);
     case 7: return launch_gemm<128, 128, 32, 2, 2, A_KIND, B_KIND>(p);
     case 8: return launch_gemm<128, 96, 32, 2, 2, A_KIND, B_KIND>(p);
-    default: return launch_gemm<64, 64, 32, 2, 2, A_KIND, B_KIND>(p);
+    case 9: return launch_gemm<64, 64, 32, 2, 2, A_KIND, B_KIND>(p);
+    case 10: return launch_gemm<64, 48, 32, 4, 1, A_KIND, B_KIND>(p);
+    case 11: return launch_gemm<32, 64, 32, 2, 2, A_KIND, B_KIND>(p);
+    default: return launch_gemm<32, 32, 32, 2, 2, A_KIND, B_KIND>(p);
   }
 }
 
