@@ -281,9 +281,9 @@ def test_depthwise_linearity_full_size(hip):
     assert np.abs(y - y12).max() <= 1e-4
 
 
-@pytest.mark.parametrize("m,n,k,act", [(24600, 24, 144, "linear"), (30001, 96, 16, "relu6"), (98309, 192, 32, "relu"),
-                                        (25000, 64, 196, "prelu"), (24576, 16, 36, "leakyrelu"), (98500, 144, 24, "relu6"),
-                                        (24600, 80, 100, "linear"), (24600, 24, 144, "sigmoid")])
+@pytest.mark.parametrize("m,n,k,act", [(65600, 24, 144, "linear"), (70001, 96, 16, "relu6"), (98309, 192, 32, "relu"),
+                                        (66000, 64, 196, "prelu"), (65536, 16, 36, "leakyrelu"), (98500, 144, 24, "relu6"),
+                                        (65600, 80, 100, "linear"), (65600, 24, 144, "sigmoid")])
 def test_matmul_tall_small_b(hip, orc, m, n, k, act):
     # tall products with a small B take the streaming kernel (sigmoid: falls back to the tiled one)
     rng = np.random.default_rng(m + n + k)

@@ -38,45 +38,15 @@ struct SkinnyArgs {
 };
 
 constexpr int kSkinnyChunk = 64;   // k per pipeline step: four float4 per lane
+constexpr int kSkinnyPad = 8;      // LDS row pitch k_pad + 8: the pitch the 16-byte fragment reads run fastest at
 
 // WAVES wavefronts per workgroup share one copy of B.
 template <int TN, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
   constexpr int kThreads = WAVES * 64;
-  extern __shared__ float lds_bt[];          // [16 * TN][k_pad + 16]: B transposed, zero padded
-  const int pitch = g.k_pad + 16;            // rows 16 banks apart: float4 reads of a wave spread over all banks
+  extern __shared__ float lds_bt[];          // [16 * TN][k_pad + kSkinnyPad]: B transposed, zero padded
+  const int pitch = g.k_pad + kSkinnyPad;
   const int tid = threadIdx.x;
-  // B -> LDS, transposed. Columns >= N and rows >= K read as zero; rows beyond
-  // the last 16-row group that holds real data are never read. Consecutive lanes
-  // take consecutive k (conflict-free LDS stores; B itself is small and cached),
-  // and eight fetches are issued before the first is stored, so the fill costs
-  // one or two memory round trips instead of one per element.
-  {
-    const int kk = ((g.K + 15) / 16) * 16;
-    const int items = kk * (16 * TN / 4);
-    for (int i0 = tid; i0 < items; i0 += kThreads * 8) {
-      float4 v[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int i = i0 + u * kThreads;
-        const int c = (i / kk) * 4, k = i - (i / kk) * kk;
-        v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (i < items && k < g.K && c < g.N) v[u] = *reinterpret_cast<const float4 *>(g.b + (long long)k * g.N + c);
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int i = i0 + u * kThreads;
-        if (i >= items) continue;
-        const int c = (i / kk) * 4, k = i - (i / kk) * kk;
-        lds_bt[(c + 0) * pitch + k] = v[u].x;
-        lds_bt[(c + 1) * pitch + k] = v[u].y;
-        lds_bt[(c + 2) * pitch + k] = v[u].z;
-        lds_bt[(c + 3) * pitch + k] = v[u].w;
-      }
-    }
-  }
-  __syncthreads();
-
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = lane >> 4, r = lane & 15;
@@ -119,8 +89,41 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
 #pragma unroll
     for (int n = 0; n < TN; ++n) acc[h][n] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
+  // the first fetch of A is issued before B is staged, so the two overlap
   float4 cur[4], nxt[4];
   if (total > 0) issue(cur, first, 0);
+
+  // B -> LDS, transposed. Columns >= N and rows >= K read as zero; rows beyond
+  // the last 16-row group that holds real data are never read. Consecutive lanes
+  // take consecutive k (conflict-free LDS stores; B itself is small and cached),
+  // and eight fetches are issued before the first is stored, so the fill costs
+  // one or two memory round trips instead of one per element.
+  {
+    const int kk = ((g.K + 15) / 16) * 16;
+    const int items = kk * (16 * TN / 4);
+    for (int i0 = tid; i0 < items; i0 += kThreads * 8) {
+      float4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * kThreads;
+        const int c = (i / kk) * 4, k = i - (i / kk) * kk;
+        v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i < items && k < g.K && c < g.N) v[u] = *reinterpret_cast<const float4 *>(g.b + (long long)k * g.N + c);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * kThreads;
+        if (i >= items) continue;
+        const int c = (i / kk) * 4, k = i - (i / kk) * kk;
+        lds_bt[(c + 0) * pitch + k] = v[u].x;
+        lds_bt[(c + 1) * pitch + k] = v[u].y;
+        lds_bt[(c + 2) * pitch + k] = v[u].z;
+        lds_bt[(c + 3) * pitch + k] = v[u].w;
+      }
+    }
+  }
+  __syncthreads();
+
   int b = first, c = 0;
   for (int q = 0; q < total; ++q) {
     int nb = b, nc = c + 1;
@@ -196,9 +199,9 @@ inline bool skinny_applies(const GemmParams &p, bool transpose_a, bool transpose
   const int tn = skinny_groups(p.N);
   if (tn == 0 || p.a_bytes == 0) return false;
   // enough 16-row blocks per wavefront to pay for the B fill (a wide B costs more)
-  if (p.M < (tn >= 9 ? 98304 : 24576)) return false;
+  if (p.M < (tn >= 9 ? 98304 : 65536)) return false;
   const long long k_pad = (p.K + kSkinnyChunk - 1) / kSkinnyChunk * kSkinnyChunk;
-  return 16LL * tn * (k_pad + 16) * 4 <= 64 * 1024;
+  return 16LL * tn * (k_pad + kSkinnyPad) * 4 <= 64 * 1024;
 }
 
 template <int TN>
@@ -207,7 +210,7 @@ inline int launch_skinny_tn(const SkinnyArgs &g) {
   // workgroups fill B fewer times but start later and pipeline less.
   constexpr int WAVES = 4;
   const int blocks = (g.M + 15) / 16;
-  const size_t lds = (size_t)16 * TN * (g.k_pad + 16) * sizeof(float);
+  const size_t lds = (size_t)16 * TN * (g.k_pad + kSkinnyPad) * sizeof(float);
   long long grid = (blocks + WAVES - 1) / WAVES;
   const long long cap = (long long)num_cus() * 3;
   if (grid > cap) grid = cap;
