@@ -164,6 +164,13 @@ def bench_model(model_dir, steps, warmup):
             s["bytes"] += nbytes
             s["launches"] += 1
         kernel_seconds = float(per_op.sum())
+        ops = []
+        for i, (op, _) in enumerate(model.plan):
+            flops, nbytes = model.op_work(i)
+            src = op["src"][0] if isinstance(op["src"], tuple) else op["src"]
+            ops.append(dict(op=op["kind"], x=list(model.shape[src]), y=list(model.shape[op["out"]]),
+                            kernel=names[i], us=round(per_op[i] * 1e6, 2),
+                            roof_us=round(max(flops / MFMA_FP32_PEAK_TFLOPS / 1e12, nbytes / HBM_PEAK_GBS / 1e9) * 1e6, 2)))
     finally:
         model.close()
     dominant = max(by_symbol, key=lambda k: by_symbol[k]["seconds"])
@@ -177,10 +184,10 @@ def bench_model(model_dir, steps, warmup):
     symbols = {k: dict(us_per_step=round(v["seconds"] * 1e6, 1), launches=v["launches"],
                        **roofline_entry(v["flops"], v["bytes"], v["seconds"])) for k, v in by_symbol.items()}
     return dict(ms_per_step=seconds / steps * 1e3, kernel_ms_per_step=kernel_seconds * 1e3, roofline=roof,
-                symbols=symbols)
+                symbols=symbols, ops=ops)
 
 
-def bench_model_node(model_dir, steps, warmup):
+def bench_model_node(model_dir, steps, warmup, prime):
     """The headline measurement: MobileNetV2 through the tfjs API in Node on the
     hip backend (KernelBackend + kernel configs + N-API addon). Returns the
     script's JSON, or None when Node or the addon is not available."""
@@ -189,7 +196,7 @@ def bench_model_node(model_dir, steps, warmup):
     addon = os.path.join(ROOT, "tfjs_amd", "lib", "tfjs_hip.node")
     if not (node and os.path.exists(addon)):
         return None
-    proc = subprocess.run([node, script, model_dir, str(BATCH), str(steps), str(warmup)], stdout=subprocess.PIPE,
+    proc = subprocess.run([node, script, model_dir, str(BATCH), str(steps), str(warmup), str(prime)], stdout=subprocess.PIPE,
                           stderr=subprocess.PIPE, text=True, timeout=900)
     if proc.returncode != 0:
         raise RuntimeError("node benchmark failed:\n%s" % proc.stderr[-3000:])
@@ -347,12 +354,17 @@ def copy_yardstick(mib):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--kernels-only", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-baseline-child", metavar="MODEL_DIR")
+    ap.add_argument("--jit-prime", type=int, default=200, metavar="N",
+                    help="batch-1 inferences the Node process runs before the warm-up steps (outside the timed "
+                         "region) so that V8 has compiled the host path; 0 disables")
+    ap.add_argument("--per-op", metavar="FILE", help="write the per-op table of the model (kernel, us, us at the "
+                                                     "roofline) to FILE as JSON")
     ap.add_argument("--copy-yardstick", type=int, metavar="MIB", default=0,
                     help="also run three device-to-device copies of this many MiB, so that a hardware-counter run "
                          "of this command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -374,11 +386,14 @@ def main():
     model_dir = tempfile.mkdtemp(prefix="tfjs_hip_mobilenet_")
     try:
         workloads.write_model(model_dir, workloads.mobilenet_v2_weights(seed=3), np.uint8)
-        js = bench_model_node(model_dir, args.steps, args.warmup)
+        js = bench_model_node(model_dir, args.steps, args.warmup, args.jit_prime)
         m = bench_model(model_dir, args.steps, args.warmup)
         cpu = None if args.no_cpu_baseline else cpu_baseline(model_dir)
     finally:
         shutil.rmtree(model_dir, ignore_errors=True)
+    if args.per_op:
+        with open(args.per_op, "w") as f:
+            json.dump(m["ops"], f, indent=0)
     kernels = None if args.no_kernels else bench_kernels()
     copy_gbs = copy_yardstick(args.copy_yardstick) if args.copy_yardstick else None
     ms_per_step = js["ms_per_step"] if js else m["ms_per_step"]
@@ -399,7 +414,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "MobileNetV2 1.0/224, batch 32, NHWC fp32, uint8-quantized random-init weights "
                                "dequantized on load (benchmark configuration 4)", "batch": BATCH,
-                   "host": host, "device": info["arch"], "cus": info["cus"]},
+                   "jit_priming_batch1_inferences": js["prime"] if js else 0, "host": host, "device": info["arch"], "cus": info["cus"]},
         "weights_load_ms": round(js["load_ms"], 2) if js else None,
         "python_host_ms_per_step": round(m["ms_per_step"], 4),
         "kernel_ms_per_step": round(m["kernel_ms_per_step"], 4),

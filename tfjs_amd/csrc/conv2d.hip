@@ -81,10 +81,124 @@ __global__ __launch_bounds__(256) void conv_few_channels(FewChannelsArgs g) {
   }
 }
 
-template <int OC>
-int launch_few_channels(const GemmParams &p, int f_h) {
+// What tap k = (r * f_w + s) * in_c + c of the filter reads, relative to the
+// top-left element of a pixel's window; rows beyond K hold a row offset that no
+// image has. Filled on the host so that the kernel does no divisions for it.
+constexpr int kMaxTaps = 36;
+struct TapTable {
+  int dh[kMaxTaps], dw[kMaxTaps];
+  unsigned off_bytes[kMaxTaps];
+};
+
+// The same convolution on the matrix cores, for filters of at most 4 * KSTEPS
+// taps (K = f_h * f_w * in_c) and 16 * NB output channels per workgroup column.
+// A wave computes 64 consecutive pixels x 16 NB channels per trip as 4 x NB
+// blocks of v_mfma_f32_16x16x4_f32 over KSTEPS k steps:
+//  * lane (r = lane % 16, kg = lane / 16) feeds tap k = 4 t + kg in k step t: of
+//    the filter (weights of channel 16 j + r, fetched once per wave and kept in
+//    registers) and of the image (pixel 16 i + r of the wave's 64: one gathered
+//    element load per block and k step, all 4 * KSTEPS of them in flight at once;
+//    buffer loads, so a tap outside the image or beyond K reads zero through an
+//    offset that the descriptor does not cover);
+//  * the operands go in swapped, so the lane ends up with channels 4 kg .. +3 of
+//    pixel 16 i + r for each block: bias (the accumulators start from it),
+//    activation and one 16-byte store per block.
+template <int KSTEPS, int NB>
+__global__ __launch_bounds__(256) void conv_few_taps(FewChannelsArgs g, TapTable taps, int chunks, unsigned x_bytes) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, kg = lane >> 4;
+  const int oc0 = blockIdx.y * (16 * NB);
+  const int K = g.f_h * g.f_w * g.in_c;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)g.x, 0, (int)x_bytes, 0x00020000);
+  float wv[KSTEPS][NB];
+  unsigned tap_off[KSTEPS];
+  int tap_dh[KSTEPS], tap_dw[KSTEPS];
+#pragma unroll
+  for (int t = 0; t < KSTEPS; ++t) {
+    const int k = 4 * t + kg;
+    tap_dh[t] = taps.dh[k];
+    tap_dw[t] = taps.dw[k];
+    tap_off[t] = taps.off_bytes[k];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) wv[t][j] = k < K ? g.w[(long long)k * g.out_c + oc0 + 16 * j + r] : 0.f;
+  }
+  float4_t bias4[NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    bias4[j] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    if (g.bias) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) bias4[j][q] = g.bias[(long long)(oc0 + 16 * j + 4 * kg + q) * g.bias_stride];
+    }
+  }
+  for (int chunk = blockIdx.x; chunk < chunks; chunk += gridDim.x) {
+    const int m_wave = chunk * 256 + wave * 64;
+    // pixel of block 0; the following blocks are 16 pixels further along the row
+    int m = m_wave + r;
+    int ow = m % g.out_w;
+    int t2 = m / g.out_w;
+    int oh = t2 % g.out_h, n = t2 / g.out_h;
+    float av[4][KSTEPS];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool live = m < g.M;
+      const int ih0 = oh * g.stride_h - g.pad_top, iw0 = ow * g.stride_w - g.pad_left;
+      // byte offset of the window's top-left element; it may lie before the
+      // image, the sum with an inside tap's offset is exact modulo 2^32
+      const unsigned base = (unsigned)(((long long)n * g.xs_n + (long long)ih0 * g.xs_h + (long long)iw0 * g.xs_w) * 4);
+#pragma unroll
+      for (int t = 0; t < KSTEPS; ++t) {
+        const bool inside = live && (unsigned)(ih0 + tap_dh[t]) < (unsigned)g.in_h &&
+                            (unsigned)(iw0 + tap_dw[t]) < (unsigned)g.in_w;
+        av[i][t] = __uint_as_float(
+            __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(inside ? base + tap_off[t] : 0xffffffffu), 0, 0));
+      }
+      m += 16;
+      ow += 16;
+      while (ow >= g.out_w) {
+        ow -= g.out_w;
+        if (++oh == g.out_h) {
+          oh = 0;
+          ++n;
+        }
+      }
+    }
+    float4_t acc[4][NB];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j) acc[i][j] = bias4[j];
+#pragma unroll
+    for (int t = 0; t < KSTEPS; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[t][j], av[i][t], acc[i][j], 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int mi = m_wave + 16 * i + r;
+      if (mi >= g.M) continue;
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        float q[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          q[k] = acc[i][j][k];
+          if (g.activation != TFHIP_LINEAR) {
+            q[k] = (q[k] > 0.f || q[k] != q[k]) ? q[k] : 0.f;   // Math.max(0, x): NaN stays, -0 becomes +0
+            if (g.activation == TFHIP_RELU6 && q[k] > 6.f) q[k] = 6.f;
+          }
+        }
+        *reinterpret_cast<float4 *>(g.y + (long long)mi * g.out_c + oc0 + 16 * j + 4 * kg) =
+            make_float4(q[0], q[1], q[2], q[3]);
+      }
+    }
+  }
+}
+
+void fill_few_channels_args(FewChannelsArgs &g, const GemmParams &p, int f_h) {
   const ConvGeom &c = p.conv;
-  FewChannelsArgs g;
   g.x = p.a; g.w = p.b; g.y = p.c;
   g.bias = p.epi.bias; g.bias_stride = p.epi.bias ? p.epi.bias_s[3] : 0;
   g.xs_n = c.xs_n; g.xs_h = c.xs_h; g.xs_w = c.xs_w;
@@ -92,6 +206,43 @@ int launch_few_channels(const GemmParams &p, int f_h) {
   g.stride_h = c.stride_h; g.stride_w = c.stride_w; g.dil_h = c.dil_h; g.dil_w = c.dil_w;
   g.pad_top = c.pad_top; g.pad_left = c.pad_left; g.out_h = c.out_h; g.out_w = c.out_w;
   g.activation = p.epi.activation;
+}
+
+template <int KSTEPS, int NB>
+int launch_few_taps(const GemmParams &p, int f_h) {
+  FewChannelsArgs g;
+  fill_few_channels_args(g, p, f_h);
+  const ConvGeom &c = p.conv;
+  TapTable taps;
+  for (int k = 0; k < kMaxTaps; ++k) {
+    const int tap = k / c.in_c, ch = k - tap * c.in_c;
+    const int fr = tap / c.f_w, fs = tap - fr * c.f_w;
+    taps.dh[k] = k < p.K ? fr * c.dil_h : (1 << 28);
+    taps.dw[k] = fs * c.dil_w;
+    taps.off_bytes[k] = (unsigned)(((long long)fr * c.dil_h * c.xs_h + (long long)fs * c.dil_w * c.xs_w + ch) * 4);
+  }
+  // 256 pixels per workgroup and trip; every workgroup makes the same number of trips
+  const int chunks = (p.M + 255) / 256;
+  const int at_once = num_cus() * 8;
+  const int trips = (chunks + at_once - 1) / at_once;
+  dim3 grid((unsigned)((chunks + trips - 1) / trips), (unsigned)(p.N / (16 * NB)), 1);
+  note_kernel("conv_few_taps<%d, %d>", KSTEPS, NB);
+  TFHIP_LAUNCH((conv_few_taps<KSTEPS, NB><<<grid, 256, 0, stream()>>>(g, taps, chunks, p.a_bytes)));
+  return kOk;
+}
+
+template <int NB>
+int launch_few_taps_k(const GemmParams &p, int f_h) {
+  if (p.K <= 12) return launch_few_taps<3, NB>(p, f_h);
+  if (p.K <= 28) return launch_few_taps<7, NB>(p, f_h);
+  return launch_few_taps<9, NB>(p, f_h);
+}
+
+template <int OC>
+int launch_few_channels(const GemmParams &p, int f_h) {
+  const ConvGeom &c = p.conv;
+  FewChannelsArgs g;
+  fill_few_channels_args(g, p, f_h);
   dim3 grid((unsigned)((p.M + 255) / 256), (unsigned)(p.N / OC), 1);
   note_kernel("conv_few_channels<%d>", OC);
   TFHIP_LAUNCH((conv_few_channels<OC><<<grid, 256, 0, stream()>>>(g)));
@@ -173,6 +324,9 @@ extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
   }
   if (!nchw && in_c <= 4 && out_c % 8 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
       p.epi.channel_operands && activation <= TFHIP_RELU6) {
+    const bool few_taps = K <= kMaxTaps && M < lim - 256 && p.a_bytes != 0;
+    if (few_taps && out_c % 32 == 0) return launch_few_taps_k<2>(p, (int)f_h);
+    if (few_taps && out_c % 16 == 0) return launch_few_taps_k<1>(p, (int)f_h);
     if (out_c % 32 == 0) return launch_few_channels<32>(p, (int)f_h);
     if (out_c % 16 == 0) return launch_few_channels<16>(p, (int)f_h);
     return launch_few_channels<8>(p, (int)f_h);

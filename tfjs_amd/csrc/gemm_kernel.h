@@ -343,11 +343,30 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   const float *a_lane = lds_a + (wm0 + (lane & 15)) * T::PITCH + (lane >> 4) * 4;
   const float *b_lane = lds_b + (wn0 + (lane & 15)) * T::PITCH + (lane >> 4) * 4;
 
+  // The accumulators start from the bias (lane l of a 16x16 block ends up with
+  // columns 4 * (l / 16) .. +3 of its row, see the epilogue): its fetch overlaps
+  // the first tiles' instead of following the k loop, and it costs no register
+  // past this point. A product that is completed by gemm_finish starts from zero.
+  const Epilogue &e = p.epi;
+  const bool fused = p.inline_epilogue != 0;
   float4_t acc[T::TM][T::TN];
+  {
+    const int lane_col = n0 + wn0 + (lane >> 4) * 4;
+    const bool with_bias = fused && e.bias != nullptr;
 #pragma unroll
-  for (int i = 0; i < T::TM; ++i)
+    for (int j = 0; j < T::TN; ++j) {
+      float4_t b4 = {0.f, 0.f, 0.f, 0.f};
+      if (with_bias) {
 #pragma unroll
-    for (int j = 0; j < T::TN; ++j) acc[i][j] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int q = 0; q < 4; ++q) {
+          const int col = lane_col + j * 16 + q;
+          b4[q] = e.bias[(long long)(col < p.N ? col : p.N - 1) * e.bias_s[3]];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i) acc[i][j] = b4;
+    }
+  }
 
   // Software pipeline over k tiles, three deep at both levels:
   //  * registers: tile t lives in ring slot t % 3 from its global fetch (issued
@@ -488,23 +507,20 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 
   // ---- epilogue: registers -> global. Lane l of a 16x16 block holds row l % 16,
   // columns 4 * (l / 16) .. +3 (the operands went into the MFMA swapped).
-  const Epilogue &e = p.epi;
   const int lane_m = lane & 15, lane_n = (lane >> 4) * 4;
-  const bool fused = p.inline_epilogue != 0;
   // destination: the output itself, or this split's dense [M][N] slab of the workspace
   const bool to_ws = p.splits > 1;
   float *C = to_ws ? p.ws + ((long long)split * p.batch + bz) * p.M * p.N : p.c + (long long)bz * p.c_batch_stride;
   const long long ldc = to_ws ? p.N : p.ldc;
   const bool conv_addr = !to_ws && e.addressing == kConv;
   const bool vec = to_ws ? p.N % 4 == 0 : p.vec_store != 0;
-  float bias_q[T::TN][4], alpha_q[T::TN][4];
+  float alpha_q[T::TN][4];
 #pragma unroll
   for (int j = 0; j < T::TN; ++j) {
     const int col = n0 + wn0 + j * 16 + lane_n;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const bool ok = fused && col + q < p.N;
-      bias_q[j][q] = (ok && e.bias) ? e.bias[(long long)(col + q) * e.bias_s[3]] : 0.f;
       alpha_q[j][q] = (ok && e.activation == TFHIP_PRELU) ? e.prelu[(long long)(col + q) * e.prelu_s[3]] : 0.f;
     }
   }
@@ -528,7 +544,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
         float out[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const float v = acc[i][j][q] + bias_q[j][q];
+          const float v = acc[i][j][q];
           if (ACT == TFHIP_RELU) {
             out[q] = (v > 0.f || v != v) ? v : 0.f;
           } else if (ACT == TFHIP_RELU6) {

@@ -80,6 +80,26 @@ struct Args {
       for (size_t k = 0; k < n; ++k) out[k] = 0;
       return true;
     }
+    // fast path: a Float64Array or Int32Array is read in place (one N-API call)
+    bool typed = false;
+    if (napi_is_typedarray(env, argv[i], &typed) == napi_ok && typed) {
+      napi_typedarray_type type;
+      size_t length = 0, offset = 0;
+      void *data = nullptr;
+      napi_value ab;
+      if (napi_get_typedarray_info(env, argv[i], &type, &length, &data, &ab, &offset) != napi_ok ||
+          length < n || (type != napi_float64_array && type != napi_int32_array)) {
+        ok = false;
+        napi_throw_type_error(env, nullptr, "tfjs_hip: expected a Float64Array or Int32Array of sufficient length");
+        return false;
+      }
+      if (type == napi_float64_array) {
+        for (size_t k = 0; k < n; ++k) out[k] = (int64_t) static_cast<const double *>(data)[k];
+      } else {
+        for (size_t k = 0; k < n; ++k) out[k] = static_cast<const int32_t *>(data)[k];
+      }
+      return true;
+    }
     for (uint32_t k = 0; k < n; ++k) {
       napi_value el;
       double v = 0;
@@ -345,12 +365,14 @@ napi_value DequantF16(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
-// add(a, aStrides, b, bStrides, out, outShape)   (rank = outShape.length <= 6)
+// add(a, aStrides, b, bStrides, out, outShape[, rank])   (rank = outShape.length <= 6)
 napi_value Add(napi_env env, napi_callback_info info) {
   Args a(env, info, 6, "add");
   uint32_t rank = 0;
-  if (a.ok && napi_get_array_length(env, a.argv[5], &rank) != napi_ok) {
-    napi_throw_type_error(env, nullptr, "tfjs_hip.add: outShape must be an array");
+  if (a.ok && a.argc > 6) {
+    rank = (uint32_t)a.i32(6);  // typed arrays: the rank comes as its own argument
+  } else if (a.ok && napi_get_array_length(env, a.argv[5], &rank) != napi_ok) {
+    napi_throw_type_error(env, nullptr, "tfjs_hip.add: outShape must be an array (or pass the rank)");
     return nullptr;
   }
   if (rank > 6) {

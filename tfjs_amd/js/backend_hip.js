@@ -14,6 +14,14 @@
  *   disposeData decrement; free the device buffer at 0 or when forced
  * Kernels only enqueue work on the library's single stream; read / readSync
  * are the sync points.
+ *
+ * Buffers released by disposeData are kept on per-size free lists here and
+ * handed out again by allocate(): an inference graph asks for the same sizes
+ * step after step, and this saves two native calls per op. Work already
+ * enqueued on the single stream runs before any later kernel that is handed
+ * the block again, so a block can be reused at once. The lists are emptied
+ * when they hold more than a quarter of the device's memory or when the
+ * native allocator reports that it is out of memory.
  */
 const tf = require('./core');
 const {addon} = require('./binding');
@@ -38,6 +46,52 @@ class HipBackend extends tf.KernelBackend {
     this.deviceInfo = addon.deviceInfo();
     this.data = new tf.DataStorage(this, tf.engine());
     this.nextEventSlot = 0;
+    this.freeLists = new Map();  // bytes -> [ptr, ...]
+    this.pooledBuffers = 0;
+    this.pooledBytes = 0;
+    this.poolLimitBytes = this.deviceInfo.hbmBytes / 4;
+  }
+
+  /** Returns every pooled buffer to the native allocator. */
+  releasePool() {
+    this.freeLists.forEach(list => list.forEach(ptr => addon.free(ptr)));
+    this.freeLists.clear();
+    this.pooledBuffers = 0;
+    this.pooledBytes = 0;
+  }
+
+  acquire(bytes) {
+    const list = this.freeLists.get(bytes);
+    if (list !== undefined && list.length > 0) {
+      this.pooledBuffers--;
+      this.pooledBytes -= bytes;
+      return list.pop();
+    }
+    try {
+      return addon.alloc(bytes);
+    } catch (e) {
+      if (this.pooledBuffers === 0) {
+        throw e;
+      }
+      this.releasePool();
+      return addon.alloc(bytes);
+    }
+  }
+
+  release(ptr, bytes) {
+    if (this.pooledBytes + bytes > this.poolLimitBytes) {
+      this.releasePool();
+      addon.free(ptr);
+      return;
+    }
+    let list = this.freeLists.get(bytes);
+    if (list === undefined) {
+      list = [];
+      this.freeLists.set(bytes, list);
+    }
+    list.push(ptr);
+    this.pooledBuffers++;
+    this.pooledBytes += bytes;
   }
 
   nextDataId() {
@@ -51,7 +105,7 @@ class HipBackend extends tf.KernelBackend {
       throw new Error(`tfjs-backend-hip does not support dtype ${dtype}`);
     }
     const bytes = size * BYTES[dtype];
-    const ptr = addon.alloc(Math.max(bytes, 1));
+    const ptr = this.acquire(Math.max(bytes, 1));
     dataId = dataId || this.nextDataId();
     this.data.set(dataId, {ptr, bytes, dtype, shape: shape.slice(), refCount: 1});
     return dataId;
@@ -144,7 +198,7 @@ class HipBackend extends tf.KernelBackend {
       if (!force && info.refCount > 0) {
         return false;
       }
-      addon.free(info.ptr);
+      this.release(info.ptr, Math.max(info.bytes, 1));
       this.data.delete(dataId);
     }
     return true;
@@ -172,9 +226,10 @@ class HipBackend extends tf.KernelBackend {
     const m = addon.memoryInfo();
     return {
       unreliable: false,
-      numDeviceBuffers: m.live,
+      numDeviceBuffers: m.live - this.pooledBuffers,
       numBytesInGPU: m.liveBytes,
-      numBytesInGPUPool: m.pooledBytes
+      numBytesInGPUPool: m.pooledBytes,
+      numBytesInBackendPool: this.pooledBytes
     };
   }
 
@@ -187,6 +242,7 @@ class HipBackend extends tf.KernelBackend {
   }
 
   dispose() {
+    this.releasePool();
     addon.shutdown();
   }
 }

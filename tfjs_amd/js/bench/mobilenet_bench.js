@@ -2,7 +2,9 @@
 /**
  * MobileNetV2 through the tfjs API on the hip backend, timed the reference's way
  * (predict plus download of the result, e2e/benchmarks/benchmark_util.js:246-286).
- *   node tfjs_amd/js/bench/mobilenet_bench.js MODEL_DIR BATCH STEPS WARMUP
+ *   node tfjs_amd/js/bench/mobilenet_bench.js MODEL_DIR BATCH STEPS WARMUP [PRIME]
+ * PRIME (default 0) batch-1 inferences run first, outside warm-up and timing, so
+ * that V8 has compiled the host path before a short measurement starts.
  * Prints one JSON line: ms_per_step (wall clock around STEPS steps, stream
  * drained on both sides), load_ms (read + upload + GPU dequant of the weights),
  * kernel_ms_per_step (device time between two events around the same steps).
@@ -18,6 +20,7 @@ async function main() {
   const batch = parseInt(process.argv[3] || '32', 10);
   const steps = parseInt(process.argv[4] || '50', 10);
   const warmup = parseInt(process.argv[5] || '5', 10);
+  const prime = parseInt(process.argv[6] || '0', 10);
   await tf.setBackend('hip');
   const t0 = tf.util.now();
   const m = model.readModel(modelDir);
@@ -33,6 +36,18 @@ async function main() {
     checksum = data[0];
     y.dispose();
   };
+  if (prime > 0) {
+    const x1 = tf.tensor(model.syntheticInput(1, 3), [1, 224, 224, 3]);
+    for (let i = 0; i < prime; i++) {
+      const y = predict(x1);
+      if (i % 16 === 15) {
+        y.dataSync();  // keeps the host at most 16 inferences ahead of the stream
+      }
+      y.dispose();
+    }
+    addon.sync();
+    x1.dispose();
+  }
   for (let i = 0; i < warmup; i++) {
     step();
   }
@@ -54,6 +69,7 @@ async function main() {
     batch,
     steps,
     warmup,
+    prime,
     checksum,
     node: process.version,
     core: tf.usingStandin ? 'standin' : '@tensorflow/tfjs-core',

@@ -11,8 +11,10 @@ export interface HipMemoryInfo {
   /** device blocks handed out and not freed */
   numDeviceBuffers: number;
   numBytesInGPU: number;
-  /** freed blocks kept by the pool for reuse */
+  /** freed blocks kept by the native pool for reuse */
   numBytesInGPUPool: number;
+  /** disposed buffers kept on the backend's own free lists (counted in numBytesInGPU) */
+  numBytesInBackendPool: number;
 }
 
 export declare class HipBackend extends KernelBackend {

@@ -11,18 +11,34 @@
 const tf = require('../core');
 const {activationCode, broadcastStrides, requireFloat32, addon} = require('./fused_util');
 
-/** Strides of `t` over the output, reordered to (n, h, w, c) for the C ABI. */
-function epilogueStrides(t, outShape, nchw) {
+// Scratch that carries the geometry and the epilogue strides to the addon.
+const geom = new Float64Array(15);
+const biasScratch = new Float64Array(4);
+const preluScratch = new Float64Array(4);
+const reshaped = [0, 1, 1];
+
+/**
+ * Strides of `t` over the output, reordered to (n, h, w, c) for the C ABI,
+ * written into `into`; null when there is no such operand.
+ */
+function epilogueStrides(t, outShape, nchw, into) {
   if (t == null) {
     return null;
   }
   let shape = t.shape;
   // For NCHW a 1-D tensor lines up with the channels (FusedConv2D.ts:55-61, :76-86)
   if (nchw && shape.length === 1 && shape[0] !== 1) {
-    shape = [shape[0], 1, 1];
+    reshaped[0] = shape[0];
+    shape = reshaped;
   }
-  const s = broadcastStrides(shape, outShape);
-  return nchw ? [s[0], s[2], s[3], s[1]] : s;
+  broadcastStrides(shape, outShape, into);
+  if (nchw) {
+    const c = into[1];
+    into[1] = into[2];
+    into[2] = into[3];
+    into[3] = c;
+  }
+  return into;
 }
 
 function convImpl(args, depthwise, fused, opName) {
@@ -54,20 +70,29 @@ function convImpl(args, depthwise, fused, opName) {
       x.shape, filter.shape, strides, dilations, pad, dimRoundingMode, depthwise,
       $dataFormat);
   const nchw = $dataFormat === 'channelsFirst';
-  const biasStrides = epilogueStrides(bias, info.outShape, nchw);
-  const preluStrides =
-      activation === 'prelu' ? epilogueStrides(prelu, info.outShape, nchw) : null;
+  const biasStrides = epilogueStrides(bias, info.outShape, nchw, biasScratch);
+  const preluStrides = activation === 'prelu' ?
+      epilogueStrides(prelu, info.outShape, nchw, preluScratch) :
+      null;
   const out = backend.makeOutput(info.outShape, 'float32');
   if (tf.util.sizeFromShape(info.outShape) === 0) {
     return out;
   }
-  const geom = [
-    info.batchSize, info.inHeight, info.inWidth, info.inChannels,
-    info.filterHeight, info.filterWidth,
-    depthwise ? info.outChannels / info.inChannels : info.outChannels,
-    info.strideHeight, info.strideWidth, info.dilationHeight, info.dilationWidth,
-    info.padInfo.top, info.padInfo.left, info.outHeight, info.outWidth
-  ];
+  geom[0] = info.batchSize;
+  geom[1] = info.inHeight;
+  geom[2] = info.inWidth;
+  geom[3] = info.inChannels;
+  geom[4] = info.filterHeight;
+  geom[5] = info.filterWidth;
+  geom[6] = depthwise ? info.outChannels / info.inChannels : info.outChannels;
+  geom[7] = info.strideHeight;
+  geom[8] = info.strideWidth;
+  geom[9] = info.dilationHeight;
+  geom[10] = info.dilationWidth;
+  geom[11] = info.padInfo.top;
+  geom[12] = info.padInfo.left;
+  geom[13] = info.outHeight;
+  geom[14] = info.outWidth;
   const alpha = args.attrs.leakyreluAlpha == null ? 0.2 : args.attrs.leakyreluAlpha;
   if (depthwise) {
     addon.fusedDepthwiseConv2D(

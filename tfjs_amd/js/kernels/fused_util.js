@@ -3,8 +3,10 @@
  * Helpers shared by the kernel configs: how a bias / PReLU-weights tensor of
  * any broadcastable shape is described to the native library (element strides
  * over the output's dims, 0 where it is stretched), and the activation codes.
+ * Shape and stride vectors travel to the addon in Float64Array scratch that
+ * the kernel configs reuse from call to call: every addon call is synchronous
+ * and has read its arguments when it returns.
  */
-const tf = require('../core');
 const {addon, FusableActivation} = require('../binding');
 
 function activationCode(activation, opName) {
@@ -20,34 +22,50 @@ function activationCode(activation, opName) {
 /**
  * Element strides of a dense tensor of `shape` over `outShape` (right-aligned
  * broadcasting, tfjs-core/src/ops/broadcast_util.ts:63-90); throws the
- * reference's error when the shapes do not broadcast to outShape.
+ * reference's error when the shapes do not broadcast to outShape. Writes into
+ * `into` (any array-like of outShape.length entries) when given.
  */
-function broadcastStrides(shape, outShape) {
-  const full = tf.backend_util.assertAndGetBroadcastShape(outShape, shape);
-  if (!tf.util.arraysEqual(full, outShape)) {
+function broadcastStrides(shape, outShape, into) {
+  const rank = outShape.length;
+  const strides = into || new Array(rank);
+  for (let i = 0; i < rank; i++) {
+    strides[i] = 0;
+  }
+  // The two common cases need no shape algebra: a vector along the last
+  // dimension (a bias) and an operand of the output's own shape.
+  if (shape.length === 1 && rank >= 1 && shape[0] === outShape[rank - 1]) {
+    strides[rank - 1] = shape[0] === 1 ? 0 : 1;
+    return strides;
+  }
+  if (shape.length > rank) {
     throw new Error(
         `Operands could not be broadcast together with shapes ` +
         `${outShape} and ${shape}.`);
   }
-  const strides = new Array(outShape.length).fill(0);
   let acc = 1;
   for (let i = 0; i < shape.length; i++) {
-    const d = shape.length - 1 - i;
-    const od = outShape.length - 1 - i;
-    strides[od] = shape[d] === 1 ? 0 : acc;
-    acc *= shape[d];
+    const d = shape[shape.length - 1 - i];
+    const od = rank - 1 - i;
+    if (d !== 1 && d !== outShape[od]) {
+      throw new Error(
+          `Operands could not be broadcast together with shapes ` +
+          `${outShape} and ${shape}.`);
+    }
+    strides[od] = d === 1 ? 0 : acc;
+    acc *= d;
   }
   return strides;
 }
 
 function requireFloat32(tensors, opName) {
-  tensors.forEach(t => {
+  for (let i = 0; i < tensors.length; i++) {
+    const t = tensors[i];
     if (t != null && t.dtype !== 'float32') {
       throw new Error(
           `${opName} for non-float32 tensors is not supported by the hip ` +
           `backend (got ${t.dtype}).`);
     }
-  });
+  }
 }
 
 module.exports = {activationCode, broadcastStrides, requireFloat32, addon};

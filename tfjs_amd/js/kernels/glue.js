@@ -9,20 +9,29 @@
 const tf = require('../core');
 const {broadcastStrides, requireFloat32, addon} = require('./fused_util');
 
+const aStrides = new Float64Array(6);
+const bStrides = new Float64Array(6);
+const outDims = new Float64Array(6);
+
 function add(args) {
   const {a, b} = args.inputs;
   const backend = args.backend;
   requireFloat32([a, b], 'Add');
-  const outShape = tf.backend_util.assertAndGetBroadcastShape(a.shape, b.shape);
+  const outShape = tf.util.arraysEqual(a.shape, b.shape) ?
+      a.shape.slice() :
+      tf.backend_util.assertAndGetBroadcastShape(a.shape, b.shape);
   if (outShape.length > 6) {
     throw new Error('Add: the hip backend supports up to rank 6');
   }
   const out = backend.makeOutput(outShape, 'float32');
   if (tf.util.sizeFromShape(outShape) > 0) {
+    for (let i = 0; i < outShape.length; i++) {
+      outDims[i] = outShape[i];
+    }
     addon.add(
-        backend.ptr(a.dataId), broadcastStrides(a.shape, outShape),
-        backend.ptr(b.dataId), broadcastStrides(b.shape, outShape),
-        backend.ptr(out.dataId), outShape);
+        backend.ptr(a.dataId), broadcastStrides(a.shape, outShape, aStrides),
+        backend.ptr(b.dataId), broadcastStrides(b.shape, outShape, bStrides),
+        backend.ptr(out.dataId), outDims, outShape.length);
   }
   return out;
 }

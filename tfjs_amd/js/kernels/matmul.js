@@ -9,6 +9,9 @@
 const tf = require('../core');
 const {activationCode, broadcastStrides, requireFloat32, addon} = require('./fused_util');
 
+const biasScratch = new Float64Array(3);
+const preluScratch = new Float64Array(3);
+
 function matMulImpl(backend, a, b, transposeA, transposeB, bias, activation, prelu, leakyreluAlpha, opName) {
   requireFloat32([a, b, bias, prelu], opName);
   const aRank = a.shape.length, bRank = b.shape.length;
@@ -31,7 +34,7 @@ function matMulImpl(backend, a, b, transposeA, transposeB, bias, activation, pre
   const batchDim = Math.max(batchDimA, batchDimB);
   // The native kernel sees the output as [batchDim, M, N]
   const view = [batchDim, outerShapeA, outerShapeB];
-  const stridesOverView = t => {
+  const stridesOverView = (t, into) => {
     if (t == null) {
       return null;
     }
@@ -61,10 +64,13 @@ function matMulImpl(backend, a, b, transposeA, transposeB, bias, activation, pre
           `stretched over only some of the batch dimensions ` +
           `[${outShapeOuterDims}] is not supported by the hip backend.`);
     }
-    return [batchStride, s[rank - 2], s[rank - 1]];
+    into[0] = batchStride;
+    into[1] = s[rank - 2];
+    into[2] = s[rank - 1];
+    return into;
   };
-  const biasStrides = stridesOverView(bias);
-  const preluStrides = stridesOverView(prelu);
+  const biasStrides = stridesOverView(bias, biasScratch);
+  const preluStrides = stridesOverView(prelu, preluScratch);
   const out = backend.makeOutput(outShape, 'float32');
   if (tf.util.sizeFromShape(outShape) > 0) {
     addon.fusedMatMul(

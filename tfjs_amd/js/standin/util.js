@@ -184,14 +184,9 @@ function assertAndGetBroadcastShape(shapeA, shapeB) {
   const l = Math.max(shapeA.length, shapeB.length);
   const result = new Array(l);
   for (let i = 0; i < l; i++) {
-    let a = shapeA[shapeA.length - i - 1];
-    if (a == null) {
-      a = 1;
-    }
-    let b = shapeB[shapeB.length - i - 1];
-    if (b == null) {
-      b = 1;
-    }
+    const ia = shapeA.length - i - 1, ib = shapeB.length - i - 1;
+    const a = ia >= 0 ? shapeA[ia] : 1;
+    const b = ib >= 0 ? shapeB[ib] : 1;
     if (a === 1) {
       result[l - i - 1] = b;
     } else if (b === 1) {
