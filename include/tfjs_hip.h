@@ -94,9 +94,10 @@ int tfhip_event_elapsed(int start_slot, int end_slot, float *ms);
  * tfhip_set_tuning(name, value): overrides a kernel-selection heuristic; value < 0
  *   restores it. Knobs: "tile" (GEMM tile shape index), "splitk" (K slices),
  *   "dw_rows" (depthwise rows per lane), "dw_halo" (1: LDS halo depthwise kernel),
- *   "no_skinny" (1: tiled GEMM also for tall products). TFHIP_TILE, TFHIP_SPLITK,
- *   TFHIP_DW_ROWS, TFHIP_DW_HALO, TFHIP_NO_SKINNY in the environment set them at
- *   tfhip_init(). */
+ *   "no_skinny" (1: tiled GEMM also for tall products), "dw_flat" (1: the
+ *   one-row-per-lane depthwise kernel always, 0: never). TFHIP_TILE, TFHIP_SPLITK,
+ *   TFHIP_DW_ROWS, TFHIP_DW_HALO, TFHIP_NO_SKINNY, TFHIP_DW_FLAT in the
+ *   environment set them at tfhip_init(). */
 int tfhip_set_launch_repeat(int n);
 int tfhip_last_kernel(char *name, size_t name_len);
 int tfhip_set_tuning(const char *name, int value);

@@ -220,6 +220,72 @@ h.test('hip kernels: argument checks happen on the host before any launch', () =
   h.assertEqual(require('./fake_addon').calls.length, calls + 1);
 });
 
+h.test('hip storage: a disposed buffer serves the next tensor of its size; releasePool frees them', () => {
+  useBackend('hip');
+  const backend = tf.backend();
+  const fake = require('./fake_addon');
+  backend.releasePool();
+  const live0 = fake.memoryInfo().live;
+  const a = tf.tensor(new Float32Array(77), [77]);
+  const ptr = backend.ptr(a.dataId);
+  a.dispose();
+  h.assertEqual(backend.memory().numDeviceBuffers, live0, 'a pooled buffer is not a live tensor buffer');
+  h.assertEqual(fake.memoryInfo().live, live0 + 1, 'but the native allocator still holds it');
+  h.assertEqual(backend.memory().numBytesInBackendPool, 77 * 4);
+  const b = tf.tensor(new Float32Array(77), [7, 11]);
+  h.assertEqual(backend.ptr(b.dataId), ptr, 'same size: same buffer');
+  const c = tf.tensor(new Float32Array(78), [78]);
+  h.assert(backend.ptr(c.dataId) !== ptr, 'another size: another buffer');
+  b.dispose();
+  c.dispose();
+  h.assertEqual(backend.memory().numBytesInBackendPool, (77 + 78) * 4);
+  backend.releasePool();
+  h.assertEqual(fake.memoryInfo().live, live0);
+  h.assertEqual(backend.memory().numBytesInBackendPool, 0);
+  // beyond the limit the lists are emptied instead of growing
+  const limit = backend.poolLimitBytes;
+  backend.poolLimitBytes = 1000;
+  const d = tf.tensor(new Float32Array(200), [200]), e = tf.tensor(new Float32Array(200), [200]);
+  d.dispose();
+  e.dispose();
+  h.assertEqual(backend.memory().numBytesInBackendPool, 0);
+  h.assertEqual(fake.memoryInfo().live, live0);
+  backend.poolLimitBytes = limit;
+});
+
+h.test('hip kernels: geometry and broadcast strides reach the addon as numbers in typed arrays', () => {
+  useBackend('hip');
+  const fake = require('./fake_addon');
+  const x = tf.tensor(new Float32Array(2 * 5 * 4 * 3), [2, 5, 4, 3]);
+  const w = tf.tensor(new Float32Array(3 * 3 * 3 * 8), [3, 3, 3, 8]);
+  tf.fused.conv2d({x, filter: w, strides: [2, 1], pad: 'same', bias: tf.tensor(new Float32Array(8)), activation: 'relu'});
+  let args = fake.lastArgs.fusedConv2D;
+  h.assertEqual(args[3], [2, 5, 4, 3, 3, 3, 8, 2, 1, 1, 1, 1, 1, 3, 4]);
+  h.assertEqual(args[6], [0, 0, 0, 1], 'a vector bias runs along the channels');
+  h.assertEqual(args[7], 1);
+  h.assertEqual(args[9], null);
+  const xc = tf.tensor(new Float32Array(2 * 3 * 5 * 4), [2, 3, 5, 4]);
+  tf.fused.conv2d({x: xc, filter: w, strides: 1, pad: 'same', dataFormat: 'NCHW', bias: tf.tensor(new Float32Array(8)),
+                   activation: 'prelu', preluActivationWeights: tf.tensor(new Float32Array(8 * 5 * 4), [8, 5, 4])});
+  args = fake.lastArgs.fusedConv2D;
+  h.assertEqual(args[4], 1);
+  h.assertEqual(args[6], [0, 0, 0, 1], 'NCHW: a vector bias still runs along the channels, strides in (n, h, w, c) order');
+  h.assertEqual(args[9], [0, 4, 1, 20]);
+  tf.fused.depthwiseConv2d({x, filter: tf.tensor(new Float32Array(3 * 3 * 3 * 2), [3, 3, 3, 2]), strides: 1, pad: 'valid'});
+  h.assertEqual(fake.lastArgs.fusedDepthwiseConv2D[3], [2, 5, 4, 3, 3, 3, 2, 1, 1, 1, 1, 0, 0, 3, 2]);
+  tf.fused.matMul({a: tf.tensor(new Float32Array(2 * 3 * 4), [2, 3, 4]), b: tf.tensor(new Float32Array(4 * 5), [1, 4, 5]),
+                   bias: tf.tensor(new Float32Array(2 * 5), [2, 1, 5])});
+  args = fake.lastArgs.fusedMatMul;
+  h.assertEqual(args.slice(3, 10), [2, 1, 3, 5, 4, 0, 0]);
+  h.assertEqual(args[11], [5, 0, 1]);
+  tf.add(tf.tensor(new Float32Array(6), [2, 3]), tf.tensor(new Float32Array(3), [3]));
+  args = fake.lastArgs.add;
+  h.assertEqual(args[1].slice(0, 2), [3, 1]);
+  h.assertEqual(args[3].slice(0, 2), [0, 1]);
+  h.assertEqual(args[5].slice(0, 2), [2, 3]);
+  h.assertEqual(args[6], 2);
+});
+
 h.test('hip decodeWeights: reference error messages, plain entries pass through', () => {
   useBackend('hip');
   h.assertThrows(() => hip.decodeWeights(new ArrayBuffer(1), [{name: 'w', dtype: 'float32', shape: [1], quantization: {dtype: 'uint8', scale: 1}}]),

@@ -4,12 +4,19 @@
  * buffers are host ArrayBuffers keyed by made-up addresses, and the kernel
  * entry points only record that they were called. It lets the storage logic of
  * HipBackend (dataIds, refCounts, moves, disposal, leak accounting) run in the
- * CPU-only test tier. It computes nothing.
+ * CPU-only test tier. It computes nothing; lastArgs keeps what each entry point
+ * was last called with.
  */
 let next = 0x1000;
 const blocks = new Map();
 const calls = [];
+const lastArgs = {};   // entry point -> its latest arguments (typed arrays copied)
 let inited = false;
+
+function record(name, args) {
+  calls.push(name);
+  lastArgs[name] = Array.from(args).map(a => ArrayBuffer.isView(a) ? Array.from(a) : a);
+}
 
 function need(ptr) {
   if (!blocks.has(ptr)) {
@@ -20,6 +27,7 @@ function need(ptr) {
 
 module.exports = {
   calls,
+  lastArgs,
   init() { inited = true; },
   shutdown() { inited = false; blocks.clear(); },
   deviceInfo() { return {name: 'fake', arch: 'gfx950:fake', cus: 256, clockKhz: 2400000, hbmBytes: 1 << 30}; },
@@ -50,11 +58,11 @@ module.exports = {
   eventElapsed() { return 0; },
   setLaunchRepeat() {},
   lastKernel() { return 'fake'; },
-  fusedMatMul() { calls.push('fusedMatMul'); },
-  fusedConv2D() { calls.push('fusedConv2D'); },
-  fusedDepthwiseConv2D() { calls.push('fusedDepthwiseConv2D'); },
-  dequantAffine() { calls.push('dequantAffine'); },
-  dequantF16() { calls.push('dequantF16'); },
-  add() { calls.push('add'); },
-  meanHW() { calls.push('meanHW'); }
+  fusedMatMul() { record('fusedMatMul', arguments); },
+  fusedConv2D() { record('fusedConv2D', arguments); },
+  fusedDepthwiseConv2D() { record('fusedDepthwiseConv2D', arguments); },
+  dequantAffine() { record('dequantAffine', arguments); },
+  dequantF16() { record('dequantF16', arguments); },
+  add() { record('add', arguments); },
+  meanHW() { record('meanHW', arguments); }
 };

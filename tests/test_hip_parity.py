@@ -235,7 +235,9 @@ def test_conv2d_epilogue_forms(hip, orc, act, bias_shape, prelu_shape):
     ((1, 11, 10, 6), (5, 3, 6, 3), (2, 1), 1, "same"), ((1, 11, 10, 8), (3, 3, 8, 1), 1, 2, "same"),
     ((1, 8, 8, 8), (3, 3, 8, 1), 1, 1, 1), ((1, 6, 6, 8), (3, 3, 8, 1), 1, 1, [[0, 0], [2, 0], [1, 3], [0, 0]]),
 ])
-def test_depthwise_shapes(hip, orc, xs, fs, stride, dil, pad):
+@pytest.mark.parametrize("flat", [0, 1])
+def test_depthwise_shapes(hip, orc, tuning, xs, fs, stride, dil, pad, flat):
+    tuning("dw_flat", flat)   # 3x3 with four-channel groups: one row per lane, or the row pipeline
     rng = np.random.default_rng(sum(xs) + sum(fs) * 3)
     x = rng.uniform(0, 1, xs).astype(np.float32)
     w = rng.normal(0, 0.5, fs).astype(np.float32)
@@ -247,8 +249,10 @@ def test_depthwise_shapes(hip, orc, xs, fs, stride, dil, pad):
 @pytest.mark.parametrize("stride", [1, 2])
 @pytest.mark.parametrize("act", ["linear", "relu", "elu", "sigmoid", "leakyrelu", "prelu"])
 @pytest.mark.parametrize("bias_shape,prelu_shape", [((8,), (8,)), ((), (1, 1, 8)), ((5, 8), (6, 5, 1)), ((2, 6, 5, 8), (1,))])
-def test_depthwise_epilogue_forms(hip, orc, act, bias_shape, prelu_shape, stride):
-    # 3x3 with four-channel groups: the row-pipeline kernel, both epilogue variants
+@pytest.mark.parametrize("flat", [0, 1])
+def test_depthwise_epilogue_forms(hip, orc, tuning, act, bias_shape, prelu_shape, stride, flat):
+    # 3x3 with four-channel groups: the row-pipeline kernel and the one-row-per-lane kernel, both epilogue variants
+    tuning("dw_flat", flat)
     rng = np.random.default_rng(29)
     x = rng.uniform(-1, 1, (2, 6 * stride, 5 * stride, 8)).astype(np.float32)
     w = rng.normal(0, 0.5, (3, 3, 8, 1)).astype(np.float32)
@@ -332,6 +336,25 @@ def test_conv2d_few_input_channels(hip, orc, xs, fs, stride, dil, pad, act, bias
     kw = dict(strides=stride, dilations=dil, pad=pad, activation=act,
               bias=None if bias_shape is None else rng.uniform(-1, 1, bias_shape).astype(np.float32),
               prelu=rng.uniform(0, 1, (16,)).astype(np.float32) if act == "prelu" else None)
+    assert_parity(hip.fused_conv2d(x, w, **kw), orc.fused_conv2d(x, w, **kw))
+
+
+@pytest.mark.parametrize("xs,fs,stride,dil,pad,act", [
+    ((3, 37, 41, 3), (3, 3, 3, 32), 2, 1, "same", "relu6"),       # several 256-pixel chunks, rows of 21 pixels
+    ((2, 20, 18, 3), (3, 3, 3, 48), 1, 1, "valid", "relu"),        # three groups of 16 channels
+    ((1, 40, 40, 2), (3, 3, 2, 64), 1, 2, "same", "linear"),       # dilated, two groups of 32 channels
+    ((5, 9, 9, 4), (3, 3, 4, 32), 3, 1, [[0, 0], [2, 1], [0, 3], [0, 0]], "relu6"),
+    ((1, 33, 5, 1), (3, 3, 1, 32), 1, 1, "same", "relu"),          # rows shorter than a block of 16 pixels
+    ((2, 12, 300, 3), (1, 7, 3, 16), (1, 2), 1, "same", "linear"), # a 1x7 filter, 21 taps
+    ((8, 600, 600, 1), (3, 3, 1, 16), 1, 1, "same", "relu6"),      # more chunks than workgroups: several trips each
+])
+def test_conv2d_few_taps_shapes(hip, orc, xs, fs, stride, dil, pad, act):
+    # the matrix-core stem kernel: at most 36 taps, 16 or 32 channels per workgroup column
+    rng = np.random.default_rng(59)
+    x = rng.uniform(-1, 1, xs).astype(np.float32)
+    w = rng.normal(0, 0.4, fs).astype(np.float32)
+    kw = dict(strides=stride, dilations=dil, pad=pad, activation=act,
+              bias=rng.uniform(-1, 1, (fs[3],)).astype(np.float32))
     assert_parity(hip.fused_conv2d(x, w, **kw), orc.fused_conv2d(x, w, **kw))
 
 
@@ -442,6 +465,10 @@ def test_add_and_mean(hip, orc):
     np.testing.assert_array_equal(hip.mean_hw(a), orc.mean_hw(a))
     big = rng.uniform(0, 6, (4, 7, 7, 1280)).astype(np.float32)
     np.testing.assert_array_equal(hip.mean_hw(big), orc.mean_hw(big))
+    # channel counts off the 16-byte path, a single position, more positions than one pass of the slices
+    for shape in [(3, 5, 4, 7), (2, 1, 1, 12), (3, 13, 11, 36), (1, 2, 3, 4)]:
+        t = rng.uniform(-3, 3, shape).astype(np.float32)
+        assert_parity(hip.mean_hw(t), orc.mean_hw(t))
 
 
 # ------------------------------------------------------------------ error paths

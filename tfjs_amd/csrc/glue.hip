@@ -60,6 +60,57 @@ __global__ __launch_bounds__(256) void mean_hw(const float *__restrict__ x, floa
   }
 }
 
+// The same for c % 4 == 0: a lane takes four channels (one 16-byte load per
+// position) and one of eight interleaved slices of the h*w positions, so that all
+// loads of a small feature map are in flight at once; the eight partial sums
+// (double, positions in ascending order within a slice) are added in slice
+// order through LDS.
+__global__ __launch_bounds__(256) void mean_hw_vec(const float *__restrict__ x, float *__restrict__ y, long long batch,
+                                                   long long hw, long long c) {
+  __shared__ double part[8][32][4];
+  const float denom = (float)hw;
+  const int slice = threadIdx.x >> 5, q = threadIdx.x & 31;
+  const long long quads = c / 4, total = batch * quads;
+  for (long long base = (long long)blockIdx.x * 32; base < total; base += (long long)gridDim.x * 32) {
+    const long long i = base + q;
+    double sum[4] = {0.0, 0.0, 0.0, 0.0};
+    if (i < total) {
+      const long long n = i / quads, cq = i - n * quads;
+      const float4 *px = reinterpret_cast<const float4 *>(x + n * hw * c + cq * 4);
+      for (long long j0 = slice; j0 < hw; j0 += 64) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const long long j = j0 + 8 * u;
+          v[u] = j < hw ? px[j * quads] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (j0 + 8 * u >= hw) continue;
+          sum[0] += (double)__fdiv_rn(v[u].x, denom);
+          sum[1] += (double)__fdiv_rn(v[u].y, denom);
+          sum[2] += (double)__fdiv_rn(v[u].z, denom);
+          sum[3] += (double)__fdiv_rn(v[u].w, denom);
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) part[slice][q][k] = sum[k];
+    __syncthreads();
+    if (threadIdx.x < 128) {
+      const int qq = threadIdx.x >> 2, k = threadIdx.x & 3;
+      const long long o = base + qq;
+      if (o < total) {
+        double t = 0.0;
+#pragma unroll
+        for (int sl = 0; sl < 8; ++sl) t += part[sl][qq][k];
+        y[o * 4 + k] = (float)t;
+      }
+    }
+    __syncthreads();
+  }
+}
+
 __global__ __launch_bounds__(256) void copy_f4(const float4 *__restrict__ src, float4 *__restrict__ dst, long long n4) {
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) dst[i] = src[i];
@@ -120,6 +171,13 @@ int tfhip_mean_hw(const float *x, float *y, int64_t batch, int64_t h, int64_t w,
   if (batch * c == 0) return kOk;
   TFHIP_CHECK_RANGE(x, batch * h * w * c, 4, "x");
   TFHIP_CHECK_RANGE(y, batch * c, 4, "y");
+  if (c % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+    long long blocks = (batch * (c / 4) + 31) / 32;
+    const long long cap = (long long)num_cus() * 32;
+    note_kernel("mean_hw_vec");
+    TFHIP_LAUNCH((mean_hw_vec<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, stream()>>>(x, y, batch, h * w, c)));
+    return kOk;
+  }
   note_kernel("mean_hw");
   TFHIP_LAUNCH((mean_hw<<<grid_for(batch * c), 256, 0, stream()>>>(x, y, batch, h * w, c)));
   return kOk;
