@@ -97,14 +97,22 @@ def last_kernel(lib):
     return buf.value.decode()
 
 
-def time_launches(lib, check, ev, fn, repeat=50, rounds=3):
+def time_launches(lib, check, ev, fn, repeat=50, rounds=3, settle_ms=20.0):
     """Average duration in seconds of one launch of the kernel `fn` enqueues:
-    `repeat` launches back to back between two events, best of `rounds`."""
+    `repeat` launches back to back between two events, best of `rounds`. The
+    GPU idles at a fraction of its clock and needs about 10 ms of work to reach
+    the sustained one, so the kernel first runs untimed for `settle_ms`."""
     fn()
     check(lib.tfhip_sync())
     check(lib.tfhip_set_launch_repeat(repeat))
     best = None
     try:
+        settled = 0.0
+        while settled < settle_ms:
+            ev.record(0)
+            fn()
+            ev.record(1)
+            settled += max(ev.elapsed_ms(0, 1), 0.01)
         for _ in range(rounds):
             ev.record(0)
             fn()

@@ -535,13 +535,16 @@ extern "C" int tfhip_fused_depthwise_conv2d(
     g.c4_total = (int)(in_c / 4);
     g.strips_w = ((int)out_w + kRowsPW - 1) / kRowsPW;
     {
-      // one output row per lane when all its wavefronts are resident at once (measured
-      // against the row pipeline: 5-15% faster up to about 3000 wavefronts, slower beyond)
+      // one output row per lane when all its wavefronts are resident at once and the
+      // input is small enough for its rows, each fetched by up to three output rows,
+      // to come from cache (measured against the row pipeline: 5-15% faster up to
+      // about 3000 wavefronts and 24 MB, slower beyond either)
       const long long flat_strips = (long long)batch * out_h * g.strips_w;
       const long long flat_blocks = (flat_strips + kSlots - 1) / kSlots;
       const long long flat_waves = flat_blocks * ((g.c4_total + kCQ - 1) / kCQ) * 4;
       const int forced = tuning(kTuneDwFlat);
-      const bool flat = forced >= 0 ? forced > 0 : (tuning(kTuneDwRows) <= 0 && flat_waves <= (long long)num_cus() * 12);
+      const bool flat = forced >= 0 ? forced > 0 : (tuning(kTuneDwRows) <= 0 && flat_waves <= (long long)num_cus() * 12 &&
+                                              batch * in_h * in_w * in_c * 4 <= 24000000);
       if (flat && flat_blocks <= 0x7fffffffLL) {
         g.rows = 1;
         g.chunks_h = (int)out_h;
