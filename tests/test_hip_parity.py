@@ -298,6 +298,20 @@ def test_matmul_tall_small_b(hip, orc, m, n, k, act):
     assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
 
 
+@pytest.mark.parametrize("regs", [0, 1])
+@pytest.mark.parametrize("m,n,k,act", [(65537, 16, 8, "relu"), (66000, 32, 12, "linear"), (65700, 48, 20, "relu6"),
+                                        (65600, 64, 28, "leakyrelu"), (65536, 96, 32, "relu6"), (98400, 144, 16, "relu"),
+                                        (98310, 136, 24, "relu6")])
+def test_matmul_tall_tiny_k(hip, orc, tuning, m, n, k, act, regs):
+    # K <= 32: B lives in registers (every column-group count, full and half k groups), or in LDS when told so
+    tuning("skinny_regs", regs)
+    rng = np.random.default_rng(m + n + k)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 0.3, (k, n)).astype(np.float32)
+    kw = dict(bias=rng.uniform(-1, 1, (n,)).astype(np.float32), activation=act, leakyrelu_alpha=0.1)
+    assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
+
+
 def test_pointwise_conv_tall(hip, orc):
     rng = np.random.default_rng(53)
     x = rng.uniform(0, 1, (14, 87, 86, 24)).astype(np.float32)

@@ -182,6 +182,150 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
   }
 }
 
+// The same product with B held in REGISTERS instead of LDS, for K <= 32: a B so
+// small that staging it through LDS - two memory round trips and a workgroup
+// barrier before the first row block - costs more than the few row blocks each
+// wavefront then has to do (measured 5-20% faster up to K = 32, 25% slower at
+// K = 96 and 144, where the LDS kernel stays). Every wavefront
+// is on its own: it fetches its share of B once (lane (g, r) keeps
+// B[k][16 n + r] for exactly the k it will feed) together with its first rows
+// of A and streams over its row blocks with the next block's A in flight.
+//   KF    full k groups of 16 (lane takes k = 16 t + 4 g + j, a float4 of A)
+//   HALF  one more group of 8 (lane takes k = 16 KF + 2 g + j, a float2 of A):
+//         K = 24 costs six matrix instructions per block instead of eight
+template <int TN, int KF, bool HALF>
+__global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
+  constexpr int STEPS = 4 * KF + (HALF ? 2 : 0);
+  const int lane = threadIdx.x & 63;
+  const int grp = lane >> 4, r = lane & 15;
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)uniform_pointer(g.a), 0, (int)g.a_bytes, 0x00020000);
+  const int blocks = (g.M + 15) / 16;
+  const int waves = gridDim.x * 4;
+  const int first = blockIdx.x * 4 + (threadIdx.x >> 6);
+
+  struct ABlock {
+    float4 full[KF > 0 ? KF : 1];
+    float2 half;
+  };
+  auto issue = [&](ABlock &dst, int b) __attribute__((always_inline)) {
+    const int row = b * 16 + r;
+    const bool row_ok = b < blocks && row < g.M;
+#pragma unroll
+    for (int t = 0; t < KF; ++t) {
+      const int k = 16 * t + 4 * grp;
+      const unsigned off = (row_ok && k < g.K) ? (unsigned)(((long long)row * g.K + k) * 4) : kNoOffset;
+      dst.full[t] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
+    }
+    if (HALF) {
+      const int k = 16 * KF + 2 * grp;
+      const unsigned off = (row_ok && k < g.K) ? (unsigned)(((long long)row * g.K + k) * 4) : kNoOffset;
+      const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)off, 0, 0);
+      dst.half = make_float2(__uint_as_float(v[0]), __uint_as_float(v[1]));
+    }
+  };
+  ABlock cur, nxt;
+  issue(cur, first);
+
+  // this lane's B values and epilogue operands
+  float breg[STEPS][TN];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const int k = s < 4 * KF ? 16 * (s / 4) + 4 * grp + s % 4 : 16 * KF + 2 * grp + (s - 4 * KF);
+#pragma unroll
+    for (int n = 0; n < TN; ++n) {
+      const int col = n * 16 + r;
+      breg[s][n] = (k < g.K && col < g.N) ? g.b[(long long)k * g.N + col] : 0.f;
+    }
+  }
+  float4_t bias4[TN];
+#pragma unroll
+  for (int n = 0; n < TN; ++n)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int col = n * 16 + grp * 4 + q;
+      bias4[n][q] = (g.bias && col < g.N) ? g.bias[(long long)col * g.bias_stride] : 0.f;
+    }
+
+  for (int b = first; b < blocks; b += waves) {
+    issue(nxt, b + waves);   // past the end: every offset is out of range, nothing is read
+    float4_t acc[TN];
+#pragma unroll
+    for (int n = 0; n < TN; ++n) acc[n] = bias4[n];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      float av;
+      if (s < 4 * KF) {
+        const float4 v = cur.full[s / 4 < KF ? s / 4 : 0];
+        av = s % 4 == 0 ? v.x : (s % 4 == 1 ? v.y : (s % 4 == 2 ? v.z : v.w));
+      } else {
+        av = s - 4 * KF == 0 ? cur.half.x : cur.half.y;
+      }
+#pragma unroll
+      for (int n = 0; n < TN; ++n) acc[n] = __builtin_amdgcn_mfma_f32_16x16x4f32(breg[s][n], av, acc[n], 0, 0, 0);
+    }
+    // lane holds row b*16 + r, columns n*16 + 4*grp .. +3
+    const int row = b * 16 + r;
+#pragma unroll
+    for (int n = 0; n < TN; ++n) {
+      const int col = n * 16 + grp * 4;
+      float out[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float v = acc[n][k];
+        switch (g.activation) {
+          case TFHIP_RELU: v = (v > 0.f || v != v) ? v : 0.f; break;
+          case TFHIP_RELU6: v = (v > 0.f || v != v) ? v : 0.f; v = v > 6.f ? 6.f : v; break;
+          case TFHIP_LEAKYRELU: v = v < 0.f ? (float)(g.leaky_alpha * (double)v) : v; break;
+          default: break;
+        }
+        out[k] = v;
+      }
+      if (row < g.M && col < g.N)
+        *reinterpret_cast<float4 *>(g.c + (long long)row * g.N + col) = make_float4(out[0], out[1], out[2], out[3]);
+    }
+    cur = nxt;
+  }
+}
+
+template <int TN, int KF, bool HALF>
+inline int launch_skinny_regs(const SkinnyArgs &g) {
+  static int resident = 0;   // workgroups per compute unit at this instantiation's register count
+  if (resident == 0) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_gemm_regs<TN, KF, HALF>, 256, 0) != hipSuccess || n < 1) {
+      (void)hipGetLastError();
+      n = 1;
+    }
+    resident = n;
+  }
+  // all workgroups resident at once; wavefront w takes row blocks w, w + waves, ...
+  const long long blocks = (g.M + 15) / 16;
+  long long grid = (blocks + 3) / 4;
+  const long long cap = (long long)num_cus() * resident;
+  if (grid > cap) grid = cap;
+  note_kernel("skinny_gemm_regs<%d, %d, %s>", TN, KF, HALF ? "true" : "false");
+  TFHIP_LAUNCH((skinny_gemm_regs<TN, KF, HALF><<<dim3((unsigned)grid), dim3(256), 0, stream()>>>(g)));
+  return kOk;
+}
+
+// Dispatch over the instantiated (columns, k) combinations; -1 when there is none.
+template <int TN>
+inline int launch_skinny_regs_tn(const SkinnyArgs &g) {
+  const int kf = g.K / 16, rest = g.K % 16;
+  if (rest == 0) {
+    if (kf == 1) return launch_skinny_regs<TN, 1, false>(g);
+    if (kf == 2) return launch_skinny_regs<TN, 2, false>(g);
+  } else if (rest <= 8) {
+    if (kf == 0) return launch_skinny_regs<TN, 0, true>(g);
+    if (kf == 1) return launch_skinny_regs<TN, 1, true>(g);
+  } else {
+    if (kf == 0) return launch_skinny_regs<TN, 1, false>(g);
+    if (kf == 1) return launch_skinny_regs<TN, 2, false>(g);
+  }
+  return -1;
+}
+
 // Instantiated widths in groups of 16 columns (0: too wide).
 inline int skinny_groups(int n) {
   const int tn = (n + 15) / 16;
@@ -228,6 +372,19 @@ inline int launch_skinny(const GemmParams &p) {
   g.k_pad = (p.K + kSkinnyChunk - 1) / kSkinnyChunk * kSkinnyChunk;
   g.a_bytes = p.a_bytes;
   g.activation = p.epi.activation;
+  if (tuning(kTuneSkinnyRegs) != 0) {   // B in registers where an instantiation fits
+    int rc = -1;
+    switch (skinny_groups(p.N)) {
+      case 1: rc = launch_skinny_regs_tn<1>(g); break;
+      case 2: rc = launch_skinny_regs_tn<2>(g); break;
+      case 3: rc = launch_skinny_regs_tn<3>(g); break;
+      case 4: rc = launch_skinny_regs_tn<4>(g); break;
+      case 6: rc = launch_skinny_regs_tn<6>(g); break;
+      case 9: rc = launch_skinny_regs_tn<9>(g); break;
+      default: break;
+    }
+    if (rc >= 0) return rc;
+  }
   switch (skinny_groups(p.N)) {
     case 1: return launch_skinny_tn<1>(g);
     case 2: return launch_skinny_tn<2>(g);
