@@ -393,7 +393,7 @@ def main():
     info = pyhost.device_info()
     model_dir = tempfile.mkdtemp(prefix="tfjs_hip_mobilenet_")
     try:
-        workloads.write_model(model_dir, workloads.mobilenet_v2_weights(seed=3), np.uint8)
+        workloads.write_graph_model(model_dir, workloads.mobilenet_v2_weights(seed=3), np.uint8)
         js = bench_model_node(model_dir, args.steps, args.warmup, args.jit_prime)
         m = bench_model(model_dir, args.steps, args.warmup)
         cpu = None if args.no_cpu_baseline else cpu_baseline(model_dir)
@@ -405,7 +405,8 @@ def main():
     kernels = None if args.no_kernels else bench_kernels()
     copy_gbs = copy_yardstick(args.copy_yardstick) if args.copy_yardstick else None
     ms_per_step = js["ms_per_step"] if js else m["ms_per_step"]
-    host = ("node %s, tfjs API -> KernelBackend 'hip' -> N-API addon -> C ABI (tfjs-core: %s)" % (js["node"], js["core"])
+    host = ("node %s, %s -> tfjs API -> KernelBackend 'hip' -> N-API addon -> C ABI (tfjs-core: %s)"
+            % (js["node"], js["model_api"], js["core"])
             if js else "python/ctypes over the C ABI (node or the addon not found)")
     line = {
         "metric": "MobileNetV2 b32 images/s + fused-op TFLOP/s & % of roofline, 1 MI355X",

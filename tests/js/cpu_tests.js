@@ -306,4 +306,118 @@ h.test('hip decodeWeights: reference error messages, plain entries pass through'
   h.assertThrows(() => hip.decodeWeights(new ArrayBuffer(0), []), /needs the 'hip' backend to be active/);
 });
 
+// ---- graph model stand-in over the JavaScript oracle backend ------------------------
+const b64 = t => Buffer.from(t).toString('base64');
+function tinyGraphArtifacts() {
+  // Placeholder -> _FusedConv2D(3x3/2, relu6) -> FusedDepthwiseConv2dNative -> AddV2 -> Mean -> _FusedMatMul -> Identity
+  const fused = (ops, n) => ({fused_ops: {list: {s: ops.map(b64)}}, num_args: {i: String(n)}, leakyrelu_alpha: {f: 0.2}});
+  const convAttrs = (stride, ops, n, pad) => Object.assign(fused(ops, n), {
+    strides: {list: {i: ['1', String(stride), String(stride), '1']}}, dilations: {list: {i: ['1', '1', '1', '1']}},
+    padding: {s: b64(pad || 'SAME')}, data_format: {s: b64('NHWC')}, explicit_paddings: {list: {}}});
+  const node = (name, op, input, attr) => ({name, op, input, attr: attr || {}});
+  const nodes = [
+    node('x', 'Placeholder', [], {dtype: {type: 'DT_FLOAT'}, shape: {shape: {dim: [{size: '-1'}, {size: '8'}, {size: '8'}, {size: '3'}]}}}),
+    node('c/w', 'Const'), node('c/b', 'Const'), node('d/w', 'Const'), node('d/b', 'Const'), node('axes', 'Const'),
+    node('f/w', 'Const'), node('f/b', 'Const'), node('f/alpha', 'Const'),
+    node('c', '_FusedConv2D', ['x', 'c/w', 'c/b'], convAttrs(2, ['BiasAdd', 'Relu6'], 1)),
+    node('d', 'FusedDepthwiseConv2dNative', ['c:0', 'd/w', 'd/b'], convAttrs(1, ['BiasAdd'], 1)),
+    node('sum', 'AddV2', ['c', 'd', '^x']),
+    node('pool', 'Mean', ['sum', 'axes'], {keep_dims: {b: false}}),
+    node('f', '_FusedMatMul', ['pool', 'f/w', 'f/b', 'f/alpha'],
+         Object.assign(fused(['BiasAdd', 'Prelu'], 2), {transpose_a: {b: false}, transpose_b: {b: true}})),
+    node('out', 'Identity', ['f'])
+  ];
+  let seed = 7;
+  const rnd = n => Float32Array.from({length: n}, () => ((seed = (Math.imul(seed, 1664525) + 1013904223) >>> 0) / 2 ** 32) - 0.5);
+  const values = {'c/w': [rnd(3 * 3 * 3 * 4), [3, 3, 3, 4]], 'c/b': [rnd(4), [4]], 'd/w': [rnd(3 * 3 * 4), [3, 3, 4, 1]],
+                  'd/b': [rnd(4), [4]], 'axes': [Int32Array.from([1, 2]), [2]], 'f/w': [rnd(5 * 4), [5, 4]],
+                  'f/b': [rnd(5), [5]], 'f/alpha': [rnd(5), [5]]};
+  const specs = [], chunks = [];
+  Object.keys(values).forEach(name => {
+    const [v, shape] = values[name];
+    specs.push({name, shape, dtype: v instanceof Int32Array ? 'int32' : 'float32'});
+    chunks.push(Buffer.from(v.buffer, v.byteOffset, v.byteLength));
+  });
+  const all = Buffer.concat(chunks);
+  return {
+    artifacts: {
+      modelTopology: {node: nodes, versions: {producer: 1, minConsumer: 0}},
+      signature: {inputs: {image: {name: 'x:0', dtype: 'DT_FLOAT'}}, outputs: {scores: {name: 'out:0', dtype: 'DT_FLOAT'}}},
+      weightSpecs: specs,
+      weightData: all.buffer.slice(all.byteOffset, all.byteOffset + all.byteLength)
+    },
+    values
+  };
+}
+
+h.test('graph model: a converter-format topology runs through the fused ops and matches the direct calls', () => {
+  useBackend('cpu');
+  const {artifacts, values} = tinyGraphArtifacts();
+  const io = {decodeWeights: oracleDecode.decodeWeights};
+  const before = tf.memory().numTensors;
+  const model = hip.loadGraphModel({load: () => artifacts}, {}, io);
+  h.assertEqual(model.inputs, [{name: 'image', shape: [-1, 8, 8, 3], dtype: 'float32'}]);
+  h.assertEqual(model.outputs, [{name: 'scores'}]);
+  h.assertEqual(model.version, '1.0');
+  const x = tf.tensor(Float32Array.from({length: 2 * 8 * 8 * 3}, (_, i) => Math.sin(i)), [2, 8, 8, 3]);
+  const t = name => tf.tensor(values[name][0], values[name][1]);
+  const want = tf.tidy(() => {
+    const c = tf.fused.conv2d({x, filter: t('c/w'), strides: [2, 2], pad: 'same', dataFormat: 'NHWC', dilations: [1, 1],
+                               bias: t('c/b'), activation: 'relu6'});
+    const d = tf.fused.depthwiseConv2d({x: c, filter: t('d/w'), strides: [1, 1], pad: 'same', dataFormat: 'NHWC',
+                                        dilations: [1, 1], bias: t('d/b')});
+    const pooled = tf.mean(tf.add(c, d), [1, 2]);
+    return tf.fused.matMul({a: pooled, b: t('f/w'), transposeB: true, bias: t('f/b'), activation: 'prelu',
+                            preluActivationWeights: t('f/alpha')}).dataSync();
+  });
+  const live = tf.memory().numTensors;
+  const y = model.predict(x);
+  h.assertEqual(y.shape, [2, 5]);
+  h.assertBitsEqual(y.dataSync(), want);
+  h.assertEqual(tf.memory().numTensors, live + 1, 'predict leaves only its result behind');
+  y.dispose();
+  // by name, an intermediate node as output, and several outputs
+  const mid = model.execute({image: x}, ['pool', 'scores']);
+  h.assertEqual(mid[0].shape, [2, 4]);
+  h.assertBitsEqual(mid[1].dataSync(), want);
+  tf.dispose(mid);
+  h.assertThrows(() => model.predict([x, x]), /Input tensor count mismatch, the graph model has 1 non-resource placeholders, while there are 2/);
+  h.assertThrows(() => model.execute({picture: x}), /keys: \[picture\] that are not part of graph/);
+  h.assertThrows(() => model.execute({image: x}, 'nowhere'), /The output 'nowhere' is not found in the graph/);
+  const thin = tf.tensor(new Float32Array(2 * 8 * 8), [2, 8, 8, 1]);
+  h.assertThrows(() => model.predict(thin),
+                 /The shape of dict\['x'\] provided in model.execute\(dict\) must be \[-1,8,8,3\], but was \[2,8,8,1\]/);
+  const ints = tf.tensor(new Int32Array(8 * 8 * 3), [1, 8, 8, 3], 'int32');
+  h.assertThrows(() => model.predict(ints),
+                 /The dtype of dict\['x'\] provided in model.execute\(dict\) must be float32, but was int32/);
+  tf.dispose([thin, ints]);
+  h.assertThrows(() => model.execute({}, 'scores'), /Missing the following inputs: \[x\]/);
+  x.dispose();
+  model.dispose();
+  h.assertEqual(tf.memory().numTensors, before);
+});
+
+h.test('graph model: unsupported nodes and malformed fused nodes throw the reference errors', () => {
+  useBackend('cpu');
+  const io = {decodeWeights: oracleDecode.decodeWeights};
+  const make = mutate => {
+    const {artifacts} = tinyGraphArtifacts();
+    mutate(artifacts.modelTopology.node);
+    return hip.loadGraphModel({load: () => artifacts}, {}, io);
+  };
+  const x = tf.tensor(new Float32Array(8 * 8 * 3), [1, 8, 8, 3]);
+  let m = make(nodes => nodes.find(n => n.name === 'sum').op = 'Einsum');
+  h.assertThrows(() => m.predict(x), /Node type Einsum is not implemented/);
+  m.dispose();
+  m = make(nodes => nodes.find(n => n.name === 'c').attr.num_args = {i: '2'});
+  h.assertThrows(() => m.predict(x), /with BiasAdd must have one extra argument: bias/);
+  m.dispose();
+  m = make(nodes => nodes.find(n => n.name === 'f').attr.num_args = {i: '1'});
+  h.assertThrows(() => m.predict(x), /Fused MatMul with BiasAdd and Prelu must have two extra arguments: bias and alpha/);
+  m.dispose();
+  h.assertThrows(() => hip.loadGraphModel(null), /modelUrl in loadGraphModel\(\) cannot be null/);
+  h.assertThrows(() => new hip.GraphModel({}, {}, io).load(), /does not have the `load` method implemented/);
+  x.dispose();
+});
+
 h.run('node cpu tests');

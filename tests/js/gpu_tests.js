@@ -166,6 +166,30 @@ h.test('config 4: MobileNetV2 batch 2 through the tfjs API, uint8 weights dequan
   h.assertParity(got, want);
 });
 
+h.test('config 4 as a converter-format graph model: loadGraphModel + injected decodeWeights == the direct model', () => {
+  const dir = process.env.TFJS_HIP_TEST_MODEL_DIR;
+  h.assert(dir && fs.existsSync(path.join(dir, 'model.json')),
+           'TFJS_HIP_TEST_MODEL_DIR must hold a model.json written by tfjs_amd.workloads.write_graph_model');
+  h.assert(tf.engine().setBackend('hip') === true);
+  const before = tf.backend().numDataIds();
+  // graph_model.ts:104-107: the io module is the third constructor argument
+  const model = hip.loadGraphModel(dir, {}, {decodeWeights: hip.decodeWeights});
+  h.assertEqual(model.inputs[0].shape, [-1, 224, 224, 3]);
+  const m = mobilenet.readModel(dir);
+  const wHip = hip.decodeWeights(m.buffer, m.specs);
+  const x = tf.tensor(mobilenet.syntheticInput(2, 3), [2, 224, 224, 3]);
+  const direct = mobilenet.buildPredict(tf, wHip)(x);
+  const y = model.predict(x);
+  h.assertEqual(y.shape, [2, 1000]);
+  h.assertBitsEqual(y.dataSync(), direct.dataSync());
+  const again = model.execute({input: x}, 'Identity');
+  h.assertBitsEqual(again.dataSync(), direct.dataSync());
+  tf.dispose([y, again, direct, x]);
+  tf.dispose(wHip);
+  model.dispose();
+  h.assertEqual(tf.backend().numDataIds(), before, 'model, weights and results are all released');
+});
+
 h.test('backend: tensors migrate cpu <-> hip with values and refCounts; tf.time reports device ms', async () => {
   h.assert(tf.engine().setBackend('cpu') === true);
   const a = tf.tensor([1, 2, 3, 4], [2, 2]);

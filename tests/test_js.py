@@ -121,7 +121,7 @@ def test_addon_loads_and_exports_every_entry_point():
 @needs_node
 def test_node_gpu_tier(tmp_path):
     from tfjs_amd import workloads
-    workloads.write_model(str(tmp_path), workloads.mobilenet_v2_weights(seed=3), np.uint8)
+    workloads.write_graph_model(str(tmp_path), workloads.mobilenet_v2_weights(seed=3), np.uint8)
     proc = run_node("tests/js/gpu_tests.js", env={"TFJS_HIP_TEST_MODEL_DIR": str(tmp_path)})
     assert proc.returncode == 0, proc.stdout[-4000:]
     assert " 0 failed" in proc.stdout

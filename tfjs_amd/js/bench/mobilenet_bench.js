@@ -9,6 +9,8 @@
  * drained on both sides), load_ms (read + upload + GPU dequant of the weights),
  * kernel_ms_per_step (device time between two events around the same steps).
  */
+const fs = require('fs');
+const path = require('path');
 const hip = require('../index');
 const model = require('../models/mobilenet_v2');
 const {addon} = require('../binding');
@@ -23,11 +25,20 @@ async function main() {
   const prime = parseInt(process.argv[6] || '0', 10);
   await tf.setBackend('hip');
   const t0 = tf.util.now();
-  const m = model.readModel(modelDir);
-  const weights = hip.decodeWeights(m.buffer, m.specs);
+  // A converter-format model.json runs as a graph model (model.predict, what a
+  // tfjs user of a converted network calls); a bare weights manifest through the
+  // same ops called directly.
+  const asGraph = fs.existsSync(path.join(modelDir, 'model.json'));
+  let predict;
+  if (asGraph) {
+    const graph = hip.loadGraphModel(modelDir, {}, {decodeWeights: hip.decodeWeights});
+    predict = x => graph.predict(x);
+  } else {
+    const m = model.readModel(modelDir);
+    predict = model.buildPredict(tf, hip.decodeWeights(m.buffer, m.specs));
+  }
   addon.sync();
   const loadMs = tf.util.now() - t0;
-  const predict = model.buildPredict(tf, weights);
   const x = tf.tensor(model.syntheticInput(batch, 3), [batch, 224, 224, 3]);
   let checksum = 0;
   const step = () => {
@@ -73,6 +84,7 @@ async function main() {
     checksum,
     node: process.version,
     core: tf.usingStandin ? 'standin' : '@tensorflow/tfjs-core',
+    model_api: asGraph ? 'GraphModel.predict (converter-format model.json)' : 'fused ops called directly',
     device: tf.backend().deviceInfo,
     num_tensors: mem.numTensors,
     num_device_buffers: mem.numDeviceBuffers

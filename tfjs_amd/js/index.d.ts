@@ -46,3 +46,24 @@ export declare function decodeWeights(
 
 export declare const kernelConfigs: KernelConfig[];
 export declare const version: string;
+
+/** Stand-in for tfjs-converter's GraphModel over the ops of the fused inference path. */
+export interface IoWithDecodeWeights {
+  decodeWeights(buffer: ArrayBuffer, specs: object[]): {[name: string]: Tensor};
+}
+export interface ModelArtifactsHandler {
+  load(): object | Promise<object>;
+}
+export declare class GraphModel {
+  constructor(handlerOrPath: string | ModelArtifactsHandler, loadOptions?: object, tfio?: IoWithDecodeWeights);
+  load(): boolean | Promise<boolean>;
+  predict(inputs: Tensor | Tensor[] | {[name: string]: Tensor}, config?: object): Tensor | Tensor[];
+  execute(inputs: Tensor | Tensor[] | {[name: string]: Tensor}, outputs?: string | string[]): Tensor | Tensor[];
+  dispose(): void;
+  readonly inputs: Array<{name: string, shape?: number[], dtype?: string}>;
+  readonly outputs: Array<{name: string}>;
+  readonly weights: {[name: string]: Tensor};
+}
+export declare function loadGraphModel(
+    modelUrl: string | ModelArtifactsHandler, options?: object, tfio?: IoWithDecodeWeights): GraphModel | Promise<GraphModel>;
+export declare function fileSystem(path: string): ModelArtifactsHandler;

@@ -15,6 +15,7 @@ const {decodeWeights} = require('./io/decode_weights');
 const matmul = require('./kernels/matmul');
 const conv = require('./kernels/conv');
 const glue = require('./kernels/glue');
+const graphModel = require('./standin/graph_model');
 
 const kernelConfigs = [
   matmul.fusedMatMulConfig, matmul.batchMatMulConfig, conv.fusedConv2DConfig,
@@ -26,4 +27,14 @@ const kernelConfigs = [
 tf.registerBackend('hip', () => new HipBackend(), 3 /* priority */);
 kernelConfigs.forEach(config => tf.registerKernel(config));
 
-module.exports = {tf, HipBackend, decodeWeights, kernelConfigs, version: '0.1.0'};
+module.exports = {
+  tf,
+  HipBackend,
+  decodeWeights,
+  kernelConfigs,
+  // graph-model loader for where @tensorflow/tfjs-converter is not installed
+  GraphModel: graphModel.GraphModel,
+  loadGraphModel: graphModel.loadGraphModel,
+  fileSystem: graphModel.fileSystem,
+  version: '0.1.0'
+};

@@ -89,6 +89,86 @@ def write_model(write_dir, weights, quantization_dtype):
     return quantization.write_weights(write_dir, [group], quantization_dtype)
 
 
+def _b64(text):
+    import base64
+    return base64.b64encode(text.encode()).decode()
+
+
+def _shape_attr(shape):
+    return {"dim": [{"size": str(d)} for d in shape]}
+
+
+def mobilenet_v2_topology():
+    """The synthetic MobileNetV2 as the `modelTopology` of a converter-format
+    graph model: a GraphDef in JSON whose nodes are the fused ops the converter's
+    grappler pass leaves for this network (the node and attribute names that
+    tfjs-converter/src/operations/op_list/convolution.ts, matrices.ts,
+    arithmetic.ts, reduction.ts and graph.ts read). Strings are base64, int64
+    values are decimal strings, as protobuf's JSON mapping writes them."""
+    ops, shapes = mobilenet_v2_graph()
+    nodes = [{"name": "input", "op": "Placeholder",
+              "attr": {"dtype": {"type": "DT_FLOAT"}, "shape": {"shape": _shape_attr([-1, 224, 224, 3])}}}]
+
+    def const(name, shape, dtype="DT_FLOAT"):
+        nodes.append({"name": name, "op": "Const",
+                      "attr": {"dtype": {"type": dtype},
+                               "value": {"tensor": {"dtype": dtype, "tensorShape": _shape_attr(shape)}}}})
+
+    def fused_attrs(act):
+        fused = ["BiasAdd"] + ({"relu6": ["Relu6"], "relu": ["Relu"]}.get(act, []))
+        return {"T": {"type": "DT_FLOAT"}, "num_args": {"i": "1"}, "epsilon": {"f": 0.0},
+                "leakyrelu_alpha": {"f": 0.2}, "fused_ops": {"list": {"s": [_b64(f) for f in fused]}}}
+
+    for op in ops:
+        k = op["kind"]
+        if k in ("conv", "dw"):
+            const(op["w"], shapes[op["w"]])
+            const(op["b"], shapes[op["b"]])
+            attr = fused_attrs(op["act"])
+            attr.update({"strides": {"list": {"i": ["1", str(op["stride"]), str(op["stride"]), "1"]}},
+                         "dilations": {"list": {"i": ["1", "1", "1", "1"]}}, "padding": {"s": _b64("SAME")},
+                         "data_format": {"s": _b64("NHWC")}, "explicit_paddings": {"list": {}}})
+            if k == "conv":
+                attr["use_cudnn_on_gpu"] = {"b": True}
+            nodes.append({"name": op["out"], "op": "_FusedConv2D" if k == "conv" else "FusedDepthwiseConv2dNative",
+                          "input": [op["src"], op["w"], op["b"]], "attr": attr})
+        elif k == "add":
+            nodes.append({"name": op["out"], "op": "AddV2", "input": list(op["src"]), "attr": {"T": {"type": "DT_FLOAT"}}})
+        elif k == "mean":
+            const(op["out"] + "/reduction_indices", [2], "DT_INT32")
+            nodes.append({"name": op["out"], "op": "Mean", "input": [op["src"], op["out"] + "/reduction_indices"],
+                          "attr": {"T": {"type": "DT_FLOAT"}, "Tidx": {"type": "DT_INT32"}, "keep_dims": {"b": False}}})
+        else:
+            const(op["w"], shapes[op["w"]])
+            const(op["b"], shapes[op["b"]])
+            attr = fused_attrs("linear")
+            attr.update({"transpose_a": {"b": False}, "transpose_b": {"b": False}})
+            nodes.append({"name": op["out"], "op": "_FusedMatMul", "input": [op["src"], op["w"], op["b"]], "attr": attr})
+    nodes.append({"name": "Identity", "op": "Identity", "input": ["logits"], "attr": {"T": {"type": "DT_FLOAT"}}})
+    return {"node": nodes, "library": {}, "versions": {"producer": 987}}
+
+
+def write_graph_model(write_dir, weights, quantization_dtype):
+    """Writes model.json (format 'graph-model': topology, signature and weights
+    manifest, the layout of tfjs-converter's output that
+    tfjs-converter/src/executor/graph_model.ts:159-181 loads) next to the
+    weight shards."""
+    full = dict(weights)
+    full["pool/reduction_indices"] = np.array([1, 2], dtype=np.int32)
+    manifest = write_model(write_dir, full, quantization_dtype)
+    model = {
+        "format": "graph-model", "generatedBy": "synthetic", "convertedBy": "tfjs_amd.workloads",
+        "signature": {
+            "inputs": {"input": {"name": "input:0", "dtype": "DT_FLOAT", "tensorShape": _shape_attr([-1, 224, 224, 3])}},
+            "outputs": {"Identity": {"name": "Identity:0", "dtype": "DT_FLOAT", "tensorShape": _shape_attr([-1, 1000])}}},
+        "modelTopology": mobilenet_v2_topology(),
+        "weightsManifest": manifest,
+    }
+    with open(os.path.join(write_dir, "model.json"), "w") as f:
+        json.dump(model, f)
+    return model
+
+
 def read_model(model_dir):
     """Returns (flat weight bytes, manifest entries) of the first group."""
     with open(os.path.join(model_dir, "weights_manifest.json")) as f:
