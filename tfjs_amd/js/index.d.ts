@@ -4,7 +4,7 @@
  * (tfjs-core/src/kernel_registry.ts:55-61), decodeWeights
  * (tfjs-core/src/io/io_utils.ts:119-135).
  */
-import {DataId, DataType, KernelBackend, KernelConfig, NamedTensorMap, TensorInfo, io} from '@tensorflow/tfjs-core';
+import {DataId, DataType, KernelBackend, KernelConfig, NamedTensorMap, Tensor, TensorInfo, io} from '@tensorflow/tfjs-core';
 
 export interface HipMemoryInfo {
   unreliable: boolean;
