@@ -125,6 +125,12 @@ bool range_is_live(const void *p, size_t bytes) {
   return a >= it->first && a + bytes <= it->first + it->second && a + bytes >= a;
 }
 
+// Copies a small result straight into pinned host memory: a kernel starts within
+// a few microseconds, the copy engine needs 10-15 for a transfer of any size.
+__global__ __launch_bounds__(256) void copy_to_host(const float4 *__restrict__ src, float4 *__restrict__ dst, int n4) {
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < n4; i += gridDim.x * 256) dst[i] = src[i];
+}
+
 }  // namespace tfhip
 
 using namespace tfhip;
@@ -327,7 +333,16 @@ int tfhip_download(void *host, const void *src, size_t src_offset, size_t bytes)
     g.next_staging = (b + 1) % kStagingBuffers;
     if (g.staging_busy[b]) TFHIP_CHECK_HIP(hipEventSynchronize(g.staging_done[b]));
     g.staging_busy[b] = false;
-    TFHIP_CHECK_HIP(hipMemcpyAsync(g.staging[b], s + done, chunk, hipMemcpyDeviceToHost, g.stream));
+    constexpr size_t kKernelCopyBytes = size_t(1) << 20;
+    if (chunk <= kKernelCopyBytes && chunk % 16 == 0 && reinterpret_cast<uintptr_t>(s + done) % 16 == 0) {
+      const int n4 = (int)(chunk / 16);
+      const int blocks = (n4 + 255) / 256 < 64 ? (n4 + 255) / 256 : 64;
+      copy_to_host<<<blocks, 256, 0, g.stream>>>(reinterpret_cast<const float4 *>(s + done),
+                                                 static_cast<float4 *>(g.staging[b]), n4);
+      TFHIP_CHECK_HIP(hipGetLastError());
+    } else {
+      TFHIP_CHECK_HIP(hipMemcpyAsync(g.staging[b], s + done, chunk, hipMemcpyDeviceToHost, g.stream));
+    }
     TFHIP_CHECK_HIP(hipStreamSynchronize(g.stream));
     memcpy(h + done, g.staging[b], chunk);
     done += chunk;
