@@ -203,6 +203,7 @@ __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
   const int blocks = (g.M + 15) / 16;
   const int waves = gridDim.x * 4;
   const int first = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int n0 = blockIdx.y * (16 * TN);   // this workgroup's slice of the columns
 
   struct ABlock {
     float4 full[KF > 0 ? KF : 1];
@@ -234,7 +235,7 @@ __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
     const int k = s < 4 * KF ? 16 * (s / 4) + 4 * grp + s % 4 : 16 * KF + 2 * grp + (s - 4 * KF);
 #pragma unroll
     for (int n = 0; n < TN; ++n) {
-      const int col = n * 16 + r;
+      const int col = n0 + n * 16 + r;
       breg[s][n] = (k < g.K && col < g.N) ? g.b[(long long)k * g.N + col] : 0.f;
     }
   }
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
   for (int n = 0; n < TN; ++n)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int col = n * 16 + grp * 4 + q;
+      const int col = n0 + n * 16 + grp * 4 + q;
       bias4[n][q] = (g.bias && col < g.N) ? g.bias[(long long)col * g.bias_stride] : 0.f;
     }
 
@@ -264,11 +265,11 @@ __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
 #pragma unroll
       for (int n = 0; n < TN; ++n) acc[n] = __builtin_amdgcn_mfma_f32_16x16x4f32(breg[s][n], av, acc[n], 0, 0, 0);
     }
-    // lane holds row b*16 + r, columns n*16 + 4*grp .. +3
+    // lane holds row b*16 + r, columns n0 + n*16 + 4*grp .. +3
     const int row = b * 16 + r;
 #pragma unroll
     for (int n = 0; n < TN; ++n) {
-      const int col = n * 16 + grp * 4;
+      const int col = n0 + n * 16 + grp * 4;
       float out[4];
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
@@ -289,7 +290,7 @@ __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
 }
 
 template <int TN, int KF, bool HALF>
-inline int launch_skinny_regs(const SkinnyArgs &g) {
+inline int launch_skinny_regs(const SkinnyArgs &g, int column_groups) {
   static int resident = 0;   // workgroups per compute unit at this instantiation's register count
   if (resident == 0) {
     int n = 0;
@@ -302,26 +303,29 @@ inline int launch_skinny_regs(const SkinnyArgs &g) {
   // all workgroups resident at once; wavefront w takes row blocks w, w + waves, ...
   const long long blocks = (g.M + 15) / 16;
   long long grid = (blocks + 3) / 4;
-  const long long cap = (long long)num_cus() * resident;
+  long long cap = (long long)num_cus() * resident / column_groups;
+  if (cap < 1) cap = 1;
   if (grid > cap) grid = cap;
   note_kernel("skinny_gemm_regs<%d, %d, %s>", TN, KF, HALF ? "true" : "false");
-  TFHIP_LAUNCH((skinny_gemm_regs<TN, KF, HALF><<<dim3((unsigned)grid), dim3(256), 0, stream()>>>(g)));
+  TFHIP_LAUNCH((skinny_gemm_regs<TN, KF, HALF>
+                <<<dim3((unsigned)grid, (unsigned)column_groups), dim3(256), 0, stream()>>>(g)));
   return kOk;
 }
 
-// Dispatch over the instantiated (columns, k) combinations; -1 when there is none.
+// Dispatch over the instantiated k combinations for TN groups of 16 columns per
+// wavefront; -1 when there is none.
 template <int TN>
-inline int launch_skinny_regs_tn(const SkinnyArgs &g) {
+inline int launch_skinny_regs_tn(const SkinnyArgs &g, int column_groups) {
   const int kf = g.K / 16, rest = g.K % 16;
   if (rest == 0) {
-    if (kf == 1) return launch_skinny_regs<TN, 1, false>(g);
-    if (kf == 2) return launch_skinny_regs<TN, 2, false>(g);
+    if (kf == 1) return launch_skinny_regs<TN, 1, false>(g, column_groups);
+    if (kf == 2) return launch_skinny_regs<TN, 2, false>(g, column_groups);
   } else if (rest <= 8) {
-    if (kf == 0) return launch_skinny_regs<TN, 0, true>(g);
-    if (kf == 1) return launch_skinny_regs<TN, 1, true>(g);
+    if (kf == 0) return launch_skinny_regs<TN, 0, true>(g, column_groups);
+    if (kf == 1) return launch_skinny_regs<TN, 1, true>(g, column_groups);
   } else {
-    if (kf == 0) return launch_skinny_regs<TN, 1, false>(g);
-    if (kf == 1) return launch_skinny_regs<TN, 2, false>(g);
+    if (kf == 0) return launch_skinny_regs<TN, 1, false>(g, column_groups);
+    if (kf == 1) return launch_skinny_regs<TN, 2, false>(g, column_groups);
   }
   return -1;
 }
@@ -373,14 +377,21 @@ inline int launch_skinny(const GemmParams &p) {
   g.a_bytes = p.a_bytes;
   g.activation = p.epi.activation;
   if (tuning(kTuneSkinnyRegs) != 0) {   // B in registers where an instantiation fits
+    // columns per wavefront: all of them up to 96; wider outputs in slices (a
+    // wavefront that keeps 144 columns of accumulators, B and bias is so heavy on
+    // registers that too few of them are resident to cover each other's stores)
+    const int total = skinny_groups(p.N);
+    int per_wave = total <= 6 ? total : 3;
+    if (tuning(kTuneSkinnyRegs) >= 2) per_wave = tuning(kTuneSkinnyRegs) - 1;   // tuning: value - 1 groups per wavefront
+    const int column_groups = (((int)p.N + 15) / 16 + per_wave - 1) / per_wave;
     int rc = -1;
-    switch (skinny_groups(p.N)) {
-      case 1: rc = launch_skinny_regs_tn<1>(g); break;
-      case 2: rc = launch_skinny_regs_tn<2>(g); break;
-      case 3: rc = launch_skinny_regs_tn<3>(g); break;
-      case 4: rc = launch_skinny_regs_tn<4>(g); break;
-      case 6: rc = launch_skinny_regs_tn<6>(g); break;
-      case 9: rc = launch_skinny_regs_tn<9>(g); break;
+    switch (per_wave) {
+      case 1: rc = launch_skinny_regs_tn<1>(g, column_groups); break;
+      case 2: rc = launch_skinny_regs_tn<2>(g, column_groups); break;
+      case 3: rc = launch_skinny_regs_tn<3>(g, column_groups); break;
+      case 4: rc = launch_skinny_regs_tn<4>(g, column_groups); break;
+      case 6: rc = launch_skinny_regs_tn<6>(g, column_groups); break;
+      case 9: rc = launch_skinny_regs_tn<9>(g, column_groups); break;
       default: break;
     }
     if (rc >= 0) return rc;
