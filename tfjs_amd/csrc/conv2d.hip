@@ -105,6 +105,7 @@ struct TapTable {
 //    activation and one 16-byte store per block.
 template <int KSTEPS, int NB>
 __global__ __launch_bounds__(256) void conv_few_taps(FewChannelsArgs g, TapTable taps, int chunks, unsigned x_bytes) {
+  // blockDim.x is 256 or 64: four wavefronts or one, 64 consecutive pixels each
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, kg = lane >> 4;
   const int oc0 = blockIdx.y * (16 * NB);
@@ -132,7 +133,7 @@ __global__ __launch_bounds__(256) void conv_few_taps(FewChannelsArgs g, TapTable
     }
   }
   for (int chunk = blockIdx.x; chunk < chunks; chunk += gridDim.x) {
-    const int m_wave = chunk * 256 + wave * 64;
+    const int m_wave = chunk * (int)blockDim.x + wave * 64;
     // pixel of block 0; the following blocks are 16 pixels further along the row
     int m = m_wave + r;
     int ow = m % g.out_w;
@@ -221,13 +222,15 @@ int launch_few_taps(const GemmParams &p, int f_h) {
     taps.dw[k] = fs * c.dil_w;
     taps.off_bytes[k] = (unsigned)(((long long)fr * c.dil_h * c.xs_h + (long long)fs * c.dil_w * c.xs_w + ch) * 4);
   }
-  // 256 pixels per workgroup and trip; every workgroup makes the same number of trips
-  const int chunks = (p.M + 255) / 256;
-  const int at_once = num_cus() * 8;
+  // 256 pixels (four wavefronts) per workgroup and trip, 64 when that would leave
+  // compute units without a workgroup; every workgroup makes the same number of trips
+  const int threads = (p.M + 255) / 256 * (p.N / (16 * NB)) >= num_cus() ? 256 : 64;
+  const int chunks = (p.M + threads - 1) / threads;
+  const int at_once = num_cus() * 8 * (256 / threads);
   const int trips = (chunks + at_once - 1) / at_once;
   dim3 grid((unsigned)((chunks + trips - 1) / trips), (unsigned)(p.N / (16 * NB)), 1);
   note_kernel("conv_few_taps<%d, %d>", KSTEPS, NB);
-  TFHIP_LAUNCH((conv_few_taps<KSTEPS, NB><<<grid, 256, 0, stream()>>>(g, taps, chunks, p.a_bytes)));
+  TFHIP_LAUNCH((conv_few_taps<KSTEPS, NB><<<grid, threads, 0, stream()>>>(g, taps, chunks, p.a_bytes)));
   return kOk;
 }
 
@@ -325,7 +328,9 @@ extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
   if (!nchw && in_c <= 4 && out_c % 8 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
       p.epi.channel_operands && activation <= TFHIP_RELU6) {
     const bool few_taps = K <= kMaxTaps && M < lim - 256 && p.a_bytes != 0;
-    if (few_taps && out_c % 32 == 0) return launch_few_taps_k<2>(p, (int)f_h);
+    // 32 channels per wavefront when there are pixels enough to fill the chip that
+    // way, else 16 (twice the wavefronts)
+    if (few_taps && out_c % 32 == 0 && M >= 64LL * 4 * num_cus()) return launch_few_taps_k<2>(p, (int)f_h);
     if (few_taps && out_c % 16 == 0) return launch_few_taps_k<1>(p, (int)f_h);
     if (out_c % 32 == 0) return launch_few_channels<32>(p, (int)f_h);
     if (out_c % 16 == 0) return launch_few_channels<16>(p, (int)f_h);
