@@ -49,19 +49,22 @@ BATCH = 32
 # cannot be read from inside this script, so the table is refreshed by hand when a
 # kernel changes; a symbol that is not listed reports null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "conv_few_channels<32>": 77654762,
-    "depthwise_3x3_rows<1, false>": 38815206,
-    "skinny_gemm<1, 4>": 77187525,
-    "skinny_gemm<6, 4>": 180155442,
-    "depthwise_3x3_rows<2, false>": 89027063,
-    "skinny_gemm<2, 4>": 58544389,
-    "skinny_gemm<9, 4>": 70722342,
-    "add_same_shape": 8326053,
-    "gemm_kernel<32, 32, 32, 2, 2, 0, 1>": 16134599,
-    "gemm_kernel<64, 64, 16, 2, 2, 0, 1>": 18573538,
-    "gemm_kernel<32, 64, 32, 2, 2, 0, 1>": 12332239,
-    "mean_hw": 8230158,
-    "gemm_finish": 900590,
+    "conv_few_taps<7, 2>": 75275220,
+    "depthwise_3x3_rows<1, false>": 63563214,
+    "skinny_gemm_regs<1, 2, false>": 77134479,
+    "skinny_gemm_regs<6, 1, false>": 180984829,
+    "depthwise_3x3_rows<2, false>": 156009789,
+    "skinny_gemm<2, 4>": 58521445,
+    "skinny_gemm_regs<3, 1, true>": 74859784,
+    "add_same_shape": 8330153,
+    "gemm_kernel<32, 32, 32, 2, 2, 0, 1>": 16139742,
+    "gemm_kernel<64, 64, 16, 2, 2, 0, 1>": 18563146,
+    "depthwise_3x3_flat<2, false>": 22006204,
+    "depthwise_3x3_flat<1, false>": 17923346,
+    "gemm_kernel<32, 64, 32, 2, 2, 0, 1>": 12331211,
+    "mean_hw_vec": 8295707,
+    "gemm_finish": 890299,
+    "copy_to_host": 277490,
 }
 
 
