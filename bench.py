@@ -385,7 +385,7 @@ def main():
         return
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build runs on one GPU; --gpus %d is not supported "
-                         "(the path shards by batch with no exchange step, see DESIGN.md)\n" % args.gpus)
+                         "(the path shards by batch with no exchange step)\n" % args.gpus)
         sys.exit(2)
     if args.kernels_only:
         print(json.dumps(dict(kernels=bench_kernels())))
