@@ -10,9 +10,9 @@ GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 TEST_EPSILON_FLOAT32 = 1e-3
 
 
-def load_cases(name):
+def load_cases(name, group="cases"):
     with open(os.path.join(GOLDEN, name)) as f:
-        return json.load(f)["cases"]
+        return json.load(f)[group]
 
 
 def tensor(j):
@@ -20,6 +20,11 @@ def tensor(j):
         return None
     if isinstance(j, list):  # tensor-like nested array in the reference's test
         return np.asarray(j, dtype=np.float32)
+    if "fill" in j:  # a constant tensor with a few elements set (hand_transcribed.json)
+        t = np.full(int(np.prod(j["shape"])), j["fill"], dtype=np.float32)
+        for i, v in j.get("set", {}).items():
+            t[int(i)] = v
+        return t.reshape(j["shape"])
     return np.asarray(j["values"], dtype=np.float32).reshape(j["shape"])
 
 

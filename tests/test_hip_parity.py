@@ -11,11 +11,12 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-from golden_util import assert_close, conv_args, ids, load_cases, tensor  # noqa: E402
+from golden_util import TEST_EPSILON_FLOAT32, assert_close, conv_args, ids, load_cases, tensor  # noqa: E402
 import synth  # noqa: E402
 
 FMM = load_cases("fused_mat_mul.json")
-MM = load_cases("mat_mul.json")
+MM = load_cases("mat_mul.json") + load_cases("hand_transcribed.json", "mat_mul")
+DILATED = load_cases("hand_transcribed.json", "dilation_equivalences")
 FCONV = load_cases("fused_conv2d.json")
 CONV = load_cases("conv2d.json")
 FDW = load_cases("fused_depthwise_conv2d.json")
@@ -98,6 +99,20 @@ def test_depthwise_golden(hip, orc, c):
     got = _run_conv(hip, c, True)
     assert_close(got, c["expected"])
     assert_parity(got, _run_conv(orc, c, True))
+
+
+@pytest.mark.parametrize("c", DILATED, ids=ids(DILATED))
+def test_dilation_equals_zero_stuffed_filter(hip, orc, c):
+    # the reference's own check: a dilated filter == the filter with zeros between its taps
+    x, w, wz = tensor(c["x"]), tensor(c["filter"]), tensor(c["filterDilated"])
+    op = hip.fused_depthwise_conv2d if c["op"] == "depthwiseConv2d" else hip.fused_conv2d
+    got = op(x, w, strides=c["strides"], pad=c["pad"], dilations=c["dilations"])
+    want = op(x, wz, strides=c["strides"], pad=c["pad"], dilations=1)
+    assert got.shape == want.shape
+    assert np.abs(got - want).max() <= TEST_EPSILON_FLOAT32
+    ref = (orc.fused_depthwise_conv2d if c["op"] == "depthwiseConv2d" else orc.fused_conv2d)(
+        x, w, strides=c["strides"], pad=c["pad"], dilations=c["dilations"])
+    assert_parity(got, ref)
 
 
 # ------------------------------------------------------- benchmark configurations

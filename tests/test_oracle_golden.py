@@ -11,7 +11,8 @@ import json
 import os
 
 FMM = load_cases("fused_mat_mul.json")
-MM = load_cases("mat_mul.json")
+MM = load_cases("mat_mul.json") + load_cases("hand_transcribed.json", "mat_mul")
+DILATED = load_cases("hand_transcribed.json", "dilation_equivalences")
 FCONV = load_cases("fused_conv2d.json")
 CONV = load_cases("conv2d.json")
 FDW = load_cases("fused_depthwise_conv2d.json")
@@ -63,6 +64,17 @@ def test_conv2d_golden(c):
 @pytest.mark.parametrize("c", FDW + DW, ids=ids(FDW + DW))
 def test_depthwise_golden(c):
     assert_close(_run_conv(c, True), c["expected"])
+
+
+@pytest.mark.parametrize("c", DILATED, ids=ids(DILATED))
+def test_dilation_equals_zero_stuffed_filter(c):
+    # the reference's own check: a dilated filter == the filter with zeros between its taps
+    x, w, wz = tensor(c["x"]), tensor(c["filter"]), tensor(c["filterDilated"])
+    op = orc.fused_depthwise_conv2d if c["op"] == "depthwiseConv2d" else orc.fused_conv2d
+    got = op(x, w, strides=c["strides"], pad=c["pad"], dilations=c["dilations"])
+    want = op(x, wz, strides=c["strides"], pad=c["pad"], dilations=1)
+    assert got.shape == want.shape
+    np.testing.assert_array_equal(got, want)   # the skipped taps contribute exact zeros
 
 
 @pytest.mark.parametrize("c", CINFO, ids=ids(CINFO))
