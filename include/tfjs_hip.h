@@ -96,9 +96,10 @@ int tfhip_event_elapsed(int start_slot, int end_slot, float *ms);
  *   "dw_rows" (depthwise rows per lane), "dw_halo" (1: LDS halo depthwise kernel),
  *   "no_skinny" (1: tiled GEMM also for tall products), "dw_flat" (1: the
  *   one-row-per-lane depthwise kernel always, 0: never), "skinny_regs" (0: the
- *   streaming GEMM always stages B in LDS). TFHIP_TILE, TFHIP_SPLITK, TFHIP_DW_ROWS,
- *   TFHIP_DW_HALO, TFHIP_NO_SKINNY, TFHIP_DW_FLAT, TFHIP_SKINNY_REGS in the
- *   environment set them at tfhip_init(). */
+ *   streaming GEMM always stages B in LDS), "small_k" (0: never the one-shot GEMM
+ *   for K <= 64, 32 / 64: that many rows per tile). TFHIP_TILE,
+ *   TFHIP_SPLITK, TFHIP_DW_ROWS, TFHIP_DW_HALO, TFHIP_NO_SKINNY, TFHIP_DW_FLAT,
+ *   TFHIP_SKINNY_REGS, TFHIP_SMALL_K in the environment set them at tfhip_init(). */
 int tfhip_set_launch_repeat(int n);
 int tfhip_last_kernel(char *name, size_t name_len);
 int tfhip_set_tuning(const char *name, int value);

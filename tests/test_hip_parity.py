@@ -327,6 +327,19 @@ def test_matmul_tall_tiny_k(hip, orc, tuning, m, n, k, act, regs):
     assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
 
 
+@pytest.mark.parametrize("rows", [32, 64])
+@pytest.mark.parametrize("batch,m,n,k,act", [(1, 600, 192, 32, "relu6"), (1, 531, 68, 64, "linear"), (3, 257, 128, 20, "relu"),
+                                              (1, 2000, 64, 4, "leakyrelu"), (2, 300, 100, 44, "relu6")])
+def test_matmul_very_short_k(hip, orc, tuning, batch, m, n, k, act, rows):
+    # K <= 64: the one-shot kernel (whole tile fetched at once), both tile heights, ragged edges, K off the 16 grid
+    tuning("small_k", rows)
+    rng = np.random.default_rng(m + n + k)
+    a = rng.uniform(-1, 1, (batch, m, k)).astype(np.float32)
+    b = rng.normal(0, 0.3, (batch if batch == 3 else 1, k, n)).astype(np.float32)
+    kw = dict(bias=rng.uniform(-1, 1, (n,)).astype(np.float32), activation=act, leakyrelu_alpha=0.1)
+    assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
+
+
 def test_pointwise_conv_tall(hip, orc):
     rng = np.random.default_rng(53)
     x = rng.uniform(0, 1, (14, 87, 86, 24)).astype(np.float32)

@@ -2,11 +2,13 @@
 // loaders the memory layout allows and a tile shape, and launches gemm_kernel.
 #include "gemm_host.h"
 #include "skinny_gemm.h"
+#include "small_k_gemm.h"
 
 using namespace tfhip;
 
 int tfhip::launch_plain_gemm(GemmParams &p, bool transpose_a, bool transpose_b, bool vec) {
   if (skinny_applies(p, transpose_a, transpose_b, vec) && tuning(kTuneNoSkinny) <= 0) return launch_skinny(p);
+  if (small_k_applies(p, transpose_a, transpose_b, vec) && tuning(kTuneSmallK) != 0) return launch_small_k(p);
   if (vec) {
     const int shape = choose_tile_shape(p.M, p.N, p.K, p.batch, num_cus());
     if (!transpose_a && !transpose_b) return launch_gemm_shape<kLoadKVec, kLoadXVec>(shape, p);
