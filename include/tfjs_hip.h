@@ -80,6 +80,30 @@ int tfhip_unregister_external(void *dptr);
 int tfhip_event_record(int slot);
 int tfhip_event_elapsed(int start_slot, int end_slot, float *ms);
 
+/* ---- recorded launch sequences (no counterpart in the reference) --------------
+ * A model whose shapes do not change enqueues the same kernels with the same
+ * arguments at every inference. Between tfhip_capture_begin() and
+ * tfhip_capture_end() the kernel entry points record their launches into a
+ * HIP graph instead of running them; tfhip_graph_launch(id) then replays the
+ * whole sequence with one call: no per-kernel host work, and shorter gaps
+ * between dependent kernels than separate launches leave.
+ *  - While recording, tfhip_alloc / tfhip_free work as usual (a block freed
+ *    while recording is kept by the graph until tfhip_graph_destroy), and the
+ *    entry points that wait for the stream or copy through the host
+ *    (tfhip_upload, tfhip_download, tfhip_sync, the event calls) fail.
+ *  - A replay reads and writes the ADDRESSES that were recorded: the caller
+ *    puts new input where the recorded input was (tfhip_copy) and takes the
+ *    result from where the recorded result was. Blocks that were live at
+ *    tfhip_capture_end and that a recorded kernel names must still be live at
+ *    every tfhip_graph_launch, which checks this and fails without launching
+ *    otherwise.
+ *  - tfhip_capture_end(NULL, &nodes) discards the recording.
+ * nodes: kernels in the graph. */
+int tfhip_capture_begin(void);
+int tfhip_capture_end(int *graph_id, int *nodes);
+int tfhip_graph_launch(int graph_id);
+int tfhip_graph_destroy(int graph_id);
+
 /* ---- measurement aids (no counterpart in the reference) ----------------------
  * tfhip_set_launch_repeat(n): every kernel entry point enqueues its kernel n
  *   times back to back (the kernels are idempotent), so that a pair of events
@@ -144,6 +168,27 @@ int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
                        const float *bias, const int64_t bias_strides[4],
                        int activation, const float *prelu_weights,
                        const int64_t prelu_strides[4], double leakyrelu_alpha);
+
+/* FusedConv2D followed by the Add of a residual connection, as one launch:
+ * y = activation(conv(x, filter) + bias) + residual, every step rounded to
+ * float32 like the separate kernels (so the result equals tfhip_fused_conv2d
+ * followed by tfhip_add bit for bit). The pair it replaces in a graph is a
+ * FusedConv2D node (tfjs-converter/src/operations/executors/
+ * convolution_executor.ts:100-137) whose only consumer is an Add / AddV2 node
+ * (arithmetic_executor.ts:30-37) with an operand of the output's shape, the
+ * form the projection convolution and the skip connection of an inverted
+ * residual block take. residual has the shape and the data format of y and
+ * must not be y itself. */
+int tfhip_fused_conv2d_add(const float *x, const float *filter, float *y,
+                           int64_t batch, int64_t in_h, int64_t in_w, int64_t in_c,
+                           int64_t f_h, int64_t f_w, int64_t out_c,
+                           int64_t stride_h, int64_t stride_w, int64_t dilation_h,
+                           int64_t dilation_w, int64_t pad_top, int64_t pad_left,
+                           int64_t out_h, int64_t out_w, int nchw,
+                           const float *bias, const int64_t bias_strides[4],
+                           int activation, const float *prelu_weights,
+                           const int64_t prelu_strides[4], double leakyrelu_alpha,
+                           const float *residual);
 
 /* ---- FusedDepthwiseConv2D ----------------------------------------------------
  * Replaces FusedDepthwiseConv2D(...)

@@ -397,6 +397,85 @@ h.test('graph model: a converter-format topology runs through the fused ops and 
   h.assertEqual(tf.memory().numTensors, before);
 });
 
+function residualGraphArtifacts() {
+  // x -> expand (1x1, relu6) -> project (1x1) -> AddV2(x, project) -> Identity: the skip connection of a residual block
+  const fused = (ops, n) => ({fused_ops: {list: {s: ops.map(b64)}}, num_args: {i: String(n)}, leakyrelu_alpha: {f: 0.2},
+                              strides: {list: {i: ['1', '1', '1', '1']}}, dilations: {list: {i: ['1', '1', '1', '1']}},
+                              padding: {s: b64('SAME')}, data_format: {s: b64('NHWC')}, explicit_paddings: {list: {}}});
+  const node = (name, op, input, attr) => ({name, op, input, attr: attr || {}});
+  const nodes = [
+    node('x', 'Placeholder', [], {dtype: {type: 'DT_FLOAT'}, shape: {shape: {dim: [{size: '-1'}, {size: '4'}, {size: '4'}, {size: '4'}]}}}),
+    node('e/w', 'Const'), node('e/b', 'Const'), node('p/w', 'Const'), node('p/b', 'Const'),
+    node('e', '_FusedConv2D', ['x', 'e/w', 'e/b'], fused(['BiasAdd', 'Relu6'], 1)),
+    node('p', '_FusedConv2D', ['e', 'p/w', 'p/b'], fused(['BiasAdd'], 1)),
+    node('sum', 'AddV2', ['x', 'p']),
+    node('twice', 'AddV2', ['sum', 'sum']),
+    node('out', 'Identity', ['twice'])
+  ];
+  let seed = 3;
+  const rnd = n => Float32Array.from({length: n}, () => ((seed = (Math.imul(seed, 1664525) + 1013904223) >>> 0) / 2 ** 32) - 0.5);
+  const values = {'e/w': [rnd(4 * 8), [1, 1, 4, 8]], 'e/b': [rnd(8), [8]], 'p/w': [rnd(8 * 4), [1, 1, 8, 4]], 'p/b': [rnd(4), [4]]};
+  const specs = [], chunks = [];
+  Object.keys(values).forEach(name => {
+    specs.push({name, shape: values[name][1], dtype: 'float32'});
+    chunks.push(Buffer.from(values[name][0].buffer));
+  });
+  const all = Buffer.concat(chunks);
+  return {modelTopology: {node: nodes, versions: {producer: 1, minConsumer: 0}}, weightSpecs: specs,
+          weightData: all.buffer.slice(all.byteOffset, all.byteOffset + all.byteLength)};
+}
+
+h.test('graph model: a convolution read by one Add only runs with it as one FusedConv2DAdd where the backend has that kernel', () => {
+  const fake = require('./fake_addon');
+  // no such kernel on the cpu backend: the plan keeps the graph's own nodes
+  useBackend('cpu');
+  const io = {decodeWeights: oracleDecode.decodeWeights};
+  let model = hip.loadGraphModel({load: () => residualGraphArtifacts()}, {}, io);
+  const xc = tf.tensor(Float32Array.from({length: 64}, (_, i) => Math.cos(i)), [1, 4, 4, 4]);
+  model.predict(xc).dispose();
+  let ops = Array.from(model.plans.values())[0].steps.filter(s => s.kind === 'op');
+  h.assertEqual(ops.map(s => s.name), ['e', 'p', 'sum', 'twice', 'out']);
+  h.assert(ops.every(s => s.conv == null));
+  xc.dispose();
+  model.dispose();
+
+  useBackend('hip');
+  model = hip.loadGraphModel({load: () => residualGraphArtifacts()}, {}, {decodeWeights: hip.decodeWeights});
+  const x = tf.tensor(new Float32Array(64), [1, 4, 4, 4]);
+  const live = tf.memory().numTensors;
+  let conv = fake.calls.filter(c => c === 'fusedConv2D').length, adds = fake.calls.filter(c => c === 'add').length;
+  const y = model.predict(x);
+  ops = Array.from(model.plans.values())[0].steps.filter(s => s.kind === 'op');
+  h.assertEqual(ops.map(s => [s.name, s.conv]), [['e', undefined], ['sum', 'p'], ['twice', undefined], ['out', undefined]]);
+  h.assertEqual(ops[1].sources, ['e', 'p/w', 'p/b', 'x']);
+  h.assertEqual(fake.calls.filter(c => c === 'fusedConv2D').length, conv + 2);
+  h.assertEqual(fake.calls.filter(c => c === 'add').length, adds + 1, 'only the Add that reads no convolution is left');
+  // the projection was handed the input's buffer as its residual: the last argument
+  h.assertEqual(fake.lastArgs.fusedConv2D[11], tf.backend().ptr(x.dataId));
+  h.assertEqual(fake.lastArgs.fusedConv2D[3], [1, 4, 4, 8, 1, 1, 4, 1, 1, 1, 1, 0, 0, 4, 4]);
+  h.assertEqual(y.shape, [1, 4, 4, 4]);
+  h.assertEqual(tf.memory().numTensors, live + 1);
+  y.dispose();
+  // switched off in the load options; and a residual that the Add would broadcast takes the two kernels
+  const plain = hip.loadGraphModel({load: () => residualGraphArtifacts()}, {fuseResidualAdd: false}, {decodeWeights: hip.decodeWeights});
+  conv = fake.calls.length;
+  plain.predict(x).dispose();
+  h.assertEqual(fake.calls.slice(conv).filter(c => c !== 'alloc' && c !== 'free'), ['fusedConv2D', 'fusedConv2D', 'add', 'add']);
+  h.assertEqual(fake.lastArgs.fusedConv2D[11], null);
+  const w = tf.tensor(new Float32Array(8 * 4), [1, 1, 8, 4]), e = tf.tensor(new Float32Array(128), [1, 4, 4, 8]);
+  const row = tf.tensor(new Float32Array(4), [4]);
+  conv = fake.calls.length;
+  const z = tf.engine().runKernel('FusedConv2DAdd', {x: e, filter: w, residual: row},
+                                  {strides: [1, 1], pad: 'same', dataFormat: 'NHWC', dilations: [1, 1]});
+  h.assertEqual(fake.calls.slice(conv).filter(c => c === 'fusedConv2D' || c === 'add'), ['fusedConv2D', 'add']);
+  h.assertEqual(z.shape, [1, 4, 4, 4]);
+  h.assertThrows(() => tf.engine().runKernel('FusedConv2DAdd', {x: e, filter: w}, {strides: [1, 1], pad: 'same'}),
+                 /residual input is missing/);
+  tf.dispose([x, w, e, row, z]);
+  plain.dispose();
+  model.dispose();
+});
+
 h.test('graph model: unsupported nodes and malformed fused nodes throw the reference errors', () => {
   useBackend('cpu');
   const io = {decodeWeights: oracleDecode.decodeWeights};

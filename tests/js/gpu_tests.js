@@ -190,6 +190,45 @@ h.test('config 4 as a converter-format graph model: loadGraphModel + injected de
   h.assertEqual(tf.backend().numDataIds(), before, 'model, weights and results are all released');
 });
 
+h.test('FusedConv2DAdd: one launch with the bits of FusedConv2D followed by Add; the graph model uses it for skip connections', () => {
+  h.assert(tf.engine().setBackend('hip') === true);
+  const before = tf.backend().numDataIds();
+  let seed = 5;
+  const rnd = n => Float32Array.from({length: n}, () => ((seed = (Math.imul(seed, 1664525) + 1013904223) >>> 0) / 2 ** 32) - 0.5);
+  const attrs = {strides: [1, 1], pad: 'same', dataFormat: 'NHWC', dilations: [1, 1], activation: 'relu6'};
+  [[2, 14, 14, 96, 1, 32], [1, 9, 7, 5, 3, 6], [2, 16, 16, 3, 3, 16]].forEach(([n, hh, ww, cin, k, cout]) => {
+    const x = tf.tensor(rnd(n * hh * ww * cin), [n, hh, ww, cin]);
+    const filter = tf.tensor(rnd(k * k * cin * cout), [k, k, cin, cout]);
+    const bias = tf.tensor(rnd(cout), [cout]);
+    const residual = tf.tensor(rnd(n * hh * ww * cout), [n, hh, ww, cout]);
+    const fused = tf.engine().runKernel('FusedConv2DAdd', {x, filter, bias, residual}, attrs);
+    const conv = tf.fused.conv2d(Object.assign({x, filter, bias}, attrs));
+    const sum = tf.add(conv, residual);
+    h.assertEqual(fused.shape, sum.shape);
+    h.assertBitsEqual(fused.dataSync(), sum.dataSync());
+    // a residual that broadcasts is the Add's business: same values through the two kernels
+    const row = tf.tensor(rnd(cout), [cout]);
+    const viaRow = tf.engine().runKernel('FusedConv2DAdd', {x, filter, bias, residual: row}, attrs);
+    const sumRow = tf.add(conv, row);
+    h.assertBitsEqual(viaRow.dataSync(), sumRow.dataSync());
+    tf.dispose([x, filter, bias, residual, fused, conv, sum, row, viaRow, sumRow]);
+  });
+  h.assertEqual(tf.backend().numDataIds(), before);
+  const dir = process.env.TFJS_HIP_TEST_MODEL_DIR;
+  const io = {decodeWeights: hip.decodeWeights};
+  const fusedModel = hip.loadGraphModel(dir, {}, io), plainModel = hip.loadGraphModel(dir, {fuseResidualAdd: false}, io);
+  const x = tf.tensor(mobilenet.syntheticInput(2, 5), [2, 224, 224, 3]);
+  const a = fusedModel.predict(x), b = plainModel.predict(x);
+  const count = model => Array.from(model.plans.values())[0].steps.filter(s => s.kind === 'op');
+  h.assertEqual(count(plainModel).length - count(fusedModel).length, 10, 'MobileNetV2 has ten skip connections');
+  h.assertEqual(count(fusedModel).filter(s => s.conv != null).length, 10);
+  h.assertBitsEqual(a.dataSync(), b.dataSync());
+  tf.dispose([a, b, x]);
+  fusedModel.dispose();
+  plainModel.dispose();
+  h.assertEqual(tf.backend().numDataIds(), before);
+});
+
 h.test('backend: tensors migrate cpu <-> hip with values and refCounts; tf.time reports device ms', async () => {
   h.assert(tf.engine().setBackend('cpu') === true);
   const a = tf.tensor([1, 2, 3, 4], [2, 2]);

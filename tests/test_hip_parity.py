@@ -534,6 +534,135 @@ def test_bad_operands_are_errors_not_faults(hip):
         hip.fused_matmul(np.zeros((2, 3), np.float32), np.zeros((4, 2), np.float32))
 
 
+# ------------------------------------------- convolution + residual in one launch
+
+RESIDUAL_CASES = [
+    # x shape, filter shape, stride, pad, format, activation: the kernel each lands on
+    ((4, 14, 14, 384), (1, 1, 384, 96), 1, "same", "NHWC", "linear"),      # pointwise, tiled GEMM
+    ((8, 112, 112, 96), (1, 1, 96, 24), 1, "same", "NHWC", "linear"),      # pointwise, streaming GEMM (B in LDS)
+    ((2, 9, 9, 2048), (1, 1, 2048, 32), 1, "valid", "NHWC", "relu"),       # pointwise, split-K + finishing pass
+    ((2, 20, 20, 32), (1, 1, 32, 128), 1, "same", "NHWC", "relu6"),        # K <= 64: tiled GEMM takes it over
+    ((2, 17, 15, 16), (3, 3, 16, 24), 1, "same", "NHWC", "linear"),        # 3x3, vector im2col GEMM
+    ((2, 17, 15, 5), (3, 3, 5, 7), 2, "same", "NHWC", "relu"),             # odd channels: scalar im2col GEMM
+    ((2, 6, 11, 9), (3, 3, 6, 10), 1, "valid", "NCHW", "linear"),          # channels first
+    ((2, 33, 33, 3), (3, 3, 3, 32), 2, "same", "NHWC", "relu6"),           # few input channels: direct kernel + add pass
+    ((1, 12, 12, 8), (1, 1, 8, 12), 1, "same", "NHWC", "sigmoid"),         # activation the finishing pass applies
+]
+
+
+@pytest.mark.parametrize("xs,ws,stride,pad,fmt,act", RESIDUAL_CASES, ids=[str(i) for i in range(len(RESIDUAL_CASES))])
+def test_conv2d_with_residual(hip, orc, xs, ws, stride, pad, fmt, act):
+    rng = np.random.default_rng(sum(xs) + sum(ws))
+    x = rng.uniform(-1, 1, xs).astype(np.float32)
+    w = rng.normal(0, 0.2, ws).astype(np.float32)
+    bias = rng.uniform(-1, 1, (ws[3],)).astype(np.float32)
+    kw = dict(strides=stride, pad=pad, data_format=fmt, bias=bias, activation=act)
+    plain = hip.fused_conv2d(x, w, **kw)
+    residual = rng.uniform(-2, 2, plain.shape).astype(np.float32)
+    residual.flat[::7] = -plain.flat[::7]          # exact cancellations: the sum must come out as +0
+    got = hip.fused_conv2d(x, w, residual=residual, **kw)
+    # the same bits as the two separate kernels, and the oracle's conv followed by its add
+    np.testing.assert_array_equal(got.view(np.uint32), hip.add(plain, residual).view(np.uint32))
+    assert_parity(got, orc.add(orc.fused_conv2d(x, w, **kw), residual))
+
+
+def test_conv2d_residual_is_checked(hip):
+    from tfjs_amd import capi
+    lib = capi.load_library()
+    with capi.DeviceBuffer(4 * 4 * 4 * 8 * 4) as x, capi.DeviceBuffer(8 * 8 * 4) as w, \
+            capi.DeviceBuffer(4 * 4 * 4 * 8 * 4) as y, capi.DeviceBuffer(64) as small:
+        geom = [4, 4, 4, 8, 1, 1, 8, 1, 1, 1, 1, 0, 0, 4, 4]
+        tail = [0, None, capi.i64_array([0] * 4), 0, None, capi.i64_array([0] * 4), 0.2]
+        assert lib.tfhip_fused_conv2d_add(x.ptr, w.ptr, y.ptr, *geom, *tail, small.ptr) != 0
+        assert b"'residual'" in lib.tfhip_last_error()
+        assert lib.tfhip_fused_conv2d_add(x.ptr, w.ptr, y.ptr, *geom, *tail, None) != 0
+        assert lib.tfhip_fused_conv2d_add(x.ptr, w.ptr, y.ptr, *geom, *tail, y.ptr) != 0
+        assert b"same buffer" in lib.tfhip_last_error()
+
+
+# -------------------------------------------------- recorded launch sequences
+
+def test_recorded_graph_replays(hip, orc):
+    """A recorded sequence gives the eager result at every replay, with eager work and
+    synchronisations between the replays, and keeps the buffers it freed while recording."""
+    from tfjs_amd import capi
+    lib, check = capi.load_library(), capi.check
+    rng = np.random.default_rng(11)
+    x = rng.uniform(-1, 1, (2, 12, 12, 16)).astype(np.float32)
+    w1 = rng.normal(0, 0.3, (1, 1, 16, 64)).astype(np.float32)
+    w2 = rng.normal(0, 0.3, (3, 3, 64, 1)).astype(np.float32)
+    w3 = rng.normal(0, 0.3, (1, 1, 64, 16)).astype(np.float32)
+    b1, b3 = rng.uniform(-1, 1, 64).astype(np.float32), rng.uniform(-1, 1, 16).astype(np.float32)
+    z4, ch = capi.i64_array([0] * 4), capi.i64_array([0, 0, 0, 1])
+    bufs = {k: capi.DeviceBuffer.from_numpy(v) for k, v in dict(x=x, w1=w1, w2=w2, w3=w3, b1=b1, b3=b3).items()}
+    out = capi.DeviceBuffer(x.nbytes)
+
+    def block(inp, result):
+        """expand -> depthwise -> project + skip connection; intermediates come from and go back to the pool"""
+        t1 = capi.DeviceBuffer(2 * 12 * 12 * 64 * 4)
+        check(lib.tfhip_fused_conv2d(inp.ptr, bufs["w1"].ptr, t1.ptr, 2, 12, 12, 16, 1, 1, 64, 1, 1, 1, 1, 0, 0, 12, 12,
+                                     0, bufs["b1"].ptr, ch, 2, None, z4, 0.2))
+        t2 = capi.DeviceBuffer(2 * 12 * 12 * 64 * 4)
+        check(lib.tfhip_fused_depthwise_conv2d(t1.ptr, bufs["w2"].ptr, t2.ptr, 2, 12, 12, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1,
+                                               12, 12, None, z4, 2, None, z4, 0.2))
+        t1.free()
+        check(lib.tfhip_fused_conv2d_add(t2.ptr, bufs["w3"].ptr, result.ptr, 2, 12, 12, 64, 1, 1, 16, 1, 1, 1, 1, 0, 0,
+                                         12, 12, 0, bufs["b3"].ptr, ch, 0, None, z4, 0.2, inp.ptr))
+        t2.free()
+
+    def expected(xv):
+        t = orc.fused_conv2d(xv, w1, bias=b1, activation="relu6")
+        t = orc.fused_depthwise_conv2d(t, w2, pad="same", activation="relu6")
+        return orc.add(orc.fused_conv2d(t, w3, bias=b3), xv)
+
+    try:
+        block(bufs["x"], out)
+        eager = out.download(np.float32, x.size).reshape(x.shape)
+        assert_parity(eager, expected(x))
+        pooled_before = hip.memory_info()["pooled_bytes"]
+        check(lib.tfhip_capture_begin())
+        try:
+            # what waits for the stream cannot be recorded
+            assert lib.tfhip_sync() != 0 and b"tfhip_capture_begin" in lib.tfhip_last_error()
+            assert lib.tfhip_capture_begin() != 0
+            block(bufs["x"], out)
+        finally:
+            gid, nodes = ctypes.c_int(), ctypes.c_int()
+            check(lib.tfhip_capture_end(ctypes.byref(gid), ctypes.byref(nodes)))
+        assert nodes.value == 3
+        # the two intermediates now belong to the graph, not to the pool
+        assert hip.memory_info()["pooled_bytes"] < pooled_before
+        for trip in range(4):
+            x2 = rng.uniform(-1, 1, x.shape).astype(np.float32)
+            bufs["x"].upload(x2)                      # new input at the recorded address
+            check(lib.tfhip_graph_launch(gid.value))
+            got = out.download(np.float32, x.size).reshape(x.shape)
+            assert_parity(got, expected(x2))
+            # eager work between replays, through the same pool
+            assert_parity(hip.fused_conv2d(x2, w1, bias=b1), orc.fused_conv2d(x2, w1, bias=b1))
+            side = capi.DeviceBuffer(x.nbytes)
+            block(bufs["x"], side)
+            np.testing.assert_array_equal(side.download(np.float32, x.size), got.reshape(-1))
+            side.free()
+        # a graph that names a freed buffer refuses to run
+        bufs.pop("b3").free()
+        assert lib.tfhip_graph_launch(gid.value) != 0
+        assert b"has been freed" in lib.tfhip_last_error()
+        check(lib.tfhip_graph_destroy(gid.value))
+        assert lib.tfhip_graph_launch(gid.value) != 0
+        assert hip.memory_info()["pooled_bytes"] >= pooled_before
+        # a discarded recording leaves nothing behind
+        check(lib.tfhip_capture_begin())
+        t = capi.DeviceBuffer(4096)
+        t.free()
+        check(lib.tfhip_capture_end(None, None))
+        assert lib.tfhip_capture_end(None, None) != 0
+    finally:
+        out.free()
+        for b in bufs.values():
+            b.free()
+
+
 # ------------------------------------------------------------- MobileNetV2 graph
 
 def test_config4_mobilenet_v2_batch1_vs_oracle(hip, orc, tmp_path):
@@ -557,7 +686,16 @@ def test_config4_mobilenet_v2_batch1_vs_oracle(hip, orc, tmp_path):
         assert_parity(got, want)
         again = model.predict()
         np.testing.assert_array_equal(got, again)
+        assert sum(1 for op, _ in model.plan if "residual" in op) == 10
     finally:
         model.close()
+    # the ten skip connections as Add kernels of their own: the same bits
+    plain = workloads.DeviceMobileNetV2(str(tmp_path), 2, fuse_residual_add=False)
+    try:
+        assert len(plain.plan) == len(model.plan) + 10
+        plain.set_input(x)
+        np.testing.assert_array_equal(plain.predict(), got)
+    finally:
+        plain.close()
     # the kernel-by-kernel host mirror agrees too
     assert_parity(workloads.run_graph(hip, ops, decoded, x[:1]), want[:1])

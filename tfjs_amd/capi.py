@@ -38,12 +38,19 @@ SIGNATURES = {
     "tfhip_event_record": [ctypes.c_int],
     "tfhip_event_elapsed": [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float)],
     "tfhip_set_launch_repeat": [ctypes.c_int],
+    "tfhip_capture_begin": [],
+    "tfhip_capture_end": [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)],
+    "tfhip_graph_launch": [ctypes.c_int],
+    "tfhip_graph_destroy": [ctypes.c_int],
     "tfhip_last_kernel": [ctypes.c_char_p, ctypes.c_size_t],
     "tfhip_fused_matmul": [c_f32p, c_f32p, c_f32p, c_i64, c_i64, c_i64, c_i64, c_i64, ctypes.c_int,
                            ctypes.c_int, c_f32p, c_i64p, ctypes.c_int, c_f32p, c_i64p, ctypes.c_double],
     "tfhip_fused_conv2d": [c_f32p, c_f32p, c_f32p] + [c_i64] * 15 + [ctypes.c_int, c_f32p, c_i64p,
                                                                       ctypes.c_int, c_f32p, c_i64p,
                                                                       ctypes.c_double],
+    "tfhip_fused_conv2d_add": [c_f32p, c_f32p, c_f32p] + [c_i64] * 15 + [ctypes.c_int, c_f32p, c_i64p,
+                                                                      ctypes.c_int, c_f32p, c_i64p,
+                                                                      ctypes.c_double, c_f32p],
     "tfhip_fused_depthwise_conv2d": [c_f32p, c_f32p, c_f32p] + [c_i64] * 15 + [c_f32p, c_i64p, ctypes.c_int,
                                                                                 c_f32p, c_i64p, ctypes.c_double],
     "tfhip_dequant_affine": [ctypes.c_void_p, ctypes.c_int, c_i64, ctypes.c_double, ctypes.c_double,

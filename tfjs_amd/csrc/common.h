@@ -30,12 +30,22 @@ void *workspace(size_t bytes);
 
 // True when [p, p + bytes) lies inside one live block (own or external).
 bool range_is_live(const void *p, size_t bytes);
+// True between tfhip_capture_begin and tfhip_capture_end.
+bool capturing();
 
 #define TFHIP_REQUIRE_INIT()                                              \
   do {                                                                    \
     if (!::tfhip::initialised())                                          \
       return ::tfhip::fail(::tfhip::kNotInitialised,                      \
                            "%s: tfhip_init has not been called", __func__); \
+  } while (0)
+
+// Entry points that wait for the stream or copy through the host cannot be recorded.
+#define TFHIP_REFUSE_WHILE_RECORDING()                                        \
+  do {                                                                        \
+    if (::tfhip::capturing())                                                 \
+      return ::tfhip::fail(::tfhip::kBadArgument,                             \
+                           "%s: not possible between tfhip_capture_begin and tfhip_capture_end", __func__); \
   } while (0)
 
 #define TFHIP_CHECK_HIP(expr)                                               \

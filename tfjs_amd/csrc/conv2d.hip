@@ -252,15 +252,28 @@ int launch_few_channels(const GemmParams &p, int f_h) {
   return kOk;
 }
 
-}  // namespace
+// y += residual for the kernels whose tail does not take a residual itself.
+__global__ __launch_bounds__(256) void add_residual(float *__restrict__ y, const float *__restrict__ residual,
+                                                    long long total) {
+  const long long stride = (long long)gridDim.x * 256;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) y[i] = y[i] + residual[i];
+}
 
-extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y, int64_t batch, int64_t in_h,
-                                  int64_t in_w, int64_t in_c, int64_t f_h, int64_t f_w, int64_t out_c,
-                                  int64_t stride_h, int64_t stride_w, int64_t dilation_h, int64_t dilation_w,
-                                  int64_t pad_top, int64_t pad_left, int64_t out_h, int64_t out_w, int nchw,
-                                  const float *bias, const int64_t bias_strides[4], int activation,
-                                  const float *prelu_weights, const int64_t prelu_strides[4],
-                                  double leakyrelu_alpha) {
+int launch_add_residual(float *y, const float *residual, long long total) {
+  long long blocks = (total + 255) / 256;
+  const long long cap = (long long)num_cus() * 16;
+  TFHIP_LAUNCH((add_residual<<<dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(256), 0, stream()>>>(y, residual,
+                                                                                                     total)));
+  return kOk;
+}
+
+int fused_conv2d(const float *x, const float *filter, float *y, int64_t batch, int64_t in_h,
+                 int64_t in_w, int64_t in_c, int64_t f_h, int64_t f_w, int64_t out_c,
+                 int64_t stride_h, int64_t stride_w, int64_t dilation_h, int64_t dilation_w,
+                 int64_t pad_top, int64_t pad_left, int64_t out_h, int64_t out_w, int nchw,
+                 const float *bias, const int64_t bias_strides[4], int activation,
+                 const float *prelu_weights, const int64_t prelu_strides[4],
+                 double leakyrelu_alpha, const float *residual) {
   TFHIP_REQUIRE_INIT();
   TFHIP_CHECK_ARG(batch >= 0 && in_h > 0 && in_w > 0 && in_c > 0 && f_h > 0 && f_w > 0 && out_c > 0 &&
                       stride_h > 0 && stride_w > 0 && dilation_h > 0 && dilation_w > 0 && out_h >= 0 && out_w >= 0,
@@ -276,6 +289,7 @@ extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
   TFHIP_CHECK_RANGE(x, batch * in_h * in_w * in_c, 4, "x");
   TFHIP_CHECK_RANGE(filter, K * out_c, 4, "filter");
   TFHIP_CHECK_RANGE(y, M * out_c, 4, "y");
+  if (residual) TFHIP_CHECK_RANGE(residual, M * out_c, 4, "residual");
 
   GemmParams p = {};
   p.a = x; p.b = filter; p.c = y;
@@ -296,6 +310,7 @@ extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
   int rc = fill_epilogue(p.epi, "tfhip_fused_conv2d", dims, 4, bias, bias_strides, activation, prelu_weights,
                          prelu_strides, leakyrelu_alpha, kConv);
   if (rc) return rc;
+  p.epi.residual = residual;   // every GEMM-shaped path below adds it in its tail
   p.epi.out_h = (int)out_h;
   p.epi.out_w = (int)out_w;
   if (nchw) {
@@ -330,11 +345,14 @@ extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
     const bool few_taps = K <= kMaxTaps && M < lim - 256 && p.a_bytes != 0;
     // 32 channels per wavefront when there are pixels enough to fill the chip that
     // way, else 16 (twice the wavefronts)
-    if (few_taps && out_c % 32 == 0 && M >= 64LL * 4 * num_cus()) return launch_few_taps_k<2>(p, (int)f_h);
-    if (few_taps && out_c % 16 == 0) return launch_few_taps_k<1>(p, (int)f_h);
-    if (out_c % 32 == 0) return launch_few_channels<32>(p, (int)f_h);
-    if (out_c % 16 == 0) return launch_few_channels<16>(p, (int)f_h);
-    return launch_few_channels<8>(p, (int)f_h);
+    if (few_taps && out_c % 32 == 0 && M >= 64LL * 4 * num_cus()) rc = launch_few_taps_k<2>(p, (int)f_h);
+    else if (few_taps && out_c % 16 == 0) rc = launch_few_taps_k<1>(p, (int)f_h);
+    else if (out_c % 32 == 0) rc = launch_few_channels<32>(p, (int)f_h);
+    else if (out_c % 16 == 0) rc = launch_few_channels<16>(p, (int)f_h);
+    else rc = launch_few_channels<8>(p, (int)f_h);
+    // these direct kernels have no residual operand: a second pass over y adds it
+    if (rc == kOk && residual) rc = launch_add_residual(y, residual, M * out_c);
+    return rc;
   }
   if (vec) {
     const int shape = choose_tile_shape(M, out_c, K, 1, num_cus());
@@ -342,4 +360,32 @@ extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y,
   }
   if (out_c <= 32) return launch_gemm<256, 32, 16, 4, 1, kLoadIm2colScalar, kLoadScalar>(p);
   return launch_gemm<64, 64, 16, 2, 2, kLoadIm2colScalar, kLoadScalar>(p);
+}
+
+}  // namespace
+
+extern "C" int tfhip_fused_conv2d(const float *x, const float *filter, float *y, int64_t batch, int64_t in_h,
+                                  int64_t in_w, int64_t in_c, int64_t f_h, int64_t f_w, int64_t out_c,
+                                  int64_t stride_h, int64_t stride_w, int64_t dilation_h, int64_t dilation_w,
+                                  int64_t pad_top, int64_t pad_left, int64_t out_h, int64_t out_w, int nchw,
+                                  const float *bias, const int64_t bias_strides[4], int activation,
+                                  const float *prelu_weights, const int64_t prelu_strides[4],
+                                  double leakyrelu_alpha) {
+  return fused_conv2d(x, filter, y, batch, in_h, in_w, in_c, f_h, f_w, out_c, stride_h, stride_w, dilation_h,
+                      dilation_w, pad_top, pad_left, out_h, out_w, nchw, bias, bias_strides, activation,
+                      prelu_weights, prelu_strides, leakyrelu_alpha, nullptr);
+}
+
+extern "C" int tfhip_fused_conv2d_add(const float *x, const float *filter, float *y, int64_t batch, int64_t in_h,
+                                      int64_t in_w, int64_t in_c, int64_t f_h, int64_t f_w, int64_t out_c,
+                                      int64_t stride_h, int64_t stride_w, int64_t dilation_h, int64_t dilation_w,
+                                      int64_t pad_top, int64_t pad_left, int64_t out_h, int64_t out_w, int nchw,
+                                      const float *bias, const int64_t bias_strides[4], int activation,
+                                      const float *prelu_weights, const int64_t prelu_strides[4],
+                                      double leakyrelu_alpha, const float *residual) {
+  TFHIP_CHECK_ARG(residual != nullptr, "tfhip_fused_conv2d_add: residual is NULL");
+  TFHIP_CHECK_ARG(residual != y, "tfhip_fused_conv2d_add: residual and y are the same buffer");
+  return fused_conv2d(x, filter, y, batch, in_h, in_w, in_c, f_h, f_w, out_c, stride_h, stride_w, dilation_h,
+                      dilation_w, pad_top, pad_left, out_h, out_w, nchw, bias, bias_strides, activation,
+                      prelu_weights, prelu_strides, leakyrelu_alpha, residual);
 }

@@ -30,6 +30,10 @@ struct Epilogue {
   // strides for (n, oh, ow, c) so NCHW outputs can be written in place.
   int out_h, out_w;
   long long y_s[4];
+  // Optional tensor of the output's own shape and layout, added to the result
+  // after the activation (a residual connection: the Add that follows the
+  // convolution in the graph, rounded like that separate float32 Add).
+  const float *residual;
 };
 
 __device__ __forceinline__ float activate(float v, int act, float alpha, double leaky) {

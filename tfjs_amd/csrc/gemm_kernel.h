@@ -514,6 +514,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   const long long ldc = to_ws ? p.N : p.ldc;
   const bool conv_addr = !to_ws && e.addressing == kConv;
   const bool vec = to_ws ? p.N % 4 == 0 : p.vec_store != 0;
+  // the residual lies where the output element does
+  const float *R = (fused && e.residual) ? e.residual + (long long)bz * p.c_batch_stride : nullptr;
   float alpha_q[T::TN][4];
 #pragma unroll
   for (int j = 0; j < T::TN; ++j) {
@@ -559,11 +561,19 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
           }
         }
         if (vec) {
+          if (R) {
+            const float4 r4 = *reinterpret_cast<const float4 *>(R + base + col);
+            out[0] += r4.x; out[1] += r4.y; out[2] += r4.z; out[3] += r4.w;
+          }
           *reinterpret_cast<float4 *>(C + base + col) = make_float4(out[0], out[1], out[2], out[3]);
         } else {
 #pragma unroll
-          for (int q = 0; q < 4; ++q)
-            if (col + q < p.N) C[base + (col + q) * col_stride] = out[q];
+          for (int q = 0; q < 4; ++q) {
+            if (col + q < p.N) {
+              const long long at = base + (col + q) * col_stride;
+              C[at] = R ? out[q] + R[at] : out[q];
+            }
+          }
         }
       }
     }
@@ -606,7 +616,8 @@ static __global__ __launch_bounds__(256) void gemm_finish(GemmParams p) {
     } else {
       v = p.c[at];
     }
-    p.c[at] = finish(e, v, bz, row, col, n, oh, ow);
+    v = finish(e, v, bz, row, col, n, oh, ow);
+    p.c[at] = e.residual ? v + e.residual[at] : v;
   }
 }
 

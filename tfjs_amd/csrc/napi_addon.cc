@@ -300,7 +300,8 @@ napi_value FusedMatMul(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
-// fusedConv2D(x, filter, y, geom[15], nchw, bias, biasStrides[4], activation, prelu, preluStrides[4], alpha)
+// fusedConv2D(x, filter, y, geom[15], nchw, bias, biasStrides[4], activation, prelu, preluStrides[4], alpha
+//             [, residual])   with a residual: tfhip_fused_conv2d_add
 // geom = [batch, inH, inW, inC, fH, fW, outC, strideH, strideW, dilH, dilW, padTop, padLeft, outH, outW]
 napi_value FusedConv2D(napi_env env, napi_callback_info info) {
   Args a(env, info, 11, "fusedConv2D");
@@ -314,6 +315,13 @@ napi_value FusedConv2D(napi_env env, napi_callback_info info) {
   const float *bias = (const float *)a.ptr(5), *prelu = (const float *)a.ptr(8);
   const double leaky = a.num(10);
   if (!a.ok) return nullptr;
+  const float *residual = a.argc > 11 ? (const float *)a.ptr(11) : nullptr;
+  if (!a.ok) return nullptr;
+  if (residual) {
+    HIP_OK(tfhip_fused_conv2d_add(x, w, y, g[0], g[1], g[2], g[3], g[4], g[5], g[6], g[7], g[8], g[9], g[10], g[11],
+                                  g[12], g[13], g[14], nchw, bias, bs, act, prelu, ps, leaky, residual));
+    return undefined(env);
+  }
   HIP_OK(tfhip_fused_conv2d(x, w, y, g[0], g[1], g[2], g[3], g[4], g[5], g[6], g[7], g[8], g[9], g[10], g[11], g[12],
                             g[13], g[14], nchw, bias, bs, act, prelu, ps, leaky));
   return undefined(env);
@@ -401,6 +409,55 @@ napi_value MeanHW(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+// copy(dst, src, bytes): device to device on the library's stream
+napi_value Copy(napi_env env, napi_callback_info info) {
+  Args a(env, info, 3, "copy");
+  void *dst = a.ptr(0), *src = a.ptr(1);
+  const double bytes = a.num(2);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_copy(dst, src, (size_t)bytes));
+  return undefined(env);
+}
+
+napi_value CaptureBegin(napi_env env, napi_callback_info) {
+  HIP_OK(tfhip_capture_begin());
+  return undefined(env);
+}
+
+// captureEnd(keep): {id, nodes}; keep == false discards the recording (id 0)
+napi_value CaptureEnd(napi_env env, napi_callback_info info) {
+  Args a(env, info, 1, "captureEnd");
+  bool keep = false;
+  if (a.ok && napi_get_value_bool(env, a.argv[0], &keep) != napi_ok) {
+    napi_throw_type_error(env, nullptr, "tfjs_hip.captureEnd: keep must be a boolean");
+    return nullptr;
+  }
+  if (!a.ok) return nullptr;
+  int id = 0, nodes = 0;
+  HIP_OK(tfhip_capture_end(keep ? &id : nullptr, &nodes));
+  napi_value obj;
+  NAPI_OK(napi_create_object(env, &obj));
+  napi_set_named_property(env, obj, "id", make_number(env, id));
+  napi_set_named_property(env, obj, "nodes", make_number(env, nodes));
+  return obj;
+}
+
+napi_value GraphLaunch(napi_env env, napi_callback_info info) {
+  Args a(env, info, 1, "graphLaunch");
+  const int id = a.i32(0);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_graph_launch(id));
+  return undefined(env);
+}
+
+napi_value GraphDestroy(napi_env env, napi_callback_info info) {
+  Args a(env, info, 1, "graphDestroy");
+  const int id = a.i32(0);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_graph_destroy(id));
+  return undefined(env);
+}
+
 napi_value Register(napi_env env, napi_value exports) {
   const napi_property_descriptor props[] = {
 #define FN(name, fn) {name, nullptr, fn, nullptr, nullptr, nullptr, napi_enumerable, nullptr}
@@ -424,6 +481,11 @@ napi_value Register(napi_env env, napi_value exports) {
       FN("dequantF16", DequantF16),
       FN("add", Add),
       FN("meanHW", MeanHW),
+      FN("copy", Copy),
+      FN("captureBegin", CaptureBegin),
+      FN("captureEnd", CaptureEnd),
+      FN("graphLaunch", GraphLaunch),
+      FN("graphDestroy", GraphDestroy),
 #undef FN
   };
   napi_define_properties(env, exports, sizeof props / sizeof props[0], props);

@@ -1,10 +1,11 @@
 // Library lifetime, the single stream, the pooled device allocator with its
-// live-block registry, host<->device copies through pinned staging, and event
-// timing.
+// live-block registry, host<->device copies through pinned staging, event
+// timing, and recording of a sequence of launches into a HIP graph.
 #include <string.h>
 
 #include <map>
 #include <mutex>
+#include <set>
 #include <unordered_map>
 #include <vector>
 
@@ -15,6 +16,13 @@ namespace {
 
 constexpr size_t kStagingBytes = size_t(32) << 20;  // per pinned staging buffer
 constexpr int kStagingBuffers = 2;
+
+struct RecordedGraph {
+  hipGraphExec_t exec = nullptr;
+  size_t nodes = 0;
+  std::vector<std::pair<void *, size_t>> owned;         // block, class size
+  std::vector<std::pair<uintptr_t, size_t>> refs;       // base, size of blocks that must stay live
+};
 
 struct Runtime {
   bool ready = false;
@@ -34,7 +42,20 @@ struct Runtime {
   size_t workspace_bytes = 0;
   hipEvent_t events[TFHIP_MAX_EVENTS] = {};
   bool event_recorded[TFHIP_MAX_EVENTS] = {};
+  // Recording (tfhip_capture_begin .. tfhip_capture_end). A recorded graph
+  // replays kernels with the addresses they were given, so it keeps what it
+  // needs: blocks freed while recording go to `capture_free` (reused by later
+  // allocations of the same recording, then owned by the graph), and every
+  // block an operand check saw is noted in `capture_refs` (checked again at
+  // each replay).
+  bool capturing = false;
+  std::unordered_map<size_t, std::vector<void *>> capture_free;
+  std::set<uintptr_t> capture_refs;
+  std::map<int, RecordedGraph> graphs;
+  int next_graph = 1;
+  std::vector<void *> retired_workspaces;  // outgrown while a graph might still name them
 };
+
 
 Runtime g;
 std::mutex g_mutex;
@@ -51,6 +72,11 @@ size_t class_size(size_t bytes) {
   const size_t lo = p >> 1;
   size_t c = lo + ((bytes - lo + step - 1) / step) * step;
   return c < 256 ? 256 : c;
+}
+
+void give_back_locked(void *p, size_t cls) {
+  g.free_lists[cls].push_back(p);
+  g.pooled_bytes += cls;
 }
 
 void release_pool_locked() {
@@ -103,8 +129,13 @@ int num_cus() { return g.prop.multiProcessorCount; }
 // ordered, so consecutive launches may share it.
 void *workspace(size_t bytes) {
   if (bytes <= g.workspace_bytes) return g.workspace;
-  (void)hipStreamSynchronize(g.stream);   // a launch in flight may still use the old block
-  if (g.workspace) (void)hipFree(g.workspace);
+  if (g.capturing || !g.graphs.empty()) {
+    // a recorded graph may name the old block: it stays allocated until shutdown
+    if (g.workspace) g.retired_workspaces.push_back(g.workspace);
+  } else {
+    (void)hipStreamSynchronize(g.stream);   // a launch in flight may still use the old block
+    if (g.workspace) (void)hipFree(g.workspace);
+  }
   g.workspace = nullptr;
   g.workspace_bytes = 0;
   const size_t want = (bytes + (size_t(1) << 24) - 1) & ~((size_t(1) << 24) - 1);
@@ -123,8 +154,12 @@ bool range_is_live(const void *p, size_t bytes) {
   auto it = g.live.upper_bound(a);
   if (it == g.live.begin()) return false;
   --it;
-  return a >= it->first && a + bytes <= it->first + it->second && a + bytes >= a;
+  const bool inside = a >= it->first && a + bytes <= it->first + it->second && a + bytes >= a;
+  if (inside && g.capturing) g.capture_refs.insert(it->first);
+  return inside;
 }
+
+bool capturing() { return g.capturing; }
 
 // Copies a small result straight into pinned host memory: a kernel starts within
 // a few microseconds, the copy engine needs 10-15 for a transfer of any size.
@@ -172,7 +207,26 @@ int tfhip_init(int device) {
 int tfhip_shutdown(void) {
   std::lock_guard<std::mutex> lock(g_mutex);
   if (!g.ready) return kOk;
+  if (g.capturing) {
+    hipGraph_t abandoned = nullptr;
+    (void)hipStreamEndCapture(g.stream, &abandoned);
+    if (abandoned) (void)hipGraphDestroy(abandoned);
+    (void)hipGetLastError();
+    g.capturing = false;
+  }
   (void)hipStreamSynchronize(g.stream);
+  for (auto &kv : g.graphs) {
+    if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
+    for (auto &b : kv.second.owned) (void)hipFree(b.first);
+  }
+  g.graphs.clear();
+  for (auto &kv : g.capture_free) {
+    for (void *p : kv.second) (void)hipFree(p);
+  }
+  g.capture_free.clear();
+  g.capture_refs.clear();
+  for (void *p : g.retired_workspaces) (void)hipFree(p);
+  g.retired_workspaces.clear();
   for (auto &kv : g.live) {
     if (g.owned[kv.first]) (void)hipFree(reinterpret_cast<void *>(kv.first));
   }
@@ -218,7 +272,10 @@ int tfhip_alloc(size_t bytes, void **dptr) {
   std::lock_guard<std::mutex> lock(g_mutex);
   void *p = nullptr;
   auto &fl = g.free_lists[cls];
-  if (!fl.empty()) {
+  if (g.capturing && !g.capture_free[cls].empty()) {
+    p = g.capture_free[cls].back();
+    g.capture_free[cls].pop_back();
+  } else if (!fl.empty()) {
     p = fl.back();
     fl.pop_back();
     g.pooled_bytes -= cls;
@@ -226,7 +283,7 @@ int tfhip_alloc(size_t bytes, void **dptr) {
     hipError_t e = hipMalloc(&p, cls);
     if (e == hipErrorOutOfMemory) {
       (void)hipGetLastError();
-      (void)hipStreamSynchronize(g.stream);
+      if (!g.capturing) (void)hipStreamSynchronize(g.stream);   // (a recording stream cannot be waited for)
       release_pool_locked();
       e = hipMalloc(&p, cls);
     }
@@ -257,8 +314,11 @@ int tfhip_free(void *dptr) {
   g.live.erase(it);
   g.owned.erase(a);
   g.live_bytes -= cls;
-  g.free_lists[cls].push_back(dptr);
-  g.pooled_bytes += cls;
+  if (g.capturing) {
+    g.capture_free[cls].push_back(dptr);   // the graph being recorded names it: the graph keeps it
+  } else {
+    give_back_locked(dptr, cls);
+  }
   return kOk;
 }
 
@@ -297,6 +357,7 @@ int tfhip_memory_info(size_t *live, size_t *live_bytes, size_t *pooled_bytes) {
 
 int tfhip_upload(void *dst, size_t dst_offset, const void *host, size_t bytes) {
   TFHIP_REQUIRE_INIT();
+  TFHIP_REFUSE_WHILE_RECORDING();
   if (bytes == 0) return kOk;
   TFHIP_CHECK_ARG(host != nullptr, "tfhip_upload: host pointer is NULL");
   char *d = static_cast<char *>(dst) + dst_offset;
@@ -319,6 +380,7 @@ int tfhip_upload(void *dst, size_t dst_offset, const void *host, size_t bytes) {
 
 int tfhip_download(void *host, const void *src, size_t src_offset, size_t bytes) {
   TFHIP_REQUIRE_INIT();
+  TFHIP_REFUSE_WHILE_RECORDING();
   if (bytes == 0) {
     TFHIP_CHECK_HIP(hipStreamSynchronize(g.stream));
     return kOk;
@@ -374,12 +436,14 @@ int tfhip_last_kernel(char *name, size_t name_len) {
 
 int tfhip_sync(void) {
   TFHIP_REQUIRE_INIT();
+  TFHIP_REFUSE_WHILE_RECORDING();
   TFHIP_CHECK_HIP(hipStreamSynchronize(g.stream));
   return kOk;
 }
 
 int tfhip_event_record(int slot) {
   TFHIP_REQUIRE_INIT();
+  TFHIP_REFUSE_WHILE_RECORDING();
   TFHIP_CHECK_ARG(slot >= 0 && slot < TFHIP_MAX_EVENTS, "tfhip_event_record: slot %d out of range", slot);
   if (!g.events[slot]) TFHIP_CHECK_HIP(hipEventCreate(&g.events[slot]));
   TFHIP_CHECK_HIP(hipEventRecord(g.events[slot], g.stream));
@@ -389,6 +453,7 @@ int tfhip_event_record(int slot) {
 
 int tfhip_event_elapsed(int start_slot, int end_slot, float *ms) {
   TFHIP_REQUIRE_INIT();
+  TFHIP_REFUSE_WHILE_RECORDING();
   TFHIP_CHECK_ARG(start_slot >= 0 && start_slot < TFHIP_MAX_EVENTS && end_slot >= 0 &&
                       end_slot < TFHIP_MAX_EVENTS && ms != nullptr,
                   "tfhip_event_elapsed: bad arguments");
@@ -396,6 +461,91 @@ int tfhip_event_elapsed(int start_slot, int end_slot, float *ms) {
                   "tfhip_event_elapsed: slot %d or %d was never recorded", start_slot, end_slot);
   TFHIP_CHECK_HIP(hipEventSynchronize(g.events[end_slot]));
   TFHIP_CHECK_HIP(hipEventElapsedTime(ms, g.events[start_slot], g.events[end_slot]));
+  return kOk;
+}
+
+int tfhip_capture_begin(void) {
+  TFHIP_REQUIRE_INIT();
+  std::lock_guard<std::mutex> lock(g_mutex);
+  TFHIP_CHECK_ARG(!g.capturing, "tfhip_capture_begin: a recording is already open");
+  // Relaxed mode: an allocation that misses the pool may still call hipMalloc.
+  TFHIP_CHECK_HIP(hipStreamBeginCapture(g.stream, hipStreamCaptureModeRelaxed));
+  g.capturing = true;
+  g.capture_refs.clear();
+  return kOk;
+}
+
+int tfhip_capture_end(int *graph_id, int *nodes) {
+  TFHIP_REQUIRE_INIT();
+  std::lock_guard<std::mutex> lock(g_mutex);
+  TFHIP_CHECK_ARG(g.capturing, "tfhip_capture_end: no recording is open");
+  g.capturing = false;
+  hipGraph_t graph = nullptr;
+  hipError_t e = hipStreamEndCapture(g.stream, &graph);
+  RecordedGraph rec;
+  if (e == hipSuccess) {
+    (void)hipGraphGetNodes(graph, nullptr, &rec.nodes);
+    if (graph_id != nullptr) e = hipGraphInstantiate(&rec.exec, graph, nullptr, nullptr, 0);
+  }
+  if (graph) (void)hipGraphDestroy(graph);
+  if (e != hipSuccess || graph_id == nullptr) {
+    // nothing will replay: the blocks set aside for the graph return to the pool
+    (void)hipGetLastError();
+    for (auto &kv : g.capture_free) {
+      for (void *p : kv.second) give_back_locked(p, kv.first);
+    }
+    g.capture_free.clear();
+    g.capture_refs.clear();
+    if (e != hipSuccess) return fail(kHipError, "tfhip_capture_end: %s", hipGetErrorString(e));
+    if (nodes) *nodes = (int)rec.nodes;
+    return kOk;
+  }
+  for (auto &kv : g.capture_free) {
+    for (void *p : kv.second) {
+      rec.owned.emplace_back(p, kv.first);
+      g.capture_refs.erase(reinterpret_cast<uintptr_t>(p));
+    }
+  }
+  g.capture_free.clear();
+  for (uintptr_t base : g.capture_refs) {
+    auto it = g.live.find(base);
+    if (it != g.live.end()) rec.refs.emplace_back(base, it->second);
+  }
+  g.capture_refs.clear();
+  const int id = g.next_graph++;
+  if (nodes) *nodes = (int)rec.nodes;
+  g.graphs[id] = std::move(rec);
+  *graph_id = id;
+  return kOk;
+}
+
+int tfhip_graph_launch(int graph_id) {
+  TFHIP_REQUIRE_INIT();
+  std::lock_guard<std::mutex> lock(g_mutex);
+  TFHIP_CHECK_ARG(!g.capturing, "tfhip_graph_launch: a recording is open");
+  auto it = g.graphs.find(graph_id);
+  TFHIP_CHECK_ARG(it != g.graphs.end(), "tfhip_graph_launch: no graph %d", graph_id);
+  for (auto &r : it->second.refs) {
+    auto b = g.live.find(r.first);
+    if (b == g.live.end() || b->second != r.second) {
+      return fail(kOutOfRange,
+                  "tfhip_graph_launch: graph %d names the device buffer at %p (%zu bytes), which has been freed since it was recorded",
+                  graph_id, reinterpret_cast<void *>(r.first), r.second);
+    }
+  }
+  for (int r = g_repeat; r > 0; --r) TFHIP_CHECK_HIP(hipGraphLaunch(it->second.exec, g.stream));
+  return kOk;
+}
+
+int tfhip_graph_destroy(int graph_id) {
+  TFHIP_REQUIRE_INIT();
+  std::lock_guard<std::mutex> lock(g_mutex);
+  auto it = g.graphs.find(graph_id);
+  TFHIP_CHECK_ARG(it != g.graphs.end(), "tfhip_graph_destroy: no graph %d", graph_id);
+  (void)hipStreamSynchronize(g.stream);   // no replay is in flight when the executable goes
+  if (it->second.exec) (void)hipGraphExecDestroy(it->second.exec);
+  for (auto &b : it->second.owned) give_back_locked(b.first, b.second);
+  g.graphs.erase(it);
   return kOk;
 }
 

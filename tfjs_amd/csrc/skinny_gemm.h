@@ -29,6 +29,7 @@ namespace tfhip {
 
 struct SkinnyArgs {
   const float *a, *b, *bias;
+  const float *residual;   // [M][N] like c, added after the activation; may be null
   float *c;
   long long bias_stride;
   double leaky_alpha;
@@ -169,8 +170,13 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
           }
           out[k] = v;
         }
-        if (row < g.M && col < g.N)
+        if (row < g.M && col < g.N) {
+          if (g.residual) {
+            const float4 r4 = *reinterpret_cast<const float4 *>(g.residual + (long long)row * g.N + col);
+            out[0] += r4.x; out[1] += r4.y; out[2] += r4.z; out[3] += r4.w;
+          }
           *reinterpret_cast<float4 *>(g.c + (long long)row * g.N + col) = make_float4(out[0], out[1], out[2], out[3]);
+        }
 #pragma unroll
         for (int h = 0; h < NA; ++h) acc[h][n] = (float4_t){0.f, 0.f, 0.f, 0.f};
       }
@@ -376,7 +382,8 @@ inline int launch_skinny(const GemmParams &p) {
   g.k_pad = (p.K + kSkinnyChunk - 1) / kSkinnyChunk * kSkinnyChunk;
   g.a_bytes = p.a_bytes;
   g.activation = p.epi.activation;
-  if (tuning(kTuneSkinnyRegs) != 0) {   // B in registers where an instantiation fits
+  g.residual = p.epi.residual;
+  if (tuning(kTuneSkinnyRegs) != 0 && !g.residual) {   // B in registers where an instantiation fits
     // columns per wavefront: all of them up to 96; wider outputs in slices (a
     // wavefront that keeps 144 columns of accumulators, B and bias is so heavy on
     // registers that too few of them are resident to cover each other's stores)

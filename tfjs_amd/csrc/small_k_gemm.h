@@ -188,7 +188,7 @@ inline bool small_k_applies(const GemmParams &p, bool transpose_a, bool transpos
   if (transpose_a || transpose_b || !vec) return false;
   if (p.K < 4 || p.K > 64 || p.K % 4 != 0 || p.N % 4 != 0 || !p.vec_store || p.ldc != p.N) return false;
   if (!p.epi.channel_operands || p.epi.activation > TFHIP_LEAKYRELU || p.epi.activation == TFHIP_PRELU) return false;
-  if (p.a_bytes == 0 || p.b_bytes == 0 || p.batch > 65535) return false;
+  if (p.a_bytes == 0 || p.b_bytes == 0 || p.batch > 65535 || p.epi.residual) return false;
   // one round trip only pays while the k loop it replaces is short against its own set-up
   return (long long)p.M * p.batch >= 512 && p.N >= 64;
 }

@@ -7,9 +7,18 @@
  * FusedDepthwiseConv2D.ts:25-61, DepthwiseConv2dNative.ts:23-102). The
  * convolution shape arithmetic is backend_util.computeConv2DInfo, exactly as
  * the reference's kernels call it; the native library receives its numbers.
+ *
+ * FusedConv2DAdd has no counterpart among the reference's kernel names: it is
+ * FusedConv2D with one more input, `residual`, the other operand of the Add
+ * node that consumes the convolution in a residual block
+ * (y = activation(conv + bias) + residual, one launch, the bits of the two
+ * separate kernels). A graph executor that finds the pair FusedConv2D -> Add
+ * runs it in their place; any shape the Add would broadcast falls back to the
+ * two kernels here.
  */
 const tf = require('../core');
 const {activationCode, broadcastStrides, requireFloat32, addon} = require('./fused_util');
+const glue = require('./glue');
 
 // Scratch that carries the geometry and the epilogue strides to the addon.
 const geom = new Float64Array(15);
@@ -41,7 +50,7 @@ function epilogueStrides(t, outShape, nchw, into) {
   return into;
 }
 
-function convImpl(args, depthwise, fused, opName) {
+function convImpl(args, depthwise, fused, opName, residual) {
   const {x, filter} = args.inputs;
   const bias = fused ? args.inputs.bias : null;
   const prelu = fused ? args.inputs.preluActivationWeights : null;
@@ -52,7 +61,7 @@ function convImpl(args, depthwise, fused, opName) {
     dilations = [1, 1];
   }
   const activation = fused ? (args.attrs.activation || 'linear') : 'linear';
-  requireFloat32([x, filter, bias, prelu], opName);
+  requireFloat32([x, filter, bias, prelu, residual], opName);
   if (activation === 'prelu' && prelu == null) {
     throw new Error(`${opName}: prelu activation needs preluActivationWeights`);
   }
@@ -74,6 +83,13 @@ function convImpl(args, depthwise, fused, opName) {
   const preluStrides = activation === 'prelu' ?
       epilogueStrides(prelu, info.outShape, nchw, preluScratch) :
       null;
+  if (residual != null && !tf.util.arraysEqual(residual.shape, info.outShape)) {
+    // an Add that broadcasts: the two kernels, as the graph had them
+    const y = convImpl(args, depthwise, fused, opName, null);
+    const sum = glue.addConfig.kernelFunc({inputs: {a: y, b: residual}, backend});
+    backend.disposeIntermediateTensorInfo(y);
+    return sum;
+  }
   const out = backend.makeOutput(info.outShape, 'float32');
   if (tf.util.sizeFromShape(info.outShape) === 0) {
     return out;
@@ -105,7 +121,8 @@ function convImpl(args, depthwise, fused, opName) {
         backend.ptr(x.dataId), backend.ptr(filter.dataId), backend.ptr(out.dataId),
         geom, nchw ? 1 : 0, bias ? backend.ptr(bias.dataId) : null, biasStrides,
         activationCode(activation, opName),
-        preluStrides ? backend.ptr(prelu.dataId) : null, preluStrides, alpha);
+        preluStrides ? backend.ptr(prelu.dataId) : null, preluStrides, alpha,
+        residual != null ? backend.ptr(residual.dataId) : null);
   }
   return out;
 }
@@ -115,6 +132,16 @@ module.exports = {
     kernelName: 'FusedConv2D',
     backendName: 'hip',
     kernelFunc: args => convImpl(args, false, true, 'FusedConv2D')
+  },
+  fusedConv2DAddConfig: {
+    kernelName: 'FusedConv2DAdd',
+    backendName: 'hip',
+    kernelFunc: args => {
+      if (args.inputs.residual == null) {
+        throw new Error('FusedConv2DAdd: the residual input is missing');
+      }
+      return convImpl(args, false, true, 'FusedConv2DAdd', args.inputs.residual);
+    }
   },
   conv2DConfig: {
     kernelName: 'Conv2D',

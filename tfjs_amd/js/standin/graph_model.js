@@ -17,6 +17,13 @@
  * {decodeWeights: require('tfjs-backend-hip').decodeWeights} to have quantized
  * weights uploaded as bytes and dequantized on the GPU.
  *
+ * One thing it does that the reference's executor does not: when the active
+ * backend registers a 'FusedConv2DAdd' kernel, a _FusedConv2D node whose only
+ * reader is an Add / AddV2 node (a projection convolution and the skip connection
+ * of a residual block) is executed together with that Add as one kernel. The
+ * result has the bits of the two separate kernels; {fuseResidualAdd: false} in
+ * the load options turns it off.
+ *
  * Where @tensorflow/tfjs-converter is installed, use its GraphModel instead; the
  * backend and the injected decodeWeights are the same.
  */
@@ -149,6 +156,30 @@ function fusedConvParams(node) {
     preluActivationWeights: isBiasAdd ? inputs[3] : inputs[2],
     leakyreluAlpha: fixed.leakyreluAlpha
   });
+}
+
+/**
+ * _FusedConv2D node + the Add that reads it -> function(inputs) => Tensor, where
+ * inputs are the convolution's own inputs followed by the Add's other operand.
+ */
+function compileConvAdd(convNode) {
+  const params = fusedConvParams(convNode);
+  const convInputs = (convNode.input || []).filter(i => i[0] !== '^').length;
+  return inputs => {
+    const p = params(inputs);
+    let x = p.x;
+    const batched = x.shape.length === 4;
+    if (!batched) {
+      x = tf.reshape(x, [1, x.shape[0], x.shape[1], x.shape[2]]);   // as tf.fused.conv2d does for rank 3
+    }
+    const out = tf.engine().runKernel(
+        'FusedConv2DAdd',
+        {x, filter: p.filter, bias: p.bias, preluActivationWeights: p.preluActivationWeights,
+         residual: inputs[convInputs]},
+        {strides: p.strides, pad: p.pad, dataFormat: p.dataFormat, dilations: p.dilations,
+         dimRoundingMode: undefined, activation: p.activation, leakyreluAlpha: p.leakyreluAlpha});
+    return out;
+  };
 }
 
 /**
@@ -387,7 +418,7 @@ class GraphModel {
       }
     });
 
-    const planKey = Object.keys(feeds).join(',') + '|' + fetches.join(',');
+    const planKey = tf.getBackend() + '|' + Object.keys(feeds).join(',') + '|' + fetches.join(',');
     let compiled = this.plans.get(planKey);
     if (compiled === undefined) {
       compiled = this.makePlan(feeds, fetches);
@@ -413,9 +444,11 @@ class GraphModel {
           for (let i = 0; i < args.length; i++) {
             args[i] = values[step.sources[i]];
           }
-          let run = this.compiled[name];
+          const key = step.conv != null ? name + '<-' + step.conv : name;
+          let run = this.compiled[key];
           if (run === undefined) {
-            run = this.compiled[name] = compileNode(this.nodes[name]);
+            run = this.compiled[key] =
+                step.conv != null ? compileConvAdd(this.nodes[step.conv]) : compileNode(this.nodes[name]);
           }
           const out = values[name] = run(args);
           // intermediates that nobody reads again can go now
@@ -457,31 +490,76 @@ class GraphModel {
           `Missing the following inputs: [${missing}]`);
     }
     const order = this.order.filter(n => needed.has(n));
-    const lastUse = {};
+    const fetchSet = new Set(fetches.map(n => parseNodeName(n)[0]));
+    const isOp = n => feeds[n] == null && this.nodes[n].op !== 'Const';
+    const dataSources = name => (this.nodes[name].input || []).filter(i => i[0] !== '^').map(i => {
+      const [src, port] = parseNodeName(i);
+      if (port !== 0) {
+        throw new Error(`Node '${name}' reads output ${port} of '${src}'; only single-output ops are supported`);
+      }
+      return src;
+    });
+
+    // _FusedConv2D read by one Add only -> one step at the convolution's place
+    // that yields the Add's value (the other operand must exist by then).
+    const position = {}, readers = {};
     order.forEach((n, idx) => {
-      if (feeds[n] == null) {
-        (this.nodes[n].input || []).forEach(i => lastUse[parseNodeName(i)[0]] = idx);
+      position[n] = idx;
+      if (isOp(n)) {
+        (this.nodes[n].input || []).forEach(i => {
+          const src = parseNodeName(i)[0];
+          readers[src] = (readers[src] || 0) + 1;
+        });
       }
     });
-    const fetchSet = new Set(fetches.map(n => parseNodeName(n)[0]));
-    const steps = order.map((name, idx) => {
-      const node = this.nodes[name];
-      if (feeds[name] != null) {
-        return {name, kind: 'feed'};
-      }
-      if (node.op === 'Const') {
-        return {name, kind: 'const'};
-      }
-      const sources = (node.input || []).filter(i => i[0] !== '^').map(i => {
-        const [src, port] = parseNodeName(i);
-        if (port !== 0) {
-          throw new Error(`Node '${name}' reads output ${port} of '${src}'; only single-output ops are supported`);
+    const fuse = this.loadOptions.fuseResidualAdd !== false && tf.getKernel != null &&
+        tf.getKernel('FusedConv2DAdd', tf.getBackend()) != null;
+    const convOf = {}, addOf = {};   // Add name -> conv name and back
+    if (fuse) {
+      order.forEach(n => {
+        const node = this.nodes[n];
+        if (!isOp(n) || (node.op !== 'Add' && node.op !== 'AddV2') || (node.input || []).length !== 2) {
+          return;
         }
-        return src;
+        const src = dataSources(n);
+        if (src.length !== 2 || src[0] === src[1]) {
+          return;
+        }
+        const candidates = [0, 1].filter(k => {
+          const c = src[k], other = src[1 - k];
+          return isOp(c) && this.nodes[c].op === '_FusedConv2D' && readers[c] === 1 && !fetchSet.has(c) &&
+              addOf[c] == null && position[other] < position[c];
+        });
+        if (candidates.length > 0) {
+          const c = src[candidates[candidates.length - 1]];
+          convOf[n] = c;
+          addOf[c] = n;
+        }
       });
-      const release = Array.from(new Set((node.input || []).map(i => parseNodeName(i)[0]))).filter(
-          src => lastUse[src] === idx && !fetchSet.has(src) && feeds[src] == null && this.nodes[src].op !== 'Const');
-      return {name, kind: 'op', sources, release};
+    }
+
+    const steps = [];
+    order.forEach(name => {
+      if (feeds[name] != null) {
+        steps.push({name, kind: 'feed'});
+      } else if (this.nodes[name].op === 'Const') {
+        steps.push({name, kind: 'const'});
+      } else if (addOf[name] != null) {
+        const add = addOf[name];
+        const other = dataSources(add).filter(srcName => srcName !== name)[0];
+        steps.push({name: add, kind: 'op', conv: name, sources: dataSources(name).concat([other])});
+      } else if (convOf[name] == null) {
+        steps.push({name, kind: 'op', sources: dataSources(name)});
+      }
+    });
+    const lastUse = {};
+    steps.forEach((step, idx) => (step.sources || []).forEach(src => lastUse[src] = idx));
+    steps.forEach((step, idx) => {
+      if (step.kind === 'op') {
+        step.release = Array.from(new Set(step.sources)).filter(
+            src => lastUse[src] === idx && !fetchSet.has(src) && feeds[src] == null &&
+                this.nodes[src].op !== 'Const');
+      }
     });
     return {steps, outputs: fetches.map(n => parseNodeName(n)[0])};
   }

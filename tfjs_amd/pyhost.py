@@ -119,9 +119,9 @@ def batch_matmul(a, b, transpose_a=False, transpose_b=False):
 
 
 def _conv_call(depthwise, x, w, strides, pad, data_format, dilations, dim_rounding_mode, bias, activation,
-               prelu, leakyrelu_alpha):
+               prelu, leakyrelu_alpha, residual=None):
     init()
-    x, w, bias, prelu = _f32(x), _f32(w), _opt(bias), _opt(prelu)
+    x, w, bias, prelu, residual = _f32(x), _f32(w), _opt(bias), _opt(prelu), _opt(residual)
     fmt = "channelsLast" if data_format == "NHWC" else "channelsFirst"
     ci = compute_conv2d_info(x.shape, w.shape, strides, dilations, pad, dim_rounding_mode, depthwise, fmt)
     nchw = fmt == "channelsFirst"
@@ -147,7 +147,12 @@ def _conv_call(depthwise, x, w, strides, pad, data_format, dilations, dim_roundi
         bufs += [dx, dw, dy]
         dbias = DeviceBuffer.from_numpy(bias) if bias is not None else None
         dprelu = DeviceBuffer.from_numpy(prelu) if prelu is not None else None
-        bufs += [b for b in (dbias, dprelu) if b is not None]
+        dres = None
+        if residual is not None:
+            if depthwise or list(residual.shape) != list(out_shape):
+                raise ValueError("residual must have the output's shape %s (FusedConv2D only)" % (out_shape,))
+            dres = DeviceBuffer.from_numpy(residual)
+        bufs += [b for b in (dbias, dprelu, dres) if b is not None]
         common = [ci["batchSize"], ci["inHeight"], ci["inWidth"], ci["inChannels"], ci["filterHeight"],
                   ci["filterWidth"]]
         tail = [ci["strideHeight"], ci["strideWidth"], ci["dilationHeight"], ci["dilationWidth"],
@@ -157,6 +162,9 @@ def _conv_call(depthwise, x, w, strides, pad, data_format, dilations, dim_roundi
         if depthwise:
             check(load_library().tfhip_fused_depthwise_conv2d(
                 dx.ptr, dw.ptr, dy.ptr, *common, w.shape[3], *tail, *epi))
+        elif dres is not None:
+            check(load_library().tfhip_fused_conv2d_add(
+                dx.ptr, dw.ptr, dy.ptr, *common, ci["outChannels"], *tail, int(nchw), *epi, dres.ptr))
         else:
             check(load_library().tfhip_fused_conv2d(
                 dx.ptr, dw.ptr, dy.ptr, *common, ci["outChannels"], *tail, int(nchw), *epi))
@@ -168,9 +176,11 @@ def _conv_call(depthwise, x, w, strides, pad, data_format, dilations, dim_roundi
 
 
 def fused_conv2d(x, w, strides=1, pad="valid", data_format="NHWC", dilations=1, dim_rounding_mode=None,
-                 bias=None, activation="linear", prelu=None, leakyrelu_alpha=0.2):
+                 bias=None, activation="linear", prelu=None, leakyrelu_alpha=0.2, residual=None):
+    """FusedConv2D; with `residual` (a tensor of the output's shape) the Add of a
+    skip connection that follows it, in the same launch."""
     return _conv_call(False, x, w, strides, pad, data_format, dilations, dim_rounding_mode, bias, activation,
-                      prelu, leakyrelu_alpha)
+                      prelu, leakyrelu_alpha, residual)
 
 
 def fused_depthwise_conv2d(x, w, strides=1, pad="valid", dilations=1, dim_rounding_mode=None, bias=None,

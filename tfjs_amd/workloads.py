@@ -225,7 +225,7 @@ class DeviceMobileNetV2:
     load (quantized shard uploaded once, one dequant kernel per tensor) and every
     activation stays in pooled device buffers between kernels."""
 
-    def __init__(self, model_dir, batch):
+    def __init__(self, model_dir, batch, fuse_residual_add=True):
         from . import pyhost
         from .capi import ACTIVATIONS, DeviceBuffer, check, i64_array, load_library
         from .conv_util import compute_conv2d_info
@@ -234,6 +234,8 @@ class DeviceMobileNetV2:
         pyhost.init()
         self.batch = batch
         self.ops, self.shapes = mobilenet_v2_graph()
+        if fuse_residual_add:
+            self.ops = self._fuse_residual_adds(self.ops)
         buf, specs = read_model(model_dir)
         self.weights = pyhost.decode_weights_to_device(buf, specs)   # name -> (DeviceBuffer, shape)
         self.input = DeviceBuffer(batch * 224 * 224 * 3 * 4)
@@ -247,6 +249,8 @@ class DeviceMobileNetV2:
             k = op["kind"]
             src = op["src"]
             if k in ("conv", "dw"):
+                if "residual" in op:
+                    src = src[0]
                 ci = compute_conv2d_info(shape[src], self.shapes[op["w"]], op["stride"], 1, "same", None, k == "dw")
                 shape[op["out"]] = tuple(ci["outShape"])
                 geom = [ci["batchSize"], ci["inHeight"], ci["inWidth"], ci["inChannels"], ci["filterHeight"],
@@ -266,6 +270,28 @@ class DeviceMobileNetV2:
         self.shape, self.last_use = shape, last_use
         self.strides_c = i64_array([0, 0, 0, 1])
         self.zero4 = i64_array([0, 0, 0, 0])
+
+    @staticmethod
+    def _fuse_residual_adds(ops):
+        """A convolution whose only reader is the Add that follows it becomes one op
+        that yields the Add's tensor (what the graph model does at load)."""
+        readers = {}
+        for op in ops:
+            for s in (op["src"] if isinstance(op["src"], tuple) else (op["src"],)):
+                readers[s] = readers.get(s, 0) + 1
+        fused, skip = [], set()
+        for i, op in enumerate(ops):
+            if i in skip:
+                continue
+            nxt = ops[i + 1] if i + 1 < len(ops) else None
+            if (op["kind"] == "conv" and nxt is not None and nxt["kind"] == "add" and op["out"] in nxt["src"]
+                    and readers.get(op["out"]) == 1 and nxt["src"][0] != nxt["src"][1]):
+                other = [s for s in nxt["src"] if s != op["out"]][0]
+                fused.append(dict(op, out=nxt["out"], src=(op["src"], other), residual=other))
+                skip.add(i + 1)
+            else:
+                fused.append(op)
+        return fused
 
     def set_input(self, x):
         self.input.upload(np.ascontiguousarray(x, dtype=np.float32))
@@ -301,7 +327,11 @@ class DeviceMobileNetV2:
             out = DeviceBuffer(n_out * 4)
             if before:
                 before(i, op)
-            if k == "conv":
+            if k == "conv" and "residual" in op:
+                check(lib.tfhip_fused_conv2d_add(t[op["src"][0]].ptr, self.weights[op["w"]][0].ptr, out.ptr, *geom, 0,
+                                                 self.weights[op["b"]][0].ptr, self.strides_c, self._ACT[op["act"]],
+                                                 None, self.zero4, 0.2, t[op["residual"]].ptr))
+            elif k == "conv":
                 check(lib.tfhip_fused_conv2d(t[op["src"]].ptr, self.weights[op["w"]][0].ptr, out.ptr, *geom, 0,
                                              self.weights[op["b"]][0].ptr, self.strides_c, self._ACT[op["act"]],
                                              None, self.zero4, 0.2))
