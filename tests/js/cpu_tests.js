@@ -476,6 +476,62 @@ h.test('graph model: a convolution read by one Add only runs with it as one Fuse
   model.dispose();
 });
 
+h.test('graph model: {recordLaunches: true} runs node by node once, records the second time, replays from then on', () => {
+  const fake = require('./fake_addon');
+  useBackend('hip');
+  const before = tf.memory().numTensors;
+  const model = hip.loadGraphModel({load: () => residualGraphArtifacts()}, {recordLaunches: true}, {decodeWeights: hip.decodeWeights});
+  const x = tf.tensor(new Float32Array(64), [1, 4, 4, 4]), x2 = tf.tensor(new Float32Array(64), [1, 4, 4, 4]);
+  const work = from => fake.calls.slice(from).filter(c => c !== 'alloc' && c !== 'free');
+  let mark = fake.calls.length;
+  model.predict(x).dispose();
+  h.assertEqual(work(mark), ['fusedConv2D', 'fusedConv2D', 'add']);
+  mark = fake.calls.length;
+  const y = model.predict(x);
+  h.assertEqual(work(mark), ['copy', 'captureBegin', 'fusedConv2D', 'fusedConv2D', 'add', 'captureEnd', 'graphLaunch', 'copy']);
+  h.assertEqual(y.shape, [1, 4, 4, 4]);
+  // while recording, buffers go straight to the native allocator: nothing of the recording sits in the free lists here
+  mark = fake.calls.length;
+  model.predict(x).dispose();
+  h.assertEqual(work(mark), ['graphLaunch', 'copy'], 'the same tensor again is not copied in');
+  mark = fake.calls.length;
+  model.predict(x2).dispose();
+  h.assertEqual(work(mark), ['copy', 'graphLaunch', 'copy']);
+  h.assertEqual(fake.lastArgs.graphLaunch, [1]);
+  // another input shape starts over, node by node
+  const wide = tf.tensor(new Float32Array(128), [2, 4, 4, 4]);
+  mark = fake.calls.length;
+  model.predict(wide).dispose();
+  h.assertEqual(work(mark), ['fusedConv2D', 'fusedConv2D', 'add']);
+  // a graph that fails while it is recorded keeps running node by node
+  const broken = hip.loadGraphModel({load: () => residualGraphArtifacts()}, {recordLaunches: true}, {decodeWeights: hip.decodeWeights});
+  broken.predict(x).dispose();
+  const realAdd = fake.add;
+  let fail = true;
+  fake.add = function() {
+    if (fail) {
+      fail = false;
+      throw new Error('not while recording');
+    }
+    return realAdd.apply(this, arguments);
+  };
+  mark = fake.calls.length;
+  broken.predict(x).dispose();
+  fake.add = realAdd;
+  h.assertEqual(work(mark), ['copy', 'captureBegin', 'fusedConv2D', 'fusedConv2D', 'captureEnd', 'fusedConv2D', 'fusedConv2D', 'add']);
+  h.assertEqual(fake.lastArgs.captureEnd, [false]);
+  h.assert(tf.backend().recording === false);
+  mark = fake.calls.length;
+  broken.predict(x).dispose();
+  h.assertEqual(work(mark), ['fusedConv2D', 'fusedConv2D', 'add']);
+  tf.dispose([x, x2, wide, y]);
+  mark = fake.calls.length;
+  model.dispose();
+  broken.dispose();
+  h.assertEqual(work(mark), ['graphDestroy']);
+  h.assertEqual(tf.memory().numTensors, before);
+});
+
 h.test('graph model: unsupported nodes and malformed fused nodes throw the reference errors', () => {
   useBackend('cpu');
   const io = {decodeWeights: oracleDecode.decodeWeights};

@@ -229,6 +229,53 @@ h.test('FusedConv2DAdd: one launch with the bits of FusedConv2D followed by Add;
   h.assertEqual(tf.backend().numDataIds(), before);
 });
 
+h.test('graph model with {recordLaunches: true}: every replay equals the node-by-node result, with other work in between', () => {
+  h.assert(tf.engine().setBackend('hip') === true);
+  const before = tf.backend().numDataIds();
+  const dir = process.env.TFJS_HIP_TEST_MODEL_DIR;
+  const io = {decodeWeights: hip.decodeWeights};
+  const eager = hip.loadGraphModel(dir, {}, io), recorded = hip.loadGraphModel(dir, {recordLaunches: true}, io);
+  const inputs = [3, 4, 5, 6].map(seed => tf.tensor(mobilenet.syntheticInput(2, seed), [2, 224, 224, 3]));
+  const want = inputs.map(x => {
+    const y = eager.predict(x);
+    const v = y.dataSync();
+    y.dispose();
+    return v;
+  });
+  // call 1 runs node by node, call 2 records and replays, the rest replay; inputs alternate and repeat
+  [0, 0, 1, 1, 2, 0, 3, 3, 2].forEach((k, call) => {
+    const y = recorded.predict(inputs[k]);
+    // unrelated work on the same stream and through the same buffer pools between the replays
+    const other = tf.add(inputs[(k + 1) % 4], inputs[(k + 2) % 4]);
+    h.assertBitsEqual(y.dataSync(), want[k], `call ${call}`);
+    tf.dispose([y, other]);
+  });
+  const rec = Array.from(recorded.recordings.values())[0];
+  h.assertEqual(rec.state, 'ready');
+  h.assertEqual(rec.nodes, 54 + 1, 'one node per kernel of the fused plan, two for the split-K classifier');
+  // a result outlives later replays: it is a copy, not the recording's own buffer
+  const first = recorded.predict(inputs[1]);
+  recorded.predict(inputs[2]).dispose();
+  h.assertBitsEqual(first.dataSync(), want[1]);
+  first.dispose();
+  // another batch size gets a recording of its own
+  const one = tf.tensor(mobilenet.syntheticInput(1, 9), [1, 224, 224, 3]);
+  const y1 = eager.predict(one);
+  for (let i = 0; i < 3; i++) {
+    const y = recorded.predict(one);
+    h.assertBitsEqual(y.dataSync(), y1.dataSync());
+    y.dispose();
+  }
+  h.assertEqual(recorded.recordings.size, 2);
+  tf.dispose(inputs);
+  tf.dispose([one, y1]);
+  eager.dispose();
+  recorded.dispose();
+  h.assertEqual(tf.backend().numDataIds(), before, 'recordings, staged inputs and results are all released');
+  const m = tf.memory();
+  h.assert(m.numDeviceBuffers >= 0);
+});
+
 h.test('backend: tensors migrate cpu <-> hip with values and refCounts; tf.time reports device ms', async () => {
   h.assert(tf.engine().setBackend('cpu') === true);
   const a = tf.tensor([1, 2, 3, 4], [2, 2]);

@@ -22,6 +22,13 @@
  * the block again, so a block can be reused at once. The lists are emptied
  * when they hold more than a quarter of the device's memory or when the
  * native allocator reports that it is out of memory.
+ *
+ * beginRecording() .. endRecording() record the kernels enqueued in between
+ * into a HIP graph (tfhip_capture_begin / tfhip_capture_end) instead of running
+ * them; replay(id) then runs the whole sequence with one native call. While
+ * recording, buffers bypass the free lists here, so that the native library
+ * sees every buffer that is released and keeps it for the graph; uploads and
+ * downloads are refused by the native library until the recording ends.
  */
 const tf = require('./core');
 const {addon} = require('./binding');
@@ -50,6 +57,46 @@ class HipBackend extends tf.KernelBackend {
     this.pooledBuffers = 0;
     this.pooledBytes = 0;
     this.poolLimitBytes = this.deviceInfo.hbmBytes / 4;
+    this.recording = false;
+  }
+
+  /** Kernels enqueued from now on are recorded, not run. */
+  beginRecording() {
+    if (this.recording) {
+      throw new Error('tfjs-backend-hip: a recording is already open');
+    }
+    addon.captureBegin();
+    this.recording = true;
+  }
+
+  /** Ends the recording: {id, nodes} of the graph, or id 0 when keep is false. */
+  endRecording(keep) {
+    if (!this.recording) {
+      throw new Error('tfjs-backend-hip: no recording is open');
+    }
+    this.recording = false;
+    return addon.captureEnd(keep !== false);
+  }
+
+  /** Runs a recorded graph once more, on the addresses it was recorded with. */
+  replay(id) {
+    addon.graphLaunch(id);
+  }
+
+  deleteRecording(id) {
+    addon.graphDestroy(id);
+  }
+
+  /** Device-to-device copy between the buffers of two dataIds of the same size. */
+  copyData(dstDataId, srcDataId) {
+    const dst = this.data.get(dstDataId), src = this.data.get(srcDataId);
+    if (dst.bytes !== src.bytes) {
+      throw new Error(`tfjs-backend-hip: copy of ${src.bytes} bytes into a tensor of ${dst.bytes} bytes`);
+    }
+    if (src.bytes > 0) {
+      // buffers come in multiples of 256 bytes: the copy kernel's 16-byte units may run past the tensor
+      addon.copy(dst.ptr, src.ptr, Math.ceil(src.bytes / 16) * 16);
+    }
   }
 
   /** Returns every pooled buffer to the native allocator. */
@@ -61,7 +108,7 @@ class HipBackend extends tf.KernelBackend {
   }
 
   acquire(bytes) {
-    const list = this.freeLists.get(bytes);
+    const list = this.recording ? undefined : this.freeLists.get(bytes);
     if (list !== undefined && list.length > 0) {
       this.pooledBuffers--;
       this.pooledBytes -= bytes;
@@ -79,6 +126,10 @@ class HipBackend extends tf.KernelBackend {
   }
 
   release(ptr, bytes) {
+    if (this.recording) {
+      addon.free(ptr);   // the native library keeps it for the graph being recorded
+      return;
+    }
     if (this.pooledBytes + bytes > this.poolLimitBytes) {
       this.releasePool();
       addon.free(ptr);
@@ -242,6 +293,9 @@ class HipBackend extends tf.KernelBackend {
   }
 
   dispose() {
+    if (this.recording) {
+      this.endRecording(false);
+    }
     this.releasePool();
     addon.shutdown();
   }

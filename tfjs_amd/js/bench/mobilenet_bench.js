@@ -2,9 +2,11 @@
 /**
  * MobileNetV2 through the tfjs API on the hip backend, timed the reference's way
  * (predict plus download of the result, e2e/benchmarks/benchmark_util.js:246-286).
- *   node tfjs_amd/js/bench/mobilenet_bench.js MODEL_DIR BATCH STEPS WARMUP [PRIME]
+ *   node tfjs_amd/js/bench/mobilenet_bench.js MODEL_DIR BATCH STEPS WARMUP [PRIME [RECORD]]
  * PRIME (default 0) batch-1 inferences run first, outside warm-up and timing, so
- * that V8 has compiled the host path before a short measurement starts.
+ * that V8 has compiled the host path before a short measurement starts. RECORD 1
+ * loads the graph model with {recordLaunches: true}: the kernels of an inference
+ * are recorded into a HIP graph once and replayed from then on.
  * Prints one JSON line: ms_per_step (wall clock around STEPS steps, stream
  * drained on both sides), load_ms (read + upload + GPU dequant of the weights),
  * kernel_ms_per_step (device time between two events around the same steps).
@@ -23,6 +25,7 @@ async function main() {
   const steps = parseInt(process.argv[4] || '50', 10);
   const warmup = parseInt(process.argv[5] || '5', 10);
   const prime = parseInt(process.argv[6] || '0', 10);
+  const record = parseInt(process.argv[7] || '0', 10) === 1;
   await tf.setBackend('hip');
   const t0 = tf.util.now();
   // A converter-format model.json runs as a graph model (model.predict, what a
@@ -31,7 +34,7 @@ async function main() {
   const asGraph = fs.existsSync(path.join(modelDir, 'model.json'));
   let predict;
   if (asGraph) {
-    const graph = hip.loadGraphModel(modelDir, {}, {decodeWeights: hip.decodeWeights});
+    const graph = hip.loadGraphModel(modelDir, {recordLaunches: record}, {decodeWeights: hip.decodeWeights});
     predict = x => graph.predict(x);
   } else {
     const m = model.readModel(modelDir);
@@ -81,6 +84,7 @@ async function main() {
     steps,
     warmup,
     prime,
+    record_launches: record && asGraph,
     checksum,
     node: process.version,
     core: tf.usingStandin ? 'standin' : '@tensorflow/tfjs-core',

@@ -21,7 +21,7 @@ const kernelConfigs = [
   matmul.fusedMatMulConfig, matmul.batchMatMulConfig, conv.fusedConv2DConfig,
   conv.fusedConv2DAddConfig, conv.conv2DConfig, conv.fusedDepthwiseConv2DConfig,
   conv.depthwiseConv2dNativeConfig, glue.addConfig, glue.meanConfig,
-  glue.reshapeConfig, glue.identityConfig
+  glue.reshapeConfig, glue.identityConfig, glue.copyConfig
 ];
 
 tf.registerBackend('hip', () => new HipBackend(), 3 /* priority */);

@@ -4,7 +4,9 @@
  * leaves the device mid-graph: Add (tfjs-backend-cpu/src/kernels/Add.ts),
  * Mean over the two spatial axes (Mean.ts:26-56 over Sum.ts:30-92), and the
  * aliasing Reshape / Identity (Reshape.ts:24-52, Identity.ts:22-30), which
- * share the input's buffer and bump its refCount.
+ * share the input's buffer and bump its refCount. HipCopy (no counterpart in
+ * the reference) duplicates a tensor on the device: what moves inputs into and
+ * results out of the fixed buffers of a recorded launch sequence.
  */
 const tf = require('../core');
 const {broadcastStrides, requireFloat32, addon} = require('./fused_util');
@@ -77,7 +79,16 @@ function identity(args) {
   return {dataId: x.dataId, shape: x.shape, dtype: x.dtype};
 }
 
+/** A copy of x in a buffer of its own (device to device). */
+function copy(args) {
+  const {x} = args.inputs;
+  const out = args.backend.makeOutput(x.shape, x.dtype);
+  args.backend.copyData(out.dataId, x.dataId);
+  return out;
+}
+
 module.exports = {
+  copyConfig: {kernelName: 'HipCopy', backendName: 'hip', kernelFunc: copy},
   addConfig: {kernelName: 'Add', backendName: 'hip', kernelFunc: add},
   meanConfig: {kernelName: 'Mean', backendName: 'hip', kernelFunc: mean},
   reshapeConfig: {kernelName: 'Reshape', backendName: 'hip', kernelFunc: reshape},

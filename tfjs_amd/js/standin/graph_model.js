@@ -24,6 +24,16 @@
  * result has the bits of the two separate kernels; {fuseResidualAdd: false} in
  * the load options turns it off.
  *
+ * And with {recordLaunches: true} in the load options, on a backend that can
+ * record (beginRecording / endRecording / replay, as the hip backend has), the
+ * kernels of one execution are recorded into a device-side graph the second time
+ * the model runs with inputs of a given shape, and every later execution with
+ * that shape replays the graph: one native call instead of one per node, which is
+ * what a small batch is bound by. The inputs are copied into buffers the recording
+ * owns (skipped while the same tensor is passed again), the results are copied
+ * out of them, so tensors keep their value semantics. A graph whose execution
+ * reads tensor values on the host cannot be recorded and keeps running node by node.
+ *
  * Where @tensorflow/tfjs-converter is installed, use its GraphModel instead; the
  * backend and the injected decodeWeights are the same.
  */
@@ -315,6 +325,7 @@ class GraphModel {
     this.nodes = {};
     this.compiled = {};
     this.plans = new Map();
+    this.recordings = new Map();
     this.order = [];
     (graph.node || []).forEach(node => {
       this.nodes[node.name] = node;
@@ -424,6 +435,14 @@ class GraphModel {
       compiled = this.makePlan(feeds, fetches);
       this.plans.set(planKey, compiled);
     }
+    if (this.loadOptions.recordLaunches === true && typeof tf.backend().beginRecording === 'function') {
+      return this.executeRecorded(planKey, compiled, feeds);
+    }
+    return this.runPlan(compiled, feeds);
+  }
+
+  /** Executes the steps of a plan node by node. */
+  runPlan(compiled, feeds) {
     const {steps, outputs: outNames} = compiled;
 
     return tf.tidy(() => {
@@ -464,6 +483,65 @@ class GraphModel {
       const result = outNames.map(n => values[n]);
       return result.length > 1 ? result : result[0];
     });
+  }
+
+  /**
+   * Execution through a recorded launch sequence: node by node the first time a
+   * combination of input shapes is seen (that run also fills the caches a
+   * recording must not touch), recorded and replayed the second time, replayed
+   * from then on.
+   */
+  executeRecorded(planKey, compiled, feeds) {
+    const backend = tf.backend();
+    const names = Object.keys(feeds);
+    const key = planKey + '|' + names.map(n => `${feeds[n].dtype}[${feeds[n].shape}]`).join(';');
+    let rec = this.recordings.get(key);
+    if (rec === undefined) {
+      this.recordings.set(key, {state: 'seen'});
+      return this.runPlan(compiled, feeds);
+    }
+    if (rec.state === 'unrecordable') {
+      return this.runPlan(compiled, feeds);
+    }
+    if (rec.state === 'seen') {
+      const staged = {}, stagedFrom = {};
+      names.forEach(n => {
+        staged[n] = tf.keep(tf.engine().runKernel('HipCopy', {x: feeds[n]}));
+        stagedFrom[n] = feeds[n].dataId;
+      });
+      let outputs = null, graph = null;
+      backend.beginRecording();
+      try {
+        outputs = this.runPlan(compiled, staged);
+        graph = backend.endRecording(true);
+      } catch (e) {
+        if (backend.recording) {
+          backend.endRecording(false);
+        }
+        tf.dispose(staged);
+        if (outputs != null) {
+          tf.dispose(outputs);
+        }
+        rec.state = 'unrecordable';
+        rec.reason = e.message;
+        return this.runPlan(compiled, feeds);
+      }
+      outputs = Array.isArray(outputs) ? outputs : [outputs];
+      outputs.forEach(t => tf.keep(t));
+      rec = {state: 'ready', id: graph.id, nodes: graph.nodes, staged, stagedFrom, outputs,
+             single: compiled.outputs.length === 1};
+      this.recordings.set(key, rec);
+    }
+    names.forEach(n => {
+      // a tensor's values never change: the same dataId again needs no copy
+      if (feeds[n].dataId !== rec.stagedFrom[n]) {
+        backend.copyData(rec.staged[n].dataId, feeds[n].dataId);
+        rec.stagedFrom[n] = feeds[n].dataId;
+      }
+    });
+    backend.replay(rec.id);
+    const results = rec.outputs.map(t => tf.engine().runKernel('HipCopy', {x: t}));
+    return rec.single ? results[0] : results;
   }
 
   /**
@@ -565,6 +643,16 @@ class GraphModel {
   }
 
   dispose() {
+    if (this.recordings != null) {
+      this.recordings.forEach(rec => {
+        if (rec.state === 'ready') {
+          tf.backend().deleteRecording(rec.id);
+          tf.dispose(rec.staged);
+          tf.dispose(rec.outputs);
+        }
+      });
+      this.recordings.clear();
+    }
     if (this.weightMap != null) {
       Object.keys(this.weightMap).forEach(k => this.weightMap[k].dispose());
       this.weightMap = null;
