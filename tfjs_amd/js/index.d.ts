@@ -38,6 +38,24 @@ export declare class HipBackend extends KernelBackend {
   makeOutput(shape: number[], dtype: DataType): TensorInfo;
   /** Device pointer of a tensor's storage, as the addon takes it. */
   ptr(dataId: DataId): number;
+  /** Device-to-device copy between two tensors of the same byte size. */
+  copyData(dst: DataId, src: DataId): void;
+  /** Kernels enqueued until endRecording() are recorded into a HIP graph, not run. */
+  beginRecording(): void;
+  /** keep === false discards the recording (id 0). */
+  endRecording(keep?: boolean): {id: number, nodes: number};
+  /** Runs a recorded graph again, on the device addresses it was recorded with. */
+  replay(id: number): void;
+  deleteRecording(id: number): void;
+  readonly recording: boolean;
+}
+
+/** Load options of the stand-in graph model beyond the reference's. */
+export interface HipGraphModelOptions {
+  /** default true: a _FusedConv2D read by one Add/AddV2 only runs with it as one FusedConv2DAdd kernel */
+  fuseResidualAdd?: boolean;
+  /** default false: record the kernels of an execution into a HIP graph and replay it for the same input shapes */
+  recordLaunches?: boolean;
 }
 
 /** decodeWeights with the dequantize step on the GPU; inject as GraphModel's tfio. */
@@ -55,7 +73,7 @@ export interface ModelArtifactsHandler {
   load(): object | Promise<object>;
 }
 export declare class GraphModel {
-  constructor(handlerOrPath: string | ModelArtifactsHandler, loadOptions?: object, tfio?: IoWithDecodeWeights);
+  constructor(handlerOrPath: string | ModelArtifactsHandler, loadOptions?: HipGraphModelOptions, tfio?: IoWithDecodeWeights);
   load(): boolean | Promise<boolean>;
   predict(inputs: Tensor | Tensor[] | {[name: string]: Tensor}, config?: object): Tensor | Tensor[];
   execute(inputs: Tensor | Tensor[] | {[name: string]: Tensor}, outputs?: string | string[]): Tensor | Tensor[];
@@ -65,5 +83,5 @@ export declare class GraphModel {
   readonly weights: {[name: string]: Tensor};
 }
 export declare function loadGraphModel(
-    modelUrl: string | ModelArtifactsHandler, options?: object, tfio?: IoWithDecodeWeights): GraphModel | Promise<GraphModel>;
+    modelUrl: string | ModelArtifactsHandler, options?: HipGraphModelOptions, tfio?: IoWithDecodeWeights): GraphModel | Promise<GraphModel>;
 export declare function fileSystem(path: string): ModelArtifactsHandler;
