@@ -49,21 +49,22 @@ BATCH = 32
 # cannot be read from inside this script, so the table is refreshed by hand when a
 # kernel changes; a symbol that is not listed reports null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "conv_few_taps<7, 2>": 75275220,
-    "depthwise_3x3_rows<1, false>": 63563214,
-    "skinny_gemm_regs<1, 2, false>": 77134479,
-    "skinny_gemm_regs<6, 1, false>": 180984829,
-    "depthwise_3x3_rows<2, false>": 156009789,
-    "skinny_gemm<2, 4>": 58521445,
-    "skinny_gemm_regs<3, 1, true>": 74859784,
-    "add_same_shape": 8330153,
-    "gemm_kernel<32, 32, 32, 2, 2, 0, 1>": 16139742,
-    "gemm_kernel<64, 64, 16, 2, 2, 0, 1>": 18563146,
-    "depthwise_3x3_flat<2, false>": 22006204,
-    "depthwise_3x3_flat<1, false>": 17923346,
-    "gemm_kernel<32, 64, 32, 2, 2, 0, 1>": 12331211,
-    "mean_hw_vec": 8295707,
-    "gemm_finish": 890299,
+    "conv_few_taps<7, 2>": 75272113,
+    "depthwise_3x3_rows<1, false>": 63685042,
+    "skinny_gemm_regs<1, 2, false>": 77140496,
+    "skinny_gemm_regs<6, 1, false>": 180978783,
+    "depthwise_3x3_rows<2, false>": 156010500,
+    "skinny_gemm<2, 4>": 64076321,
+    "skinny_gemm_regs<3, 1, true>": 75048140,
+    "gemm_kernel<32, 32, 32, 2, 2, 0, 1>": 17343831,
+    "small_k_gemm<64, 2, 2, 16>": 29245333,
+    "depthwise_3x3_flat<2, false>": 22006171,
+    "small_k_gemm<32, 2, 2, 16>": 19741783,
+    "depthwise_3x3_flat<1, false>": 17923334,
+    "gemm_kernel<64, 64, 16, 2, 2, 0, 1>": 20597758,
+    "gemm_kernel<32, 64, 32, 2, 2, 0, 1>": 12344502,
+    "mean_hw_vec": 8295726,
+    "gemm_finish": 896441,
     "copy_to_host": 277490,
 }
 

@@ -205,6 +205,35 @@ int tfhip_fused_depthwise_conv2d(
     const float *prelu_weights, const int64_t prelu_strides[4],
     double leakyrelu_alpha);
 
+/* ---- pointwise + depthwise convolution in one launch ---------------------------
+ * y = dw_act(depthwise3x3(pw_act(conv1x1(x, pw_filter) + pw_bias), dw_filter) + dw_bias):
+ * the expansion and the depthwise stage of an inverted-residual block without the
+ * expanded tensor ever reaching memory. In a graph this is a FusedConv2D node with
+ * a 1x1 filter, stride 1 (convolution_executor.ts:100-137) whose only consumer is a
+ * FusedDepthwiseConv2dNative node with a 3x3 filter, channel multiplier 1, dilation
+ * 1 (convolution_executor.ts:139-173). Every intermediate value is rounded as the
+ * two separate kernels round it (the result equals tfhip_fused_conv2d followed by
+ * tfhip_fused_depthwise_conv2d). NHWC; x is [batch,in_h,in_w,in_c], pw_filter
+ * [in_c,mid_c], dw_filter [3,3,mid_c], biases [mid_c] or NULL, y
+ * [batch,out_h,out_w,mid_c]; stride, pad_top, pad_left, out_h, out_w are those of
+ * the depthwise stage; both activations relu or both relu6.
+ * The fused kernel takes in_c 8 / 16 / 24 / 32, mid_c a multiple of 16 up to
+ * 256, stride 1 or 2; for any other shape or activation pair
+ * tfhip_fused_pointwise_depthwise fails and the caller runs the two
+ * convolutions. tfhip_pointwise_depthwise_pays returns 1 when the kernel takes
+ * the shape AND is expected to be faster than the two (an expanded tensor large
+ * enough that writing and re-reading it is what the pair costs): what a graph
+ * executor asks before it fuses the two nodes. */
+int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_filter,
+                                    const float *pw_bias, int pw_activation,
+                                    const float *dw_filter, const float *dw_bias,
+                                    int dw_activation, float *y, int64_t batch,
+                                    int64_t in_h, int64_t in_w, int64_t in_c,
+                                    int64_t mid_c, int64_t stride, int64_t pad_top,
+                                    int64_t pad_left, int64_t out_h, int64_t out_w);
+int tfhip_pointwise_depthwise_pays(int64_t batch, int64_t in_c, int64_t mid_c,
+                                        int64_t stride, int64_t out_h, int64_t out_w);
+
 /* ---- weight dequantisation on load -----------------------------------------
  * The quantization branch of decodeWeight, tfjs-core/src/io/io_utils.ts:196-251,
  * which the reference runs in JavaScript before backend.write(). `q` points at

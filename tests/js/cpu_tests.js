@@ -476,6 +476,78 @@ h.test('graph model: a convolution read by one Add only runs with it as one Fuse
   model.dispose();
 });
 
+function blockGraphArtifacts() {
+  // an inverted-residual block: x -> expand 1x1 (relu6) -> depthwise 3x3 (relu6) -> project 1x1 -> AddV2(x, .) -> Identity
+  const fused = (ops, extra) => Object.assign({
+    fused_ops: {list: {s: ops.map(b64)}}, num_args: {i: '1'}, leakyrelu_alpha: {f: 0.2},
+    strides: {list: {i: ['1', '1', '1', '1']}}, dilations: {list: {i: ['1', '1', '1', '1']}},
+    padding: {s: b64('SAME')}, data_format: {s: b64('NHWC')}, explicit_paddings: {list: {}}}, extra || {});
+  const node = (name, op, input, attr) => ({name, op, input, attr: attr || {}});
+  const nodes = [
+    node('x', 'Placeholder', [], {dtype: {type: 'DT_FLOAT'}, shape: {shape: {dim: [{size: '-1'}, {size: '6'}, {size: '6'}, {size: '8'}]}}}),
+    node('e/w', 'Const'), node('e/b', 'Const'), node('d/w', 'Const'), node('d/b', 'Const'), node('p/w', 'Const'), node('p/b', 'Const'),
+    node('e', '_FusedConv2D', ['x', 'e/w', 'e/b'], fused(['BiasAdd', 'Relu6'])),
+    node('d', 'FusedDepthwiseConv2dNative', ['e', 'd/w', 'd/b'], fused(['BiasAdd', 'Relu6'], {strides: {list: {i: ['1', '2', '2', '1']}}})),
+    node('p', '_FusedConv2D', ['d', 'p/w', 'p/b'], fused(['BiasAdd'])),
+    node('out', 'Identity', ['p'])
+  ];
+  const shapes = {'e/w': [1, 1, 8, 16], 'e/b': [16], 'd/w': [3, 3, 16, 1], 'd/b': [16], 'p/w': [1, 1, 16, 8], 'p/b': [8]};
+  const specs = [], chunks = [];
+  Object.keys(shapes).forEach(name => {
+    const n = shapes[name].reduce((a, b) => a * b, 1);
+    specs.push({name, shape: shapes[name], dtype: 'float32'});
+    chunks.push(Buffer.from(Float32Array.from({length: n}, (_, i) => Math.sin(i + n)).buffer));
+  });
+  const all = Buffer.concat(chunks);
+  return {modelTopology: {node: nodes, versions: {producer: 1, minConsumer: 0}}, weightSpecs: specs,
+          weightData: all.buffer.slice(all.byteOffset, all.byteOffset + all.byteLength)};
+}
+
+h.test('graph model: a 1x1 convolution read by one 3x3 depthwise convolution only is one step; the kernel picks one launch or two', () => {
+  const fake = require('./fake_addon');
+  useBackend('hip');
+  const before = tf.memory().numTensors;
+  const io = {decodeWeights: hip.decodeWeights};
+  const model = hip.loadGraphModel({load: () => blockGraphArtifacts()}, {}, io);
+  const x1 = tf.tensor(new Float32Array(6 * 6 * 8), [1, 6, 6, 8]), x4 = tf.tensor(new Float32Array(4 * 6 * 6 * 8), [4, 6, 6, 8]);
+  const work = from => fake.calls.slice(from).filter(c => c !== 'alloc' && c !== 'free');
+  fake.paysFromBatch = 4;
+  let mark = fake.calls.length;
+  const y1 = model.predict(x1);
+  const ops = Array.from(model.plans.values())[0].steps.filter(s => s.kind === 'op');
+  h.assertEqual(ops.map(s => [s.name, s.pointwise]), [['d', 'e'], ['p', undefined], ['out', undefined]]);
+  h.assertEqual(ops[0].sources, ['x', 'e/w', 'e/b', 'd/w', 'd/b']);
+  // one image: the native library says the fused kernel does not pay, the kernel runs the two convolutions
+  h.assertEqual(work(mark), ['fusedConv2D', 'fusedDepthwiseConv2D', 'fusedConv2D']);
+  h.assertEqual(y1.shape, [1, 3, 3, 8]);
+  mark = fake.calls.length;
+  const live = tf.memory().numTensors;
+  const y4 = model.predict(x4);
+  h.assertEqual(work(mark), ['fusedPointwiseDepthwise', 'fusedConv2D']);
+  h.assertEqual(tf.memory().numTensors, live + 1);
+  // geometry of the depthwise stage: batch, inH, inW, inC, midC, stride, padTop, padLeft, outH, outW; relu6 for both stages
+  h.assertEqual(fake.lastArgs.fusedPointwiseDepthwise[8], [4, 6, 6, 8, 16, 2, 0, 0, 3, 3]);
+  h.assertEqual([fake.lastArgs.fusedPointwiseDepthwise[3], fake.lastArgs.fusedPointwiseDepthwise[6]], [2, 2]);
+  h.assertEqual(y4.shape, [4, 3, 3, 8]);
+  // switched off: the graph's own nodes
+  const plain = hip.loadGraphModel({load: () => blockGraphArtifacts()}, {fusePointwiseDepthwise: false}, io);
+  mark = fake.calls.length;
+  plain.predict(x4).dispose();
+  h.assertEqual(work(mark), ['fusedConv2D', 'fusedDepthwiseConv2D', 'fusedConv2D']);
+  // a pair with different activations stays two steps
+  const mixed = blockGraphArtifacts();
+  mixed.modelTopology.node.find(nd => nd.name === 'd').attr.fused_ops = {list: {s: ['BiasAdd', 'Relu'].map(b64)}};
+  const other = hip.loadGraphModel({load: () => mixed}, {}, io);
+  other.predict(x4).dispose();
+  h.assert(Array.from(other.plans.values())[0].steps.every(s => s.pointwise == null));
+  fake.paysFromBatch = null;
+  tf.dispose([x1, x4, y1, y4]);
+  model.dispose();
+  plain.dispose();
+  other.dispose();
+  h.assertEqual(tf.memory().numTensors, before);
+});
+
 h.test('graph model: {recordLaunches: true} runs node by node once, records the second time, replays from then on', () => {
   const fake = require('./fake_addon');
   useBackend('hip');

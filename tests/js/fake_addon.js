@@ -65,6 +65,9 @@ module.exports = {
   dequantF16() { record('dequantF16', arguments); },
   add() { record('add', arguments); },
   meanHW() { record('meanHW', arguments); },
+  fusedPointwiseDepthwise() { record('fusedPointwiseDepthwise', arguments); },
+  pointwiseDepthwisePays(batch) { return module.exports.paysFromBatch != null && batch >= module.exports.paysFromBatch; },
+  paysFromBatch: null,   // tests set the batch size from which the fused kernel "pays"
   copy() { record('copy', arguments); },
   captureBegin() { record('captureBegin', arguments); },
   captureEnd(keep) { record('captureEnd', arguments); return {id: keep ? 1 : 0, nodes: 0}; },

@@ -229,6 +229,44 @@ h.test('FusedConv2DAdd: one launch with the bits of FusedConv2D followed by Add;
   h.assertEqual(tf.backend().numDataIds(), before);
 });
 
+h.test('FusedPointwiseDepthwiseConv2D: expansion + depthwise stage in one launch, the bits of the two kernels; used by the graph model at batch 32', () => {
+  h.assert(tf.engine().setBackend('hip') === true);
+  const before = tf.backend().numDataIds();
+  let seed = 11;
+  const rnd = n => Float32Array.from({length: n}, () => ((seed = (Math.imul(seed, 1664525) + 1013904223) >>> 0) / 2 ** 32) - 0.5);
+  const addon = require('../../tfjs_amd/js/binding').addon;
+  // [batch, size, inC, midC, stride]: the first two are shapes the native library fuses, the third it does not
+  [[32, 112, 16, 96, 2], [32, 56, 24, 144, 2], [2, 20, 16, 32, 1]].forEach(([n, size, cin, mid, stride]) => {
+    const x = tf.tensor(rnd(n * size * size * cin), [n, size, size, cin]);
+    const filter = tf.tensor(rnd(cin * mid), [1, 1, cin, mid]), bias = tf.tensor(rnd(mid), [mid]);
+    const dwFilter = tf.tensor(rnd(9 * mid), [3, 3, mid, 1]), dwBias = tf.tensor(rnd(mid), [mid]);
+    const out = Math.ceil(size / stride);
+    h.assertEqual(addon.pointwiseDepthwisePays(n, cin, mid, stride, out, out), n === 32);
+    const fused = tf.engine().runKernel('FusedPointwiseDepthwiseConv2D', {x, filter, bias, dwFilter, dwBias},
+                                        {strides: [stride, stride], pad: 'same', activation: 'relu6'});
+    h.assertEqual(addon.lastKernel().startsWith('expand_dw_3x3'), n === 32);
+    const expanded = tf.fused.conv2d({x, filter, strides: [1, 1], pad: 'valid', dataFormat: 'NHWC', dilations: [1, 1], bias, activation: 'relu6'});
+    const two = tf.fused.depthwiseConv2d({x: expanded, filter: dwFilter, strides: [stride, stride], pad: 'same', dataFormat: 'NHWC',
+                                          dilations: [1, 1], bias: dwBias, activation: 'relu6'});
+    h.assertEqual(fused.shape, two.shape);
+    h.assertBitsEqual(fused.dataSync(), two.dataSync());
+    tf.dispose([x, filter, bias, dwFilter, dwBias, fused, expanded, two]);
+  });
+  h.assertEqual(tf.backend().numDataIds(), before);
+  const dir = process.env.TFJS_HIP_TEST_MODEL_DIR;
+  const io = {decodeWeights: hip.decodeWeights};
+  const fusedModel = hip.loadGraphModel(dir, {}, io), plainModel = hip.loadGraphModel(dir, {fusePointwiseDepthwise: false}, io);
+  const x = tf.tensor(mobilenet.syntheticInput(32, 7), [32, 224, 224, 3]);
+  const a = fusedModel.predict(x), b = plainModel.predict(x);
+  const steps = model => Array.from(model.plans.values())[0].steps.filter(s => s.kind === 'op');
+  h.assertEqual(steps(plainModel).length - steps(fusedModel).length, 16, 'every expansion but the first block, which has none');
+  h.assertBitsEqual(a.dataSync(), b.dataSync());
+  tf.dispose([a, b, x]);
+  fusedModel.dispose();
+  plainModel.dispose();
+  h.assertEqual(tf.backend().numDataIds(), before);
+});
+
 h.test('graph model with {recordLaunches: true}: every replay equals the node-by-node result, with other work in between', () => {
   h.assert(tf.engine().setBackend('hip') === true);
   const before = tf.backend().numDataIds();

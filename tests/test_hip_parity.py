@@ -580,6 +580,73 @@ def test_conv2d_residual_is_checked(hip):
         assert b"same buffer" in lib.tfhip_last_error()
 
 
+# ---------------------------------- pointwise + depthwise convolution in one launch
+
+PW_DW_CASES = [
+    # batch, h, w, in_c, mid_c, stride, pad, activations
+    (6, 112, 112, 16, 96, 2, "same", "relu6", "relu6"),     # MobileNetV2's first expansion: halo on every side of a tile
+    (22, 56, 56, 24, 144, 1, "same", "relu6", "relu6"),     # K = 24: one full k group and a half one
+    (2, 56, 56, 24, 144, 2, "same", "relu6", "relu6"),
+    (2, 28, 28, 32, 192, 1, "same", "relu6", "relu6"),      # K = 32: two k groups
+    (2, 28, 28, 32, 192, 2, "same", "relu", "relu"),
+    (1, 9, 23, 8, 16, 1, "valid", "relu6", "relu6"),        # K = 8, one channel block, ragged tiles, no padding
+    (2, 17, 31, 16, 48, 2, "same", "relu", "relu"),         # odd sizes: partial last tile and row chunk
+    (1, 5, 5, 16, 256, 1, [[0, 0], [2, 0], [1, 2], [0, 0]], "relu6", "relu6"),   # explicit, lopsided padding; widest channel count
+    (40, 20, 14, 24, 64, 1, "same", "relu6", "relu6"),      # many images: several row chunks per image are not needed
+]
+
+
+@pytest.mark.parametrize("case", PW_DW_CASES, ids=[str(i) for i in range(len(PW_DW_CASES))])
+def test_pointwise_depthwise_fused(hip, orc, case):
+    from tfjs_amd import capi
+    n, h, w, cin, mid, stride, pad, act1, act2 = case
+    rng = np.random.default_rng(n * 131 + h + w + cin + mid)
+    x = rng.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    w1 = rng.normal(0, 0.5, (1, 1, cin, mid)).astype(np.float32)
+    b1 = rng.uniform(-1, 2, (mid,)).astype(np.float32)       # positive: relu6(bias) is far from the zero padding
+    w2 = rng.normal(0, 0.5, (3, 3, mid, 1)).astype(np.float32)
+    b2 = rng.uniform(-1, 1, (mid,)).astype(np.float32)
+    got = hip.fused_pointwise_depthwise(x, w1, w2, strides=stride, pad=pad, pw_bias=b1, pw_activation=act1,
+                                        dw_bias=b2, dw_activation=act2)
+    mid_hip = hip.fused_conv2d(x, w1, bias=b1, activation=act1)
+    name = ctypes.create_string_buffer(256)
+    capi.load_library().tfhip_last_kernel(name, 256)
+    two = hip.fused_depthwise_conv2d(mid_hip, w2, strides=stride, pad=pad, bias=b2, activation=act2)
+    want = orc.fused_depthwise_conv2d(orc.fused_conv2d(x, w1, bias=b1, activation=act1), w2, strides=stride, pad=pad,
+                                      bias=b2, activation=act2)
+    assert_parity(got, want)
+    # where the separate expansion is the streaming kernel whose instruction order the fused one keeps
+    # (the large layers: that is where the fusion is used), the two launches give the same bits
+    if name.value.decode().startswith("skinny_gemm_regs"):
+        np.testing.assert_array_equal(got.view(np.uint32), two.view(np.uint32))
+    else:
+        assert_parity(got, two, 1e-5)
+
+
+def test_pointwise_depthwise_without_biases_and_unsupported_shapes(hip, orc):
+    from tfjs_amd import capi
+    rng = np.random.default_rng(77)
+    x = rng.uniform(-1, 1, (2, 12, 12, 16)).astype(np.float32)
+    w1 = rng.normal(0, 0.5, (1, 1, 16, 32)).astype(np.float32)
+    w2 = rng.normal(0, 0.5, (3, 3, 32, 1)).astype(np.float32)
+    got = hip.fused_pointwise_depthwise(x, w1, w2, strides=1, pad="same", pw_activation="relu", dw_activation="relu")
+    assert_parity(got, orc.fused_depthwise_conv2d(orc.fused_conv2d(x, w1, activation="relu"), w2, pad="same",
+                                                  activation="relu"))
+    with pytest.raises(capi.HipBackendError, match="run the two convolutions"):   # a pair of activations it does not take
+        hip.fused_pointwise_depthwise(x, w1, w2, pw_activation="relu6", dw_activation="linear")
+    lib = capi.load_library()
+    assert lib.tfhip_pointwise_depthwise_pays(32, 16, 96, 2, 56, 56) == 1
+    assert lib.tfhip_pointwise_depthwise_pays(32, 24, 144, 2, 28, 28) == 1
+    assert lib.tfhip_pointwise_depthwise_pays(32, 32, 192, 1, 28, 28) == 0     # taken, but the two kernels are faster
+    assert lib.tfhip_pointwise_depthwise_pays(1, 16, 96, 2, 56, 56) == 0       # one image: the expanded tensor is small
+    assert lib.tfhip_pointwise_depthwise_pays(32, 64, 384, 1, 14, 14) == 0     # too many input channels
+    assert lib.tfhip_pointwise_depthwise_pays(64, 16, 40, 2, 112, 112) == 0    # channels no multiple of 16
+    assert lib.tfhip_pointwise_depthwise_pays(64, 16, 96, 3, 112, 112) == 0    # stride 3
+    with pytest.raises(capi.HipBackendError, match="run the two convolutions"):
+        hip.fused_pointwise_depthwise(rng.uniform(-1, 1, (1, 8, 8, 12)).astype(np.float32),
+                                      rng.normal(0, 1, (1, 1, 12, 32)).astype(np.float32), w2)
+
+
 # -------------------------------------------------- recorded launch sequences
 
 def test_recorded_graph_replays(hip, orc):
@@ -689,13 +756,27 @@ def test_config4_mobilenet_v2_batch1_vs_oracle(hip, orc, tmp_path):
         assert sum(1 for op, _ in model.plan if "residual" in op) == 10
     finally:
         model.close()
-    # the ten skip connections as Add kernels of their own: the same bits
-    plain = workloads.DeviceMobileNetV2(str(tmp_path), 2, fuse_residual_add=False)
+    # the ten skip connections as Add kernels of their own, expansions and depthwise stages as two kernels
+    plain = workloads.DeviceMobileNetV2(str(tmp_path), 2, fuse_residual_add=False, fuse_expand_depthwise=False)
     try:
-        assert len(plain.plan) == len(model.plan) + 10
+        fused_pairs = sum(1 for op, _ in model.plan if op["kind"] == "pwdw")   # none at this small batch
+        assert len(plain.plan) == len(model.plan) + 10 + fused_pairs
         plain.set_input(x)
-        np.testing.assert_array_equal(plain.predict(), got)
+        # (at this small batch the separate expansions run on the tiled kernel, whose k order differs)
+        assert_parity(plain.predict(), got, 1e-4)
     finally:
         plain.close()
+    # at batch 32 the first expansions run fused with their depthwise stage: the same bits as the separate kernels
+    x32 = workloads.mobilenet_v2_input(32)
+    outs = []
+    for fuse in (True, False):
+        m32 = workloads.DeviceMobileNetV2(str(tmp_path), 32, fuse_expand_depthwise=fuse)
+        try:
+            assert sum(1 for op, _ in m32.plan if op["kind"] == "pwdw") == (2 if fuse else 0)
+            m32.set_input(x32)
+            outs.append(m32.predict())
+        finally:
+            m32.close()
+    np.testing.assert_array_equal(outs[0], outs[1])
     # the kernel-by-kernel host mirror agrees too
     assert_parity(workloads.run_graph(hip, ops, decoded, x[:1]), want[:1])

@@ -1,0 +1,370 @@
+// Pointwise (1x1) convolution + depthwise 3x3 convolution in one kernel: the
+// expansion and the depthwise stage of an inverted-residual block.
+//
+// Run as two kernels, the expanded tensor - the largest of the whole network -
+// is written to memory by the first and read back by the second. Here a
+// workgroup produces a tile of the expanded tensor row by row into a ring of
+// rows in LDS (matrix cores, the operand layout and instruction order of
+// skinny_gemm_regs, so the same bits), and the depthwise stage reads its 3x3
+// windows from that ring (the multiply-add order of depthwise_3x3_rows: taps
+// by row then column from zero, then the bias, then the activation): only the
+// block's input and the depthwise output touch memory.
+//
+//   workgroup  = one image, `rows` output rows, `tile_w` output columns, all channels
+//   ring       = 3 + S expanded rows of ecols = 16 * pblocks pixels (tile + halo),
+//                pixel pitch c + 4 floats (16-byte accesses of a wave then spread
+//                over all banks)
+//   step o     = depthwise output row o from ring rows S o .. S o + 2, and the S
+//                expanded rows the next step needs into the free ring slots; one
+//                barrier per step
+//   expansion  = tasks of 16 pixels x 16 channels dealt to the four waves in turn:
+//                A (16 pixels x K input channels) comes from memory as one 16-byte
+//                (+ one 8-byte) load per lane, issued a step ahead; the weights
+//                come from LDS, transposed so that a lane's four k values are one
+//                16-byte read
+//   padding    = positions of the expanded tensor outside the image are zero (what
+//                the depthwise stage pads with), not activation(bias)
+#include "common.h"
+#include "epilogue.h"
+
+namespace tfhip {
+namespace {
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+constexpr unsigned kNoOff = 0xffffffffu;   // an offset no buffer descriptor covers: loads return 0
+
+struct ExpandDwArgs {
+  const float *x, *w1, *b1, *w2, *b2;
+  float *y;
+  int batch, in_h, in_w, cin, c;   // x [batch, in_h, in_w, cin]; expanded [batch, in_h, in_w, c]
+  int pad_top, pad_left, out_h, out_w;
+  int act1, act2;                  // both relu or both relu6
+  int tile_w, tiles_w, rows, chunks_h, pblocks, pitch;
+  unsigned x_bytes;
+};
+
+template <int ACT>
+__device__ __forceinline__ float relu_like(float v) {
+  const float t = (v > 0.f || v != v) ? v : 0.f;     // Math.max(0, x): NaN stays, -0 becomes +0
+  return (ACT == TFHIP_RELU6 && t > 6.f) ? 6.f : t;
+}
+
+constexpr int kMaxTasks = 6;    // expansion tasks per wave and step
+constexpr int kMaxPasses = 4;   // depthwise pixels per lane and step
+
+// S: stride of the depthwise stage. K = 16 KF + (HALF ? 8 : 0) input channels.
+// ACT: the activation of both stages, relu or relu6.
+template <int S, int KF, bool HALF, int ACT>
+__global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g) {
+  constexpr int K = 16 * KF + (HALF ? 8 : 0);
+  constexpr int KP = K + 4;             // floats per column of the transposed weights in LDS
+  constexpr int RING = 3 + S;
+  extern __shared__ float lds[];
+  const int ecols = 16 * g.pblocks;
+  const int row_floats = ecols * g.pitch;
+  float *ring = lds;                                  // [RING][ecols][pitch]
+  float *w1t = ring + RING * row_floats;              // [c][KP]
+  float *b1s = w1t + g.c * KP;                        // [c]
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int grp = lane >> 4, r = lane & 15;
+  int rem = blockIdx.x;
+  const int tw = rem % g.tiles_w;
+  rem /= g.tiles_w;
+  const int chunk = rem % g.chunks_h;
+  const int n = rem / g.chunks_h;
+  const int oh0 = chunk * g.rows, ow0 = tw * g.tile_w;
+  const int ih0 = oh0 * S - g.pad_top, iw0 = ow0 * S - g.pad_left;   // image position of expanded (0, 0)
+  const int rows = oh0 + g.rows <= g.out_h ? g.rows : g.out_h - oh0;
+  const int cblocks = g.c / 16;
+  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)g.x, 0, (int)g.x_bytes, 0x00020000);
+
+  // weights of the expansion, transposed, and its bias
+  for (int k = 0; k < K; ++k) {
+    for (int col = threadIdx.x; col < g.c; col += 256) w1t[col * KP + k] = g.w1[k * g.c + col];
+  }
+  for (int i = threadIdx.x; i < g.c; i += 256) b1s[i] = g.b1 ? g.b1[i] : 0.f;
+
+  // depthwise stage: this lane's four channels and its pixels of a row
+  const int cq = g.c / 4, groups = 256 / cq;
+  const int c4 = (int)threadIdx.x % cq, pxg = (int)threadIdx.x / cq;
+  const bool dw_lane = pxg < groups;
+  float4 w2q[9], b2q = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int t = 0; t < 9; ++t) {
+    w2q[t] = dw_lane ? *reinterpret_cast<const float4 *>(g.w2 + (long long)t * g.c + 4 * c4) : b2q;
+  }
+  if (dw_lane && g.b2) b2q = *reinterpret_cast<const float4 *>(g.b2 + 4 * c4);
+
+  // Expansion work of one step: S expanded rows x pblocks blocks of 16 pixels ("row blocks"), each
+  // with c / 16 blocks of 16 channels. The (row block, channel block) pairs are cut into four
+  // contiguous shares, one per wave: a share spans at most two row blocks, and all its channel
+  // blocks of one row block use the same 16 pixels x K inputs (one load per lane).
+  const int per_step = S * g.pblocks * cblocks;
+  const int share = (per_step + 3) / 4;
+  const int t_lo = wave * share < per_step ? wave * share : per_step;
+  const int t_hi = t_lo + share < per_step ? t_lo + share : per_step;
+  const int rb0 = t_lo / cblocks;
+  const int cb0_lo = t_lo - rb0 * cblocks;
+  const int end0 = t_hi < (rb0 + 1) * cblocks ? t_hi : (rb0 + 1) * cblocks;
+  const int cb0_hi = end0 - rb0 * cblocks;           // first row block: channel blocks [cb0_lo, cb0_hi)
+  const int cb1_hi = t_hi - end0;                     // second row block: channel blocks [0, cb1_hi)
+  const int row0 = rb0 / g.pblocks, pb0 = rb0 - row0 * g.pblocks;
+  const int row1 = (rb0 + 1) / g.pblocks, pb1 = (rb0 + 1) - row1 * g.pblocks;
+
+  struct AFrag {
+    float4 full[KF > 0 ? KF : 1];
+    float2 half;
+  };
+  auto load_a = [&](AFrag &a, int erow, int pb) __attribute__((always_inline)) {
+    const int ih = ih0 + erow, iw = iw0 + 16 * pb + r;
+    const bool inside = ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
+    const unsigned base = (unsigned)((((long long)n * g.in_h + ih) * g.in_w + iw) * K * 4);
+#pragma unroll
+    for (int t = 0; t < KF; ++t) {
+      const auto v = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)(inside ? base + (16 * t + 4 * grp) * 4 : kNoOff), 0, 0);
+      a.full[t] = make_float4(__uint_as_float(v[0]), __uint_as_float(v[1]), __uint_as_float(v[2]), __uint_as_float(v[3]));
+    }
+    if (HALF) {
+      const auto v = __builtin_amdgcn_raw_buffer_load_b64(rx, (int)(inside ? base + (16 * KF + 2 * grp) * 4 : kNoOff), 0, 0);
+      a.half = make_float2(__uint_as_float(v[0]), __uint_as_float(v[1]));
+    }
+  };
+  // channel blocks [cb_lo, cb_hi) of the row block (erow, pb) into ring slot `slot`
+  auto expand_blocks = [&](const AFrag &a, int erow, int slot, int pb, int cb_lo, int cb_hi) __attribute__((always_inline)) {
+    const int ih = ih0 + erow, iw = iw0 + 16 * pb + r;
+    const bool inside = ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
+    float *dst = ring + slot * row_floats + (16 * pb + r) * g.pitch + 4 * grp;
+    const float *wcol = w1t + r * KP + 4 * grp;
+    const float *bias = b1s + 4 * grp;
+    for (int cb = cb_lo; cb < cb_hi; ++cb) {
+      float4_t acc = *reinterpret_cast<const float4_t *>(bias + 16 * cb);
+#pragma unroll
+      for (int t = 0; t < KF; ++t) {
+        const float4 b = *reinterpret_cast<const float4 *>(wcol + 16 * cb * KP + 16 * t);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.x, a.full[t].x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.y, a.full[t].y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.z, a.full[t].z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.w, a.full[t].w, acc, 0, 0, 0);
+      }
+      if (HALF) {
+        const float2 b = *reinterpret_cast<const float2 *>(w1t + (16 * cb + r) * KP + 16 * KF + 2 * grp);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.x, a.half.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.y, a.half.y, acc, 0, 0, 0);
+      }
+      // the lane holds pixel 16 pb + r, channels 16 cb + 4 grp .. +3; outside the image the
+      // expanded tensor is the zero padding of the depthwise stage
+      float4 e;
+      e.x = inside ? relu_like<ACT>(acc[0]) : 0.f;
+      e.y = inside ? relu_like<ACT>(acc[1]) : 0.f;
+      e.z = inside ? relu_like<ACT>(acc[2]) : 0.f;
+      e.w = inside ? relu_like<ACT>(acc[3]) : 0.f;
+      *reinterpret_cast<float4 *>(dst + 16 * cb) = e;
+    }
+  };
+  // this wave's share of expanded rows first .. first + S - 1 (only those below first + nrows), whose
+  // first row goes to ring slot `slot`
+  AFrag a0, a1;
+  auto issue_rows = [&](int first, int nrows) __attribute__((always_inline)) {
+    if (cb0_hi > cb0_lo && row0 < nrows) load_a(a0, first + row0, pb0);
+    if (cb1_hi > 0 && row1 < nrows) load_a(a1, first + row1, pb1);
+  };
+  auto expand_rows = [&](int first, int nrows, int slot) __attribute__((always_inline)) {
+    if (cb0_hi > cb0_lo && row0 < nrows) {
+      const int s0 = slot + row0 >= RING ? slot + row0 - RING : slot + row0;
+      expand_blocks(a0, first + row0, s0, pb0, cb0_lo, cb0_hi);
+    }
+    if (cb1_hi > 0 && row1 < nrows) {
+      const int s1 = slot + row1 >= RING ? slot + row1 - RING : slot + row1;
+      expand_blocks(a1, first + row1, s1, pb1, 0, cb1_hi);
+    }
+  };
+
+  // prologue: expanded rows 0, 1, 2
+  __syncthreads();   // w1t, b1s
+#pragma unroll
+  for (int first = 0; first < 3; first += S) {
+    const int nrows = 3 - first < S ? 3 - first : S;
+    issue_rows(first, nrows);
+    expand_rows(first, nrows, first);
+  }
+  __syncthreads();
+
+  int slot0 = 0;            // ring slot of expanded row S o
+  int new_slot = 3 % RING;  // ring slot of expanded row S o + 3
+  for (int o = 0; o < rows; ++o) {
+    // the rows the next step reads: S o + 3 .. S o + 2 + S (none after the last step)
+    const bool more = o + 1 < rows;
+    const int first = S * o + 3;
+    if (more) issue_rows(first, S);
+    // depthwise output row o
+    const int oh = oh0 + o;
+    if (dw_lane) {
+#pragma unroll
+      for (int pass = 0; pass < kMaxPasses; ++pass) {
+        const int q = pxg + pass * groups;
+        if (q >= g.tile_w || ow0 + q >= g.out_w) break;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int wr = 0; wr < 3; ++wr) {
+          const int slot = slot0 + wr >= RING ? slot0 + wr - RING : slot0 + wr;
+          const float *erow = ring + slot * row_floats + (S * q) * g.pitch + 4 * c4;
+#pragma unroll
+          for (int wc = 0; wc < 3; ++wc) {
+            const float4 e = *reinterpret_cast<const float4 *>(erow + wc * g.pitch);
+            const float4 w = w2q[wr * 3 + wc];
+            acc.x = fmaf(e.x, w.x, acc.x);
+            acc.y = fmaf(e.y, w.y, acc.y);
+            acc.z = fmaf(e.z, w.z, acc.z);
+            acc.w = fmaf(e.w, w.w, acc.w);
+          }
+        }
+        float4 out;
+        out.x = relu_like<ACT>(acc.x + b2q.x);
+        out.y = relu_like<ACT>(acc.y + b2q.y);
+        out.z = relu_like<ACT>(acc.z + b2q.z);
+        out.w = relu_like<ACT>(acc.w + b2q.w);
+        *reinterpret_cast<float4 *>(g.y + (((long long)n * g.out_h + oh) * g.out_w + ow0 + q) * g.c + 4 * c4) = out;
+      }
+    }
+    if (more) expand_rows(first, S, new_slot);
+    slot0 = slot0 + S >= RING ? slot0 + S - RING : slot0 + S;
+    new_slot = new_slot + S >= RING ? new_slot + S - RING : new_slot + S;
+    __syncthreads();
+  }
+}
+
+template <int S, int KF, bool HALF, int ACT>
+int launch_expand_dw_act(const ExpandDwArgs &g, size_t lds_bytes) {
+  static bool raised = false;   // dynamic LDS above the default limit needs the attribute once per instantiation
+  if (!raised) {
+    TFHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(expand_dw_3x3<S, KF, HALF, ACT>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    raised = true;
+  }
+  const long long wgs = (long long)g.batch * g.chunks_h * g.tiles_w;
+  note_kernel("expand_dw_3x3<%d, %d, %s, %d>", S, KF, HALF ? "true" : "false", ACT);
+  TFHIP_LAUNCH((expand_dw_3x3<S, KF, HALF, ACT><<<dim3((unsigned)wgs), dim3(256), lds_bytes, stream()>>>(g)));
+  return kOk;
+}
+
+template <int S, int KF, bool HALF>
+int launch_expand_dw(const ExpandDwArgs &g, size_t lds_bytes) {
+  if (g.act1 == TFHIP_RELU6) return launch_expand_dw_act<S, KF, HALF, TFHIP_RELU6>(g, lds_bytes);
+  return launch_expand_dw_act<S, KF, HALF, TFHIP_RELU>(g, lds_bytes);
+}
+
+}  // namespace
+
+// Fills the tiling of `g` for the fused kernel; false when the shape is one it does not take.
+bool plan_expand_dw(ExpandDwArgs &g, int stride, size_t *lds_bytes) {
+  const int K = g.cin;
+  if (!(K == 8 || K == 16 || K == 24 || K == 32) || g.c % 16 != 0 || g.c > 256 || (stride != 1 && stride != 2)) return false;
+  const int cq = g.c / 4, cblocks = g.c / 16;
+  const int groups = 256 / cq;
+  if (groups < 1) return false;
+  // output columns per workgroup: with its halo the tile is one or two blocks of 16 expanded
+  // pixels; the wider candidate unless only the narrower one divides the row
+  const int candidates[2][2] = {{14, 30}, {7, 15}};
+  int pick = 0;
+  for (int i = 1; i >= 0; --i) {
+    const int tile_w = candidates[stride - 1][i] > g.out_w ? g.out_w : candidates[stride - 1][i];
+    const int pblocks = ((tile_w - 1) * stride + 3 + 15) / 16;
+    const size_t bytes = ((size_t)(3 + stride) * 16 * pblocks * (g.c + 4) + (size_t)g.c * (K + 4) + g.c) * sizeof(float);
+    const bool fits = pblocks <= 2 && (tile_w + groups - 1) / groups <= kMaxPasses && bytes <= 156 * 1024;
+    if (!fits) continue;
+    if (pick == 0 || (g.out_w % pick != 0 && g.out_w % tile_w == 0)) pick = tile_w;
+  }
+  if (pick == 0) return false;
+  g.tile_w = pick;
+  g.pblocks = ((pick - 1) * stride + 3 + 15) / 16;
+  g.pitch = g.c + 4;
+  *lds_bytes = ((size_t)(3 + stride) * 16 * g.pblocks * g.pitch + (size_t)g.c * (K + 4) + g.c) * sizeof(float);
+  g.tiles_w = (g.out_w + g.tile_w - 1) / g.tile_w;
+  // output rows per workgroup: every row chunk recomputes two expanded rows of halo, so as
+  // many rows as still give each compute unit the workgroups its LDS holds (four at most)
+  long long resident = (long long)(160 * 1024 / *lds_bytes);
+  resident = resident > 4 ? 4 : resident;
+  int rows = g.out_h;
+  while (rows > 14 && (long long)g.batch * ((g.out_h + rows - 1) / rows) * g.tiles_w < resident * num_cus()) rows = (rows + 1) / 2;
+  g.rows = rows;
+  g.chunks_h = (g.out_h + rows - 1) / rows;
+  return true;
+}
+
+}  // namespace tfhip
+
+using namespace tfhip;
+
+extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_filter, const float *pw_bias,
+                                               int pw_activation, const float *dw_filter, const float *dw_bias,
+                                               int dw_activation, float *y, int64_t batch, int64_t in_h,
+                                               int64_t in_w, int64_t in_c, int64_t mid_c, int64_t stride,
+                                               int64_t pad_top, int64_t pad_left, int64_t out_h, int64_t out_w) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_ARG(batch >= 0 && in_h > 0 && in_w > 0 && in_c > 0 && mid_c > 0 && stride > 0 && out_h >= 0 && out_w >= 0 &&
+                      pad_top >= 0 && pad_left >= 0,
+                  "tfhip_fused_pointwise_depthwise: bad dimension");
+  const int64_t lim = 0x7fffffff;
+  TFHIP_CHECK_ARG(batch * in_h * in_w * (in_c > mid_c ? in_c : mid_c) < lim && batch * out_h * out_w * mid_c < lim,
+                  "tfhip_fused_pointwise_depthwise: tensor exceeds the supported range");
+  TFHIP_CHECK_ARG(pw_activation >= TFHIP_LINEAR && pw_activation <= TFHIP_ELU && dw_activation >= TFHIP_LINEAR &&
+                      dw_activation <= TFHIP_ELU,
+                  "tfhip_fused_pointwise_depthwise: unknown activation");
+  if (batch * out_h * out_w == 0) return kOk;
+  TFHIP_CHECK_RANGE(x, batch * in_h * in_w * in_c, 4, "x");
+  TFHIP_CHECK_RANGE(pw_filter, in_c * mid_c, 4, "pw_filter");
+  TFHIP_CHECK_RANGE(dw_filter, 9 * mid_c, 4, "dw_filter");
+  if (pw_bias) TFHIP_CHECK_RANGE(pw_bias, mid_c, 4, "pw_bias");
+  if (dw_bias) TFHIP_CHECK_RANGE(dw_bias, mid_c, 4, "dw_bias");
+  TFHIP_CHECK_RANGE(y, batch * out_h * out_w * mid_c, 4, "y");
+
+  ExpandDwArgs g = {};
+  g.x = x; g.w1 = pw_filter; g.b1 = pw_bias; g.w2 = dw_filter; g.b2 = dw_bias; g.y = y;
+  g.batch = (int)batch; g.in_h = (int)in_h; g.in_w = (int)in_w; g.cin = (int)in_c; g.c = (int)mid_c;
+  g.pad_top = (int)pad_top; g.pad_left = (int)pad_left; g.out_h = (int)out_h; g.out_w = (int)out_w;
+  g.act1 = pw_activation; g.act2 = dw_activation;
+  g.x_bytes = (unsigned)(batch * in_h * in_w * in_c * 4);
+  size_t lds_bytes = 0;
+  const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(dw_filter) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+                       (dw_bias == nullptr || reinterpret_cast<uintptr_t>(dw_bias) % 16 == 0);
+  const bool same_relu = pw_activation == dw_activation && (pw_activation == TFHIP_RELU || pw_activation == TFHIP_RELU6);
+  if (!aligned || !same_relu || !plan_expand_dw(g, (int)stride, &lds_bytes)) {
+    return fail(kBadArgument,
+                "tfhip_fused_pointwise_depthwise: form not taken by the fused kernel (in_c 8/16/24/32, mid_c a "
+                "multiple of 16 up to 256, stride 1 or 2, both activations relu or both relu6, 16-byte aligned "
+                "operands); run the two convolutions");
+  }
+  const int key = (int)stride * 100 + (int)in_c;
+  switch (key) {
+    case 108: return launch_expand_dw<1, 0, true>(g, lds_bytes);
+    case 116: return launch_expand_dw<1, 1, false>(g, lds_bytes);
+    case 124: return launch_expand_dw<1, 1, true>(g, lds_bytes);
+    case 132: return launch_expand_dw<1, 2, false>(g, lds_bytes);
+    case 208: return launch_expand_dw<2, 0, true>(g, lds_bytes);
+    case 216: return launch_expand_dw<2, 1, false>(g, lds_bytes);
+    case 224: return launch_expand_dw<2, 1, true>(g, lds_bytes);
+    default: return launch_expand_dw<2, 2, false>(g, lds_bytes);
+  }
+}
+
+// 1 when tfhip_fused_pointwise_depthwise takes this shape and is expected to beat the two
+// kernels, else 0. Measured at batch 32 (in sequence, where the expanded tensor really goes
+// to memory and back): 16 -> 96 channels at 112x112, stride 2, 44 us against 95 us; 24 -> 144
+// at 56x56, stride 2, 28 against 41; the same with stride 1 about even (55 / 56); 32 -> 192 at
+// 28x28 slower (25 against 19 + 7, the expanded tensor stays in cache there). So: an
+// expanded tensor of at least 48 MB for stride 2, 96 MB for stride 1.
+extern "C" int tfhip_pointwise_depthwise_pays(int64_t batch, int64_t in_c, int64_t mid_c, int64_t stride,
+                                              int64_t out_h, int64_t out_w) {
+  if (!initialised() || batch <= 0 || out_h <= 0 || out_w <= 0 || mid_c <= 0 || mid_c > 0x7fffffff || in_c > 64 ||
+      batch > 0x7fffffff || out_h > 0x7fffffff || out_w > 0x7fffffff) {
+    return 0;
+  }
+  ExpandDwArgs g = {};
+  g.batch = (int)batch; g.cin = (int)in_c; g.c = (int)mid_c; g.out_h = (int)out_h; g.out_w = (int)out_w;
+  size_t lds_bytes = 0;
+  if (!plan_expand_dw(g, (int)stride, &lds_bytes)) return 0;
+  const int64_t expanded_bytes = batch * out_h * stride * out_w * stride * mid_c * 4;
+  return expanded_bytes >= (stride == 2 ? 48LL : 96LL) * 1000 * 1000 ? 1 : 0;
+}

@@ -409,6 +409,32 @@ napi_value MeanHW(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+// fusedPointwiseDepthwise(x, pwFilter, pwBias, pwActivation, dwFilter, dwBias, dwActivation, y,
+//                         geom[10] = [batch, inH, inW, inC, midC, stride, padTop, padLeft, outH, outW])
+napi_value FusedPointwiseDepthwise(napi_env env, napi_callback_info info) {
+  Args a(env, info, 9, "fusedPointwiseDepthwise");
+  int64_t g[10];
+  a.ints(8, g, 10);
+  const float *x = (const float *)a.ptr(0), *w1 = (const float *)a.ptr(1), *b1 = (const float *)a.ptr(2);
+  const float *w2 = (const float *)a.ptr(4), *b2 = (const float *)a.ptr(5);
+  float *y = (float *)a.ptr(7);
+  const int act1 = a.i32(3), act2 = a.i32(6);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_fused_pointwise_depthwise(x, w1, b1, act1, w2, b2, act2, y, g[0], g[1], g[2], g[3], g[4], g[5], g[6], g[7],
+                                         g[8], g[9]));
+  return undefined(env);
+}
+
+// pointwiseDepthwisePays(batch, inC, midC, stride, outH, outW): boolean
+napi_value PointwiseDepthwisePays(napi_env env, napi_callback_info info) {
+  Args a(env, info, 6, "pointwiseDepthwisePays");
+  const int64_t b = a.i64(0), ic = a.i64(1), mc = a.i64(2), s = a.i64(3), oh = a.i64(4), ow = a.i64(5);
+  if (!a.ok) return nullptr;
+  napi_value r;
+  NAPI_OK(napi_get_boolean(env, tfhip_pointwise_depthwise_pays(b, ic, mc, s, oh, ow) == 1, &r));
+  return r;
+}
+
 // copy(dst, src, bytes): device to device on the library's stream
 napi_value Copy(napi_env env, napi_callback_info info) {
   Args a(env, info, 3, "copy");
@@ -481,6 +507,8 @@ napi_value Register(napi_env env, napi_value exports) {
       FN("dequantF16", DequantF16),
       FN("add", Add),
       FN("meanHW", MeanHW),
+      FN("fusedPointwiseDepthwise", FusedPointwiseDepthwise),
+      FN("pointwiseDepthwisePays", PointwiseDepthwisePays),
       FN("copy", Copy),
       FN("captureBegin", CaptureBegin),
       FN("captureEnd", CaptureEnd),

@@ -54,6 +54,8 @@ export declare class HipBackend extends KernelBackend {
 export interface HipGraphModelOptions {
   /** default true: a _FusedConv2D read by one Add/AddV2 only runs with it as one FusedConv2DAdd kernel */
   fuseResidualAdd?: boolean;
+  /** default true: a 1x1 _FusedConv2D read by one 3x3 FusedDepthwiseConv2dNative only is one FusedPointwiseDepthwiseConv2D step */
+  fusePointwiseDepthwise?: boolean;
   /** default false: record the kernels of an execution into a HIP graph and replay it for the same input shapes */
   recordLaunches?: boolean;
 }

@@ -19,7 +19,7 @@ const graphModel = require('./standin/graph_model');
 
 const kernelConfigs = [
   matmul.fusedMatMulConfig, matmul.batchMatMulConfig, conv.fusedConv2DConfig,
-  conv.fusedConv2DAddConfig, conv.conv2DConfig, conv.fusedDepthwiseConv2DConfig,
+  conv.fusedConv2DAddConfig, conv.fusedPointwiseDepthwiseConfig, conv.conv2DConfig, conv.fusedDepthwiseConv2DConfig,
   conv.depthwiseConv2dNativeConfig, glue.addConfig, glue.meanConfig,
   glue.reshapeConfig, glue.identityConfig, glue.copyConfig
 ];

@@ -127,7 +127,75 @@ function convImpl(args, depthwise, fused, opName, residual) {
   return out;
 }
 
+const pwdwGeom = new Float64Array(10);
+
+/**
+ * FusedPointwiseDepthwiseConv2D (no counterpart among the reference's kernel
+ * names): a FusedConv2D with a 1x1 filter, stride 1, followed by the
+ * FusedDepthwiseConv2D that is its only reader - the expansion and the
+ * depthwise stage of an inverted-residual block - as one launch in which the
+ * expanded tensor never reaches memory.
+ *   inputs  x, filter [1,1,inC,midC], bias [midC], dwFilter [3,3,midC,1], dwBias [midC]
+ *   attrs   activation ('relu' | 'relu6', of both stages), and of the depthwise
+ *           stage: strides, pad, dimRoundingMode
+ * Where the native library does not expect the fused kernel to be faster (or
+ * does not take the shape), the two kernels run one after the other here; the
+ * result is the same either way.
+ */
+function fusedPointwiseDepthwise(args) {
+  const {x, filter, bias, dwFilter, dwBias} = args.inputs;
+  const {strides, pad, dimRoundingMode, activation} = args.attrs;
+  const backend = args.backend;
+  const opName = 'FusedPointwiseDepthwiseConv2D';
+  requireFloat32([x, filter, bias, dwFilter, dwBias], opName);
+  const midC = filter.shape[3];
+  const fusable = x.shape.length === 4 && filter.shape[0] === 1 && filter.shape[1] === 1 &&
+      dwFilter.shape[0] === 3 && dwFilter.shape[1] === 3 && dwFilter.shape[2] === midC && dwFilter.shape[3] === 1 &&
+      bias != null && bias.shape.length === 1 && bias.shape[0] === midC &&
+      dwBias != null && dwBias.shape.length === 1 && dwBias.shape[0] === midC &&
+      (activation === 'relu' || activation === 'relu6');
+  if (fusable) {
+    const info = tf.backend_util.computeConv2DInfo(
+        [x.shape[0], x.shape[1], x.shape[2], midC], dwFilter.shape, strides, [1, 1], pad, dimRoundingMode, true,
+        'channelsLast');
+    if (info.strideHeight === info.strideWidth && tf.util.sizeFromShape(info.outShape) > 0 &&
+        addon.pointwiseDepthwisePays(
+            info.batchSize, x.shape[3], midC, info.strideHeight, info.outHeight, info.outWidth)) {
+      const out = backend.makeOutput(info.outShape, 'float32');
+      pwdwGeom[0] = info.batchSize;
+      pwdwGeom[1] = x.shape[1];
+      pwdwGeom[2] = x.shape[2];
+      pwdwGeom[3] = x.shape[3];
+      pwdwGeom[4] = midC;
+      pwdwGeom[5] = info.strideHeight;
+      pwdwGeom[6] = info.padInfo.top;
+      pwdwGeom[7] = info.padInfo.left;
+      pwdwGeom[8] = info.outHeight;
+      pwdwGeom[9] = info.outWidth;
+      const code = activationCode(activation, opName);
+      addon.fusedPointwiseDepthwise(
+          backend.ptr(x.dataId), backend.ptr(filter.dataId), backend.ptr(bias.dataId), code,
+          backend.ptr(dwFilter.dataId), backend.ptr(dwBias.dataId), code, backend.ptr(out.dataId), pwdwGeom);
+      return out;
+    }
+  }
+  const expanded = convImpl(
+      {inputs: {x, filter, bias}, backend, attrs: {strides: [1, 1], pad: 'valid', dataFormat: 'NHWC', dilations: [1, 1], activation}},
+      false, true, 'FusedConv2D');
+  const out = convImpl(
+      {inputs: {x: expanded, filter: dwFilter, bias: dwBias}, backend,
+       attrs: {strides, pad, dataFormat: 'NHWC', dilations: [1, 1], dimRoundingMode, activation}},
+      true, true, 'FusedDepthwiseConv2D');
+  backend.disposeIntermediateTensorInfo(expanded);
+  return out;
+}
+
 module.exports = {
+  fusedPointwiseDepthwiseConfig: {
+    kernelName: 'FusedPointwiseDepthwiseConv2D',
+    backendName: 'hip',
+    kernelFunc: fusedPointwiseDepthwise
+  },
   fusedConv2DConfig: {
     kernelName: 'FusedConv2D',
     backendName: 'hip',

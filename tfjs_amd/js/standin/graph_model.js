@@ -22,7 +22,12 @@
  * reader is an Add / AddV2 node (a projection convolution and the skip connection
  * of a residual block) is executed together with that Add as one kernel. The
  * result has the bits of the two separate kernels; {fuseResidualAdd: false} in
- * the load options turns it off.
+ * the load options turns it off. Likewise, with a 'FusedPointwiseDepthwiseConv2D'
+ * kernel, a 1x1 _FusedConv2D whose only reader is a 3x3 FusedDepthwiseConv2dNative
+ * with the same relu / relu6 activation (the expansion and the depthwise stage of
+ * an inverted-residual block) is one step, and the kernel decides per shape
+ * whether one launch or the two are faster; {fusePointwiseDepthwise: false} turns
+ * that off.
  *
  * And with {recordLaunches: true} in the load options, on a backend that can
  * record (beginRecording / endRecording / replay, as the hip backend has), the
@@ -190,6 +195,42 @@ function compileConvAdd(convNode) {
          dimRoundingMode: undefined, activation: p.activation, leakyreluAlpha: p.leakyreluAlpha});
     return out;
   };
+}
+
+/**
+ * 1x1 _FusedConv2D + the FusedDepthwiseConv2dNative that reads it -> function(inputs) => Tensor,
+ * inputs = [x, filter, bias, dwFilter, dwBias]; null when the pair is not of the form the
+ * FusedPointwiseDepthwiseConv2D kernel covers (checked on the attributes; shapes are checked by
+ * the kernel, which runs the two convolutions itself where it must).
+ */
+function compilePointwiseDepthwise(convNode, dwNode, weightMap) {
+  let conv, dw;
+  try {
+    conv = fusedConvParams(convNode)([null, null, null]);
+    dw = fusedConvParams(dwNode)([null, null, null]);
+  } catch (e) {
+    return null;   // a malformed node throws when it is executed on its own, as in the reference
+  }
+  const dataInputs = node => (node.input || []).filter(i => i[0] !== '^');
+  const fusedOps = node => getStringArrayParam(node.attr || {}, 'fused_ops', []);
+  const act = conv.activation;
+  const filter = weightMap[parseNodeName(dataInputs(convNode)[1] || '')[0]];
+  const dwFilter = weightMap[parseNodeName(dataInputs(dwNode)[1] || '')[0]];
+  const ok = dataInputs(convNode).length === 3 && dataInputs(dwNode).length === 3 &&
+      fusedOps(convNode)[0] === 'biasadd' && fusedOps(dwNode)[0] === 'biasadd' &&
+      (act === 'relu' || act === 'relu6') && dw.activation === act &&
+      conv.dataFormat === 'NHWC' && dw.dataFormat === 'NHWC' &&
+      conv.strides[0] === 1 && conv.strides[1] === 1 &&
+      conv.dilations[0] === 1 && conv.dilations[1] === 1 && dw.dilations[0] === 1 && dw.dilations[1] === 1 &&
+      filter != null && filter.shape.length === 4 && filter.shape[0] === 1 && filter.shape[1] === 1 &&
+      dwFilter != null && dwFilter.shape.length === 4 && dwFilter.shape[0] === 3 && dwFilter.shape[1] === 3;
+  if (!ok) {
+    return null;
+  }
+  const attrs = {strides: dw.strides, pad: dw.pad, dimRoundingMode: undefined, activation: act};
+  return inputs => tf.engine().runKernel(
+      'FusedPointwiseDepthwiseConv2D',
+      {x: inputs[0], filter: inputs[1], bias: inputs[2], dwFilter: inputs[3], dwBias: inputs[4]}, attrs);
 }
 
 /**
@@ -463,11 +504,17 @@ class GraphModel {
           for (let i = 0; i < args.length; i++) {
             args[i] = values[step.sources[i]];
           }
-          const key = step.conv != null ? name + '<-' + step.conv : name;
+          const key = step.conv != null ? name + '<-' + step.conv : (step.pointwise != null ? name + '<=' + step.pointwise : name);
           let run = this.compiled[key];
           if (run === undefined) {
-            run = this.compiled[key] =
-                step.conv != null ? compileConvAdd(this.nodes[step.conv]) : compileNode(this.nodes[name]);
+            if (step.conv != null) {
+              run = compileConvAdd(this.nodes[step.conv]);
+            } else if (step.pointwise != null) {
+              run = step.run;
+            } else {
+              run = compileNode(this.nodes[name]);
+            }
+            this.compiled[key] = run;
           }
           const out = values[name] = run(args);
           // intermediates that nobody reads again can go now
@@ -616,8 +663,41 @@ class GraphModel {
       });
     }
 
+    // 1x1 _FusedConv2D read by one 3x3 FusedDepthwiseConv2dNative only -> one step at the depthwise node's place
+    const pointwiseOf = {}, depthwiseOf = {}, pairRun = {};
+    const fusePair = this.loadOptions.fusePointwiseDepthwise !== false && tf.getKernel != null &&
+        tf.getKernel('FusedPointwiseDepthwiseConv2D', tf.getBackend()) != null;
+    if (fusePair) {
+      order.forEach(n => {
+        const node = this.nodes[n];
+        if (!isOp(n) || node.op !== 'FusedDepthwiseConv2dNative') {
+          return;
+        }
+        const c = dataSources(n)[0];
+        if (c == null || !isOp(c) || this.nodes[c].op !== '_FusedConv2D' || readers[c] !== 1 || fetchSet.has(c) ||
+            addOf[c] != null) {
+          return;
+        }
+        const run = compilePointwiseDepthwise(this.nodes[c], node, this.weightMap);
+        if (run != null) {
+          pointwiseOf[n] = c;
+          depthwiseOf[c] = n;
+          pairRun[n] = run;
+        }
+      });
+    }
+
     const steps = [];
     order.forEach(name => {
+      if (depthwiseOf[name] != null) {
+        return;   // runs inside the step of the depthwise node that reads it
+      }
+      if (pointwiseOf[name] != null) {
+        const conv = pointwiseOf[name];
+        steps.push({name, kind: 'op', pointwise: conv, run: pairRun[name],
+                    sources: dataSources(conv).concat(dataSources(name).slice(1))});
+        return;
+      }
       if (feeds[name] != null) {
         steps.push({name, kind: 'feed'});
       } else if (this.nodes[name].op === 'Const') {

@@ -189,6 +189,36 @@ def fused_depthwise_conv2d(x, w, strides=1, pad="valid", dilations=1, dim_roundi
                       leakyrelu_alpha)
 
 
+def fused_pointwise_depthwise(x, pw_filter, dw_filter, strides=1, pad="same", pw_bias=None, pw_activation="linear",
+                              dw_bias=None, dw_activation="linear"):
+    """1x1 convolution + depthwise 3x3 convolution (NHWC) as one launch; raises
+    HipBackendError for a shape the fused kernel does not take."""
+    init()
+    x, w1, w2 = _f32(x), _f32(pw_filter), _f32(dw_filter)
+    b1, b2 = _opt(pw_bias), _opt(dw_bias)
+    mid = w1.shape[3]
+    ci = compute_conv2d_info([x.shape[0], x.shape[1], x.shape[2], mid], w2.shape, strides, 1, pad, None, True,
+                             "channelsLast")
+    assert ci["strideHeight"] == ci["strideWidth"] and w2.shape[:2] == (3, 3) and w2.shape[3] == 1
+    total = int(np.prod(ci["outShape"], dtype=np.int64))
+    bufs = []
+    try:
+        dx, dw1, dw2, dy = (DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(w1), DeviceBuffer.from_numpy(w2),
+                            DeviceBuffer(total * 4))
+        bufs += [dx, dw1, dw2, dy]
+        db1 = DeviceBuffer.from_numpy(b1) if b1 is not None else None
+        db2 = DeviceBuffer.from_numpy(b2) if b2 is not None else None
+        bufs += [b for b in (db1, db2) if b is not None]
+        check(load_library().tfhip_fused_pointwise_depthwise(
+            dx.ptr, dw1.ptr, db1.ptr if db1 else None, ACTIVATIONS[pw_activation], dw2.ptr, db2.ptr if db2 else None,
+            ACTIVATIONS[dw_activation], dy.ptr, x.shape[0], x.shape[1], x.shape[2], x.shape[3], mid,
+            ci["strideHeight"], ci["padInfo"]["top"], ci["padInfo"]["left"], ci["outHeight"], ci["outWidth"]))
+        return dy.download(np.float32, total).reshape(ci["outShape"])
+    finally:
+        for buf in bufs:
+            buf.free()
+
+
 def add(a, b):
     init()
     a, b = _f32(a), _f32(b)

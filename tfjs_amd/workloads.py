@@ -225,7 +225,7 @@ class DeviceMobileNetV2:
     load (quantized shard uploaded once, one dequant kernel per tensor) and every
     activation stays in pooled device buffers between kernels."""
 
-    def __init__(self, model_dir, batch, fuse_residual_add=True):
+    def __init__(self, model_dir, batch, fuse_residual_add=True, fuse_expand_depthwise=True):
         from . import pyhost
         from .capi import ACTIVATIONS, DeviceBuffer, check, i64_array, load_library
         from .conv_util import compute_conv2d_info
@@ -236,6 +236,8 @@ class DeviceMobileNetV2:
         self.ops, self.shapes = mobilenet_v2_graph()
         if fuse_residual_add:
             self.ops = self._fuse_residual_adds(self.ops)
+        if fuse_expand_depthwise:
+            self.ops = self._fuse_expand_depthwise(self.ops, self.shapes, batch, self._lib)
         buf, specs = read_model(model_dir)
         self.weights = pyhost.decode_weights_to_device(buf, specs)   # name -> (DeviceBuffer, shape)
         self.input = DeviceBuffer(batch * 224 * 224 * 3 * 4)
@@ -257,6 +259,14 @@ class DeviceMobileNetV2:
                         ci["filterWidth"], ci["outChannels"] if k == "conv" else 1, ci["strideHeight"],
                         ci["strideWidth"], 1, 1, ci["padInfo"]["top"], ci["padInfo"]["left"], ci["outHeight"],
                         ci["outWidth"]]
+                self.plan.append((op, geom))
+            elif k == "pwdw":
+                n, h, w, _ = shape[src]
+                mid = self.shapes[op["w"]][3]
+                ci = compute_conv2d_info((n, h, w, mid), self.shapes[op["w2"]], op["stride"], 1, "same", None, True)
+                shape[op["out"]] = tuple(ci["outShape"])
+                geom = [n, h, w, self.shapes[op["w"]][2], mid, op["stride"], ci["padInfo"]["top"], ci["padInfo"]["left"],
+                        ci["outHeight"], ci["outWidth"]]
                 self.plan.append((op, geom))
             elif k == "add":
                 shape[op["out"]] = shape[src[0]]
@@ -293,6 +303,38 @@ class DeviceMobileNetV2:
                 fused.append(op)
         return fused
 
+    @staticmethod
+    def _fuse_expand_depthwise(ops, shapes, batch, lib):
+        """A 1x1 convolution whose only reader is the depthwise 3x3 convolution that
+        follows it becomes one op, where the fused kernel takes the shape (what the
+        graph model does at load)."""
+        readers, size = {}, {"input": 224}
+        for op in ops:
+            for s in (op["src"] if isinstance(op["src"], tuple) else (op["src"],)):
+                readers[s] = readers.get(s, 0) + 1
+        fused, skip = [], set()
+        for i, op in enumerate(ops):
+            src = op["src"][0] if isinstance(op["src"], tuple) else op["src"]
+            if op["kind"] in ("conv", "dw"):
+                size[op["out"]] = (size[src] + op["stride"] - 1) // op["stride"]
+            elif op["kind"] == "add":
+                size[op["out"]] = size[src]
+            if i in skip:
+                continue
+            nxt = ops[i + 1] if i + 1 < len(ops) else None
+            if (op["kind"] == "conv" and "residual" not in op and shapes[op["w"]][:2] == (1, 1) and op["stride"] == 1
+                    and nxt is not None and nxt["kind"] == "dw" and nxt["src"] == op["out"]
+                    and readers.get(op["out"]) == 1):
+                cin, mid = shapes[op["w"]][2], shapes[op["w"]][3]
+                out_size = (size[src] + nxt["stride"] - 1) // nxt["stride"]
+                if lib.tfhip_pointwise_depthwise_pays(batch, cin, mid, nxt["stride"], out_size, out_size) == 1:
+                    fused.append(dict(kind="pwdw", src=src, out=nxt["out"], w=op["w"], b=op["b"], act=op["act"],
+                                      w2=nxt["w"], b2=nxt["b"], act2=nxt["act"], stride=nxt["stride"]))
+                    skip.add(i + 1)
+                    continue
+            fused.append(op)
+        return fused
+
     def set_input(self, x):
         self.input.upload(np.ascontiguousarray(x, dtype=np.float32))
 
@@ -304,8 +346,12 @@ class DeviceMobileNetV2:
         n_out = int(np.prod(self.shape[op["out"]]))
         srcs = op["src"] if isinstance(op["src"], tuple) else (op["src"],)
         n_in = sum(int(np.prod(self.shape[s])) for s in srcs)
-        n_w = sum(int(np.prod(self.shapes[op[key]])) for key in ("w", "b") if key in op)
-        if k == "conv":
+        n_w = sum(int(np.prod(self.shapes[op[key]])) for key in ("w", "b", "w2", "b2") if key in op)
+        if k == "pwdw":
+            _, _, cin, mid = self.shapes[op["w"]]
+            n_mid = int(np.prod(self.shape[op["src"]][:3])) * mid
+            flops = 2 * n_mid * cin + 2 * n_out * 9
+        elif k == "conv":
             fh, fw, cin, _ = self.shapes[op["w"]]
             flops = 2 * n_out * fh * fw * cin
         elif k == "dw":
@@ -335,6 +381,10 @@ class DeviceMobileNetV2:
                 check(lib.tfhip_fused_conv2d(t[op["src"]].ptr, self.weights[op["w"]][0].ptr, out.ptr, *geom, 0,
                                              self.weights[op["b"]][0].ptr, self.strides_c, self._ACT[op["act"]],
                                              None, self.zero4, 0.2))
+            elif k == "pwdw":
+                check(lib.tfhip_fused_pointwise_depthwise(
+                    t[op["src"]].ptr, self.weights[op["w"]][0].ptr, self.weights[op["b"]][0].ptr, self._ACT[op["act"]],
+                    self.weights[op["w2"]][0].ptr, self.weights[op["b2"]][0].ptr, self._ACT[op["act2"]], out.ptr, *geom))
             elif k == "dw":
                 check(lib.tfhip_fused_depthwise_conv2d(t[op["src"]].ptr, self.weights[op["w"]][0].ptr, out.ptr,
                                                        *geom, self.weights[op["b"]][0].ptr, self.strides_c,
