@@ -144,29 +144,39 @@ def bench_model(model_dir, steps, warmup):
         check(lib.tfhip_sync())
         seconds = time.perf_counter() - t0
 
-        # per-op durations on the stream: each op's kernel enqueued `repeat` times
-        # between two events, after the timed region
+        # Per-op durations, in sequence: a series of inferences with an event at every
+        # op boundary; interval i = op i's kernel(s) plus one marker. The marker's cost
+        # is what the instrumented inference takes longer than the plain one, per
+        # boundary, so that the per-op times add up to the plain inference. (Launching
+        # an op's kernel many times back to back instead would flatter every layer
+        # whose operands fit the 256 MB memory-side cache: in a real inference an
+        # activation is written by one kernel and read by the next through memory.)
         ev = Events(lib, check)
-        repeat = 20
         names = {}
-        check(lib.tfhip_set_launch_repeat(repeat))
-        try:
-            def before(i, op):
-                ev.record(2 * i)
+        n_ops = len(model.plan)
 
-            def after(i, op):
-                ev.record(2 * i + 1)
-                names[i] = last_kernel(lib)
-            per_op = np.zeros(len(model.plan))
-            rounds = 3
-            for r in range(rounds):
-                out = model.forward(before, after)
-                check(lib.tfhip_sync())
-                out.free()
-                d = np.array([ev.elapsed_ms(2 * i, 2 * i + 1) / repeat * 1e-3 for i in range(len(model.plan))])
-                per_op = d if r == 0 else np.minimum(per_op, d)
-        finally:
-            check(lib.tfhip_set_launch_repeat(1))
+        def before(i, op):
+            ev.record(i)
+
+        def after(i, op):
+            names[i] = last_kernel(lib)
+            if i == n_ops - 1:
+                ev.record(n_ops)
+        plain_rounds = 50
+        ev.record(n_ops + 1)
+        for _ in range(plain_rounds):
+            model.forward().free()
+        ev.record(n_ops + 2)
+        plain_ms = ev.elapsed_ms(n_ops + 1, n_ops + 2) / plain_rounds
+        series = []
+        for r in range(25):
+            out = model.forward(before, after)
+            check(lib.tfhip_sync())
+            out.free()
+            series.append([ev.elapsed_ms(i, i + 1) for i in range(n_ops)])
+        intervals = np.median(np.array(series[5:]), axis=0)
+        marker_ms = max(0.0, (float(intervals.sum()) - plain_ms) / n_ops)
+        per_op = np.maximum(intervals - marker_ms, 1e-4) * 1e-3
         by_symbol = {}
         for i in range(len(model.plan)):
             flops, nbytes = model.op_work(i)
@@ -196,7 +206,7 @@ def bench_model(model_dir, steps, warmup):
     symbols = {k: dict(us_per_step=round(v["seconds"] * 1e6, 1), launches=v["launches"],
                        **roofline_entry(v["flops"], v["bytes"], v["seconds"])) for k, v in by_symbol.items()}
     return dict(ms_per_step=seconds / steps * 1e3, kernel_ms_per_step=kernel_seconds * 1e3, roofline=roof,
-                symbols=symbols, ops=ops)
+                symbols=symbols, ops=ops, marker_us=marker_ms * 1e3)
 
 
 def bench_model_node(model_dir, steps, warmup, prime):
@@ -433,6 +443,7 @@ def main():
         "weights_load_ms": round(js["load_ms"], 2) if js else None,
         "python_host_ms_per_step": round(m["ms_per_step"], 4),
         "kernel_ms_per_step": round(m["kernel_ms_per_step"], 4),
+        "event_marker_us": round(m["marker_us"], 2),
         "tflops_model": round(BATCH * workloads.mobilenet_v2_flops_per_image() / (ms_per_step * 1e-3) / 1e12, 3),
         "roofline": m["roofline"],
         "cpu_baseline": cpu,

@@ -120,8 +120,8 @@ int tfhip_graph_destroy(int graph_id);
  *   "dw_rows" (depthwise rows per lane), "dw_halo" (1: LDS halo depthwise kernel),
  *   "no_skinny" (1: tiled GEMM also for tall products), "dw_flat" (1: the
  *   one-row-per-lane depthwise kernel always, 0: never), "skinny_regs" (0: the
- *   streaming GEMM always stages B in LDS), "small_k" (0: never the one-shot GEMM
- *   for K <= 64, 32 / 64: that many rows per tile). TFHIP_TILE,
+ *   streaming GEMM always stages B in LDS), "small_k" (32 / 64: the one-shot GEMM for
+ *   K <= 64 with that many rows per tile; unset or 0: never). TFHIP_TILE,
  *   TFHIP_SPLITK, TFHIP_DW_ROWS, TFHIP_DW_HALO, TFHIP_NO_SKINNY, TFHIP_DW_FLAT,
  *   TFHIP_SKINNY_REGS, TFHIP_SMALL_K in the environment set them at tfhip_init(). */
 int tfhip_set_launch_repeat(int n);

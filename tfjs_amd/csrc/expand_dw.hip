@@ -286,7 +286,7 @@ bool plan_expand_dw(ExpandDwArgs &g, int stride, size_t *lds_bytes) {
   long long resident = (long long)(160 * 1024 / *lds_bytes);
   resident = resident > 4 ? 4 : resident;
   int rows = g.out_h;
-  while (rows > 14 && (long long)g.batch * ((g.out_h + rows - 1) / rows) * g.tiles_w < resident * num_cus()) rows = (rows + 1) / 2;
+  while (rows > 7 && (long long)g.batch * ((g.out_h + rows - 1) / rows) * g.tiles_w < resident * num_cus()) rows = (rows + 1) / 2;
   g.rows = rows;
   g.chunks_h = (g.out_h + rows - 1) / rows;
   return true;
@@ -351,10 +351,10 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
 
 // 1 when tfhip_fused_pointwise_depthwise takes this shape and is expected to beat the two
 // kernels, else 0. Measured at batch 32 (in sequence, where the expanded tensor really goes
-// to memory and back): 16 -> 96 channels at 112x112, stride 2, 44 us against 95 us; 24 -> 144
-// at 56x56, stride 2, 28 against 41; the same with stride 1 about even (55 / 56); 32 -> 192 at
-// 28x28 slower (25 against 19 + 7, the expanded tensor stays in cache there). So: an
-// expanded tensor of at least 48 MB for stride 2, 96 MB for stride 1.
+// to memory and back): 16 -> 96 channels at 112x112, stride 2, 46 us against 91 us; 24 -> 144
+// at 56x56, stride 2, 33 against 36; the same with stride 1 about even; 32 -> 192 at 28x28
+// slower (the expanded tensor stays in cache there). So: an expanded tensor of at least 48 MB
+// for stride 2, 96 MB for stride 1.
 extern "C" int tfhip_pointwise_depthwise_pays(int64_t batch, int64_t in_c, int64_t mid_c, int64_t stride,
                                               int64_t out_h, int64_t out_w) {
   if (!initialised() || batch <= 0 || out_h <= 0 || out_w <= 0 || mid_c <= 0 || mid_c > 0x7fffffff || in_c > 64 ||

@@ -2,8 +2,14 @@
 // (the first expansion convolutions of a mobile network: K = 32, 64, N = 6 K).
 //
 // With one to four k tiles the pipelined kernel of gemm_kernel.h is all prologue
-// and epilogue (measured: 6-10% slower than this kernel at K = 32 and 64; from
-// K = 96 on its overlap of fetches and matrix instructions wins, by 12-30%).
+// and epilogue (measured with launches back to back: 6-10% slower than this kernel
+// at K = 32 and 64; from K = 96 on its overlap of fetches and matrix instructions
+// wins, by 12-30%). Inside a network the picture turns: operands then come from
+// memory, not from the cache a repeated launch leaves them in, and waiting for one
+// long round trip before the first matrix instruction costs more than the tiled
+// kernel's staggered fetches (seven MobileNetV2 layers, in sequence: 99.7 us with
+// this kernel, 88.7 us with the tiled one). So it is only used when the "small_k"
+// knob asks for it.
 // Here a workgroup fetches ALL of its A rows and B columns at once (every load
 // of the tile in flight together: one memory round trip), stores them to LDS
 // in the x-major layout of gemm_kernel.h (row pitch k_pad + 8 floats, B transposed
