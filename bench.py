@@ -49,23 +49,21 @@ BATCH = 32
 # cannot be read from inside this script, so the table is refreshed by hand when a
 # kernel changes; a symbol that is not listed reports null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "conv_few_taps<7, 2>": 75272113,
-    "depthwise_3x3_rows<1, false>": 63685042,
-    "skinny_gemm_regs<1, 2, false>": 77140496,
-    "skinny_gemm_regs<6, 1, false>": 180978783,
-    "depthwise_3x3_rows<2, false>": 156010500,
-    "skinny_gemm<2, 4>": 64076321,
-    "skinny_gemm_regs<3, 1, true>": 75048140,
-    "gemm_kernel<32, 32, 32, 2, 2, 0, 1>": 17343831,
-    "small_k_gemm<64, 2, 2, 16>": 29245333,
-    "depthwise_3x3_flat<2, false>": 22006171,
-    "small_k_gemm<32, 2, 2, 16>": 19741783,
-    "depthwise_3x3_flat<1, false>": 17923334,
-    "gemm_kernel<64, 64, 16, 2, 2, 0, 1>": 20597758,
-    "gemm_kernel<32, 64, 32, 2, 2, 0, 1>": 12344502,
-    "mean_hw_vec": 8295726,
-    "gemm_finish": 896441,
-    "copy_to_host": 277490,
+    "conv_few_taps<7, 2>": 75272724,
+    "depthwise_3x3_rows<1, false>": 64029862,
+    "skinny_gemm_regs<1, 2, false>": 77141123,
+    "expand_dw_3x3<2, 1, false, 2>": 75185994,
+    "skinny_gemm<2, 4>": 64055529,
+    "skinny_gemm_regs<3, 1, true>": 75046363,
+    "expand_dw_3x3<2, 1, true, 2>": 29123101,
+    "gemm_kernel<32, 32, 32, 2, 2, 0, 1>": 17343914,
+    "gemm_kernel<64, 64, 16, 2, 2, 0, 1>": 18571414,
+    "depthwise_3x3_flat<2, false>": 22006284,
+    "depthwise_3x3_flat<1, false>": 17923385,
+    "gemm_kernel<32, 64, 32, 2, 2, 0, 1>": 12344544,
+    "mean_hw_vec": 8295765,
+    "gemm_finish": 896445,
+    "copy_to_host": 277491,
 }
 
 
