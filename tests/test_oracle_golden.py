@@ -386,3 +386,39 @@ def test_mean_hw_closed_form():
     got = orc.mean_hw(x)
     want = (x.astype(np.float64) / np.float64(np.float32(49))).astype(np.float32).astype(np.float64).sum(axis=(1, 2))
     np.testing.assert_array_equal(got, want.astype(np.float32))
+
+
+# -------------------------------------------- plan-level fusions of the device model
+
+def test_device_model_fuses_skip_connections_and_expansion_pairs():
+    """Host logic only (no GPU): which ops of the MobileNetV2 op list merge, and that the merged
+    lists still name every tensor the graph produces for its readers."""
+    from tfjs_amd import workloads
+    ops, shapes = workloads.mobilenet_v2_graph()
+    fused = workloads.DeviceMobileNetV2._fuse_residual_adds(ops)
+    assert len(ops) - len(fused) == 10 and sum(1 for op in fused if "residual" in op) == 10
+    for op in fused:
+        if "residual" in op:
+            # the projection convolution now yields the Add's tensor and reads the block input as well
+            assert op["kind"] == "conv" and op["act"] == "linear" and op["src"][1] == op["residual"]
+    assert not any(op["kind"] == "add" for op in fused)
+
+    class Lib:   # the native library's answer, replaced by a rule of thumb: only stride 2 at 56x56 or larger pays
+        asked = []
+
+        def tfhip_pointwise_depthwise_pays(self, batch, cin, mid, stride, out_h, out_w):
+            self.asked.append((cin, mid, stride, out_h))
+            return 1 if stride == 2 and out_h * stride >= 56 and cin <= 32 else 0
+    lib = Lib()
+    paired = workloads.DeviceMobileNetV2._fuse_expand_depthwise(fused, shapes, 32, lib)
+    # every expansion that feeds one depthwise stage is offered; the stem (3x3) and the first block (no expansion) are not
+    assert len(lib.asked) == 16 and (16, 96, 2, 56) in lib.asked and (24, 144, 2, 28) in lib.asked
+    pw = [op for op in paired if op["kind"] == "pwdw"]
+    assert [(shapes[op["w"]][2], shapes[op["w"]][3], op["stride"]) for op in pw] == [(16, 96, 2), (24, 144, 2)]
+    assert len(fused) - len(paired) == len(pw)
+    produced = {"input"}
+    for op in paired:
+        for s in (op["src"] if isinstance(op["src"], tuple) else (op["src"],)):
+            assert s in produced, "%s is read before it is produced" % s
+        produced.add(op["out"])
+    assert "logits" in produced

@@ -49,7 +49,6 @@ __device__ __forceinline__ float relu_like(float v) {
   return (ACT == TFHIP_RELU6 && t > 6.f) ? 6.f : t;
 }
 
-constexpr int kMaxTasks = 6;    // expansion tasks per wave and step
 constexpr int kMaxPasses = 4;   // depthwise pixels per lane and step
 
 // S: stride of the depthwise stage. K = 16 KF + (HALF ? 8 : 0) input channels.
