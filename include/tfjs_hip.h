@@ -121,9 +121,12 @@ int tfhip_graph_destroy(int graph_id);
  *   "no_skinny" (1: tiled GEMM also for tall products), "dw_flat" (1: the
  *   one-row-per-lane depthwise kernel always, 0: never), "skinny_regs" (0: the
  *   streaming GEMM always stages B in LDS), "small_k" (32 / 64: the one-shot GEMM for
- *   K <= 64 with that many rows per tile; unset or 0: never). TFHIP_TILE,
+ *   K <= 64 with that many rows per tile; unset or 0: never), "fuse_pw_dw"
+ *   (tfhip_pointwise_depthwise_pays: 1: yes for every shape the fused kernel
+ *   takes, 0: never). TFHIP_TILE,
  *   TFHIP_SPLITK, TFHIP_DW_ROWS, TFHIP_DW_HALO, TFHIP_NO_SKINNY, TFHIP_DW_FLAT,
- *   TFHIP_SKINNY_REGS, TFHIP_SMALL_K in the environment set them at tfhip_init(). */
+ *   TFHIP_SKINNY_REGS, TFHIP_SMALL_K, TFHIP_FUSE_PW_DW in the environment set them at
+ *   tfhip_init(). */
 int tfhip_set_launch_repeat(int n);
 int tfhip_last_kernel(char *name, size_t name_len);
 int tfhip_set_tuning(const char *name, int value);

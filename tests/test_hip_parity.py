@@ -637,6 +637,7 @@ def test_pointwise_depthwise_without_biases_and_unsupported_shapes(hip, orc):
     lib = capi.load_library()
     assert lib.tfhip_pointwise_depthwise_pays(32, 16, 96, 2, 56, 56) == 1
     assert lib.tfhip_pointwise_depthwise_pays(32, 24, 144, 2, 28, 28) == 1
+    assert lib.tfhip_pointwise_depthwise_pays(32, 24, 144, 1, 56, 56) == 1
     assert lib.tfhip_pointwise_depthwise_pays(32, 32, 192, 1, 28, 28) == 0     # taken, but the two kernels are faster
     assert lib.tfhip_pointwise_depthwise_pays(1, 16, 96, 2, 56, 56) == 0       # one image: the expanded tensor is small
     assert lib.tfhip_pointwise_depthwise_pays(32, 64, 384, 1, 14, 14) == 0     # too many input channels
@@ -772,7 +773,7 @@ def test_config4_mobilenet_v2_batch1_vs_oracle(hip, orc, tmp_path):
     for fuse in (True, False):
         m32 = workloads.DeviceMobileNetV2(str(tmp_path), 32, fuse_expand_depthwise=fuse)
         try:
-            assert sum(1 for op, _ in m32.plan if op["kind"] == "pwdw") == (2 if fuse else 0)
+            assert sum(1 for op, _ in m32.plan if op["kind"] == "pwdw") == (3 if fuse else 0)
             m32.set_input(x32)
             outs.append(m32.predict())
         finally:

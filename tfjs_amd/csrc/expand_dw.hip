@@ -78,9 +78,30 @@ __global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g) {
   const int cblocks = g.c / 16;
   const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)g.x, 0, (int)g.x_bytes, 0x00020000);
 
-  // weights of the expansion, transposed, and its bias
-  for (int k = 0; k < K; ++k) {
-    for (int col = threadIdx.x; col < g.c; col += 256) w1t[col * KP + k] = g.w1[k * g.c + col];
+  // weights of the expansion, transposed, and its bias: 16-byte loads along the channels, eight of
+  // a lane in flight at once (the fill is a memory round trip per batch of loads, paid by every
+  // workgroup before its first matrix instruction)
+  {
+    const int quads = g.c / 4, total = quads * K;   // w1 is [K][c]
+    for (int i0 = threadIdx.x; i0 < total; i0 += 256 * 8) {
+      float4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * 256;
+        v[u] = *reinterpret_cast<const float4 *>(g.w1 + 4 * (i < total ? i : total - 1));
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * 256;
+        if (i < total) {
+          const int k = i / quads, col = 4 * (i - k * quads);
+          w1t[(col + 0) * KP + k] = v[u].x;
+          w1t[(col + 1) * KP + k] = v[u].y;
+          w1t[(col + 2) * KP + k] = v[u].z;
+          w1t[(col + 3) * KP + k] = v[u].w;
+        }
+      }
+    }
   }
   for (int i = threadIdx.x; i < g.c; i += 256) b1s[i] = g.b1 ? g.b1[i] : 0.f;
 
@@ -325,7 +346,8 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
   g.act1 = pw_activation; g.act2 = dw_activation;
   g.x_bytes = (unsigned)(batch * in_h * in_w * in_c * 4);
   size_t lds_bytes = 0;
-  const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(dw_filter) % 16 == 0 &&
+  const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(pw_filter) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(dw_filter) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
                        (dw_bias == nullptr || reinterpret_cast<uintptr_t>(dw_bias) % 16 == 0);
   const bool same_relu = pw_activation == dw_activation && (pw_activation == TFHIP_RELU || pw_activation == TFHIP_RELU6);
@@ -349,11 +371,12 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
 }
 
 // 1 when tfhip_fused_pointwise_depthwise takes this shape and is expected to beat the two
-// kernels, else 0. Measured at batch 32 (in sequence, where the expanded tensor really goes
-// to memory and back): 16 -> 96 channels at 112x112, stride 2, 46 us against 91 us; 24 -> 144
-// at 56x56, stride 2, 33 against 36; the same with stride 1 about even; 32 -> 192 at 28x28
-// slower (the expanded tensor stays in cache there). So: an expanded tensor of at least 48 MB
-// for stride 2, 96 MB for stride 1.
+// kernels, else 0. Measured at batch 32 in sequence, where the expanded tensor really goes to
+// memory and back (fused against expansion + depthwise stage): 16 -> 96 channels at 112x112,
+// stride 2: 43 us against 38 + 55; 24 -> 144 at 56x56, stride 2: 27 against 19 + 18, stride 1:
+// 49 against 19 + 36; 32 -> 192 at 28x28, where the expanded tensor (19 MB) stays in cache:
+// 24 and 27 against 27 and 25 at stride 1, 38 against 21 at stride 2. So: an expanded
+// tensor of at least 48 MB.
 extern "C" int tfhip_pointwise_depthwise_pays(int64_t batch, int64_t in_c, int64_t mid_c, int64_t stride,
                                               int64_t out_h, int64_t out_w) {
   if (!initialised() || batch <= 0 || out_h <= 0 || out_w <= 0 || mid_c <= 0 || mid_c > 0x7fffffff || in_c > 64 ||
@@ -364,6 +387,7 @@ extern "C" int tfhip_pointwise_depthwise_pays(int64_t batch, int64_t in_c, int64
   g.batch = (int)batch; g.cin = (int)in_c; g.c = (int)mid_c; g.out_h = (int)out_h; g.out_w = (int)out_w;
   size_t lds_bytes = 0;
   if (!plan_expand_dw(g, (int)stride, &lds_bytes)) return 0;
+  if (tuning(kTuneFusePwDw) >= 0) return tuning(kTuneFusePwDw) > 0 ? 1 : 0;   // knob: always / never
   const int64_t expanded_bytes = batch * out_h * stride * out_w * stride * mid_c * 4;
-  return expanded_bytes >= (stride == 2 ? 48LL : 96LL) * 1000 * 1000 ? 1 : 0;
+  return expanded_bytes >= 48LL * 1000 * 1000 ? 1 : 0;
 }

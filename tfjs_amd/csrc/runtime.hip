@@ -106,14 +106,14 @@ void note_kernel(const char *fmt, ...) {
 
 int launch_repeat() { return g_repeat; }
 
-int g_tuning[kTuneCount] = {-1, -1, -1, -1, -1, -1, -1, -1};
-const char *const kTuningNames[kTuneCount] = {"tile", "splitk", "dw_rows", "dw_halo", "no_skinny", "dw_flat", "skinny_regs", "small_k"};
+int g_tuning[kTuneCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1};
+const char *const kTuningNames[kTuneCount] = {"tile", "splitk", "dw_rows", "dw_halo", "no_skinny", "dw_flat", "skinny_regs", "small_k", "fuse_pw_dw"};
 int tuning(int key) { return g_tuning[key]; }
 
 void read_tuning_from_environment() {
   static const char *const env_names[kTuneCount] = {"TFHIP_TILE", "TFHIP_SPLITK", "TFHIP_DW_ROWS", "TFHIP_DW_HALO",
                                                     "TFHIP_NO_SKINNY", "TFHIP_DW_FLAT", "TFHIP_SKINNY_REGS",
-                                                    "TFHIP_SMALL_K"};
+                                                    "TFHIP_SMALL_K", "TFHIP_FUSE_PW_DW"};
   for (int i = 0; i < kTuneCount; ++i) {
     const char *e = getenv(env_names[i]);
     g_tuning[i] = e ? atoi(e) : -1;
