@@ -237,6 +237,26 @@ int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_filter,
 int tfhip_pointwise_depthwise_pays(int64_t batch, int64_t in_c, int64_t mid_c,
                                         int64_t stride, int64_t out_h, int64_t out_w);
 
+/* The same with a convolution over few input channels as the first stage (a network's
+ * stem followed by the first block's depthwise stage): x [batch,in_h,in_w,in_c] with
+ * in_c <= 4, filter [f_h,f_w,in_c,mid_c] of at most 36 taps (f_h * f_w * in_c), its
+ * stride and padding, the intermediate tensor [batch,mid_h,mid_w,mid_c], then the
+ * depthwise 3x3 stage as above. The nodes it stands for are a FusedConv2D and the
+ * FusedDepthwiseConv2dNative that is its only reader; the result equals
+ * tfhip_fused_conv2d followed by tfhip_fused_depthwise_conv2d bit for bit.
+ * tfhip_conv2d_depthwise_pays: as tfhip_pointwise_depthwise_pays. */
+int tfhip_fused_conv2d_depthwise(const float *x, const float *filter, const float *bias,
+                                 int activation, const float *dw_filter,
+                                 const float *dw_bias, int dw_activation, float *y,
+                                 int64_t batch, int64_t in_h, int64_t in_w, int64_t in_c,
+                                 int64_t f_h, int64_t f_w, int64_t mid_c, int64_t stride,
+                                 int64_t pad_top, int64_t pad_left, int64_t mid_h,
+                                 int64_t mid_w, int64_t dw_stride, int64_t dw_pad_top,
+                                 int64_t dw_pad_left, int64_t out_h, int64_t out_w);
+int tfhip_conv2d_depthwise_pays(int64_t batch, int64_t in_c, int64_t f_h, int64_t f_w,
+                                int64_t mid_c, int64_t mid_h, int64_t mid_w,
+                                int64_t dw_stride, int64_t out_h, int64_t out_w);
+
 /* ---- weight dequantisation on load -----------------------------------------
  * The quantization branch of decodeWeight, tfjs-core/src/io/io_utils.ts:196-251,
  * which the reference runs in JavaScript before backend.write(). `q` points at

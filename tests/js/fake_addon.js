@@ -58,6 +58,7 @@ module.exports = {
   eventElapsed() { return 0; },
   setLaunchRepeat() {},
   lastKernel() { return 'fake'; },
+  setTuning() {},
   fusedMatMul() { record('fusedMatMul', arguments); },
   fusedConv2D() { record('fusedConv2D', arguments); },
   fusedDepthwiseConv2D() { record('fusedDepthwiseConv2D', arguments); },
@@ -67,6 +68,8 @@ module.exports = {
   meanHW() { record('meanHW', arguments); },
   fusedPointwiseDepthwise() { record('fusedPointwiseDepthwise', arguments); },
   pointwiseDepthwisePays(batch) { return module.exports.paysFromBatch != null && batch >= module.exports.paysFromBatch; },
+  fusedConv2DDepthwise() { record('fusedConv2DDepthwise', arguments); },
+  conv2dDepthwisePays(batch) { return module.exports.paysFromBatch != null && batch >= module.exports.paysFromBatch; },
   paysFromBatch: null,   // tests set the batch size from which the fused kernel "pays"
   copy() { record('copy', arguments); },
   captureBegin() { record('captureBegin', arguments); },

@@ -252,6 +252,23 @@ h.test('FusedPointwiseDepthwiseConv2D: expansion + depthwise stage in one launch
     h.assertBitsEqual(fused.dataSync(), two.dataSync());
     tf.dispose([x, filter, bias, dwFilter, dwBias, fused, expanded, two]);
   });
+  // a stem: 3x3 stride 2 over three channels, then the depthwise stage; fused at batch 32, two kernels at batch 2
+  [32, 2].forEach(n => {
+    const x = tf.tensor(rnd(n * 64 * 64 * 3), [n, 64, 64, 3]);
+    const filter = tf.tensor(rnd(27 * 32), [3, 3, 3, 32]), bias = tf.tensor(rnd(32), [32]);
+    const dwFilter = tf.tensor(rnd(9 * 32), [3, 3, 32, 1]), dwBias = tf.tensor(rnd(32), [32]);
+    addon.setTuning('fuse_pw_dw', n === 32 ? 1 : -1);   // (64x64 images are below the size from which it pays)
+    const fused = tf.engine().runKernel('FusedPointwiseDepthwiseConv2D', {x, filter, bias, dwFilter, dwBias},
+                                        {strides: [1, 1], pad: 'same', activation: 'relu6', convStrides: [2, 2], convPad: 'same'});
+    h.assertEqual(addon.lastKernel().startsWith('expand_dw_3x3<1, stem 7'), n === 32);
+    addon.setTuning('fuse_pw_dw', -1);
+    const mid = tf.fused.conv2d({x, filter, strides: [2, 2], pad: 'same', dataFormat: 'NHWC', dilations: [1, 1], bias, activation: 'relu6'});
+    const two = tf.fused.depthwiseConv2d({x: mid, filter: dwFilter, strides: [1, 1], pad: 'same', dataFormat: 'NHWC',
+                                          dilations: [1, 1], bias: dwBias, activation: 'relu6'});
+    h.assertEqual(fused.shape, [n, 32, 32, 32]);
+    h.assertBitsEqual(fused.dataSync(), two.dataSync());
+    tf.dispose([x, filter, bias, dwFilter, dwBias, fused, mid, two]);
+  });
   h.assertEqual(tf.backend().numDataIds(), before);
   const dir = process.env.TFJS_HIP_TEST_MODEL_DIR;
   const io = {decodeWeights: hip.decodeWeights};
@@ -259,7 +276,7 @@ h.test('FusedPointwiseDepthwiseConv2D: expansion + depthwise stage in one launch
   const x = tf.tensor(mobilenet.syntheticInput(32, 7), [32, 224, 224, 3]);
   const a = fusedModel.predict(x), b = plainModel.predict(x);
   const steps = model => Array.from(model.plans.values())[0].steps.filter(s => s.kind === 'op');
-  h.assertEqual(steps(plainModel).length - steps(fusedModel).length, 16, 'every expansion but the first block, which has none');
+  h.assertEqual(steps(plainModel).length - steps(fusedModel).length, 17, 'the stem with the first depthwise stage, and every expansion');
   h.assertBitsEqual(a.dataSync(), b.dataSync());
   tf.dispose([a, b, x]);
   fusedModel.dispose();

@@ -623,6 +623,36 @@ def test_pointwise_depthwise_fused(hip, orc, case):
         assert_parity(got, two, 1e-5)
 
 
+STEM_DW_CASES = [
+    # x shape, filter shape, conv stride, conv pad, depthwise stride, depthwise pad, activation
+    ((3, 64, 64, 3), (3, 3, 3, 32), 2, "same", 1, "same", "relu6"),        # MobileNetV2's stem and first depthwise stage
+    ((2, 33, 47, 3), (3, 3, 3, 32), 2, "same", 2, "same", "relu"),         # odd sizes, stride 2 twice
+    ((2, 20, 30, 1), (3, 3, 1, 16), 1, "valid", 1, "same", "relu6"),       # 9 taps: three k steps, one channel block
+    ((1, 18, 18, 4), (3, 3, 4, 48), 1, "same", 1, "valid", "relu6"),       # 36 taps: nine k steps
+    ((2, 24, 40, 2), (1, 7, 2, 64), 1, [[0, 0], [0, 0], [3, 3], [0, 0]], 2, "same", "relu6"),   # 1x7 filter, explicit padding
+]
+
+
+@pytest.mark.parametrize("case", STEM_DW_CASES, ids=[str(i) for i in range(len(STEM_DW_CASES))])
+def test_conv2d_depthwise_fused(hip, orc, case):
+    xs, fs, stride, pad, dw_stride, dw_pad, act = case
+    rng = np.random.default_rng(sum(xs) + sum(fs))
+    x = rng.uniform(-1, 1, xs).astype(np.float32)
+    w1 = rng.normal(0, 0.5, fs).astype(np.float32)
+    b1 = rng.uniform(-1, 2, (fs[3],)).astype(np.float32)
+    w2 = rng.normal(0, 0.5, (3, 3, fs[3], 1)).astype(np.float32)
+    b2 = rng.uniform(-1, 1, (fs[3],)).astype(np.float32)
+    got = hip.fused_conv2d_depthwise(x, w1, w2, strides=stride, pad=pad, dw_strides=dw_stride, dw_pad=dw_pad, bias=b1,
+                                     dw_bias=b2, activation=act)
+    mid = hip.fused_conv2d(x, w1, strides=stride, pad=pad, bias=b1, activation=act)
+    two = hip.fused_depthwise_conv2d(mid, w2, strides=dw_stride, pad=dw_pad, bias=b2, activation=act)
+    want = orc.fused_depthwise_conv2d(orc.fused_conv2d(x, w1, strides=stride, pad=pad, bias=b1, activation=act), w2,
+                                      strides=dw_stride, pad=dw_pad, bias=b2, activation=act)
+    assert_parity(got, want)
+    # the separate stem kernels feed the matrix cores in the same order: the same bits
+    np.testing.assert_array_equal(got.view(np.uint32), two.view(np.uint32))
+
+
 def test_pointwise_depthwise_without_biases_and_unsupported_shapes(hip, orc):
     from tfjs_amd import capi
     rng = np.random.default_rng(77)
@@ -773,7 +803,7 @@ def test_config4_mobilenet_v2_batch1_vs_oracle(hip, orc, tmp_path):
     for fuse in (True, False):
         m32 = workloads.DeviceMobileNetV2(str(tmp_path), 32, fuse_expand_depthwise=fuse)
         try:
-            assert sum(1 for op, _ in m32.plan if op["kind"] == "pwdw") == (3 if fuse else 0)
+            assert sum(1 for op, _ in m32.plan if op["kind"] in ("pwdw", "cvdw")) == (4 if fuse else 0)
             m32.set_input(x32)
             outs.append(m32.predict())
         finally:

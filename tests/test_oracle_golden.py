@@ -409,13 +409,19 @@ def test_device_model_fuses_skip_connections_and_expansion_pairs():
         def tfhip_pointwise_depthwise_pays(self, batch, cin, mid, stride, out_h, out_w):
             self.asked.append((cin, mid, stride, out_h))
             return 1 if stride == 2 and out_h * stride >= 56 and cin <= 32 else 0
+
+        def tfhip_conv2d_depthwise_pays(self, batch, cin, fh, fw, mid, mid_h, mid_w, stride, out_h, out_w):
+            self.stem = (cin, fh, fw, mid, mid_h, stride, out_h)
+            return 1
     lib = Lib()
     paired = workloads.DeviceMobileNetV2._fuse_expand_depthwise(fused, shapes, 32, lib)
     # every expansion that feeds one depthwise stage is offered; the stem (3x3) and the first block (no expansion) are not
     assert len(lib.asked) == 16 and (16, 96, 2, 56) in lib.asked and (24, 144, 2, 28) in lib.asked
+    assert lib.stem == (3, 3, 3, 32, 112, 1, 112)   # the stem convolution and the first block's depthwise stage
+    assert paired[0]["kind"] == "cvdw" and paired[0]["conv_stride"] == 2 and paired[0]["src"] == "input"
     pw = [op for op in paired if op["kind"] == "pwdw"]
     assert [(shapes[op["w"]][2], shapes[op["w"]][3], op["stride"]) for op in pw] == [(16, 96, 2), (24, 144, 2)]
-    assert len(fused) - len(paired) == len(pw)
+    assert len(fused) - len(paired) == len(pw) + 1
     produced = {"input"}
     for op in paired:
         for s in (op["src"] if isinstance(op["src"], tuple) else (op["src"],)):

@@ -54,6 +54,9 @@ SIGNATURES = {
     "tfhip_fused_pointwise_depthwise": [c_f32p, c_f32p, c_f32p, ctypes.c_int, c_f32p, c_f32p, ctypes.c_int, c_f32p] +
                                        [c_i64] * 10,
     "tfhip_pointwise_depthwise_pays": [c_i64] * 6,
+    "tfhip_fused_conv2d_depthwise": [c_f32p, c_f32p, c_f32p, ctypes.c_int, c_f32p, c_f32p, ctypes.c_int, c_f32p] +
+                                    [c_i64] * 17,
+    "tfhip_conv2d_depthwise_pays": [c_i64] * 10,
     "tfhip_fused_depthwise_conv2d": [c_f32p, c_f32p, c_f32p] + [c_i64] * 15 + [c_f32p, c_i64p, ctypes.c_int,
                                                                                 c_f32p, c_i64p, ctypes.c_double],
     "tfhip_dequant_affine": [ctypes.c_void_p, ctypes.c_int, c_i64, ctypes.c_double, ctypes.c_double,

@@ -41,6 +41,17 @@ struct ExpandDwArgs {
   int act1, act2;                  // both relu or both relu6
   int tile_w, tiles_w, rows, chunks_h, pblocks, pitch;
   unsigned x_bytes;
+  // first stage a convolution over few input channels instead of a 1x1 one (TAPS > 0): x is
+  // [batch, xh, xw, xc], the "expanded" tensor [batch, in_h, in_w, c] is its output
+  int xh, xw, xc, conv_stride, conv_pad_top, conv_pad_left, k;
+};
+
+// Tap k = (fr * f_w + fs) * xc + ch of the first-stage filter: row / column relative to a
+// window's top-left input element, and byte offset from it (rows beyond K: a row no image has).
+constexpr int kMaxStemTaps = 36;
+struct StemTaps {
+  int dh[kMaxStemTaps], dw[kMaxStemTaps];
+  unsigned off_bytes[kMaxStemTaps];
 };
 
 template <int ACT>
@@ -53,9 +64,13 @@ constexpr int kMaxPasses = 4;   // depthwise pixels per lane and step
 
 // S: stride of the depthwise stage. K = 16 KF + (HALF ? 8 : 0) input channels.
 // ACT: the activation of both stages, relu or relu6.
-template <int S, int KF, bool HALF, int ACT>
-__global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g) {
-  constexpr int K = 16 * KF + (HALF ? 8 : 0);
+// TAPS > 0: the first stage is a convolution of at most 4 TAPS taps (filter height x width x
+// input channels, a network stem) gathered element by element with the lane layout and
+// instruction order of conv_few_taps (lane (grp, r) feeds tap 4 t + grp in k step t); KF and
+// HALF are then unused.
+template <int S, int KF, bool HALF, int ACT, int TAPS>
+__global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g, StemTaps taps) {
+  constexpr int K = TAPS > 0 ? 4 * TAPS : 16 * KF + (HALF ? 8 : 0);   // k extent of the weights in LDS
   constexpr int KP = K + 4;             // floats per column of the transposed weights in LDS
   constexpr int RING = 3 + S;
   extern __shared__ float lds[];
@@ -81,8 +96,12 @@ __global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g) {
   // weights of the expansion, transposed, and its bias: 16-byte loads along the channels, eight of
   // a lane in flight at once (the fill is a memory round trip per batch of loads, paid by every
   // workgroup before its first matrix instruction)
+  if (TAPS > 0) {   // rows beyond the filter's taps multiply zeros
+    for (int i = threadIdx.x; i < g.c * KP; i += 256) w1t[i] = 0.f;
+    __syncthreads();
+  }
   {
-    const int quads = g.c / 4, total = quads * K;   // w1 is [K][c]
+    const int quads = g.c / 4, total = quads * (TAPS > 0 ? g.k : K);   // w1 is [K][c]
     for (int i0 = threadIdx.x; i0 < total; i0 += 256 * 8) {
       float4 v[8];
 #pragma unroll
@@ -135,11 +154,34 @@ __global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g) {
   struct AFrag {
     float4 full[KF > 0 ? KF : 1];
     float2 half;
+    float tap[TAPS > 0 ? TAPS : 1];
   };
+  int tap_dh[TAPS > 0 ? TAPS : 1], tap_dw[TAPS > 0 ? TAPS : 1];
+  unsigned tap_off[TAPS > 0 ? TAPS : 1];
+  if (TAPS > 0) {
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t) {
+      tap_dh[t] = taps.dh[4 * t + grp];
+      tap_dw[t] = taps.dw[4 * t + grp];
+      tap_off[t] = taps.off_bytes[4 * t + grp];
+    }
+  }
   auto load_a = [&](AFrag &a, int erow, int pb) __attribute__((always_inline)) {
     const int ih = ih0 + erow, iw = iw0 + 16 * pb + r;
     const bool inside = ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
-    const unsigned base = (unsigned)((((long long)n * g.in_h + ih) * g.in_w + iw) * K * 4);
+    if (TAPS > 0) {
+      // the window of first-stage output pixel (ih, iw); its top-left element may lie before
+      // the image, the sum with an inside tap's offset is exact modulo 2^32
+      const int xh0 = ih * g.conv_stride - g.conv_pad_top, xw0 = iw * g.conv_stride - g.conv_pad_left;
+      const unsigned base = (unsigned)((((long long)n * g.xh + xh0) * g.xw + xw0) * g.xc * 4);
+#pragma unroll
+      for (int t = 0; t < TAPS; ++t) {
+        const bool ok = inside && (unsigned)(xh0 + tap_dh[t]) < (unsigned)g.xh && (unsigned)(xw0 + tap_dw[t]) < (unsigned)g.xw;
+        a.tap[t] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rx, (int)(ok ? base + tap_off[t] : kNoOff), 0, 0));
+      }
+      return;
+    }
+    const unsigned base = (unsigned)((((long long)n * g.in_h + ih) * g.in_w + iw) * (16 * KF + (HALF ? 8 : 0)) * 4);
 #pragma unroll
     for (int t = 0; t < KF; ++t) {
       const auto v = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)(inside ? base + (16 * t + 4 * grp) * 4 : kNoOff), 0, 0);
@@ -159,15 +201,21 @@ __global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g) {
     const float *bias = b1s + 4 * grp;
     for (int cb = cb_lo; cb < cb_hi; ++cb) {
       float4_t acc = *reinterpret_cast<const float4_t *>(bias + 16 * cb);
+      if (TAPS > 0) {
 #pragma unroll
-      for (int t = 0; t < KF; ++t) {
+        for (int t = 0; t < TAPS; ++t) {
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w1t[(16 * cb + r) * KP + 4 * t + grp], a.tap[t], acc, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < (TAPS > 0 ? 0 : KF); ++t) {
         const float4 b = *reinterpret_cast<const float4 *>(wcol + 16 * cb * KP + 16 * t);
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.x, a.full[t].x, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.y, a.full[t].y, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.z, a.full[t].z, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.w, a.full[t].w, acc, 0, 0, 0);
       }
-      if (HALF) {
+      if (HALF && TAPS == 0) {
         const float2 b = *reinterpret_cast<const float2 *>(w1t + (16 * cb + r) * KP + 16 * KF + 2 * grp);
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.x, a.half.x, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b.y, a.half.y, acc, 0, 0, 0);
@@ -254,32 +302,44 @@ __global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g) {
   }
 }
 
-template <int S, int KF, bool HALF, int ACT>
-int launch_expand_dw_act(const ExpandDwArgs &g, size_t lds_bytes) {
+template <int S, int KF, bool HALF, int ACT, int TAPS>
+int launch_expand_dw_act(const ExpandDwArgs &g, const StemTaps &taps, size_t lds_bytes) {
   static bool raised = false;   // dynamic LDS above the default limit needs the attribute once per instantiation
   if (!raised) {
-    TFHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(expand_dw_3x3<S, KF, HALF, ACT>),
+    TFHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(expand_dw_3x3<S, KF, HALF, ACT, TAPS>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     raised = true;
   }
   const long long wgs = (long long)g.batch * g.chunks_h * g.tiles_w;
-  note_kernel("expand_dw_3x3<%d, %d, %s, %d>", S, KF, HALF ? "true" : "false", ACT);
-  TFHIP_LAUNCH((expand_dw_3x3<S, KF, HALF, ACT><<<dim3((unsigned)wgs), dim3(256), lds_bytes, stream()>>>(g)));
+  if (TAPS > 0) {
+    note_kernel("expand_dw_3x3<%d, stem %d, %d>", S, TAPS, ACT);
+  } else {
+    note_kernel("expand_dw_3x3<%d, %d, %s, %d>", S, KF, HALF ? "true" : "false", ACT);
+  }
+  TFHIP_LAUNCH((expand_dw_3x3<S, KF, HALF, ACT, TAPS><<<dim3((unsigned)wgs), dim3(256), lds_bytes, stream()>>>(g, taps)));
   return kOk;
 }
 
 template <int S, int KF, bool HALF>
 int launch_expand_dw(const ExpandDwArgs &g, size_t lds_bytes) {
-  if (g.act1 == TFHIP_RELU6) return launch_expand_dw_act<S, KF, HALF, TFHIP_RELU6>(g, lds_bytes);
-  return launch_expand_dw_act<S, KF, HALF, TFHIP_RELU>(g, lds_bytes);
+  const StemTaps none = {};
+  if (g.act1 == TFHIP_RELU6) return launch_expand_dw_act<S, KF, HALF, TFHIP_RELU6, 0>(g, none, lds_bytes);
+  return launch_expand_dw_act<S, KF, HALF, TFHIP_RELU, 0>(g, none, lds_bytes);
+}
+
+template <int S, int TAPS>
+int launch_stem_dw(const ExpandDwArgs &g, const StemTaps &taps, size_t lds_bytes) {
+  if (g.act1 == TFHIP_RELU6) return launch_expand_dw_act<S, 0, false, TFHIP_RELU6, TAPS>(g, taps, lds_bytes);
+  return launch_expand_dw_act<S, 0, false, TFHIP_RELU, TAPS>(g, taps, lds_bytes);
 }
 
 }  // namespace
 
 // Fills the tiling of `g` for the fused kernel; false when the shape is one it does not take.
-bool plan_expand_dw(ExpandDwArgs &g, int stride, size_t *lds_bytes) {
-  const int K = g.cin;
-  if (!(K == 8 || K == 16 || K == 24 || K == 32) || g.c % 16 != 0 || g.c > 256 || (stride != 1 && stride != 2)) return false;
+// K: the k extent of the first stage's weights in LDS (input channels of a 1x1 first stage, 4 x k
+// steps of a few-channel convolution).
+bool plan_expand_dw(ExpandDwArgs &g, int stride, int K, size_t *lds_bytes) {
+  if (g.c % 16 != 0 || g.c > 256 || (stride != 1 && stride != 2)) return false;
   const int cq = g.c / 4, cblocks = g.c / 16;
   const int groups = 256 / cq;
   if (groups < 1) return false;
@@ -293,7 +353,9 @@ bool plan_expand_dw(ExpandDwArgs &g, int stride, size_t *lds_bytes) {
     const size_t bytes = ((size_t)(3 + stride) * 16 * pblocks * (g.c + 4) + (size_t)g.c * (K + 4) + g.c) * sizeof(float);
     const bool fits = pblocks <= 2 && (tile_w + groups - 1) / groups <= kMaxPasses && bytes <= 156 * 1024;
     if (!fits) continue;
-    if (pick == 0 || (g.out_w % pick != 0 && g.out_w % tile_w == 0)) pick = tile_w;
+    // (a narrow tile that gives the four waves fewer than four blocks per step only when nothing else fits)
+    const bool idle_waves = stride * pblocks * cblocks < 4;
+    if (pick == 0 || (g.out_w % pick != 0 && g.out_w % tile_w == 0 && !idle_waves)) pick = tile_w;
   }
   if (pick == 0) return false;
   g.tile_w = pick;
@@ -351,7 +413,8 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
                        reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
                        (dw_bias == nullptr || reinterpret_cast<uintptr_t>(dw_bias) % 16 == 0);
   const bool same_relu = pw_activation == dw_activation && (pw_activation == TFHIP_RELU || pw_activation == TFHIP_RELU6);
-  if (!aligned || !same_relu || !plan_expand_dw(g, (int)stride, &lds_bytes)) {
+  const bool k_ok = in_c == 8 || in_c == 16 || in_c == 24 || in_c == 32;
+  if (!aligned || !same_relu || !k_ok || !plan_expand_dw(g, (int)stride, (int)in_c, &lds_bytes)) {
     return fail(kBadArgument,
                 "tfhip_fused_pointwise_depthwise: form not taken by the fused kernel (in_c 8/16/24/32, mid_c a "
                 "multiple of 16 up to 256, stride 1 or 2, both activations relu or both relu6, 16-byte aligned "
@@ -386,8 +449,100 @@ extern "C" int tfhip_pointwise_depthwise_pays(int64_t batch, int64_t in_c, int64
   ExpandDwArgs g = {};
   g.batch = (int)batch; g.cin = (int)in_c; g.c = (int)mid_c; g.out_h = (int)out_h; g.out_w = (int)out_w;
   size_t lds_bytes = 0;
-  if (!plan_expand_dw(g, (int)stride, &lds_bytes)) return 0;
+  const bool k_ok = in_c == 8 || in_c == 16 || in_c == 24 || in_c == 32;
+  if (!k_ok || !plan_expand_dw(g, (int)stride, (int)in_c, &lds_bytes)) return 0;
   if (tuning(kTuneFusePwDw) >= 0) return tuning(kTuneFusePwDw) > 0 ? 1 : 0;   // knob: always / never
   const int64_t expanded_bytes = batch * out_h * stride * out_w * stride * mid_c * 4;
   return expanded_bytes >= 48LL * 1000 * 1000 ? 1 : 0;
+}
+
+namespace {
+
+// k steps of the instantiated few-channel first stages for a filter of `taps` taps (0: none)
+int stem_k_steps(int64_t taps) { return taps <= 12 ? 3 : (taps <= 28 ? 7 : (taps <= 36 ? 9 : 0)); }
+
+}  // namespace
+
+extern "C" int tfhip_fused_conv2d_depthwise(const float *x, const float *filter, const float *bias, int activation,
+                                            const float *dw_filter, const float *dw_bias, int dw_activation, float *y,
+                                            int64_t batch, int64_t in_h, int64_t in_w, int64_t in_c, int64_t f_h,
+                                            int64_t f_w, int64_t mid_c, int64_t stride, int64_t pad_top,
+                                            int64_t pad_left, int64_t mid_h, int64_t mid_w, int64_t dw_stride,
+                                            int64_t dw_pad_top, int64_t dw_pad_left, int64_t out_h, int64_t out_w) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_ARG(batch >= 0 && in_h > 0 && in_w > 0 && in_c > 0 && f_h > 0 && f_w > 0 && mid_c > 0 && stride > 0 &&
+                      mid_h >= 0 && mid_w >= 0 && dw_stride > 0 && out_h >= 0 && out_w >= 0 && pad_top >= 0 &&
+                      pad_left >= 0 && dw_pad_top >= 0 && dw_pad_left >= 0,
+                  "tfhip_fused_conv2d_depthwise: bad dimension");
+  const int64_t lim = 0x7fffffff;
+  TFHIP_CHECK_ARG(batch * in_h * in_w * in_c < lim && batch * mid_h * mid_w * mid_c < lim && batch * out_h * out_w * mid_c < lim,
+                  "tfhip_fused_conv2d_depthwise: tensor exceeds the supported range");
+  TFHIP_CHECK_ARG(activation >= TFHIP_LINEAR && activation <= TFHIP_ELU && dw_activation >= TFHIP_LINEAR &&
+                      dw_activation <= TFHIP_ELU,
+                  "tfhip_fused_conv2d_depthwise: unknown activation");
+  if (batch * out_h * out_w == 0) return kOk;
+  const int64_t K = f_h * f_w * in_c;
+  TFHIP_CHECK_RANGE(x, batch * in_h * in_w * in_c, 4, "x");
+  TFHIP_CHECK_RANGE(filter, K * mid_c, 4, "filter");
+  TFHIP_CHECK_RANGE(dw_filter, 9 * mid_c, 4, "dw_filter");
+  if (bias) TFHIP_CHECK_RANGE(bias, mid_c, 4, "bias");
+  if (dw_bias) TFHIP_CHECK_RANGE(dw_bias, mid_c, 4, "dw_bias");
+  TFHIP_CHECK_RANGE(y, batch * out_h * out_w * mid_c, 4, "y");
+
+  ExpandDwArgs g = {};
+  g.x = x; g.w1 = filter; g.b1 = bias; g.w2 = dw_filter; g.b2 = dw_bias; g.y = y;
+  g.batch = (int)batch; g.in_h = (int)mid_h; g.in_w = (int)mid_w; g.cin = (int)in_c; g.c = (int)mid_c;
+  g.pad_top = (int)dw_pad_top; g.pad_left = (int)dw_pad_left; g.out_h = (int)out_h; g.out_w = (int)out_w;
+  g.act1 = activation; g.act2 = dw_activation;
+  g.x_bytes = (unsigned)(batch * in_h * in_w * in_c * 4);
+  g.xh = (int)in_h; g.xw = (int)in_w; g.xc = (int)in_c; g.conv_stride = (int)stride;
+  g.conv_pad_top = (int)pad_top; g.conv_pad_left = (int)pad_left; g.k = (int)K;
+  const int k_steps = in_c <= 4 ? stem_k_steps(K) : 0;
+  size_t lds_bytes = 0;
+  const bool aligned = reinterpret_cast<uintptr_t>(filter) % 16 == 0 && reinterpret_cast<uintptr_t>(dw_filter) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+                       (dw_bias == nullptr || reinterpret_cast<uintptr_t>(dw_bias) % 16 == 0);
+  const bool same_relu = activation == dw_activation && (activation == TFHIP_RELU || activation == TFHIP_RELU6);
+  if (!aligned || !same_relu || k_steps == 0 || batch * in_h * in_w * in_c * 4 > 0xfffffffeLL ||
+      !plan_expand_dw(g, (int)dw_stride, 4 * k_steps, &lds_bytes)) {
+    return fail(kBadArgument,
+                "tfhip_fused_conv2d_depthwise: form not taken by the fused kernel (at most 4 input channels and 36 "
+                "filter taps, mid_c a multiple of 16 up to 256, depthwise stride 1 or 2, both activations relu or "
+                "both relu6, 16-byte aligned operands); run the two convolutions");
+  }
+  StemTaps taps;
+  for (int k = 0; k < kMaxStemTaps; ++k) {
+    const int tap = k / (int)in_c, ch = k - tap * (int)in_c;
+    const int fr = tap / (int)f_w, fs = tap - fr * (int)f_w;
+    taps.dh[k] = k < K ? fr : (1 << 28);
+    taps.dw[k] = fs;
+    taps.off_bytes[k] = (unsigned)((((long long)fr * in_w + fs) * in_c + ch) * 4);
+  }
+  const int key = (int)dw_stride * 10 + k_steps;
+  switch (key) {
+    case 13: return launch_stem_dw<1, 3>(g, taps, lds_bytes);
+    case 17: return launch_stem_dw<1, 7>(g, taps, lds_bytes);
+    case 19: return launch_stem_dw<1, 9>(g, taps, lds_bytes);
+    case 23: return launch_stem_dw<2, 3>(g, taps, lds_bytes);
+    case 27: return launch_stem_dw<2, 7>(g, taps, lds_bytes);
+    default: return launch_stem_dw<2, 9>(g, taps, lds_bytes);
+  }
+}
+
+// 1 when tfhip_fused_conv2d_depthwise takes this shape and is expected to beat the two kernels (the
+// tensor between the stages of at least 48 MB, as for the pointwise first stage), else 0.
+extern "C" int tfhip_conv2d_depthwise_pays(int64_t batch, int64_t in_c, int64_t f_h, int64_t f_w, int64_t mid_c,
+                                           int64_t mid_h, int64_t mid_w, int64_t dw_stride, int64_t out_h,
+                                           int64_t out_w) {
+  if (!initialised() || batch <= 0 || out_h <= 0 || out_w <= 0 || mid_c <= 0 || mid_c > 0x7fffffff || in_c <= 0 ||
+      in_c > 4 || f_h <= 0 || f_w <= 0 || f_h * f_w * in_c > 36 || batch > 0x7fffffff || out_h > 0x7fffffff ||
+      out_w > 0x7fffffff || mid_h <= 0 || mid_w <= 0) {
+    return 0;
+  }
+  ExpandDwArgs g = {};
+  g.batch = (int)batch; g.cin = (int)in_c; g.c = (int)mid_c; g.out_h = (int)out_h; g.out_w = (int)out_w;
+  size_t lds_bytes = 0;
+  if (!plan_expand_dw(g, (int)dw_stride, 4 * stem_k_steps(f_h * f_w * in_c), &lds_bytes)) return 0;
+  if (tuning(kTuneFusePwDw) >= 0) return tuning(kTuneFusePwDw) > 0 ? 1 : 0;
+  return batch * mid_h * mid_w * mid_c * 4 >= 48LL * 1000 * 1000 ? 1 : 0;
 }

@@ -273,6 +273,21 @@ napi_value SetLaunchRepeat(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+// setTuning(name, value): overrides a kernel-selection heuristic (value < 0 restores it)
+napi_value SetTuning(napi_env env, napi_callback_info info) {
+  Args a(env, info, 2, "setTuning");
+  char name[64] = "";
+  size_t len = 0;
+  if (a.ok && napi_get_value_string_utf8(env, a.argv[0], name, sizeof name, &len) != napi_ok) {
+    napi_throw_type_error(env, nullptr, "tfjs_hip.setTuning: name must be a string");
+    return nullptr;
+  }
+  const int value = a.i32(1);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_set_tuning(name, value));
+  return undefined(env);
+}
+
 napi_value LastKernel(napi_env env, napi_callback_info) {
   char name[256] = "";
   HIP_OK(tfhip_last_kernel(name, sizeof name));
@@ -425,6 +440,35 @@ napi_value FusedPointwiseDepthwise(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+// fusedConv2DDepthwise(x, filter, bias, activation, dwFilter, dwBias, dwActivation, y,
+//                      geom[17] = [batch, inH, inW, inC, fH, fW, midC, stride, padTop, padLeft, midH, midW,
+//                                  dwStride, dwPadTop, dwPadLeft, outH, outW])
+napi_value FusedConv2DDepthwise(napi_env env, napi_callback_info info) {
+  Args a(env, info, 9, "fusedConv2DDepthwise");
+  int64_t g[17];
+  a.ints(8, g, 17);
+  const float *x = (const float *)a.ptr(0), *w1 = (const float *)a.ptr(1), *b1 = (const float *)a.ptr(2);
+  const float *w2 = (const float *)a.ptr(4), *b2 = (const float *)a.ptr(5);
+  float *y = (float *)a.ptr(7);
+  const int act1 = a.i32(3), act2 = a.i32(6);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_fused_conv2d_depthwise(x, w1, b1, act1, w2, b2, act2, y, g[0], g[1], g[2], g[3], g[4], g[5], g[6], g[7],
+                                      g[8], g[9], g[10], g[11], g[12], g[13], g[14], g[15], g[16]));
+  return undefined(env);
+}
+
+// conv2dDepthwisePays(batch, inC, fH, fW, midC, midH, midW, dwStride, outH, outW): boolean
+napi_value Conv2DDepthwisePays(napi_env env, napi_callback_info info) {
+  Args a(env, info, 10, "conv2dDepthwisePays");
+  int64_t v[10];
+  for (int i = 0; i < 10; ++i) v[i] = a.i64(i);
+  if (!a.ok) return nullptr;
+  napi_value r;
+  NAPI_OK(napi_get_boolean(env, tfhip_conv2d_depthwise_pays(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], v[9]) == 1,
+                           &r));
+  return r;
+}
+
 // pointwiseDepthwisePays(batch, inC, midC, stride, outH, outW): boolean
 napi_value PointwiseDepthwisePays(napi_env env, napi_callback_info info) {
   Args a(env, info, 6, "pointwiseDepthwisePays");
@@ -500,6 +544,7 @@ napi_value Register(napi_env env, napi_value exports) {
       FN("eventElapsed", EventElapsed),
       FN("setLaunchRepeat", SetLaunchRepeat),
       FN("lastKernel", LastKernel),
+      FN("setTuning", SetTuning),
       FN("fusedMatMul", FusedMatMul),
       FN("fusedConv2D", FusedConv2D),
       FN("fusedDepthwiseConv2D", FusedDepthwiseConv2D),
@@ -509,6 +554,8 @@ napi_value Register(napi_env env, napi_value exports) {
       FN("meanHW", MeanHW),
       FN("fusedPointwiseDepthwise", FusedPointwiseDepthwise),
       FN("pointwiseDepthwisePays", PointwiseDepthwisePays),
+      FN("fusedConv2DDepthwise", FusedConv2DDepthwise),
+      FN("conv2dDepthwisePays", Conv2DDepthwisePays),
       FN("copy", Copy),
       FN("captureBegin", CaptureBegin),
       FN("captureEnd", CaptureEnd),

@@ -128,16 +128,19 @@ function convImpl(args, depthwise, fused, opName, residual) {
 }
 
 const pwdwGeom = new Float64Array(10);
+const cvdwGeom = new Float64Array(17);
 
 /**
  * FusedPointwiseDepthwiseConv2D (no counterpart among the reference's kernel
- * names): a FusedConv2D with a 1x1 filter, stride 1, followed by the
- * FusedDepthwiseConv2D that is its only reader - the expansion and the
- * depthwise stage of an inverted-residual block - as one launch in which the
- * expanded tensor never reaches memory.
- *   inputs  x, filter [1,1,inC,midC], bias [midC], dwFilter [3,3,midC,1], dwBias [midC]
- *   attrs   activation ('relu' | 'relu6', of both stages), and of the depthwise
- *           stage: strides, pad, dimRoundingMode
+ * names): a FusedConv2D followed by the FusedDepthwiseConv2D that is its only
+ * reader, as one launch in which the tensor between them never reaches memory.
+ * Two forms of the first stage are fused: a 1x1 filter with stride 1 (the
+ * expansion of an inverted-residual block) and a filter over at most 4 input
+ * channels and 36 taps (a network's stem).
+ *   inputs  x, filter, bias [midC], dwFilter [3,3,midC,1], dwBias [midC]
+ *   attrs   activation ('relu' | 'relu6', of both stages); of the first stage
+ *           convStrides, convPad (default [1, 1], 'valid'); of the depthwise
+ *           stage strides, pad, dimRoundingMode
  * Where the native library does not expect the fused kernel to be faster (or
  * does not take the shape), the two kernels run one after the other here; the
  * result is the same either way.
@@ -145,20 +148,29 @@ const pwdwGeom = new Float64Array(10);
 function fusedPointwiseDepthwise(args) {
   const {x, filter, bias, dwFilter, dwBias} = args.inputs;
   const {strides, pad, dimRoundingMode, activation} = args.attrs;
+  const convStrides = args.attrs.convStrides == null ? [1, 1] : args.attrs.convStrides;
+  const convPad = args.attrs.convPad == null ? 'valid' : args.attrs.convPad;
   const backend = args.backend;
   const opName = 'FusedPointwiseDepthwiseConv2D';
   requireFloat32([x, filter, bias, dwFilter, dwBias], opName);
   const midC = filter.shape[3];
-  const fusable = x.shape.length === 4 && filter.shape[0] === 1 && filter.shape[1] === 1 &&
+  const fusable = x.shape.length === 4 && filter.shape.length === 4 && filter.shape[2] === x.shape[3] &&
       dwFilter.shape[0] === 3 && dwFilter.shape[1] === 3 && dwFilter.shape[2] === midC && dwFilter.shape[3] === 1 &&
       bias != null && bias.shape.length === 1 && bias.shape[0] === midC &&
       dwBias != null && dwBias.shape.length === 1 && dwBias.shape[0] === midC &&
       (activation === 'relu' || activation === 'relu6');
   if (fusable) {
+    const first = tf.backend_util.computeConv2DInfo(
+        x.shape, filter.shape, convStrides, [1, 1], convPad, undefined, false, 'channelsLast');
     const info = tf.backend_util.computeConv2DInfo(
-        [x.shape[0], x.shape[1], x.shape[2], midC], dwFilter.shape, strides, [1, 1], pad, dimRoundingMode, true,
-        'channelsLast');
-    if (info.strideHeight === info.strideWidth && tf.util.sizeFromShape(info.outShape) > 0 &&
+        first.outShape, dwFilter.shape, strides, [1, 1], pad, dimRoundingMode, true, 'channelsLast');
+    const pointwise = first.filterHeight === 1 && first.filterWidth === 1 && first.strideHeight === 1 &&
+        first.strideWidth === 1 && first.padInfo.top === 0 && first.padInfo.left === 0 &&
+        first.outHeight === x.shape[1] && first.outWidth === x.shape[2];
+    const square = info.strideHeight === info.strideWidth && first.strideHeight === first.strideWidth &&
+        tf.util.sizeFromShape(info.outShape) > 0;
+    const code = activationCode(activation, opName);
+    if (square && pointwise &&
         addon.pointwiseDepthwisePays(
             info.batchSize, x.shape[3], midC, info.strideHeight, info.outHeight, info.outWidth)) {
       const out = backend.makeOutput(info.outShape, 'float32');
@@ -172,15 +184,31 @@ function fusedPointwiseDepthwise(args) {
       pwdwGeom[7] = info.padInfo.left;
       pwdwGeom[8] = info.outHeight;
       pwdwGeom[9] = info.outWidth;
-      const code = activationCode(activation, opName);
       addon.fusedPointwiseDepthwise(
           backend.ptr(x.dataId), backend.ptr(filter.dataId), backend.ptr(bias.dataId), code,
           backend.ptr(dwFilter.dataId), backend.ptr(dwBias.dataId), code, backend.ptr(out.dataId), pwdwGeom);
       return out;
     }
+    if (square && !pointwise &&
+        addon.conv2dDepthwisePays(
+            info.batchSize, x.shape[3], first.filterHeight, first.filterWidth, midC, first.outHeight, first.outWidth,
+            info.strideHeight, info.outHeight, info.outWidth)) {
+      const out = backend.makeOutput(info.outShape, 'float32');
+      const v = [info.batchSize, x.shape[1], x.shape[2], x.shape[3], first.filterHeight, first.filterWidth, midC,
+                 first.strideHeight, first.padInfo.top, first.padInfo.left, first.outHeight, first.outWidth,
+                 info.strideHeight, info.padInfo.top, info.padInfo.left, info.outHeight, info.outWidth];
+      for (let i = 0; i < 17; i++) {
+        cvdwGeom[i] = v[i];
+      }
+      addon.fusedConv2DDepthwise(
+          backend.ptr(x.dataId), backend.ptr(filter.dataId), backend.ptr(bias.dataId), code,
+          backend.ptr(dwFilter.dataId), backend.ptr(dwBias.dataId), code, backend.ptr(out.dataId), cvdwGeom);
+      return out;
+    }
   }
   const expanded = convImpl(
-      {inputs: {x, filter, bias}, backend, attrs: {strides: [1, 1], pad: 'valid', dataFormat: 'NHWC', dilations: [1, 1], activation}},
+      {inputs: {x, filter, bias}, backend,
+       attrs: {strides: convStrides, pad: convPad, dataFormat: 'NHWC', dilations: [1, 1], activation}},
       false, true, 'FusedConv2D');
   const out = convImpl(
       {inputs: {x: expanded, filter: dwFilter, bias: dwBias}, backend,

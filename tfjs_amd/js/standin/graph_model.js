@@ -23,9 +23,9 @@
  * of a residual block) is executed together with that Add as one kernel. The
  * result has the bits of the two separate kernels; {fuseResidualAdd: false} in
  * the load options turns it off. Likewise, with a 'FusedPointwiseDepthwiseConv2D'
- * kernel, a 1x1 _FusedConv2D whose only reader is a 3x3 FusedDepthwiseConv2dNative
- * with the same relu / relu6 activation (the expansion and the depthwise stage of
- * an inverted-residual block) is one step, and the kernel decides per shape
+ * kernel, a 1x1 _FusedConv2D (or one over at most 4 input channels: a stem) whose only
+ * reader is a 3x3 FusedDepthwiseConv2dNative with the same relu / relu6 activation
+ * (the expansion and the depthwise stage of an inverted-residual block) is one step, and the kernel decides per shape
  * whether one launch or the two are faster; {fusePointwiseDepthwise: false} turns
  * that off.
  *
@@ -198,7 +198,7 @@ function compileConvAdd(convNode) {
 }
 
 /**
- * 1x1 _FusedConv2D + the FusedDepthwiseConv2dNative that reads it -> function(inputs) => Tensor,
+ * _FusedConv2D (1x1, or over few input channels) + the FusedDepthwiseConv2dNative that reads it -> function(inputs) => Tensor,
  * inputs = [x, filter, bias, dwFilter, dwBias]; null when the pair is not of the form the
  * FusedPointwiseDepthwiseConv2D kernel covers (checked on the attributes; shapes are checked by
  * the kernel, which runs the two convolutions itself where it must).
@@ -220,14 +220,16 @@ function compilePointwiseDepthwise(convNode, dwNode, weightMap) {
       fusedOps(convNode)[0] === 'biasadd' && fusedOps(dwNode)[0] === 'biasadd' &&
       (act === 'relu' || act === 'relu6') && dw.activation === act &&
       conv.dataFormat === 'NHWC' && dw.dataFormat === 'NHWC' &&
-      conv.strides[0] === 1 && conv.strides[1] === 1 &&
       conv.dilations[0] === 1 && conv.dilations[1] === 1 && dw.dilations[0] === 1 && dw.dilations[1] === 1 &&
-      filter != null && filter.shape.length === 4 && filter.shape[0] === 1 && filter.shape[1] === 1 &&
+      filter != null && filter.shape.length === 4 &&
+      ((filter.shape[0] === 1 && filter.shape[1] === 1 && conv.strides[0] === 1 && conv.strides[1] === 1) ||
+       (filter.shape[2] <= 4 && filter.shape[0] * filter.shape[1] * filter.shape[2] <= 36)) &&
       dwFilter != null && dwFilter.shape.length === 4 && dwFilter.shape[0] === 3 && dwFilter.shape[1] === 3;
   if (!ok) {
     return null;
   }
-  const attrs = {strides: dw.strides, pad: dw.pad, dimRoundingMode: undefined, activation: act};
+  const attrs = {strides: dw.strides, pad: dw.pad, dimRoundingMode: undefined, activation: act,
+                 convStrides: conv.strides, convPad: conv.pad};
   return inputs => tf.engine().runKernel(
       'FusedPointwiseDepthwiseConv2D',
       {x: inputs[0], filter: inputs[1], bias: inputs[2], dwFilter: inputs[3], dwBias: inputs[4]}, attrs);

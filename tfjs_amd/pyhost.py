@@ -219,6 +219,37 @@ def fused_pointwise_depthwise(x, pw_filter, dw_filter, strides=1, pad="same", pw
             buf.free()
 
 
+def fused_conv2d_depthwise(x, filter, dw_filter, strides=1, pad="same", dw_strides=1, dw_pad="same", bias=None,
+                           dw_bias=None, activation="relu6"):
+    """Convolution over few input channels + depthwise 3x3 convolution (NHWC, the same activation
+    for both) as one launch; raises HipBackendError for a form the fused kernel does not take."""
+    init()
+    x, w1, w2 = _f32(x), _f32(filter), _f32(dw_filter)
+    b1, b2 = _opt(bias), _opt(dw_bias)
+    c1 = compute_conv2d_info(x.shape, w1.shape, strides, 1, pad, None, False, "channelsLast")
+    c2 = compute_conv2d_info(c1["outShape"], w2.shape, dw_strides, 1, dw_pad, None, True, "channelsLast")
+    assert c1["strideHeight"] == c1["strideWidth"] and c2["strideHeight"] == c2["strideWidth"]
+    total = int(np.prod(c2["outShape"], dtype=np.int64))
+    bufs = []
+    try:
+        dx, dw1, dw2, dy = (DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(w1), DeviceBuffer.from_numpy(w2),
+                            DeviceBuffer(total * 4))
+        bufs += [dx, dw1, dw2, dy]
+        db1 = DeviceBuffer.from_numpy(b1) if b1 is not None else None
+        db2 = DeviceBuffer.from_numpy(b2) if b2 is not None else None
+        bufs += [b for b in (db1, db2) if b is not None]
+        check(load_library().tfhip_fused_conv2d_depthwise(
+            dx.ptr, dw1.ptr, db1.ptr if db1 else None, ACTIVATIONS[activation], dw2.ptr, db2.ptr if db2 else None,
+            ACTIVATIONS[activation], dy.ptr, x.shape[0], x.shape[1], x.shape[2], x.shape[3], w1.shape[0], w1.shape[1],
+            w1.shape[3], c1["strideHeight"], c1["padInfo"]["top"], c1["padInfo"]["left"], c1["outHeight"],
+            c1["outWidth"], c2["strideHeight"], c2["padInfo"]["top"], c2["padInfo"]["left"], c2["outHeight"],
+            c2["outWidth"]))
+        return dy.download(np.float32, total).reshape(c2["outShape"])
+    finally:
+        for buf in bufs:
+            buf.free()
+
+
 def add(a, b):
     init()
     a, b = _f32(a), _f32(b)

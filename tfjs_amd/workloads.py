@@ -260,6 +260,15 @@ class DeviceMobileNetV2:
                         ci["strideWidth"], 1, 1, ci["padInfo"]["top"], ci["padInfo"]["left"], ci["outHeight"],
                         ci["outWidth"]]
                 self.plan.append((op, geom))
+            elif k == "cvdw":
+                c1 = compute_conv2d_info(shape[src], self.shapes[op["w"]], op["conv_stride"], 1, "same", None, False)
+                c2 = compute_conv2d_info(c1["outShape"], self.shapes[op["w2"]], op["stride"], 1, "same", None, True)
+                shape[op["out"]] = tuple(c2["outShape"])
+                fh, fw, cin, mid = self.shapes[op["w"]]
+                geom = [c1["batchSize"], c1["inHeight"], c1["inWidth"], cin, fh, fw, mid, op["conv_stride"],
+                        c1["padInfo"]["top"], c1["padInfo"]["left"], c1["outHeight"], c1["outWidth"], op["stride"],
+                        c2["padInfo"]["top"], c2["padInfo"]["left"], c2["outHeight"], c2["outWidth"]]
+                self.plan.append((op, geom))
             elif k == "pwdw":
                 n, h, w, _ = shape[src]
                 mid = self.shapes[op["w"]][3]
@@ -322,14 +331,21 @@ class DeviceMobileNetV2:
             if i in skip:
                 continue
             nxt = ops[i + 1] if i + 1 < len(ops) else None
-            if (op["kind"] == "conv" and "residual" not in op and shapes[op["w"]][:2] == (1, 1) and op["stride"] == 1
-                    and nxt is not None and nxt["kind"] == "dw" and nxt["src"] == op["out"]
-                    and readers.get(op["out"]) == 1):
-                cin, mid = shapes[op["w"]][2], shapes[op["w"]][3]
-                out_size = (size[src] + nxt["stride"] - 1) // nxt["stride"]
-                if lib.tfhip_pointwise_depthwise_pays(batch, cin, mid, nxt["stride"], out_size, out_size) == 1:
-                    fused.append(dict(kind="pwdw", src=src, out=nxt["out"], w=op["w"], b=op["b"], act=op["act"],
-                                      w2=nxt["w"], b2=nxt["b"], act2=nxt["act"], stride=nxt["stride"]))
+            if (op["kind"] == "conv" and "residual" not in op and nxt is not None and nxt["kind"] == "dw"
+                    and nxt["src"] == op["out"] and readers.get(op["out"]) == 1):
+                fh, fw, cin, mid = shapes[op["w"]]
+                mid_size = size[op["out"]]
+                out_size = (mid_size + nxt["stride"] - 1) // nxt["stride"]
+                pointwise = (fh, fw) == (1, 1) and op["stride"] == 1
+                if pointwise:
+                    pays = lib.tfhip_pointwise_depthwise_pays(batch, cin, mid, nxt["stride"], out_size, out_size)
+                else:
+                    pays = lib.tfhip_conv2d_depthwise_pays(batch, cin, fh, fw, mid, mid_size, mid_size, nxt["stride"],
+                                                           out_size, out_size)
+                if pays == 1:
+                    fused.append(dict(kind="pwdw" if pointwise else "cvdw", src=src, out=nxt["out"], w=op["w"], b=op["b"],
+                                      act=op["act"], w2=nxt["w"], b2=nxt["b"], act2=nxt["act"], stride=nxt["stride"],
+                                      conv_stride=op["stride"]))
                     skip.add(i + 1)
                     continue
             fused.append(op)
@@ -347,7 +363,12 @@ class DeviceMobileNetV2:
         srcs = op["src"] if isinstance(op["src"], tuple) else (op["src"],)
         n_in = sum(int(np.prod(self.shape[s])) for s in srcs)
         n_w = sum(int(np.prod(self.shapes[op[key]])) for key in ("w", "b", "w2", "b2") if key in op)
-        if k == "pwdw":
+        if k == "cvdw":
+            fh, fw, cin, mid = self.shapes[op["w"]]
+            geom = self.plan[i][1]
+            n_mid = geom[0] * geom[10] * geom[11] * mid
+            flops = 2 * n_mid * fh * fw * cin + 2 * n_out * 9
+        elif k == "pwdw":
             _, _, cin, mid = self.shapes[op["w"]]
             n_mid = int(np.prod(self.shape[op["src"]][:3])) * mid
             flops = 2 * n_mid * cin + 2 * n_out * 9
@@ -381,6 +402,10 @@ class DeviceMobileNetV2:
                 check(lib.tfhip_fused_conv2d(t[op["src"]].ptr, self.weights[op["w"]][0].ptr, out.ptr, *geom, 0,
                                              self.weights[op["b"]][0].ptr, self.strides_c, self._ACT[op["act"]],
                                              None, self.zero4, 0.2))
+            elif k == "cvdw":
+                check(lib.tfhip_fused_conv2d_depthwise(
+                    t[op["src"]].ptr, self.weights[op["w"]][0].ptr, self.weights[op["b"]][0].ptr, self._ACT[op["act"]],
+                    self.weights[op["w2"]][0].ptr, self.weights[op["b2"]][0].ptr, self._ACT[op["act2"]], out.ptr, *geom))
             elif k == "pwdw":
                 check(lib.tfhip_fused_pointwise_depthwise(
                     t[op["src"]].ptr, self.weights[op["w"]][0].ptr, self.weights[op["b"]][0].ptr, self._ACT[op["act"]],
