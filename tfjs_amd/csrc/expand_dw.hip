@@ -311,11 +311,7 @@ int launch_expand_dw_act(const ExpandDwArgs &g, const StemTaps &taps, size_t lds
     raised = true;
   }
   const long long wgs = (long long)g.batch * g.chunks_h * g.tiles_w;
-  if (TAPS > 0) {
-    note_kernel("expand_dw_3x3<%d, stem %d, %d>", S, TAPS, ACT);
-  } else {
-    note_kernel("expand_dw_3x3<%d, %d, %s, %d>", S, KF, HALF ? "true" : "false", ACT);
-  }
+  note_kernel("expand_dw_3x3<%d, %d, %s, %d, %d>", S, KF, HALF ? "true" : "false", ACT, TAPS);
   TFHIP_LAUNCH((expand_dw_3x3<S, KF, HALF, ACT, TAPS><<<dim3((unsigned)wgs), dim3(256), lds_bytes, stream()>>>(g, taps)));
   return kOk;
 }
