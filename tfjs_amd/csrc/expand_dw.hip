@@ -256,7 +256,7 @@ __global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g, StemTaps ta
     issue_rows(first, nrows);
     expand_rows(first, nrows, first);
   }
-  __syncthreads();
+  lds_barrier();
 
   int slot0 = 0;            // ring slot of expanded row S o
   int new_slot = 3 % RING;  // ring slot of expanded row S o + 3
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g, StemTaps ta
     if (more) expand_rows(first, S, new_slot);
     slot0 = slot0 + S >= RING ? slot0 + S - RING : slot0 + S;
     new_slot = new_slot + S >= RING ? new_slot + S - RING : new_slot + S;
-    __syncthreads();
+    lds_barrier();   // the ring lives in LDS alone: no wait for the stores of the output row
   }
 }
 

@@ -53,16 +53,6 @@
 
 namespace tfhip {
 
-// Workgroup barrier that orders LDS traffic only. __syncthreads() also fences
-// global memory, which makes every wave wait for all of its outstanding global
-// loads (vmcnt(0)) at each barrier and so drains the prefetch ring once per k
-// tile; the tiles exchanged between waves here live in LDS alone.
-__device__ __forceinline__ void lds_barrier() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
 enum LoadKind { kLoadKVec = 0, kLoadXVec = 1, kLoadScalar = 2, kLoadIm2colVec = 3, kLoadIm2colScalar = 4 };
 
 struct ConvGeom {
