@@ -99,7 +99,10 @@ def last_kernel(lib):
     return buf.value.decode()
 
 
-def time_launches(lib, check, ev, fn, repeat=50, rounds=3, settle_ms=20.0):
+SETTLE_MS = 20.0   # --settle-ms: a counter-collecting profiler run needs no settled clock
+
+
+def time_launches(lib, check, ev, fn, repeat=50, rounds=3, settle_ms=None):
     """Average duration in seconds of one launch of the kernel `fn` enqueues:
     `repeat` launches back to back between two events, best of `rounds`. The
     GPU idles at a fraction of its clock and needs about 10 ms of work to reach
@@ -110,6 +113,7 @@ def time_launches(lib, check, ev, fn, repeat=50, rounds=3, settle_ms=20.0):
     best = None
     try:
         settled = 0.0
+        settle_ms = SETTLE_MS if settle_ms is None else settle_ms
         while settled < settle_ms:
             ev.record(0)
             fn()
@@ -385,12 +389,17 @@ def main():
     ap.add_argument("--jit-prime", type=int, default=200, metavar="N",
                     help="batch-1 inferences the Node process runs before the warm-up steps (outside the timed "
                          "region) so that V8 has compiled the host path; 0 disables")
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_MS, metavar="MS",
+                    help="untimed run of each configuration's kernel before its timed launches (default 20: the GPU "
+                         "reaches its sustained clock); small under a counter-collecting profiler, where only "
+                         "counts matter")
     ap.add_argument("--per-op", metavar="FILE", help="write the per-op table of the model (kernel, us, us at the "
                                                      "roofline) to FILE as JSON")
     ap.add_argument("--copy-yardstick", type=int, metavar="MIB", default=0,
                     help="also run three device-to-device copies of this many MiB, so that a hardware-counter run "
                          "of this command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
+    globals()["SETTLE_MS"] = args.settle_ms
     if args.cpu_baseline_child:
         cpu_baseline_child(args.cpu_baseline_child)
         return
