@@ -811,3 +811,26 @@ def test_config4_mobilenet_v2_batch1_vs_oracle(hip, orc, tmp_path):
     np.testing.assert_array_equal(outs[0], outs[1])
     # the kernel-by-kernel host mirror agrees too
     assert_parity(workloads.run_graph(hip, ops, decoded, x[:1]), want[:1])
+
+
+def test_shutdown_and_init_again(hip, orc):
+    """Per-kernel set-up made at first use (the raised LDS limit of the fused expansion kernel) is
+    redone after tfhip_shutdown + tfhip_init: the second life of the library runs the same kernels."""
+    rng = np.random.default_rng(77)
+    x = rng.uniform(-1, 1, (2, 20, 28, 24)).astype(np.float32)
+    w1 = rng.normal(0, 0.5, (1, 1, 24, 144)).astype(np.float32)     # 144 channels: more than 64 KB of LDS
+    w2 = rng.normal(0, 0.5, (3, 3, 144, 1)).astype(np.float32)
+    b1 = rng.uniform(-1, 2, (144,)).astype(np.float32)
+    want = orc.fused_depthwise_conv2d(orc.fused_conv2d(x, w1, bias=b1, activation="relu6"), w2, strides=1, pad="same",
+                                      activation="relu6")
+    for life in range(2):
+        got = hip.fused_pointwise_depthwise(x, w1, w2, strides=1, pad="same", pw_bias=b1, pw_activation="relu6",
+                                            dw_activation="relu6")
+        assert_parity(got, want)
+        a = rng.uniform(-1, 1, (1, 64, 96)).astype(np.float32)
+        b = rng.uniform(-1, 1, (1, 96, 48)).astype(np.float32)
+        assert_parity(hip.fused_matmul(a, b), orc.fused_matmul(a, b))
+        assert hip.memory_info()["live"] == 0
+        if life == 0:
+            hip.shutdown()
+            hip.init(0)

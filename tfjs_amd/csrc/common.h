@@ -23,6 +23,7 @@ enum Status {
 };
 
 bool initialised();
+int init_count();          // how many times tfhip_init has set a device up: per-device set-up keyed on it is redone after a shutdown
 hipStream_t stream();
 int num_cus();
 // Device scratch of at least `bytes` (nullptr if it cannot be allocated); valid until the next call.

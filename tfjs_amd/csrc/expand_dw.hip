@@ -304,11 +304,12 @@ __global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g, StemTaps ta
 
 template <int S, int KF, bool HALF, int ACT, int TAPS>
 int launch_expand_dw_act(const ExpandDwArgs &g, const StemTaps &taps, size_t lds_bytes) {
-  static bool raised = false;   // dynamic LDS above the default limit needs the attribute once per instantiation
-  if (!raised) {
+  // dynamic LDS above the default limit needs the attribute once per instantiation and device set-up
+  static int raised = 0;
+  if (raised != init_count()) {
     TFHIP_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(expand_dw_3x3<S, KF, HALF, ACT, TAPS>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    raised = true;
+    raised = init_count();
   }
   const long long wgs = (long long)g.batch * g.chunks_h * g.tiles_w;
   note_kernel("expand_dw_3x3<%d, %d, %s, %d, %d>", S, KF, HALF ? "true" : "false", ACT, TAPS);

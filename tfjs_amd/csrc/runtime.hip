@@ -106,6 +106,7 @@ void note_kernel(const char *fmt, ...) {
 
 int launch_repeat() { return g_repeat; }
 
+int g_init_count = 0;
 int g_tuning[kTuneCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1};
 const char *const kTuningNames[kTuneCount] = {"tile", "splitk", "dw_rows", "dw_halo", "no_skinny", "dw_flat", "skinny_regs", "small_k", "fuse_pw_dw"};
 int tuning(int key) { return g_tuning[key]; }
@@ -121,6 +122,7 @@ void read_tuning_from_environment() {
 }
 
 bool initialised() { return g.ready; }
+int init_count() { return g_init_count; }
 hipStream_t stream() { return g.stream; }
 int num_cus() { return g.prop.multiProcessorCount; }
 
@@ -199,6 +201,7 @@ int tfhip_init(int device) {
     g.staging_busy[i] = false;
   }
   g.device = device;
+  ++g_init_count;
   read_tuning_from_environment();
   g.ready = true;
   return kOk;
