@@ -151,6 +151,30 @@ int tfhip_fused_matmul(const float *a, const float *b, float *out,
                        int activation, const float *prelu_weights,
                        const int64_t prelu_strides[3], double leakyrelu_alpha);
 
+/* tfhip_fused_matmul for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It
+ * has no counterpart in the reference. Same arguments, same kernels and the
+ * same result bit for bit; the one difference is where a product whose K is
+ * cut into slices keeps its partial sums: not in the library's growing
+ * workspace but in a static device array of TFHIP_NOALLOC_SCRATCH_BYTES that
+ * each GPU holds until the process ends. The call makes no hipMalloc / hipFree.
+ * A product whose partial sums (slices x batch x M x N x 4 bytes, with the
+ * slices the library chooses: at most 8, and 1 whenever the tiles already
+ * fill the GPU or K is short) exceed the array fails with a message that
+ * states both sizes, and launches nothing. Every call on a GPU shares that
+ * GPU's array: calls that overlap on one GPU (other threads, other streams)
+ * race. Nothing is cleared between calls because each call writes every
+ * element it later reads. */
+#define TFHIP_NOALLOC_SCRATCH_BYTES (16u << 20)
+int tfhip_fused_matmul_noalloc(const float *a, const float *b, float *out,
+                               int64_t batch_a, int64_t batch_b, int64_t M,
+                               int64_t N, int64_t K, int transpose_a,
+                               int transpose_b, const float *bias,
+                               const int64_t bias_strides[3], int activation,
+                               const float *prelu_weights,
+                               const int64_t prelu_strides[3],
+                               double leakyrelu_alpha);
+
 /* ---- FusedConv2D -----------------------------------------------------------
  * Replaces FusedConv2D(x_id, batch_size, input_height, ..., out_id)
  * (tfjs-backend-wasm/src/cc/kernels/FusedConv2D.cc:33-54); semantics of

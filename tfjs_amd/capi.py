@@ -45,6 +45,8 @@ SIGNATURES = {
     "tfhip_last_kernel": [ctypes.c_char_p, ctypes.c_size_t],
     "tfhip_fused_matmul": [c_f32p, c_f32p, c_f32p, c_i64, c_i64, c_i64, c_i64, c_i64, ctypes.c_int,
                            ctypes.c_int, c_f32p, c_i64p, ctypes.c_int, c_f32p, c_i64p, ctypes.c_double],
+    "tfhip_fused_matmul_noalloc": [c_f32p, c_f32p, c_f32p, c_i64, c_i64, c_i64, c_i64, c_i64, ctypes.c_int,
+                                   ctypes.c_int, c_f32p, c_i64p, ctypes.c_int, c_f32p, c_i64p, ctypes.c_double],
     "tfhip_fused_conv2d": [c_f32p, c_f32p, c_f32p] + [c_i64] * 15 + [ctypes.c_int, c_f32p, c_i64p,
                                                                       ctypes.c_int, c_f32p, c_i64p,
                                                                       ctypes.c_double],

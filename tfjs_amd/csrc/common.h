@@ -26,8 +26,22 @@ bool initialised();
 int init_count();          // how many times tfhip_init has set a device up: per-device set-up keyed on it is redone after a shutdown
 hipStream_t stream();
 int num_cus();
+int device_index();        // the device tfhip_init was given
 // Device scratch of at least `bytes` (nullptr if it cannot be allocated); valid until the next call.
 void *workspace(size_t bytes);
+// While a FixedWorkspace object lives, workspace() hands out the caller's block
+// instead of the library's growing one and allocates nothing: a request beyond
+// `bytes` returns nullptr, and workspace_is_fixed() tells a launcher to fail
+// rather than fall back.
+struct FixedWorkspace {
+  FixedWorkspace(void *ptr, size_t bytes);
+  ~FixedWorkspace();
+};
+bool workspace_is_fixed();
+size_t fixed_workspace_bytes();
+// Resolves the device address of gemm.hip's static scratch array for `device`
+// (which must be current). Called by tfhip_init.
+int setup_static_scratch(int device);
 
 // True when [p, p + bytes) lies inside one live block (own or external).
 bool range_is_live(const void *p, size_t bytes);

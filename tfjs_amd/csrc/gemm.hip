@@ -22,23 +22,96 @@ int tfhip::launch_plain_gemm(GemmParams &p, bool transpose_a, bool transpose_b, 
   return launch_gemm<64, 64, 16, 2, 2, kLoadScalar, kLoadScalar>(p);
 }
 
+namespace tfhip {
+namespace {
+
+// Scratch of tfhip_fused_matmul_noalloc: the split-K partial sums that
+// tfhip_fused_matmul keeps in the library's growing workspace. Every GPU the
+// library runs on holds its own copy of the array, at its own address, until
+// the process ends; in host code the name below is only a stand-in for the
+// symbol, and the per-device address is resolved once by setup_static_scratch
+// (with that device current) and used from then on.
+static __device__ __align__(256) float scratch[TFHIP_NOALLOC_SCRATCH_BYTES / sizeof(float)];
+
+constexpr int kMaxDevices = 64;
+float *g_scratch_ptr[kMaxDevices] = {};
+
+}  // namespace
+
+int setup_static_scratch(int device) {
+  if (device < 0 || device >= kMaxDevices)
+    return fail(kBadArgument, "tfhip_init: device %d is beyond the %d devices the static scratch table covers", device,
+                kMaxDevices);
+  if (g_scratch_ptr[device] != nullptr) return kOk;
+  void *ptr = nullptr;
+  const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || ptr == nullptr) {
+    (void)hipGetLastError();
+    return fail(kHipError, "tfhip_init: hipGetSymbolAddress(scratch) on device %d failed: %s", device,
+                hipGetErrorString(e));
+  }
+  g_scratch_ptr[device] = static_cast<float *>(ptr);
+  return kOk;
+}
+
+}  // namespace tfhip
+
+static int fused_matmul_impl(const char *who, const float *a, const float *b, float *out, int64_t batch_a,
+                             int64_t batch_b, int64_t M, int64_t N, int64_t K, int transpose_a, int transpose_b,
+                             const float *bias, const int64_t bias_strides[3], int activation,
+                             const float *prelu_weights, const int64_t prelu_strides[3], double leakyrelu_alpha);
+
 extern "C" int tfhip_fused_matmul(const float *a, const float *b, float *out, int64_t batch_a, int64_t batch_b,
                                   int64_t M, int64_t N, int64_t K, int transpose_a, int transpose_b,
                                   const float *bias, const int64_t bias_strides[3], int activation,
                                   const float *prelu_weights, const int64_t prelu_strides[3],
                                   double leakyrelu_alpha) {
+  return fused_matmul_impl("tfhip_fused_matmul", a, b, out, batch_a, batch_b, M, N, K, transpose_a, transpose_b, bias,
+                           bias_strides, activation, prelu_weights, prelu_strides, leakyrelu_alpha);
+}
+
+extern "C" int tfhip_fused_matmul_noalloc(const float *a, const float *b, float *out, int64_t batch_a,
+                                          int64_t batch_b, int64_t M, int64_t N, int64_t K, int transpose_a,
+                                          int transpose_b, const float *bias, const int64_t bias_strides[3],
+                                          int activation, const float *prelu_weights,
+                                          const int64_t prelu_strides[3], double leakyrelu_alpha) {
   TFHIP_REQUIRE_INIT();
-  TFHIP_CHECK_ARG(batch_a >= 0 && batch_b >= 0 && M >= 0 && N >= 0 && K >= 0, "tfhip_fused_matmul: negative dimension");
+  float *ptr = g_scratch_ptr[device_index()];
+  if (ptr == nullptr)
+    return fail(kHipError, "tfhip_fused_matmul_noalloc: the static scratch array was not resolved on device %d",
+                device_index());
+  // Same kernels and the same choice of K slices as tfhip_fused_matmul; only the
+  // home of the partial sums differs, so the two agree bit for bit. Nothing needs
+  // clearing between calls: every slab element that gemm_finish reads was written
+  // by this call's gemm_kernel.
+  FixedWorkspace fixed(ptr, TFHIP_NOALLOC_SCRATCH_BYTES);
+  return fused_matmul_impl("tfhip_fused_matmul_noalloc", a, b, out, batch_a, batch_b, M, N, K, transpose_a,
+                           transpose_b, bias, bias_strides, activation, prelu_weights, prelu_strides,
+                           leakyrelu_alpha);
+}
+
+static int fused_matmul_impl(const char *who, const float *a, const float *b, float *out, int64_t batch_a,
+                             int64_t batch_b, int64_t M, int64_t N, int64_t K, int transpose_a, int transpose_b,
+                             const float *bias, const int64_t bias_strides[3], int activation,
+                             const float *prelu_weights, const int64_t prelu_strides[3], double leakyrelu_alpha) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_ARG(batch_a >= 0 && batch_b >= 0 && M >= 0 && N >= 0 && K >= 0, "%s: negative dimension", who);
   const int64_t lim = 0x7fffffff;
   TFHIP_CHECK_ARG(M < lim && N < lim && K < lim && batch_a < lim && batch_b < lim,
-                  "tfhip_fused_matmul: dimension exceeds 2^31-1");
+                  "%s: dimension exceeds 2^31-1", who);
   const int64_t batch = batch_a > batch_b ? batch_a : batch_b;
+  int rc = kOk;
   if (batch_a == 0 || batch_b == 0 || M == 0 || N == 0) return kOk;
+  auto live = [&](const void *ptr, int64_t elems, const char *name) {
+    if (ptr != nullptr && range_is_live(ptr, (size_t)elems * 4)) return (int)kOk;
+    return fail(kOutOfRange, "%s: operand '%s' (%lld elements of 4 bytes at %p) is not inside a live device buffer",
+                who, name, (long long)elems, ptr);
+  };
   if (K > 0) {
-    TFHIP_CHECK_RANGE(a, batch_a * M * K, 4, "a");
-    TFHIP_CHECK_RANGE(b, batch_b * K * N, 4, "b");
+    if ((rc = live(a, batch_a * M * K, "a")) != kOk) return rc;
+    if ((rc = live(b, batch_b * K * N, "b")) != kOk) return rc;
   }
-  TFHIP_CHECK_RANGE(out, batch * M * N, 4, "out");
+  if ((rc = live(out, batch * M * N, "out")) != kOk) return rc;
 
   GemmParams p = {};
   p.a = a; p.b = b; p.c = out;
@@ -50,7 +123,7 @@ extern "C" int tfhip_fused_matmul(const float *a, const float *b, float *out, in
   p.b_sx = transpose_b ? K : 1; p.b_sk = transpose_b ? 1 : N;
   p.ldc = N;
   const int64_t dims[3] = {batch, M, N};
-  int rc = fill_epilogue(p.epi, "tfhip_fused_matmul", dims, 3, bias, bias_strides, activation, prelu_weights,
+  rc = fill_epilogue(p.epi, who, dims, 3, bias, bias_strides, activation, prelu_weights,
                          prelu_strides, leakyrelu_alpha, kMatmul);
   if (rc) return rc;
 

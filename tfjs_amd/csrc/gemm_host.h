@@ -102,6 +102,11 @@ inline int launch_gemm(GemmParams &p) {
     if (best > 1) {
       const size_t bytes = (size_t)best * p.batch * p.M * p.N * sizeof(float);
       float *ws = bytes <= (size_t(1) << 30) ? static_cast<float *>(workspace(bytes)) : nullptr;
+      if (!ws && workspace_is_fixed())
+        return fail(kBadArgument,
+                    "gemm: %d K slices of a %d x %d x %d output need %zu bytes of scratch; the static array of the "
+                    "entry point that allocates nothing holds %zu",
+                    best, p.batch, p.M, p.N, bytes, fixed_workspace_bytes());
       if (ws) {
         p.splits = best;
         p.k_per_split = ((k_tiles + best - 1) / best) * BK;

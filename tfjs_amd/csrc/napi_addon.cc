@@ -298,8 +298,9 @@ napi_value LastKernel(napi_env env, napi_callback_info) {
 
 // fusedMatMul(a, b, out, batchA, batchB, M, N, K, transposeA, transposeB,
 //             bias, biasStrides[3], activation, prelu, preluStrides[3], leakyreluAlpha)
-napi_value FusedMatMul(napi_env env, napi_callback_info info) {
-  Args a(env, info, 16, "fusedMatMul");
+// fusedMatMulNoAlloc: the same arguments, through tfhip_fused_matmul_noalloc.
+static napi_value FusedMatMulAny(napi_env env, napi_callback_info info, bool noalloc) {
+  Args a(env, info, 16, noalloc ? "fusedMatMulNoAlloc" : "fusedMatMul");
   int64_t bs[3], ps[3];
   a.ints(11, bs, 3);
   a.ints(14, ps, 3);
@@ -311,9 +312,15 @@ napi_value FusedMatMul(napi_env env, napi_callback_info info) {
   const int act = a.i32(12);
   const double leaky = a.num(15);
   if (!a.ok) return nullptr;
-  HIP_OK(tfhip_fused_matmul(pa, pb, out, bA, bB, M, N, K, tA, tB, bias, bs, act, prelu, ps, leaky));
+  if (noalloc) {
+    HIP_OK(tfhip_fused_matmul_noalloc(pa, pb, out, bA, bB, M, N, K, tA, tB, bias, bs, act, prelu, ps, leaky));
+  } else {
+    HIP_OK(tfhip_fused_matmul(pa, pb, out, bA, bB, M, N, K, tA, tB, bias, bs, act, prelu, ps, leaky));
+  }
   return undefined(env);
 }
+napi_value FusedMatMul(napi_env env, napi_callback_info info) { return FusedMatMulAny(env, info, false); }
+napi_value FusedMatMulNoAlloc(napi_env env, napi_callback_info info) { return FusedMatMulAny(env, info, true); }
 
 // fusedConv2D(x, filter, y, geom[15], nchw, bias, biasStrides[4], activation, prelu, preluStrides[4], alpha
 //             [, residual])   with a residual: tfhip_fused_conv2d_add
@@ -546,6 +553,7 @@ napi_value Register(napi_env env, napi_value exports) {
       FN("lastKernel", LastKernel),
       FN("setTuning", SetTuning),
       FN("fusedMatMul", FusedMatMul),
+      FN("fusedMatMulNoAlloc", FusedMatMulNoAlloc),
       FN("fusedConv2D", FusedConv2D),
       FN("fusedDepthwiseConv2D", FusedDepthwiseConv2D),
       FN("dequantAffine", DequantAffine),

@@ -123,13 +123,32 @@ void read_tuning_from_environment() {
 
 bool initialised() { return g.ready; }
 int init_count() { return g_init_count; }
+int device_index() { return g.device; }
 hipStream_t stream() { return g.stream; }
 int num_cus() { return g.prop.multiProcessorCount; }
 
 // Scratch for kernels that need device memory beyond their operands (split-K
 // partial sums). One block that only grows; work on the single stream is
 // ordered, so consecutive launches may share it.
+void *g_fixed_ws = nullptr;
+size_t g_fixed_ws_bytes = 0;
+bool g_ws_fixed = false;
+
+FixedWorkspace::FixedWorkspace(void *ptr, size_t bytes) {
+  g_fixed_ws = ptr;
+  g_fixed_ws_bytes = bytes;
+  g_ws_fixed = true;
+}
+FixedWorkspace::~FixedWorkspace() {
+  g_ws_fixed = false;
+  g_fixed_ws = nullptr;
+  g_fixed_ws_bytes = 0;
+}
+bool workspace_is_fixed() { return g_ws_fixed; }
+size_t fixed_workspace_bytes() { return g_fixed_ws_bytes; }
+
 void *workspace(size_t bytes) {
+  if (g_ws_fixed) return bytes <= g_fixed_ws_bytes ? g_fixed_ws : nullptr;
   if (bytes <= g.workspace_bytes) return g.workspace;
   if (g.capturing || !g.graphs.empty()) {
     // a recorded graph may name the old block: it stays allocated until shutdown
@@ -193,6 +212,10 @@ int tfhip_init(int device) {
     return fail(kBadArgument,
                 "tfhip_init: device %d is %s; this library carries gfx950 code only",
                 device, g.prop.gcnArchName);
+  }
+  {
+    const int rc = setup_static_scratch(device);   // this device's copy of the static scratch array
+    if (rc != kOk) return rc;
   }
   TFHIP_CHECK_HIP(hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking));
   for (int i = 0; i < kStagingBuffers; ++i) {
