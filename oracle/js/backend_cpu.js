@@ -14,7 +14,11 @@
  * Registers itself as backend 'cpu' with whichever tfjs-core the product
  * resolves (the offline stand-in when the real package is absent).
  */
+// The engine (registry, KernelBackend, DataStorage) is the one the package under
+// test registers with: a backend can only be compared through the same engine.
+// All shape arithmetic comes from the oracle's own restatement.
 const tf = require('../../tfjs_amd/js/core');
+const shapes = require('./shape_util');
 
 const BLOCK_SIZE = 48;  // tfjs-backend-cpu/src/backend_cpu.ts:38
 
@@ -86,11 +90,11 @@ function vals(backend, t) {
 // ---- aliasing kernels: Reshape.ts:24-52, Identity.ts:22-30 ---------------------
 function reshape({inputs, backend, attrs}) {
   const x = inputs.x;
-  const xSize = tf.util.sizeFromShape(x.shape);
-  const shape = tf.util.inferFromImplicitShape(attrs.shape, xSize);
-  tf.util.assert(
-      xSize === tf.util.sizeFromShape(shape),
-      () => `The new shape (${shape}) has ${tf.util.sizeFromShape(shape)} ` +
+  const xSize = shapes.util.sizeFromShape(x.shape);
+  const shape = shapes.util.inferFromImplicitShape(attrs.shape, xSize);
+  shapes.util.assert(
+      xSize === shapes.util.sizeFromShape(shape),
+      () => `The new shape (${shape}) has ${shapes.util.sizeFromShape(shape)} ` +
           `elements and the old shape (${x.shape}) has ${xSize} elements. ` +
           `The new shape and old shape must have the same number of elements.`);
   backend.incRef(x.dataId);
@@ -104,28 +108,28 @@ function identity({inputs, backend}) {
 
 // ---- broadcasting binary template: utils/binary_impl.ts:25-68 -----------------
 function binaryImpl(op, aShape, bShape, aVals, bVals) {
-  const newShape = tf.backend_util.assertAndGetBroadcastShape(aShape, bShape);
+  const newShape = shapes.backend_util.assertAndGetBroadcastShape(aShape, bShape);
   const rank = newShape.length;
-  const strides = tf.util.computeStrides(newShape);
-  const result = new Float32Array(tf.util.sizeFromShape(newShape));
+  const strides = shapes.util.computeStrides(newShape);
+  const result = new Float32Array(shapes.util.sizeFromShape(newShape));
   const aRank = aShape.length, bRank = bShape.length;
-  const aStrides = tf.util.computeStrides(aShape);
-  const bStrides = tf.util.computeStrides(bShape);
-  const aBroadcast = tf.backend_util.getBroadcastDims(aShape, newShape);
-  const bBroadcast = tf.backend_util.getBroadcastDims(bShape, newShape);
+  const aStrides = shapes.util.computeStrides(aShape);
+  const bStrides = shapes.util.computeStrides(bShape);
+  const aBroadcast = shapes.backend_util.getBroadcastDims(aShape, newShape);
+  const bBroadcast = shapes.backend_util.getBroadcastDims(bShape, newShape);
   if (aBroadcast.length + bBroadcast.length === 0) {
     for (let i = 0; i < result.length; ++i) {
       result[i] = op(aVals[i % aVals.length], bVals[i % bVals.length]);
     }
   } else {
     for (let i = 0; i < result.length; ++i) {
-      const loc = tf.util.indexToLoc(i, rank, strides);
+      const loc = shapes.util.indexToLoc(i, rank, strides);
       const aLoc = loc.slice(-aRank);
       aBroadcast.forEach(d => aLoc[d] = 0);
-      const aIndex = tf.util.locToIndex(aLoc, aRank, aStrides);
+      const aIndex = shapes.util.locToIndex(aLoc, aRank, aStrides);
       const bLoc = loc.slice(-bRank);
       bBroadcast.forEach(d => bLoc[d] = 0);
-      const bIndex = tf.util.locToIndex(bLoc, bRank, bStrides);
+      const bIndex = shapes.util.locToIndex(bLoc, bRank, bStrides);
       result[i] = op(aVals[aIndex], bVals[bIndex]);
     }
   }
@@ -190,12 +194,12 @@ function batchMatMul({inputs, backend, attrs}) {
   const innerB = transposeB ? b.shape[bRank - 1] : b.shape[bRank - 2];
   const outerA = transposeA ? a.shape[aRank - 1] : a.shape[aRank - 2];
   const outerB = transposeB ? b.shape[bRank - 2] : b.shape[bRank - 1];
-  const batchDimA = tf.util.sizeFromShape(a.shape.slice(0, -2));
-  const batchDimB = tf.util.sizeFromShape(b.shape.slice(0, -2));
-  const outOuter = tf.backend_util.assertAndGetBroadcastShape(
+  const batchDimA = shapes.util.sizeFromShape(a.shape.slice(0, -2));
+  const batchDimB = shapes.util.sizeFromShape(b.shape.slice(0, -2));
+  const outOuter = shapes.backend_util.assertAndGetBroadcastShape(
       a.shape.slice(0, -2), b.shape.slice(0, -2));
   const outShape = outOuter.concat([outerA, outerB]);
-  tf.util.assert(
+  shapes.util.assert(
       innerA === innerB,
       () => `Error in matMul: inner shapes (${innerA}) and (` +
           `${innerB}) of Tensors with shapes ${a.shape} and ` +
@@ -206,7 +210,7 @@ function batchMatMul({inputs, backend, attrs}) {
   const sharedDim = innerA, leftDim = outerA, rightDim = outerB;
   const batchDim = Math.max(batchDimA, batchDimB);
   const aValues = vals(backend, a), bValues = vals(backend, b);
-  const aS = tf.util.computeStrides(a3dShape), bS = tf.util.computeStrides(b3dShape);
+  const aS = shapes.util.computeStrides(a3dShape), bS = shapes.util.computeStrides(b3dShape);
   const aBatch = aS[0], aOuterStep = transposeA ? 1 : aS[1], aInnerStep = transposeA ? aS[1] : 1;
   const bInnerStep = transposeB ? 1 : bS[1], bOuterStep = transposeB ? bS[1] : 1, bBatch = bS[0];
   const size = leftDim * rightDim;
@@ -278,16 +282,16 @@ function fusedMatMul({inputs, backend, attrs}) {
 // ---- Conv2D.ts:23-103 ----------------------------------------------------------
 function conv2D({inputs, backend, attrs}) {
   const x = inputs.x, filter = inputs.filter;
-  const $dataFormat = tf.backend_util.convertConv2DDataFormat(attrs.dataFormat || 'NHWC');
-  const info = tf.backend_util.computeConv2DInfo(
+  const $dataFormat = shapes.backend_util.convertConv2DDataFormat(attrs.dataFormat || 'NHWC');
+  const info = shapes.backend_util.computeConv2DInfo(
       x.shape, filter.shape, attrs.strides, attrs.dilations == null ? [1, 1] : attrs.dilations,
       attrs.pad, attrs.dimRoundingMode, false, $dataFormat);
   const channelsLast = info.dataFormat === 'channelsLast';
   const padLeft = info.padInfo.left, padTop = info.padInfo.top;
-  const yVals = new Float32Array(tf.util.sizeFromShape(info.outShape));
-  const xS = tf.util.computeStrides(x.shape);
-  const fS = tf.util.computeStrides(filter.shape);
-  const yS = tf.util.computeStrides(info.outShape);
+  const yVals = new Float32Array(shapes.util.sizeFromShape(info.outShape));
+  const xS = shapes.util.computeStrides(x.shape);
+  const fS = shapes.util.computeStrides(filter.shape);
+  const yS = shapes.util.computeStrides(info.outShape);
   const xBatch = xS[0], xRow = channelsLast ? xS[1] : xS[2], xCol = channelsLast ? xS[2] : 1,
         xChan = channelsLast ? 1 : xS[1];
   const yBatch = yS[0], yRow = channelsLast ? yS[1] : yS[2], yCol = channelsLast ? yS[2] : 1,
@@ -343,18 +347,18 @@ function fusedConv2D({inputs, backend, attrs}) {
 function depthwiseConv2dNative({inputs, backend, attrs}) {
   const x = inputs.x, filter = inputs.filter;
   const dilations = attrs.dilations == null ? [1, 1] : attrs.dilations;
-  tf.util.assert(
-      tf.backend_util.eitherStridesOrDilationsAreOne(attrs.strides, dilations),
+  shapes.util.assert(
+      shapes.backend_util.eitherStridesOrDilationsAreOne(attrs.strides, dilations),
       () => 'Error in depthwiseConv2d: Either strides or dilations must be ' +
           `1. Got strides ${attrs.strides} and dilations '${dilations}'`);
-  const info = tf.backend_util.computeConv2DInfo(
+  const info = shapes.backend_util.computeConv2DInfo(
       x.shape, filter.shape, attrs.strides, dilations, attrs.pad, attrs.dimRoundingMode, true);
   const padLeft = info.padInfo.left, padTop = info.padInfo.top;
   const chMul = info.outChannels / info.inChannels;
-  const xS = tf.util.computeStrides(x.shape);
-  const fS = tf.util.computeStrides(filter.shape);
-  const yS = tf.util.computeStrides(info.outShape);
-  const yVals = new Float32Array(tf.util.sizeFromShape(info.outShape));
+  const xS = shapes.util.computeStrides(x.shape);
+  const fS = shapes.util.computeStrides(filter.shape);
+  const yS = shapes.util.computeStrides(info.outShape);
+  const yVals = new Float32Array(shapes.util.sizeFromShape(info.outShape));
   const xVals = vals(backend, x), wVals = vals(backend, filter);
   for (let b = 0; b < info.batchSize; ++b) {
     const xOffset1 = b * xS[0];
@@ -409,7 +413,7 @@ function fusedDepthwiseConv2D({inputs, backend, attrs}) {
  * innermost and accumulates each output in a double. */
 function mean({inputs, backend, attrs}) {
   const x = inputs.x;
-  const axes = tf.util.parseAxisParam(attrs.axis, x.shape).slice().sort((p, q) => p - q);
+  const axes = shapes.util.parseAxisParam(attrs.axis, x.shape).slice().sort((p, q) => p - q);
   if (x.shape.length !== 4 || axes.length !== 2 || axes[0] !== 1 || axes[1] !== 2) {
     throw new Error('oracle Mean: only axes [1, 2] of a rank-4 tensor are restated');
   }

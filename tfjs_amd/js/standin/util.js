@@ -1,426 +1,307 @@
 'use strict';
 /**
  * Offline stand-in for the slice of @tensorflow/tfjs-core's `util`,
- * `backend_util` and `broadcast_util` namespaces that a backend package touches
- * (tfjs-core/src/util_base.ts, ops/conv_util.ts, ops/broadcast_util.ts). Used
- * only when the real package cannot be resolved; same names, arguments and
- * error behaviour.
+ * `backend_util` and `broadcast_util` namespaces that a backend package touches.
+ * Used only when the real package cannot be resolved. The exported names,
+ * argument orders, result fields and the error texts callers match on are the
+ * interface of tfjs-core/src/util_base.ts, ops/conv_util.ts and
+ * ops/broadcast_util.ts; the bodies are this package's own (the shape
+ * arithmetic is the one tfjs_amd/conv_util.py states, written again for JS).
  */
 
-function assert(expr, msg) {
-  if (!expr) {
-    throw new Error(typeof msg === 'string' ? msg : msg());
-  }
+function assert(condition, message) {
+  if (condition) return;
+  throw new Error(typeof message === 'function' ? message() : message);
 }
 
-function sizeFromShape(shape) {
-  if (shape.length === 0) {
-    return 1;
-  }
-  let size = shape[0];
-  for (let i = 1; i < shape.length; i++) {
-    size *= shape[i];
-  }
-  return size;
+const sizeFromShape = shape => shape.reduce((n, d) => n * d, 1);
+
+function arraysEqual(a, b) {
+  if (a === b) return true;
+  if (a == null || b == null || a.length !== b.length) return false;
+  return Array.prototype.every.call(a, (v, i) => v === b[i]);
 }
 
-function arraysEqual(n1, n2) {
-  if (n1 === n2) {
-    return true;
-  }
-  if (n1 == null || n2 == null || n1.length !== n2.length) {
-    return false;
-  }
-  for (let i = 0; i < n1.length; i++) {
-    if (n1[i] !== n2[i]) {
-      return false;
-    }
-  }
-  return true;
-}
-
-/** util.computeStrides: rank-1 entries (util_base.ts:565-579). */
+/**
+ * Row-major element strides of all axes but the last (whose stride is 1 and is
+ * left out): the convention of util.computeStrides (util_base.ts:565-579).
+ */
 function computeStrides(shape) {
-  const rank = shape.length;
-  if (rank < 2) {
-    return [];
-  }
-  const strides = new Array(rank - 1);
-  strides[rank - 2] = shape[rank - 1];
-  for (let i = rank - 3; i >= 0; --i) {
-    strides[i] = strides[i + 1] * shape[i + 1];
+  const strides = [];
+  let run = 1;
+  for (let axis = shape.length - 1; axis >= 1; --axis) {
+    run *= shape[axis];
+    strides.unshift(run);
   }
   return strides;
 }
 
-function isInt(a) {
-  return a % 1 === 0;
-}
+const isInt = value => value % 1 === 0;
 
-/** util.inferFromImplicitShape (util_base.ts:335-372). */
+/**
+ * Fills in the one -1 of a reshape target from the element count
+ * (util.inferFromImplicitShape, util_base.ts:335).
+ */
 function inferFromImplicitShape(shape, size) {
-  let shapeProd = 1;
-  let implicitIdx = -1;
-  for (let i = 0; i < shape.length; ++i) {
-    if (shape[i] >= 0) {
-      shapeProd *= shape[i];
-    } else if (shape[i] === -1) {
-      if (implicitIdx !== -1) {
-        throw Error(
-            `Shapes can only have 1 implicit size. ` +
-            `Found -1 at dim ${implicitIdx} and dim ${i}`);
-      }
-      implicitIdx = i;
-    } else if (shape[i] < 0) {
-      throw Error(`Shapes can not be < 0. Found ${shape[i]} at dim ${i}`);
+  const holes = [];
+  let known = 1;
+  shape.forEach((d, axis) => {
+    if (d === -1) {
+      holes.push(axis);
+    } else if (d < 0) {
+      throw new Error(`Shapes can not be < 0. Found ${d} at dim ${axis}`);
+    } else {
+      known *= d;
     }
+  });
+  if (holes.length > 1) {
+    throw new Error(`Shapes can only have 1 implicit size. Found -1 at dim ${holes[0]} and dim ${holes[1]}`);
   }
-  if (implicitIdx === -1) {
-    if (size > 0 && size !== shapeProd) {
-      throw Error(`Size(${size}) must match the product of shape ${shape}`);
+  if (holes.length === 0) {
+    if (size > 0 && size !== known) {
+      throw new Error(`Size(${size}) must match the product of shape ${shape}`);
     }
     return shape;
   }
-  if (shapeProd === 0) {
-    throw Error(
-        `Cannot infer the missing size in [${shape}] when ` +
-        `there are 0 elements`);
+  if (known === 0) {
+    throw new Error(`Cannot infer the missing size in [${shape}] when there are 0 elements`);
   }
-  if (size % shapeProd !== 0) {
-    throw Error(
-        `The implicit shape can't be a fractional number. ` +
-        `Got ${size} / ${shapeProd}`);
+  const missing = size / known;
+  if (!isInt(missing)) {
+    throw new Error(`The implicit shape can't be a fractional number. Got ${size} / ${known}`);
   }
-  const newShape = shape.slice();
-  newShape[implicitIdx] = size / shapeProd;
-  return newShape;
+  return shape.map(d => (d === -1 ? missing : d));
 }
 
+/** Normalises an axis argument (number, list or null = all axes) to non-negative axes. */
 function parseAxisParam(axis, shape) {
   const rank = shape.length;
-  axis = axis == null ? shape.map((s, i) => i) : [].concat(axis);
-  assert(
-      axis.every(ax => ax >= -rank && ax < rank),
-      () => `All values in axis param must be in range [-${rank}, ${rank}) but ` +
-          `got axis ${axis}`);
-  assert(
-      axis.every(ax => isInt(ax)),
-      () => `All values in axis param must be integers but got axis ${axis}`);
-  return axis.map(a => a < 0 ? rank + a : a);
+  const list = axis == null ? shape.map((_, i) => i) : (Array.isArray(axis) ? axis.slice() : [axis]);
+  for (const a of list) {
+    assert(a >= -rank && a < rank,
+           `All values in axis param must be in range [-${rank}, ${rank}) but got axis ${list}`);
+    assert(isInt(a), `All values in axis param must be integers but got axis ${list}`);
+  }
+  return list.map(a => (a < 0 ? a + rank : a));
 }
 
+const ELEMENT_BYTES = {float32: 4, int32: 4, complex64: 8, bool: 1};
+const TYPED_ARRAYS = {float32: Float32Array, int32: Int32Array, bool: Uint8Array};
+
 function bytesPerElement(dtype) {
-  if (dtype === 'float32' || dtype === 'int32') {
-    return 4;
-  } else if (dtype === 'complex64') {
-    return 8;
-  } else if (dtype === 'bool') {
-    return 1;
-  }
-  throw new Error(`Unknown dtype ${dtype}`);
+  if (!(dtype in ELEMENT_BYTES)) throw new Error(`Unknown dtype ${dtype}`);
+  return ELEMENT_BYTES[dtype];
 }
 
 function getTypedArrayFromDType(dtype, size) {
-  if (dtype == null || dtype === 'float32') {
-    return new Float32Array(size);
-  } else if (dtype === 'int32') {
-    return new Int32Array(size);
-  } else if (dtype === 'bool') {
-    return new Uint8Array(size);
-  }
-  throw new Error(`Unknown data type ${dtype}`);
+  const Ctor = TYPED_ARRAYS[dtype == null ? 'float32' : dtype];
+  if (!Ctor) throw new Error(`Unknown data type ${dtype}`);
+  return new Ctor(size);
 }
 
 function now() {
-  const t = process.hrtime();
-  return t[0] * 1000 + t[1] / 1e6;
+  const [s, ns] = process.hrtime();
+  return s * 1e3 + ns * 1e-6;
 }
 
+/** Flat index -> coordinates, with the rank-1 strides of computeStrides. */
 function indexToLoc(index, rank, strides) {
-  if (rank === 0) {
-    return [];
-  } else if (rank === 1) {
-    return [index];
+  const loc = [];
+  let rest = index;
+  for (let axis = 0; axis < rank - 1; ++axis) {
+    const q = Math.floor(rest / strides[axis]);
+    loc.push(q);
+    rest -= q * strides[axis];
   }
-  const locs = new Array(rank);
-  for (let i = 0; i < locs.length - 1; ++i) {
-    locs[i] = Math.floor(index / strides[i]);
-    index -= locs[i] * strides[i];
-  }
-  locs[locs.length - 1] = index;
-  return locs;
+  if (rank > 0) loc.push(rest);
+  return loc;
 }
 
-function locToIndex(locs, rank, strides) {
-  if (rank === 0) {
-    return 0;
-  } else if (rank === 1) {
-    return locs[0];
-  }
-  let index = locs[locs.length - 1];
-  for (let i = 0; i < locs.length - 1; ++i) {
-    index += strides[i] * locs[i];
-  }
+/** Coordinates -> flat index. */
+function locToIndex(loc, rank, strides) {
+  if (rank === 0) return 0;
+  let index = loc[rank - 1];
+  for (let axis = 0; axis < rank - 1; ++axis) index += loc[axis] * strides[axis];
   return index;
 }
 
-// ---- broadcast_util (tfjs-core/src/ops/broadcast_util.ts) -------------------
+// ---- broadcasting ------------------------------------------------------------
 
+/** Axes of inShape (aligned at the right with outShape) that are stretched from 1. */
 function getBroadcastDims(inShape, outShape) {
-  const inRank = inShape.length;
-  const dims = [];
-  for (let i = 0; i < inRank; i++) {
-    const dim = inRank - 1 - i;
-    const a = inShape[dim] || 1;
-    const b = outShape[outShape.length - 1 - i] || 1;
-    if (b > 1 && a === 1) {
-      dims.unshift(dim);
-    }
-  }
-  return dims;
+  const shift = outShape.length - inShape.length;
+  const stretched = [];
+  inShape.forEach((d, axis) => {
+    const out = axis + shift >= 0 ? outShape[axis + shift] : 1;
+    if ((d || 1) === 1 && (out || 1) > 1) stretched.push(axis);
+  });
+  return stretched;
 }
 
+/** The numpy-style broadcast of two shapes, or an Error when they do not combine. */
 function assertAndGetBroadcastShape(shapeA, shapeB) {
-  const l = Math.max(shapeA.length, shapeB.length);
-  const result = new Array(l);
-  for (let i = 0; i < l; i++) {
-    const ia = shapeA.length - i - 1, ib = shapeB.length - i - 1;
-    const a = ia >= 0 ? shapeA[ia] : 1;
-    const b = ib >= 0 ? shapeB[ib] : 1;
-    if (a === 1) {
-      result[l - i - 1] = b;
-    } else if (b === 1) {
-      result[l - i - 1] = a;
-    } else if (a !== b) {
-      const errMsg = `Operands could not be broadcast together with shapes ` +
-          `${shapeA} and ${shapeB}.`;
-      throw Error(errMsg);
-    } else {
-      result[l - i - 1] = a;
+  const rank = Math.max(shapeA.length, shapeB.length);
+  const at = (shape, axis) => {
+    const i = axis - (rank - shape.length);
+    return i < 0 ? 1 : shape[i];
+  };
+  const out = [];
+  for (let axis = 0; axis < rank; ++axis) {
+    const a = at(shapeA, axis), b = at(shapeB, axis);
+    if (a !== b && a !== 1 && b !== 1) {
+      throw new Error(`Operands could not be broadcast together with shapes ${shapeA} and ${shapeB}.`);
     }
+    out.push(a === 1 ? b : a);
   }
-  return result;
+  return out;
 }
 
-// ---- conv_util (tfjs-core/src/ops/conv_util.ts) -----------------------------
+// ---- convolution geometry ------------------------------------------------------
 
-function parseTupleParam(param) {
-  if (typeof param === 'number') {
-    return [param, param, param];
-  }
-  if (param.length === 2) {
-    return [param[0], param[1], 1];
-  }
-  return param;
+/** A stride / dilation argument as [h, w, d]: a number repeats, a pair gets depth 1. */
+function tuple3(param) {
+  if (typeof param === 'number') return [param, param, param];
+  return param.length === 2 ? [param[0], param[1], 1] : param;
 }
 
-function tupleValuesAreOne(param) {
-  const t = parseTupleParam(param);
-  return t[0] === 1 && t[1] === 1 && t[2] === 1;
-}
+const tupleValuesAreOne = param => tuple3(param).every(v => v === 1);
 
-function eitherStridesOrDilationsAreOne(strides, dilations) {
-  return tupleValuesAreOne(strides) || tupleValuesAreOne(dilations);
-}
+const eitherStridesOrDilationsAreOne = (strides, dilations) =>
+    tupleValuesAreOne(strides) || tupleValuesAreOne(dilations);
 
 function convertConv2DDataFormat(dataFormat) {
-  if (dataFormat === 'NHWC') {
-    return 'channelsLast';
-  } else if (dataFormat === 'NCHW') {
-    return 'channelsFirst';
-  }
-  throw new Error(`Unknown dataFormat ${dataFormat}`);
+  const names = {NHWC: 'channelsLast', NCHW: 'channelsFirst'};
+  if (!(dataFormat in names)) throw new Error(`Unknown dataFormat ${dataFormat}`);
+  return names[dataFormat];
 }
 
-function roundValue(value, roundingMode) {
-  if (!roundingMode) {
-    return Math.trunc(value);
-  }
-  switch (roundingMode) {
-    case 'round':
-      return Math.round(value);
-    case 'ceil':
-      return Math.ceil(value);
-    case 'floor':
-      return Math.floor(value);
-    default:
-      throw new Error(`Unknown roundingMode ${roundingMode}`);
-  }
+const ROUNDERS = {round: Math.round, ceil: Math.ceil, floor: Math.floor};
+
+function roundExtent(value, mode) {
+  if (!mode) return Math.trunc(value);
+  if (!(mode in ROUNDERS)) throw new Error(`Unknown roundingMode ${mode}`);
+  return ROUNDERS[mode](value);
 }
 
-function getEffectiveFilterSize(filterSize, dilation) {
-  if (dilation <= 1) {
-    return filterSize;
-  }
-  return filterSize + (filterSize - 1) * (dilation - 1);
-}
+/** Span of a filter axis once dilation spreads its taps. */
+const dilatedExtent = (taps, dilation) => (dilation <= 1 ? taps : taps + (taps - 1) * (dilation - 1));
 
-function getPadAndOutInfo(
-    pad, inHeight, inWidth, strideHeight, strideWidth, filterHeight, filterWidth,
-    roundingMode, dataFormat) {
-  let padInfo;
-  let outHeight;
-  let outWidth;
+/**
+ * Output extent and padding of both image axes. `fh`, `fw` are dilated filter
+ * extents. Per axis, with input n, stride s, filter f:
+ *   'same'    out = ceil(n / s); total pad = max(0, (out-1)*s + f - n), the
+ *             smaller half in front
+ *   'valid'   out = ceil((n - f + 1) / s), no pad
+ *   explicit  out = round_mode((n - f + before + after) / s + 1)
+ *   number p  out = round_mode((n - FH + 2p) / SH + 1) on BOTH axes with the
+ *             height's filter extent and stride (conv_util.ts:443-446 does so,
+ *             and results must match it)
+ */
+function padAndOutput(pad, inH, inW, sh, sw, fh, fw, mode, dataFormat) {
   if (typeof pad === 'number') {
-    const padType = (pad === 0) ? 'VALID' : 'NUMBER';
-    padInfo = {top: pad, bottom: pad, left: pad, right: pad, type: padType};
-    // conv_util.ts:443-446: both output dims use the filter height and the
-    // stride height
-    outHeight = roundValue(
-        (inHeight - filterHeight + 2 * pad) / strideHeight + 1, roundingMode);
-    outWidth = roundValue(
-        (inWidth - filterHeight + 2 * pad) / strideHeight + 1, roundingMode);
-  } else if (pad === 'same') {
-    outHeight = Math.ceil(inHeight / strideHeight);
-    outWidth = Math.ceil(inWidth / strideWidth);
-    const padAlongHeight =
-        Math.max(0, (outHeight - 1) * strideHeight + filterHeight - inHeight);
-    const padAlongWidth =
-        Math.max(0, (outWidth - 1) * strideWidth + filterWidth - inWidth);
-    const top = Math.floor(padAlongHeight / 2);
-    const bottom = padAlongHeight - top;
-    const left = Math.floor(padAlongWidth / 2);
-    const right = padAlongWidth - left;
-    padInfo = {top, bottom, left, right, type: 'SAME'};
-  } else if (pad === 'valid') {
-    padInfo = {top: 0, bottom: 0, left: 0, right: 0, type: 'VALID'};
-    outHeight = Math.ceil((inHeight - filterHeight + 1) / strideHeight);
-    outWidth = Math.ceil((inWidth - filterWidth + 1) / strideWidth);
-  } else if (typeof pad === 'object') {
-    const top = dataFormat === 'channelsLast' ? pad[1][0] : pad[2][0];
-    const bottom = dataFormat === 'channelsLast' ? pad[1][1] : pad[2][1];
-    const left = dataFormat === 'channelsLast' ? pad[2][0] : pad[3][0];
-    const right = dataFormat === 'channelsLast' ? pad[2][1] : pad[3][1];
-    const padType = (top === 0 && bottom === 0 && left === 0 && right === 0) ?
-        'VALID' :
-        'EXPLICIT';
-    padInfo = {top, bottom, left, right, type: padType};
-    outHeight = roundValue(
-        (inHeight - filterHeight + top + bottom) / strideHeight + 1,
-        roundingMode);
-    outWidth = roundValue(
-        (inWidth - filterWidth + left + right) / strideWidth + 1, roundingMode);
-  } else {
-    throw Error(`Unknown padding parameter: ${pad}`);
+    const extent = n => roundExtent((n - fh + 2 * pad) / sh + 1, mode);
+    return {
+      padInfo: {top: pad, bottom: pad, left: pad, right: pad, type: pad === 0 ? 'VALID' : 'NUMBER'},
+      outHeight: extent(inH),
+      outWidth: extent(inW)
+    };
   }
-  return {padInfo, outHeight, outWidth};
+  if (pad === 'same') {
+    const axis = (n, s, f) => {
+      const out = Math.ceil(n / s);
+      const total = Math.max(0, (out - 1) * s + f - n);
+      const before = Math.floor(total / 2);
+      return {out, before, after: total - before};
+    };
+    const h = axis(inH, sh, fh), w = axis(inW, sw, fw);
+    return {
+      padInfo: {top: h.before, bottom: h.after, left: w.before, right: w.after, type: 'SAME'},
+      outHeight: h.out,
+      outWidth: w.out
+    };
+  }
+  if (pad === 'valid') {
+    return {
+      padInfo: {top: 0, bottom: 0, left: 0, right: 0, type: 'VALID'},
+      outHeight: Math.ceil((inH - fh + 1) / sh),
+      outWidth: Math.ceil((inW - fw + 1) / sw)
+    };
+  }
+  if (pad !== null && typeof pad === 'object') {
+    // one [before, after] pair per tensor axis, in the tensor's own axis order
+    const hAxis = dataFormat === 'channelsLast' ? 1 : 2;
+    const [top, bottom] = pad[hAxis];
+    const [left, right] = pad[hAxis + 1];
+    const none = top === 0 && bottom === 0 && left === 0 && right === 0;
+    return {
+      padInfo: {top, bottom, left, right, type: none ? 'VALID' : 'EXPLICIT'},
+      outHeight: roundExtent((inH - fh + top + bottom) / sh + 1, mode),
+      outWidth: roundExtent((inW - fw + left + right) / sw + 1, mode)
+    };
+  }
+  throw new Error(`Unknown padding parameter: ${pad}`);
 }
 
-/** computeConv2DInfo (conv_util.ts:177-236). */
-function computeConv2DInfo(
-    inShape, filterShape, strides, dilations, pad, roundingMode, depthwise,
-    dataFormat) {
-  depthwise = depthwise || false;
+/**
+ * The Conv2DInfo record (field names of conv_util.ts:30-74) for an input shape,
+ * an HWIO filter shape, strides, dilations and a pad argument.
+ */
+function computeConv2DInfo(inShape, filterShape, strides, dilations, pad, roundingMode, depthwise, dataFormat) {
   dataFormat = dataFormat || 'channelsLast';
-  let batchSize = -1, inHeight = -1, inWidth = -1, inChannels = -1;
-  if (dataFormat === 'channelsLast') {
-    batchSize = inShape[0];
-    inHeight = inShape[1];
-    inWidth = inShape[2];
-    inChannels = inShape[3];
-  } else if (dataFormat === 'channelsFirst') {
-    batchSize = inShape[0];
-    inChannels = inShape[1];
-    inHeight = inShape[2];
-    inWidth = inShape[3];
-  } else {
+  if (dataFormat !== 'channelsLast' && dataFormat !== 'channelsFirst') {
     throw new Error(`Unknown dataFormat ${dataFormat}`);
   }
-  const filterHeight = filterShape[0];
-  const filterWidth = filterShape[1];
-  const filterChannels = filterShape[3];
-  const s = parseTupleParam(strides);
-  const d = parseTupleParam(dilations);
-  const strideHeight = s[0], strideWidth = s[1];
-  const dilationHeight = d[0], dilationWidth = d[1];
-  const effectiveFilterHeight =
-      getEffectiveFilterSize(filterHeight, dilationHeight);
-  const effectiveFilterWidth =
-      getEffectiveFilterSize(filterWidth, dilationWidth);
-  const info = getPadAndOutInfo(
-      pad, inHeight, inWidth, strideHeight, strideWidth, effectiveFilterHeight,
-      effectiveFilterWidth, roundingMode, dataFormat);
+  const last = dataFormat === 'channelsLast';
+  const batchSize = inShape[0];
+  const inChannels = inShape[last ? 3 : 1];
+  const inHeight = inShape[last ? 1 : 2], inWidth = inShape[last ? 2 : 3];
+  const [filterHeight, filterWidth, , filterChannels] = filterShape;
+  const [strideHeight, strideWidth] = tuple3(strides);
+  const [dilationHeight, dilationWidth] = tuple3(dilations);
+  const effectiveFilterHeight = dilatedExtent(filterHeight, dilationHeight);
+  const effectiveFilterWidth = dilatedExtent(filterWidth, dilationWidth);
+  const {padInfo, outHeight, outWidth} = padAndOutput(
+      pad, inHeight, inWidth, strideHeight, strideWidth, effectiveFilterHeight, effectiveFilterWidth, roundingMode,
+      dataFormat);
   const outChannels = depthwise ? filterChannels * inChannels : filterChannels;
-  let outShape;
-  if (dataFormat === 'channelsFirst') {
-    outShape = [batchSize, outChannels, info.outHeight, info.outWidth];
-  } else {
-    outShape = [batchSize, info.outHeight, info.outWidth, outChannels];
-  }
+  const outShape = last ? [batchSize, outHeight, outWidth, outChannels] : [batchSize, outChannels, outHeight, outWidth];
   return {
-    batchSize,
-    dataFormat,
-    inHeight,
-    inWidth,
-    inChannels,
-    outHeight: info.outHeight,
-    outWidth: info.outWidth,
-    outChannels,
-    padInfo: info.padInfo,
-    strideHeight,
-    strideWidth,
-    filterHeight,
-    filterWidth,
-    effectiveFilterHeight,
-    effectiveFilterWidth,
-    dilationHeight,
-    dilationWidth,
-    inShape,
-    outShape,
-    filterShape
+    batchSize, dataFormat, inHeight, inWidth, inChannels, outHeight, outWidth, outChannels, padInfo,
+    strideHeight, strideWidth, filterHeight, filterWidth, effectiveFilterHeight, effectiveFilterWidth,
+    dilationHeight, dilationWidth, inShape, outShape, filterShape
   };
 }
 
-/** checkPadOnDimRoundingMode (conv_util.ts:607-631). */
+/** A dimRoundingMode only makes sense with whole-number padding (conv_util.ts:607-631). */
 function checkPadOnDimRoundingMode(opDesc, pad, dimRoundingMode) {
-  if (dimRoundingMode != null) {
-    if (typeof pad === 'string') {
-      throw Error(
-          `Error in ${opDesc}: pad must be an integer when using ` +
-          `dimRoundingMode ${dimRoundingMode} but got pad ${pad}.`);
-    } else if (typeof pad === 'number') {
-      assert(
-          isInt(pad),
-          () => `Error in ${opDesc}: pad must be an integer when using ` +
-              `dimRoundingMode ${dimRoundingMode} but got pad ${pad}.`);
-    } else if (typeof pad === 'object') {
-      pad.forEach(p => {
-        p.forEach(v => {
-          assert(
-              isInt(v),
-              () => `Error in ${opDesc}: pad must be an integer when using ` +
-                  `dimRoundingMode ${dimRoundingMode} but got pad ${v}.`);
-        });
-      });
-    } else {
-      throw Error(`Error in ${opDesc}: Unknown padding parameter: ${pad}`);
+  if (dimRoundingMode == null) return;
+  const complain = got => {
+    throw new Error(`Error in ${opDesc}: pad must be an integer when using dimRoundingMode ${dimRoundingMode} ` +
+                    `but got pad ${got}.`);
+  };
+  if (typeof pad === 'string') {
+    complain(pad);
+  } else if (typeof pad === 'number') {
+    if (!isInt(pad)) complain(pad);
+  } else if (pad !== null && typeof pad === 'object') {
+    for (const pair of pad) {
+      for (const v of pair) {
+        if (!isInt(v)) complain(v);
+      }
     }
+  } else {
+    throw new Error(`Error in ${opDesc}: Unknown padding parameter: ${pad}`);
   }
 }
 
 module.exports = {
   util: {
-    assert,
-    sizeFromShape,
-    arraysEqual,
-    computeStrides,
-    isInt,
-    inferFromImplicitShape,
-    parseAxisParam,
-    bytesPerElement,
-    getTypedArrayFromDType,
-    now,
-    indexToLoc,
-    locToIndex
+    assert, sizeFromShape, arraysEqual, computeStrides, isInt, inferFromImplicitShape, parseAxisParam,
+    bytesPerElement, getTypedArrayFromDType, now, indexToLoc, locToIndex
   },
   broadcast_util: {getBroadcastDims, assertAndGetBroadcastShape},
   backend_util: {
-    computeConv2DInfo,
-    convertConv2DDataFormat,
-    eitherStridesOrDilationsAreOne,
-    tupleValuesAreOne,
-    checkPadOnDimRoundingMode,
-    getBroadcastDims,
-    assertAndGetBroadcastShape
+    computeConv2DInfo, convertConv2DDataFormat, eitherStridesOrDilationsAreOne, tupleValuesAreOne,
+    checkPadOnDimRoundingMode, getBroadcastDims, assertAndGetBroadcastShape
   }
 };

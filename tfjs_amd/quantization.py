@@ -1,15 +1,18 @@
-"""Producer side of the quantized weight format: what the converter writes and the
+"""Producer side of the quantized weight format: what a converter writes and the
 dequantize-on-load path consumes.
 
-quantize_weights / dequantize_weights / get_affine_quantization_range follow
-tfjs-converter/python/tensorflowjs/quantization.py (:93-147, :151-173, :175-216);
-write_weights follows the byte layout and manifest of
-tfjs-converter/python/tensorflowjs/write_weights.py (:241-337): the entries of a
-group are concatenated in manifest order, quantized entries as their uint8 /
-uint16 / float16 bytes, and the stream is cut into shards of shard_size_bytes.
+The format is the one tfjs-converter/python/tensorflowjs/quantization.py defines
+(public names quantize_weights :93, dequantize_weights :151) and
+write_weights.py lays out (:241-337): the entries of a group are concatenated in
+manifest order, quantized entries as their uint8 / uint16 / float16 bytes, and
+the stream is cut into shards of shard_size_bytes.
 
-All range arithmetic is float64, as in the reference (min/max are cast with
-astype(np.float64) at quantization.py:123-124).
+Affine codes, in float64 throughout: with L = 255 or 65535 levels a tensor whose
+values span [lo, hi] gets step = (hi - lo) / L and code = rint((x - lo) / step);
+a reader computes code * step + lo. When lo <= 0 <= hi the grid is slid by less
+than half a step so that 0.0 itself is a code: lo' = -rint(-lo / step) * step,
+hi' = lo' + L * step, and values are clamped to [lo', hi'] first. A constant
+tensor is all-zero codes with step 1 and lo = its value.
 """
 import json
 import math
@@ -17,66 +20,61 @@ import os
 
 import numpy as np
 
+_LEVELS = {np.dtype(np.uint8): 255, np.dtype(np.uint16): 65535}
 
-def get_affine_quantization_range(min_val, max_val, quantization_dtype):
-    if quantization_dtype not in (np.uint8, np.uint16):
-        raise ValueError("Invalid `quantization_dtype`: %r" % quantization_dtype)
-    quant_max = np.iinfo(quantization_dtype).max
-    scale = (max_val - min_val) / quant_max
-    if min_val <= 0 <= max_val:
-        quantized_zero_point = (0 - min_val) / scale
-        nudged_zero_point = np.round(quantized_zero_point)
-        # Solve 0 = nudged_zero_point * scale + nudged_min for nudged_min.
-        nudged_min = -nudged_zero_point * scale
-        nudged_max = quant_max * scale + nudged_min
-    else:
-        nudged_min, nudged_max = min_val, max_val
-    return scale, nudged_min, nudged_max
+
+def _code_dtype(kind):
+    try:
+        return np.dtype(kind)
+    except TypeError:
+        return None
+
+
+def _affine_grid(lo, hi, levels):
+    """(step, lo, hi) of the code grid for values spanning [lo, hi], lo < hi."""
+    step = (hi - lo) / levels
+    if lo <= 0.0 <= hi:
+        lo = -np.rint(-lo / step) * step      # zero lands on a code
+        hi = lo + levels * step
+    return step, lo, hi
 
 
 def quantize_weights(data, quantization_dtype):
-    """Returns (quantized ndarray, metadata dict). metadata is {'min', 'scale'}
-    for uint8/uint16 and {} for float16."""
-    if quantization_dtype in (np.uint8, np.uint16):
-        min_val = data.min().astype(np.float64)
-        max_val = data.max().astype(np.float64)
-        if min_val == max_val:
-            quantized = np.zeros_like(data, dtype=quantization_dtype)
-            scale = 1.0
-        else:
-            scale, min_val, max_val = get_affine_quantization_range(
-                min_val, max_val, quantization_dtype)
-            quantized = np.round(
-                (data.astype(np.float64).clip(min_val, max_val) - min_val) / scale
-            ).astype(quantization_dtype)
-        return quantized, {"min": float(min_val), "scale": float(scale)}
-    if quantization_dtype == np.float16:
+    """Encodes `data`; returns (codes, metadata): {'min', 'scale'} for the affine
+    kinds (np.uint8, np.uint16), {} for np.float16 (a plain narrowing cast of
+    float32 data)."""
+    kind = _code_dtype(quantization_dtype)
+    if kind == np.float16:
         if data.dtype != np.float32:
-            raise ValueError(
-                "Invalid data dtype %r\nfloat16 quantization only supports "
-                "float32 dtype" % data.dtype)
+            raise ValueError("float16 quantization takes float32 data, not %s" % data.dtype)
         return data.astype(np.float16), {}
-    raise ValueError("Invalid `quantization_dtype`: %r" % quantization_dtype)
+    if kind not in _LEVELS:
+        raise ValueError("cannot quantize to %r: uint8, uint16 or float16" % (quantization_dtype,))
+    values = np.asarray(data, dtype=np.float64)
+    lo, hi = float(values.min()), float(values.max())
+    if lo == hi:
+        return np.zeros(data.shape, dtype=kind), {"min": lo, "scale": 1.0}
+    step, lo, hi = _affine_grid(lo, hi, _LEVELS[kind])
+    codes = np.rint((np.clip(values, lo, hi) - lo) / step).astype(kind)
+    return codes, {"min": float(lo), "scale": float(step)}
 
 
 def dequantize_weights(data, metadata, original_dtype=np.float32):
-    dtype = data.dtype
-    if dtype in (np.uint8, np.uint16):
-        if not ("scale" in metadata and "min" in metadata):
-            raise ValueError("Missing metadata min or scale for dtype %s" % dtype.name)
-        scale, min_val = metadata["scale"], metadata["min"]
-        if original_dtype == np.int32:
-            return np.round(data * scale + min_val).astype(original_dtype)
-        return (data * scale + min_val).astype(original_dtype)
-    if dtype == np.float16:
+    """Decodes what quantize_weights wrote, with numpy's arithmetic (the device
+    decoder and its CPU restatement follow the JavaScript reader instead)."""
+    kind = data.dtype
+    if kind == np.float16:
         if original_dtype != np.float32:
-            raise ValueError(
-                "Invalid data dtype %r\nfloat16 quantization only supports "
-                "float32 dtype" % data.dtype)
-        return data.astype(original_dtype)
-    raise ValueError(
-        "Invalid dtype %s for dequantization\nSupported dtypes are uint8, "
-        "uint16, float16" % dtype.name)
+            raise ValueError("float16 codes decode to float32 only, not %s" % np.dtype(original_dtype))
+        return data.astype(np.float32)
+    if kind not in _LEVELS:
+        raise ValueError("cannot dequantize %s codes: uint8, uint16 or float16" % kind)
+    if "min" not in metadata or "scale" not in metadata:
+        raise ValueError("%s codes need both 'min' and 'scale'" % kind)
+    values = data * metadata["scale"] + metadata["min"]
+    if original_dtype == np.int32:
+        values = np.round(values)
+    return values.astype(original_dtype)
 
 
 def write_weights(write_dir, weight_groups, quantization_dtype=None, shard_size_bytes=4 * 1024 * 1024):
