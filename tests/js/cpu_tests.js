@@ -397,14 +397,15 @@ h.test('graph model: a converter-format topology runs through the fused ops and 
   h.assertEqual(tf.memory().numTensors, before);
 });
 
-function residualGraphArtifacts() {
+function residualGraphArtifacts(unbatched) {
   // x -> expand (1x1, relu6) -> project (1x1) -> AddV2(x, project) -> Identity: the skip connection of a residual block
   const fused = (ops, n) => ({fused_ops: {list: {s: ops.map(b64)}}, num_args: {i: String(n)}, leakyrelu_alpha: {f: 0.2},
                               strides: {list: {i: ['1', '1', '1', '1']}}, dilations: {list: {i: ['1', '1', '1', '1']}},
                               padding: {s: b64('SAME')}, data_format: {s: b64('NHWC')}, explicit_paddings: {list: {}}});
   const node = (name, op, input, attr) => ({name, op, input, attr: attr || {}});
   const nodes = [
-    node('x', 'Placeholder', [], {dtype: {type: 'DT_FLOAT'}, shape: {shape: {dim: [{size: '-1'}, {size: '4'}, {size: '4'}, {size: '4'}]}}}),
+    node('x', 'Placeholder', [], {dtype: {type: 'DT_FLOAT'}, shape: {shape: {dim:
+        (unbatched ? [] : [{size: '-1'}]).concat([{size: '4'}, {size: '4'}, {size: '4'}])}}}),
     node('e/w', 'Const'), node('e/b', 'Const'), node('p/w', 'Const'), node('p/b', 'Const'),
     node('e', '_FusedConv2D', ['x', 'e/w', 'e/b'], fused(['BiasAdd', 'Relu6'], 1)),
     node('p', '_FusedConv2D', ['e', 'p/w', 'p/b'], fused(['BiasAdd'], 1)),
@@ -474,6 +475,16 @@ h.test('graph model: a convolution read by one Add only runs with it as one Fuse
   tf.dispose([x, w, e, row, z]);
   plain.dispose();
   model.dispose();
+  // an unbatched [h, w, c] input comes back unbatched, as from tf.fused.conv2d followed by tf.add
+  const single = hip.loadGraphModel({load: () => residualGraphArtifacts(true)}, {}, {decodeWeights: hip.decodeWeights});
+  const x3 = tf.tensor(new Float32Array(64), [4, 4, 4]);
+  const live3 = tf.memory().numTensors;
+  const y3 = single.predict(x3);
+  h.assertEqual(y3.shape, [4, 4, 4]);
+  h.assertEqual(fake.lastArgs.fusedConv2D[3], [1, 4, 4, 8, 1, 1, 4, 1, 1, 1, 1, 0, 0, 4, 4]);
+  h.assertEqual(tf.memory().numTensors, live3 + 1);
+  tf.dispose([x3, y3]);
+  single.dispose();
 });
 
 function blockGraphArtifacts() {
@@ -602,6 +613,34 @@ h.test('graph model: {recordLaunches: true} runs node by node once, records the 
   broken.dispose();
   h.assertEqual(work(mark), ['graphDestroy']);
   h.assertEqual(tf.memory().numTensors, before);
+});
+
+h.test('hip storage: while a recorded graph is alive, released buffers go back to the native allocator', () => {
+  const fake = require('./fake_addon');
+  useBackend('hip');
+  const backend = tf.backend();
+  backend.releasePool();
+  const live = () => fake.memoryInfo().live;
+  const base = live();
+  const w = tf.tensor(new Float32Array(8), [8]);
+  h.assertEqual(live(), base + 1);
+  backend.beginRecording();
+  const graph = backend.endRecording(true);
+  h.assertEqual(backend.liveRecordings, 1);
+  // a buffer the graph may name is given up: the native side (which checks replays) must see it go
+  w.dispose();
+  h.assertEqual(live(), base, 'not parked on a free list of the backend');
+  h.assertEqual(backend.pooledBuffers, 0);
+  backend.deleteRecording(graph.id);
+  h.assertEqual(backend.liveRecordings, 0);
+  // a discarded recording does not count
+  backend.beginRecording();
+  backend.endRecording(false);
+  h.assertEqual(backend.liveRecordings, 0);
+  const v = tf.tensor(new Float32Array(8), [8]);
+  v.dispose();
+  h.assertEqual(backend.pooledBuffers, 1, 'no graph alive: the free lists serve again');
+  backend.releasePool();
 });
 
 h.test('graph model: unsupported nodes and malformed fused nodes throw the reference errors', () => {

@@ -400,6 +400,42 @@ def test_conv2d_few_taps_shapes(hip, orc, xs, fs, stride, dil, pad, act):
     assert_parity(hip.fused_conv2d(x, w, **kw), orc.fused_conv2d(x, w, **kw))
 
 
+@pytest.mark.parametrize("tile", range(13))
+def test_every_gemm_tile_shape_with_every_loader(hip, orc, tuning, tile):
+    # each of the 13 tile shapes forced in turn (five of them ask for more than 64 KB of LDS) over the four
+    # operand layouts of the vector loaders, the vector im2col loader, and the scalar loaders on shapes no
+    # float4 fetch can take; ragged against every tile edge
+    from tfjs_amd.capi import load_library
+    tuning("tile", tile)
+    tuning("no_skinny", 1)
+    rng = np.random.default_rng(1300 + tile)
+    m, n, k = 268, 132, 72
+    name = ctypes.create_string_buffer(256)
+    seen = set()
+    for ta, tb in [(0, 0), (0, 1), (1, 0), (1, 1)]:
+        a = rng.uniform(-1, 1, (k, m) if ta else (m, k)).astype(np.float32)
+        b = rng.uniform(-1, 1, (n, k) if tb else (k, n)).astype(np.float32)
+        kw = dict(bias=rng.uniform(-1, 1, (n,)).astype(np.float32), activation="relu", transpose_a=bool(ta),
+                  transpose_b=bool(tb))
+        assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
+        load_library().tfhip_last_kernel(name, 256)
+        seen.add(name.value.decode())
+    assert len(seen) == 4 and all(s.startswith("gemm_kernel<") for s in seen), seen
+    x = rng.uniform(-1, 1, (2, 13, 11, 8)).astype(np.float32)
+    w = rng.normal(0, 0.3, (3, 3, 8, 20)).astype(np.float32)
+    kw = dict(pad="same", strides=2, bias=rng.uniform(-1, 1, (20,)).astype(np.float32), activation="relu6")
+    assert_parity(hip.fused_conv2d(x, w, **kw), orc.fused_conv2d(x, w, **kw))
+    load_library().tfhip_last_kernel(name, 256)
+    assert name.value.decode().endswith("3, 1>"), name.value      # vector im2col A, row-major B
+    # odd extents: the scalar loaders (their tile shape is fixed, the knob must not break them)
+    a = rng.uniform(-1, 1, (37, 23)).astype(np.float32)
+    b = rng.uniform(-1, 1, (23, 19)).astype(np.float32)
+    assert_parity(hip.fused_matmul(a, b), orc.fused_matmul(a, b))
+    x = rng.uniform(-1, 1, (1, 9, 7, 5)).astype(np.float32)
+    w = rng.normal(0, 0.3, (3, 3, 5, 6)).astype(np.float32)
+    assert_parity(hip.fused_conv2d(x, w, pad="same"), orc.fused_conv2d(x, w, pad="same"))
+
+
 @pytest.mark.parametrize("fmt", ["NHWC", "NCHW"])
 def test_conv2d_split_k(hip, orc, tuning, fmt):
     tuning("splitk", 3)
@@ -743,9 +779,18 @@ def test_recorded_graph_replays(hip, orc):
             np.testing.assert_array_equal(side.download(np.float32, x.size), got.reshape(-1))
             side.free()
         # a graph that names a freed buffer refuses to run
-        bufs.pop("b3").free()
+        b3_ptr = bufs.pop("b3")
+        b3_addr = b3_ptr.ptr
+        b3_ptr.free()
         assert lib.tfhip_graph_launch(gid.value) != 0
         assert b"has been freed" in lib.tfhip_last_error()
+        # ... also when the same address has been handed out again for a block of the same size class:
+        # it is another tensor's memory now
+        again = capi.DeviceBuffer(16 * 4)
+        assert again.ptr == b3_addr, "the pool hands a freed block of the class out again"
+        assert lib.tfhip_graph_launch(gid.value) != 0
+        assert b"has been freed" in lib.tfhip_last_error()
+        again.free()
         check(lib.tfhip_graph_destroy(gid.value))
         assert lib.tfhip_graph_launch(gid.value) != 0
         assert hip.memory_info()["pooled_bytes"] >= pooled_before

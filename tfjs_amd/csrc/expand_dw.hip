@@ -387,6 +387,8 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
   const int64_t lim = 0x7fffffff;
   TFHIP_CHECK_ARG(batch * in_h * in_w * (in_c > mid_c ? in_c : mid_c) < lim && batch * out_h * out_w * mid_c < lim,
                   "tfhip_fused_pointwise_depthwise: tensor exceeds the supported range");
+  TFHIP_CHECK_ARG(batch * in_h * in_w * in_c * 4 <= 0xfffffffeLL,
+                  "tfhip_fused_pointwise_depthwise: x exceeds the 4 GiB one buffer descriptor addresses");
   TFHIP_CHECK_ARG(pw_activation >= TFHIP_LINEAR && pw_activation <= TFHIP_ELU && dw_activation >= TFHIP_LINEAR &&
                       dw_activation <= TFHIP_ELU,
                   "tfhip_fused_pointwise_depthwise: unknown activation");

@@ -125,6 +125,16 @@ inline int launch_gemm(GemmParams &p) {
     p.group_m = g > p.tiles_m ? p.tiles_m : g;
   }
   if (grid > 0x7fffffffLL) return fail(kBadArgument, "gemm: %lld tiles exceed the grid limit", grid);
+  if (T::LDS_FLOATS * sizeof(float) > 64 * 1024) {
+    // dynamic LDS above the default limit: the attribute once per instantiation and device set-up
+    static int raised = 0;
+    if (raised != init_count()) {
+      TFHIP_CHECK_HIP(hipFuncSetAttribute(
+          reinterpret_cast<const void *>(gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>),
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)(T::LDS_FLOATS * sizeof(float))));
+      raised = init_count();
+    }
+  }
   note_kernel("gemm_kernel<%d, %d, %d, %d, %d, %d, %d>", BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND);
   // The fused epilogue covers per-column operands with a relu-family activation;
   // anything else leaves raw sums for gemm_finish.

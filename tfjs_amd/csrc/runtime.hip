@@ -21,7 +21,12 @@ struct RecordedGraph {
   hipGraphExec_t exec = nullptr;
   size_t nodes = 0;
   std::vector<std::pair<void *, size_t>> owned;         // block, class size
-  std::vector<std::pair<uintptr_t, size_t>> refs;       // base, size of blocks that must stay live
+  struct Ref {
+    uintptr_t base;
+    size_t size;
+    uint64_t generation;
+  };
+  std::vector<Ref> refs;   // blocks a recorded kernel names and that were live when the recording ended
 };
 
 struct Runtime {
@@ -32,6 +37,10 @@ struct Runtime {
   // live blocks: base address -> usable size. `owned` blocks came from the pool.
   std::map<uintptr_t, size_t> live;
   std::map<uintptr_t, bool> owned;
+  // Every hand-out of an address (tfhip_alloc, tfhip_register_external) gets a new
+  // number: an address that was freed and handed out again is a different block.
+  std::map<uintptr_t, uint64_t> generation;
+  uint64_t next_generation = 1;
   std::unordered_map<size_t, std::vector<void *>> free_lists;  // by class size
   size_t live_bytes = 0, pooled_bytes = 0;
   void *staging[kStagingBuffers] = {nullptr, nullptr};
@@ -258,6 +267,7 @@ int tfhip_shutdown(void) {
   }
   g.live.clear();
   g.owned.clear();
+  g.generation.clear();
   g.live_bytes = 0;
   release_pool_locked();
   for (int i = 0; i < kStagingBuffers; ++i) {
@@ -321,6 +331,7 @@ int tfhip_alloc(size_t bytes, void **dptr) {
   }
   g.live[reinterpret_cast<uintptr_t>(p)] = cls;
   g.owned[reinterpret_cast<uintptr_t>(p)] = true;
+  g.generation[reinterpret_cast<uintptr_t>(p)] = g.next_generation++;
   g.live_bytes += cls;
   *dptr = p;
   return kOk;
@@ -339,6 +350,7 @@ int tfhip_free(void *dptr) {
   const size_t cls = it->second;
   g.live.erase(it);
   g.owned.erase(a);
+  g.generation.erase(a);
   g.live_bytes -= cls;
   if (g.capturing) {
     g.capture_free[cls].push_back(dptr);   // the graph being recorded names it: the graph keeps it
@@ -354,6 +366,7 @@ int tfhip_register_external(void *dptr, size_t bytes) {
   std::lock_guard<std::mutex> lock(g_mutex);
   g.live[reinterpret_cast<uintptr_t>(dptr)] = bytes;
   g.owned[reinterpret_cast<uintptr_t>(dptr)] = false;
+  g.generation[reinterpret_cast<uintptr_t>(dptr)] = g.next_generation++;
   return kOk;
 }
 
@@ -367,6 +380,7 @@ int tfhip_unregister_external(void *dptr) {
   }
   g.live.erase(it);
   g.owned.erase(a);
+  g.generation.erase(a);
   return kOk;
 }
 
@@ -535,7 +549,7 @@ int tfhip_capture_end(int *graph_id, int *nodes) {
   g.capture_free.clear();
   for (uintptr_t base : g.capture_refs) {
     auto it = g.live.find(base);
-    if (it != g.live.end()) rec.refs.emplace_back(base, it->second);
+    if (it != g.live.end()) rec.refs.push_back({base, it->second, g.generation[base]});
   }
   g.capture_refs.clear();
   const int id = g.next_graph++;
@@ -552,11 +566,14 @@ int tfhip_graph_launch(int graph_id) {
   auto it = g.graphs.find(graph_id);
   TFHIP_CHECK_ARG(it != g.graphs.end(), "tfhip_graph_launch: no graph %d", graph_id);
   for (auto &r : it->second.refs) {
-    auto b = g.live.find(r.first);
-    if (b == g.live.end() || b->second != r.second) {
+    // the same address, size AND hand-out: a block that was freed and handed out again
+    // at the same address belongs to someone else now
+    auto b = g.live.find(r.base);
+    auto gen = g.generation.find(r.base);
+    if (b == g.live.end() || b->second != r.size || gen == g.generation.end() || gen->second != r.generation) {
       return fail(kOutOfRange,
                   "tfhip_graph_launch: graph %d names the device buffer at %p (%zu bytes), which has been freed since it was recorded",
-                  graph_id, reinterpret_cast<void *>(r.first), r.second);
+                  graph_id, reinterpret_cast<void *>(r.base), r.size);
     }
   }
   for (int r = g_repeat; r > 0; --r) TFHIP_CHECK_HIP(hipGraphLaunch(it->second.exec, g.stream));

@@ -28,7 +28,12 @@
  * them; replay(id) then runs the whole sequence with one native call. While
  * recording, buffers bypass the free lists here, so that the native library
  * sees every buffer that is released and keeps it for the graph; uploads and
- * downloads are refused by the native library until the recording ends.
+ * downloads are refused by the native library until the recording ends. While
+ * any recorded graph is alive, released buffers keep going straight back to the
+ * native allocator: it alone can tell that a buffer a graph names has been given
+ * up (a replay is then refused instead of reading a buffer that meanwhile
+ * belongs to another tensor), and a buffer parked on a free list here would
+ * still count as live there.
  */
 const tf = require('./core');
 const {addon} = require('./binding');
@@ -58,6 +63,7 @@ class HipBackend extends tf.KernelBackend {
     this.pooledBytes = 0;
     this.poolLimitBytes = this.deviceInfo.hbmBytes / 4;
     this.recording = false;
+    this.liveRecordings = 0;
   }
 
   /** Kernels enqueued from now on are recorded, not run. */
@@ -75,7 +81,11 @@ class HipBackend extends tf.KernelBackend {
       throw new Error('tfjs-backend-hip: no recording is open');
     }
     this.recording = false;
-    return addon.captureEnd(keep !== false);
+    const graph = addon.captureEnd(keep !== false);
+    if (graph.id) {
+      this.liveRecordings++;
+    }
+    return graph;
   }
 
   /** Runs a recorded graph once more, on the addresses it was recorded with. */
@@ -85,6 +95,7 @@ class HipBackend extends tf.KernelBackend {
 
   deleteRecording(id) {
     addon.graphDestroy(id);
+    this.liveRecordings--;
   }
 
   /** Device-to-device copy between the buffers of two dataIds of the same size. */
@@ -126,8 +137,10 @@ class HipBackend extends tf.KernelBackend {
   }
 
   release(ptr, bytes) {
-    if (this.recording) {
-      addon.free(ptr);   // the native library keeps it for the graph being recorded
+    if (this.recording || this.liveRecordings > 0) {
+      // recording: the native library keeps it for the graph; a graph is alive: the
+      // native library must see the release to refuse a replay that names the buffer
+      addon.free(ptr);
       return;
     }
     if (this.pooledBytes + bytes > this.poolLimitBytes) {

@@ -182,18 +182,29 @@ function compileConvAdd(convNode) {
   const convInputs = (convNode.input || []).filter(i => i[0] !== '^').length;
   return inputs => {
     const p = params(inputs);
-    let x = p.x;
+    let x = p.x, residual = inputs[convInputs];
     const batched = x.shape.length === 4;
     if (!batched) {
-      x = tf.reshape(x, [1, x.shape[0], x.shape[1], x.shape[2]]);   // as tf.fused.conv2d does for rank 3
+      // as tf.fused.conv2d does for rank 3: a batch of one going in, rank 3 coming out
+      x = tf.reshape(x, [1, x.shape[0], x.shape[1], x.shape[2]]);
+      if (residual.shape.length === 3) {
+        residual = tf.reshape(residual, [1, residual.shape[0], residual.shape[1], residual.shape[2]]);
+      }
     }
     const out = tf.engine().runKernel(
         'FusedConv2DAdd',
-        {x, filter: p.filter, bias: p.bias, preluActivationWeights: p.preluActivationWeights,
-         residual: inputs[convInputs]},
+        {x, filter: p.filter, bias: p.bias, preluActivationWeights: p.preluActivationWeights, residual},
         {strides: p.strides, pad: p.pad, dataFormat: p.dataFormat, dilations: p.dilations,
          dimRoundingMode: undefined, activation: p.activation, leakyreluAlpha: p.leakyreluAlpha});
-    return out;
+    if (batched) {
+      return out;
+    }
+    const squeezed = tf.reshape(out, [out.shape[1], out.shape[2], out.shape[3]]);
+    tf.dispose([x, out]);
+    if (residual !== inputs[convInputs]) {
+      residual.dispose();
+    }
+    return squeezed;
   };
 }
 
