@@ -659,6 +659,66 @@ def test_pointwise_depthwise_fused(hip, orc, case):
         assert_parity(got, two, 1e-5)
 
 
+TILE_CASES = [
+    # batch, h, w, in_c, mid_c, stride, pad, activation, knobs (tile_slice, tile_chunks)
+    (2, 14, 14, 64, 384, 1, "same", "relu6", {}),                  # MobileNetV2's 14x14 blocks: whole image per tile
+    (3, 14, 14, 96, 576, 1, "same", "relu6", {}),
+    (2, 14, 14, 96, 576, 2, "same", "relu6", {}),                  # stride 2: 15x15 expanded tile, 7x7 out
+    (2, 7, 7, 160, 960, 1, "same", "relu6", {}),                   # ten k groups; 7 columns: two row parts per column
+    (2, 28, 28, 32, 192, 1, "same", "relu6", {}),                  # row chunks with halo rows
+    (2, 28, 28, 32, 192, 2, "same", "relu", {}),
+    (1, 28, 28, 16, 96, 1, "same", "relu6", {"tile_slice": 32}),   # one k group, slices of two channel blocks
+    (2, 20, 14, 24, 64, 1, "same", "relu6", {}),                   # K = 24: a full k group and a half one; one slice of 64
+    (1, 9, 23, 16, 96, 1, "valid", "relu6", {}),                   # no padding: every tile position lies in the image
+    (2, 17, 13, 32, 96, 2, "same", "relu", {"tile_chunks": 3}),    # odd sizes, ragged last chunk
+    (1, 5, 5, 64, 192, 1, [[0, 0], [2, 0], [1, 2], [0, 0]], "relu6", {"tile_slice": 64}),   # explicit, lopsided padding
+    (2, 14, 14, 64, 384, 1, "same", "relu6", {"tile_slice": 64, "tile_chunks": 2}),
+    (2, 14, 14, 64, 384, 1, "same", "relu6", {"tile_slice": 32, "tile_chunks": 14}),        # one output row per chunk
+    (32, 14, 14, 64, 384, 1, "same", "relu6", {}),                 # the full batch
+]
+
+
+@pytest.mark.parametrize("case", TILE_CASES, ids=[str(i) for i in range(len(TILE_CASES))])
+def test_pointwise_depthwise_tile_kernel(hip, orc, tuning, case):
+    """The channel-sliced fused kernel against the oracle's two convolutions and against the two
+    separate launches (whose instruction order it keeps: the same bits)."""
+    from tfjs_amd import capi
+    n, h, w, cin, mid, stride, pad, act, knobs = case
+    tuning("pw_dw_tile", 1)
+    for k, v in knobs.items():
+        tuning(k, v)
+    rng = np.random.default_rng(n * 17 + h * 3 + w + cin + mid + stride)
+    x = rng.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    w1 = rng.normal(0, 0.4, (1, 1, cin, mid)).astype(np.float32)
+    b1 = rng.uniform(-1, 2, (mid,)).astype(np.float32)       # positive: relu6(bias) is far from the zero padding
+    w2 = rng.normal(0, 0.5, (3, 3, mid, 1)).astype(np.float32)
+    b2 = rng.uniform(-1, 1, (mid,)).astype(np.float32)
+    got = hip.fused_pointwise_depthwise(x, w1, w2, strides=stride, pad=pad, pw_bias=b1, pw_activation=act,
+                                        dw_bias=b2, dw_activation=act)
+    name = ctypes.create_string_buffer(256)
+    capi.load_library().tfhip_last_kernel(name, 256)
+    assert name.value.decode().startswith("expand_dw_tile<"), name.value
+    mid_hip = hip.fused_conv2d(x, w1, bias=b1, activation=act)
+    capi.load_library().tfhip_last_kernel(name, 256)
+    two = hip.fused_depthwise_conv2d(mid_hip, w2, strides=stride, pad=pad, bias=b2, activation=act)
+    if n <= 4:
+        want = orc.fused_depthwise_conv2d(orc.fused_conv2d(x, w1, bias=b1, activation=act), w2, strides=stride, pad=pad,
+                                          bias=b2, activation=act)
+        assert_parity(got, want)
+    # the tiled GEMM feeds the matrix cores in the same order when K is whole k groups of 16 (it
+    # pads a half group with zeros where this kernel, like the streaming GEMM, runs two instructions)
+    first = name.value.decode()
+    if first.startswith("skinny_gemm_regs") or (first.startswith("gemm_kernel") and cin % 16 == 0):
+        np.testing.assert_array_equal(got.view(np.uint32), two.view(np.uint32))
+    else:
+        assert_parity(got, two, 1e-5)
+    # without biases
+    got = hip.fused_pointwise_depthwise(x[:1], w1, w2, strides=stride, pad=pad, pw_activation=act, dw_activation=act)
+    want = orc.fused_depthwise_conv2d(orc.fused_conv2d(x[:1], w1, activation=act), w2, strides=stride, pad=pad,
+                                      activation=act)
+    assert_parity(got, want)
+
+
 STEM_DW_CASES = [
     # x shape, filter shape, conv stride, conv pad, depthwise stride, depthwise pad, activation
     ((3, 64, 64, 3), (3, 3, 3, 32), 2, "same", 1, "same", "relu6"),        # MobileNetV2's stem and first depthwise stage
@@ -704,9 +764,12 @@ def test_pointwise_depthwise_without_biases_and_unsupported_shapes(hip, orc):
     assert lib.tfhip_pointwise_depthwise_pays(32, 16, 96, 2, 56, 56) == 1
     assert lib.tfhip_pointwise_depthwise_pays(32, 24, 144, 2, 28, 28) == 1
     assert lib.tfhip_pointwise_depthwise_pays(32, 24, 144, 1, 56, 56) == 1
-    assert lib.tfhip_pointwise_depthwise_pays(32, 32, 192, 1, 28, 28) == 0     # taken, but the two kernels are faster
+    assert lib.tfhip_pointwise_depthwise_pays(32, 32, 192, 1, 28, 28) == 1     # the channel-sliced kernel
+    assert lib.tfhip_pointwise_depthwise_pays(32, 64, 384, 1, 14, 14) == 1
+    assert lib.tfhip_pointwise_depthwise_pays(32, 160, 960, 1, 7, 7) == 1
     assert lib.tfhip_pointwise_depthwise_pays(1, 16, 96, 2, 56, 56) == 0       # one image: the expanded tensor is small
-    assert lib.tfhip_pointwise_depthwise_pays(32, 64, 384, 1, 14, 14) == 0     # too many input channels
+    assert lib.tfhip_pointwise_depthwise_pays(1, 64, 384, 1, 14, 14) == 0      # ... and too few workgroups to fill the chip
+    assert lib.tfhip_pointwise_depthwise_pays(32, 128, 384, 1, 14, 14) == 0    # a count of input channels neither kernel has
     assert lib.tfhip_pointwise_depthwise_pays(64, 16, 40, 2, 112, 112) == 0    # channels no multiple of 16
     assert lib.tfhip_pointwise_depthwise_pays(64, 16, 96, 3, 112, 112) == 0    # stride 3
     with pytest.raises(capi.HipBackendError, match="run the two convolutions"):
@@ -842,17 +905,22 @@ def test_config4_mobilenet_v2_batch1_vs_oracle(hip, orc, tmp_path):
         assert_parity(plain.predict(), got, 1e-4)
     finally:
         plain.close()
-    # at batch 32 the first expansions run fused with their depthwise stage: the same bits as the separate kernels
+    # at batch 32 (the benchmark's workload) the stem and every expansion run fused with their depthwise
+    # stage, with the kernels that batch selects: against the oracle end to end, and the same bits as the
+    # separate kernels
     x32 = workloads.mobilenet_v2_input(32)
+    want32 = workloads.run_graph(orc, ops, decoded, x32)
     outs = []
     for fuse in (True, False):
         m32 = workloads.DeviceMobileNetV2(str(tmp_path), 32, fuse_expand_depthwise=fuse)
         try:
-            assert sum(1 for op, _ in m32.plan if op["kind"] in ("pwdw", "cvdw")) == (4 if fuse else 0)
+            assert sum(1 for op, _ in m32.plan if op["kind"] in ("pwdw", "cvdw")) == (17 if fuse else 0)
             m32.set_input(x32)
             outs.append(m32.predict())
         finally:
             m32.close()
+    assert_parity(outs[0], want32)
+    assert_parity(outs[1], want32)
     np.testing.assert_array_equal(outs[0], outs[1])
     # the kernel-by-kernel host mirror agrees too
     assert_parity(workloads.run_graph(hip, ops, decoded, x[:1]), want[:1])

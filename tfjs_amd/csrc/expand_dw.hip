@@ -26,6 +26,7 @@
 //                the depthwise stage pads with), not activation(bias)
 #include "common.h"
 #include "epilogue.h"
+#include "expand_dw_tile.h"
 
 namespace tfhip {
 namespace {
@@ -375,6 +376,18 @@ bool plan_expand_dw(ExpandDwArgs &g, int stride, int K, size_t *lds_bytes) {
 
 using namespace tfhip;
 
+namespace {
+
+// Where both fused kernels take a shape: the row-ring kernel for the wide maps of the first
+// blocks (its workgroups split the map, and every one needs all expanded channels), the tile
+// kernel from 28x28 down (its workgroups split the channels).
+bool prefer_tile_kernel(int64_t batch, int64_t in_c, int64_t mid_c, int64_t stride, int64_t out_h, int64_t out_w) {
+  (void)batch; (void)in_c; (void)mid_c; (void)out_h;
+  return out_w * stride <= 28;
+}
+
+}  // namespace
+
 extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_filter, const float *pw_bias,
                                                int pw_activation, const float *dw_filter, const float *dw_bias,
                                                int dw_activation, float *y, int64_t batch, int64_t in_h,
@@ -400,6 +413,13 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
   if (dw_bias) TFHIP_CHECK_RANGE(dw_bias, mid_c, 4, "dw_bias");
   TFHIP_CHECK_RANGE(y, batch * out_h * out_w * mid_c, 4, "y");
 
+  const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(pw_filter) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(dw_filter) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+                       (dw_bias == nullptr || reinterpret_cast<uintptr_t>(dw_bias) % 16 == 0);
+  const bool same_relu = pw_activation == dw_activation && (pw_activation == TFHIP_RELU || pw_activation == TFHIP_RELU6);
+
+  // the row-ring kernel (all channels per workgroup: wide maps, few channels)
   ExpandDwArgs g = {};
   g.x = x; g.w1 = pw_filter; g.b1 = pw_bias; g.w2 = dw_filter; g.b2 = dw_bias; g.y = y;
   g.batch = (int)batch; g.in_h = (int)in_h; g.in_w = (int)in_w; g.cin = (int)in_c; g.c = (int)mid_c;
@@ -407,16 +427,32 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
   g.act1 = pw_activation; g.act2 = dw_activation;
   g.x_bytes = (unsigned)(batch * in_h * in_w * in_c * 4);
   size_t lds_bytes = 0;
-  const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(pw_filter) % 16 == 0 &&
-                       reinterpret_cast<uintptr_t>(dw_filter) % 16 == 0 &&
-                       reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
-                       (dw_bias == nullptr || reinterpret_cast<uintptr_t>(dw_bias) % 16 == 0);
-  const bool same_relu = pw_activation == dw_activation && (pw_activation == TFHIP_RELU || pw_activation == TFHIP_RELU6);
   const bool k_ok = in_c == 8 || in_c == 16 || in_c == 24 || in_c == 32;
-  if (!aligned || !same_relu || !k_ok || !plan_expand_dw(g, (int)stride, (int)in_c, &lds_bytes)) {
+  const bool ring_ok = aligned && same_relu && k_ok && plan_expand_dw(g, (int)stride, (int)in_c, &lds_bytes);
+
+  // the channel-sliced tile kernel (small maps, many channels)
+  ExpandDwTileArgs t = {};
+  t.x = x; t.w1 = pw_filter; t.b1 = pw_bias; t.w2 = dw_filter; t.b2 = dw_bias; t.y = y;
+  t.batch = (int)batch; t.in_h = (int)in_h; t.in_w = (int)in_w; t.cin = (int)in_c; t.c = (int)mid_c;
+  t.stride = (int)stride; t.pad_top = (int)pad_top; t.pad_left = (int)pad_left; t.out_h = (int)out_h; t.out_w = (int)out_w;
+  t.cap = pw_activation == TFHIP_RELU6 ? 6.f : __builtin_inff();
+  t.x_bytes = g.x_bytes;
+  size_t tile_lds_bytes = 0;
+  const bool tile_ok = aligned && same_relu &&
+                       (pw_bias == nullptr || reinterpret_cast<uintptr_t>(pw_bias) % 16 == 0) &&
+                       plan_expand_dw_tile(t, &tile_lds_bytes);
+
+  bool use_tile = tile_ok && !ring_ok;
+  if (tile_ok && ring_ok) {
+    const int knob = tuning(kTunePwDwTile);
+    use_tile = knob >= 0 ? knob > 0 : prefer_tile_kernel(batch, in_c, mid_c, stride, out_h, out_w);
+  }
+  if (use_tile) return launch_expand_dw_tile(t, tile_lds_bytes);
+  if (!ring_ok) {
     return fail(kBadArgument,
-                "tfhip_fused_pointwise_depthwise: form not taken by the fused kernel (in_c 8/16/24/32, mid_c a "
-                "multiple of 16 up to 256, stride 1 or 2, both activations relu or both relu6, 16-byte aligned "
+                "tfhip_fused_pointwise_depthwise: form not taken by the fused kernels (in_c 8/16/24/32 with mid_c a "
+                "multiple of 16 up to 256, or in_c 16/24/32/64/96/160 with mid_c a multiple of 32 on a map that "
+                "fits the kernel's tile; stride 1 or 2, both activations relu or both relu6, 16-byte aligned "
                 "operands); run the two convolutions");
   }
   const int key = (int)stride * 100 + (int)in_c;
@@ -441,18 +477,24 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
 // tensor of at least 48 MB.
 extern "C" int tfhip_pointwise_depthwise_pays(int64_t batch, int64_t in_c, int64_t mid_c, int64_t stride,
                                               int64_t out_h, int64_t out_w) {
-  if (!initialised() || batch <= 0 || out_h <= 0 || out_w <= 0 || mid_c <= 0 || mid_c > 0x7fffffff || in_c > 64 ||
-      batch > 0x7fffffff || out_h > 0x7fffffff || out_w > 0x7fffffff) {
+  if (!initialised() || batch <= 0 || out_h <= 0 || out_w <= 0 || mid_c <= 0 || mid_c > 0x7fffffff || in_c <= 0 ||
+      in_c > 0x7fffffff || batch > 0x7fffffff || out_h > 0x7fffffff || out_w > 0x7fffffff) {
     return 0;
   }
   ExpandDwArgs g = {};
   g.batch = (int)batch; g.cin = (int)in_c; g.c = (int)mid_c; g.out_h = (int)out_h; g.out_w = (int)out_w;
   size_t lds_bytes = 0;
   const bool k_ok = in_c == 8 || in_c == 16 || in_c == 24 || in_c == 32;
-  if (!k_ok || !plan_expand_dw(g, (int)stride, (int)in_c, &lds_bytes)) return 0;
+  const bool ring_ok = k_ok && plan_expand_dw(g, (int)stride, (int)in_c, &lds_bytes);
+  ExpandDwTileArgs t = {};
+  t.batch = (int)batch; t.cin = (int)in_c; t.c = (int)mid_c; t.stride = (int)stride; t.out_h = (int)out_h; t.out_w = (int)out_w;
+  const bool tile_ok = plan_expand_dw_tile(t, &lds_bytes);
+  if (!ring_ok && !tile_ok) return 0;
   if (tuning(kTuneFusePwDw) >= 0) return tuning(kTuneFusePwDw) > 0 ? 1 : 0;   // knob: always / never
   const int64_t expanded_bytes = batch * out_h * stride * out_w * stride * mid_c * 4;
-  return expanded_bytes >= 48LL * 1000 * 1000 ? 1 : 0;
+  if (ring_ok && expanded_bytes >= 48LL * 1000 * 1000) return 1;
+  // the tile kernel: one launch instead of two once the launch has enough workgroups to fill the chip
+  return tile_ok && (long long)t.batch * t.chunks_h * t.slices >= num_cus() / 2 ? 1 : 0;
 }
 
 namespace {
