@@ -123,7 +123,11 @@ int tfhip_graph_destroy(int graph_id);
  *   streaming GEMM always stages B in LDS), "small_k" (32 / 64: the one-shot GEMM for
  *   K <= 64 with that many rows per tile; unset or 0: never), "fuse_pw_dw"
  *   (tfhip_pointwise_depthwise_pays: 1: yes for every shape the fused kernel
- *   takes, 0: never). TFHIP_TILE,
+ *   takes, 0: never), "pw_dw_tile" (1 / 0: the channel-sliced / the row-ring
+ *   pointwise + depthwise kernel where both take a shape), "tile_slice" (32 / 48 /
+ *   64 channels per workgroup of the channel-sliced kernel), "tile_chunks" (its row
+ *   chunks per image), "block_rows" (output rows per workgroup of the whole-block
+ *   kernel), "fuse_block" (tfhip_inverted_residual_pays: 1 always, 0 never). TFHIP_TILE,
  *   TFHIP_SPLITK, TFHIP_DW_ROWS, TFHIP_DW_HALO, TFHIP_NO_SKINNY, TFHIP_DW_FLAT,
  *   TFHIP_SKINNY_REGS, TFHIP_SMALL_K, TFHIP_FUSE_PW_DW in the environment set them at
  *   tfhip_init(). */
@@ -280,6 +284,47 @@ int tfhip_fused_conv2d_depthwise(const float *x, const float *filter, const floa
 int tfhip_conv2d_depthwise_pays(int64_t batch, int64_t in_c, int64_t f_h, int64_t f_w,
                                 int64_t mid_c, int64_t mid_h, int64_t mid_w,
                                 int64_t dw_stride, int64_t out_h, int64_t out_w);
+
+/* ---- a whole inverted-residual block in one launch -------------------------------
+ * y = conv1x1(dw_act(depthwise3x3(pw_act(conv1x1(x, pw) + pw_bias), dw) + dw_bias), proj) + proj_bias
+ *     [+ residual]:
+ * the expansion, the depthwise stage and the linear projection of an inverted-residual
+ * block, and the Add of its skip connection where `residual` is not NULL, without the
+ * expanded tensor or the depthwise output ever reaching memory. In a graph these are a
+ * FusedConv2D node with a 1x1 filter (convolution_executor.ts:100-137), the
+ * FusedDepthwiseConv2dNative node that is its only reader (3x3, channel multiplier 1,
+ * dilation 1; convolution_executor.ts:139-173), the 1x1 FusedConv2D with no activation
+ * that is that node's only reader, and the Add / AddV2 node (arithmetic_executor.ts:30-37)
+ * that reads the projection and a tensor of its shape. Every intermediate value is
+ * rounded as the separate kernels round it: the result equals tfhip_fused_conv2d,
+ * tfhip_fused_depthwise_conv2d and tfhip_fused_conv2d_add in turn.
+ * NHWC; x [batch,in_h,in_w,in_c]; y and residual [batch,out_h,out_w,out_c]; stride,
+ * pad_top, pad_left, out_h, out_w are the depthwise stage's; `activation` (relu or
+ * relu6) is that of the expansion and of the depthwise stage; the projection is linear.
+ * The two 1x1 filters come TRANSPOSED, k-contiguous per output channel:
+ * pw_filter_t [mid_c,in_c] and proj_filter_t [out_c,mid_c] (tfhip_transpose2d of the
+ * HWIO filters' [in,out] matrices: a caller does it once per model); dw_filter is
+ * [3,3,mid_c]; biases may be NULL.
+ * The kernel takes in_c 32 / 64 / 96 / 160, mid_c a multiple of 64, out_c a multiple
+ * of 4 up to 160, stride 1 or 2, maps up to about 28 columns wide; for any other form
+ * it fails and the caller runs the separate convolutions. tfhip_inverted_residual_pays
+ * returns 1 when the kernel takes the shape AND is expected to be faster than them.
+ *
+ * tfhip_transpose2d: y[c][r] = x[r][c] for a row-major [rows, cols] matrix (the
+ * Transpose kernel of tfjs-backend-cpu/src/kernels/Transpose.ts for rank 2, perm [1,0]). */
+int tfhip_fused_inverted_residual(const float *x, const float *pw_filter_t,
+                                  const float *pw_bias, int activation,
+                                  const float *dw_filter, const float *dw_bias,
+                                  const float *proj_filter_t, const float *proj_bias,
+                                  const float *residual, float *y, int64_t batch,
+                                  int64_t in_h, int64_t in_w, int64_t in_c,
+                                  int64_t mid_c, int64_t out_c, int64_t stride,
+                                  int64_t pad_top, int64_t pad_left, int64_t out_h,
+                                  int64_t out_w);
+int tfhip_inverted_residual_pays(int64_t batch, int64_t in_h, int64_t in_w,
+                                 int64_t in_c, int64_t mid_c, int64_t out_c,
+                                 int64_t stride, int64_t out_h, int64_t out_w);
+int tfhip_transpose2d(const float *x, float *y, int64_t rows, int64_t cols);
 
 /* ---- weight dequantisation on load -----------------------------------------
  * The quantization branch of decodeWeight, tfjs-core/src/io/io_utils.ts:196-251,

@@ -719,6 +719,70 @@ def test_pointwise_depthwise_tile_kernel(hip, orc, tuning, case):
     assert_parity(got, want)
 
 
+BLOCK_CASES = [
+    # batch, h, w, in_c, mid_c, out_c, stride, pad, activation, residual, block_rows knob
+    (2, 14, 14, 64, 384, 64, 1, "same", "relu6", True, None),       # MobileNetV2 b7-b9: two waves per pixel block
+    (2, 14, 14, 64, 384, 96, 1, "same", "relu6", False, None),      # b10: six channel blocks out
+    (2, 14, 14, 96, 576, 96, 1, "same", "relu6", True, None),       # b11, b12: six k groups, nine slices
+    (2, 14, 14, 96, 576, 160, 2, "same", "relu6", False, None),     # b13: stride 2, ten channel blocks out
+    (2, 28, 28, 32, 192, 32, 1, "same", "relu6", True, None),       # b4, b5: a pixel block per wave
+    (2, 28, 28, 32, 192, 64, 2, "same", "relu6", False, None),      # b6
+    (2, 7, 7, 160, 960, 160, 1, "same", "relu", True, None),        # ten k groups, fifteen slices; relu
+    (3, 14, 14, 64, 128, 24, 1, "same", "relu6", False, 1),         # out_c no multiple of 16; one row per workgroup
+    (2, 14, 14, 64, 128, 64, 1, "same", "relu6", True, 3),          # ragged last chunk (3, 3, 3, 3, 2)
+    (1, 9, 13, 32, 64, 16, 1, "valid", "relu6", False, None),       # no padding
+    (2, 11, 9, 32, 128, 32, 2, "same", "relu6", False, None),       # odd sizes at stride 2
+    (1, 6, 5, 64, 64, 64, 1, [[0, 0], [2, 0], [1, 2], [0, 0]], "relu6", False, None),   # explicit, lopsided padding
+    (32, 14, 14, 64, 384, 64, 1, "same", "relu6", True, None),      # the full batch
+]
+
+
+@pytest.mark.parametrize("case", BLOCK_CASES, ids=[str(i) for i in range(len(BLOCK_CASES))])
+def test_inverted_residual_block_kernel(hip, orc, tuning, case):
+    """The whole-block kernel against the oracle's three convolutions (+ Add) and against the
+    separate launches, whose instruction order it keeps (the same bits)."""
+    from tfjs_amd import capi
+    n, h, w, cin, mid, cout, stride, pad, act, with_res, knob = case
+    if knob:
+        tuning("block_rows", knob)
+    rng = np.random.default_rng(n * 19 + h * 5 + w + cin + mid + cout + stride)
+    x = rng.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    w1 = rng.normal(0, 0.4, (1, 1, cin, mid)).astype(np.float32)
+    b1 = rng.uniform(-1, 2, (mid,)).astype(np.float32)        # positive: act(bias) is far from the zero padding
+    w2 = rng.normal(0, 0.5, (3, 3, mid, 1)).astype(np.float32)
+    b2 = rng.uniform(-1, 1, (mid,)).astype(np.float32)
+    w3 = rng.normal(0, 0.1, (1, 1, mid, cout)).astype(np.float32)
+    b3 = rng.uniform(-1, 1, (cout,)).astype(np.float32)
+    e = hip.fused_conv2d(x, w1, bias=b1, activation=act)
+    d = hip.fused_depthwise_conv2d(e, w2, strides=stride, pad=pad, bias=b2, activation=act)
+    res = rng.uniform(-2, 2, d.shape[:3] + (cout,)).astype(np.float32) if with_res else None
+    got = hip.fused_inverted_residual(x, w1, w2, w3, strides=stride, pad=pad, pw_bias=b1, dw_bias=b2, proj_bias=b3,
+                                      activation=act, residual=res)
+    name = ctypes.create_string_buffer(256)
+    capi.load_library().tfhip_last_kernel(name, 256)
+    assert name.value.decode().startswith("inverted_residual_block<"), name.value
+    three = hip.fused_conv2d(d, w3, bias=b3, residual=res) if with_res else hip.fused_conv2d(d, w3, bias=b3)
+    if n <= 4:
+        want = orc.fused_conv2d(orc.fused_depthwise_conv2d(orc.fused_conv2d(x, w1, bias=b1, activation=act), w2,
+                                                           strides=stride, pad=pad, bias=b2, activation=act), w3, bias=b3)
+        if with_res:
+            want = orc.add(want, res)
+        assert_parity(got, want)
+    assert_parity(got, three, 1e-5)
+    # no biases at all
+    got = hip.fused_inverted_residual(x[:1], w1, w2, w3, strides=stride, pad=pad, activation=act)
+    want = orc.fused_conv2d(orc.fused_depthwise_conv2d(orc.fused_conv2d(x[:1], w1, activation=act), w2, strides=stride,
+                                                       pad=pad, activation=act), w3)
+    assert_parity(got, want)
+
+
+def test_transpose2d(hip):
+    rng = np.random.default_rng(3)
+    for shape in [(1, 1), (5, 3), (32, 32), (33, 65), (64, 384), (960, 160), (1, 100), (100, 1)]:
+        x = rng.uniform(-1, 1, shape).astype(np.float32)
+        np.testing.assert_array_equal(hip.transpose2d(x), x.T)
+
+
 STEM_DW_CASES = [
     # x shape, filter shape, conv stride, conv pad, depthwise stride, depthwise pad, activation
     ((3, 64, 64, 3), (3, 3, 3, 32), 2, "same", 1, "same", "relu6"),        # MobileNetV2's stem and first depthwise stage

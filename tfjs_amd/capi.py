@@ -61,6 +61,10 @@ SIGNATURES = {
     "tfhip_conv2d_depthwise_pays": [c_i64] * 10,
     "tfhip_fused_depthwise_conv2d": [c_f32p, c_f32p, c_f32p] + [c_i64] * 15 + [c_f32p, c_i64p, ctypes.c_int,
                                                                                 c_f32p, c_i64p, ctypes.c_double],
+    "tfhip_fused_inverted_residual": [c_f32p, c_f32p, c_f32p, ctypes.c_int, c_f32p, c_f32p, c_f32p, c_f32p, c_f32p, c_f32p] +
+                                     [c_i64] * 11,
+    "tfhip_inverted_residual_pays": [c_i64] * 9,
+    "tfhip_transpose2d": [c_f32p, c_f32p, c_i64, c_i64],
     "tfhip_dequant_affine": [ctypes.c_void_p, ctypes.c_int, c_i64, ctypes.c_double, ctypes.c_double,
                              ctypes.c_void_p, ctypes.c_int],
     "tfhip_dequant_f16": [ctypes.c_void_p, c_i64, ctypes.c_void_p],

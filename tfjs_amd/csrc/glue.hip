@@ -128,7 +128,37 @@ int grid_for(long long items) {
 
 using namespace tfhip;
 
+// y[c][r] = x[r][c] through a 32 x 33 LDS tile: reads and writes both run along rows.
+__global__ __launch_bounds__(256) void transpose2d(const float *__restrict__ x, float *__restrict__ y, int rows, int cols) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int r0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
+  for (int i = ty; i < 32; i += 8) {
+    const int r = r0 + i, c = c0 + tx;
+    if (r < rows && c < cols) tile[i][tx] = x[(long long)r * cols + c];
+  }
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8) {
+    const int c = c0 + i, r = r0 + tx;
+    if (r < rows && c < cols) y[(long long)c * rows + r] = tile[tx][i];
+  }
+}
+
 extern "C" {
+
+int tfhip_transpose2d(const float *x, float *y, int64_t rows, int64_t cols) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_ARG(rows >= 0 && cols >= 0 && rows < 0x7fffffff && cols < 0x7fffffff, "tfhip_transpose2d: bad dimensions");
+  if (rows * cols == 0) return kOk;
+  TFHIP_CHECK_ARG((rows + 31) / 32 <= 65535, "tfhip_transpose2d: more than 2 097 120 rows");
+  TFHIP_CHECK_RANGE(x, rows * cols, 4, "x");
+  TFHIP_CHECK_RANGE(y, rows * cols, 4, "y");
+  TFHIP_CHECK_ARG(x != y, "tfhip_transpose2d: x and y are the same buffer");
+  note_kernel("transpose2d");
+  const dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32));
+  TFHIP_LAUNCH((transpose2d<<<grid, 256, 0, stream()>>>(x, y, (int)rows, (int)cols)));
+  return kOk;
+}
 
 int tfhip_add(const float *a, const int64_t *a_strides, const float *b, const int64_t *b_strides, float *out,
               const int64_t *out_shape, int rank) {

@@ -219,6 +219,55 @@ def fused_pointwise_depthwise(x, pw_filter, dw_filter, strides=1, pad="same", pw
             buf.free()
 
 
+def transpose2d(x):
+    """y[c][r] = x[r][c] of a rank-2 array, on the device."""
+    init()
+    x = _f32(x)
+    rows, cols = x.shape
+    dx, dy = DeviceBuffer.from_numpy(x), DeviceBuffer(max(1, x.size) * 4)
+    try:
+        check(load_library().tfhip_transpose2d(dx.ptr, dy.ptr, rows, cols))
+        return dy.download(np.float32, x.size).reshape(cols, rows)
+    finally:
+        dx.free()
+        dy.free()
+
+
+def fused_inverted_residual(x, pw_filter, dw_filter, proj_filter, strides=1, pad="same", pw_bias=None, dw_bias=None,
+                            proj_bias=None, activation="relu6", residual=None):
+    """Expansion (1x1, HWIO filter [1,1,in,mid]) + depthwise 3x3 + linear projection (1x1, [1,1,mid,out])
+    (+ residual) as one launch; the two 1x1 filters are transposed on the device first, as a caller
+    does once per model. Raises HipBackendError for a form the block kernel does not take."""
+    init()
+    x, w1, w2, w3 = _f32(x), _f32(pw_filter), _f32(dw_filter), _f32(proj_filter)
+    b1, b2, b3, res = _opt(pw_bias), _opt(dw_bias), _opt(proj_bias), _opt(residual)
+    cin, mid, out_c = w1.shape[2], w1.shape[3], w3.shape[3]
+    ci = compute_conv2d_info([x.shape[0], x.shape[1], x.shape[2], mid], w2.shape, strides, 1, pad, None, True,
+                             "channelsLast")
+    assert ci["strideHeight"] == ci["strideWidth"] and w2.shape[:2] == (3, 3) and w2.shape[3] == 1
+    out_shape = [x.shape[0], ci["outHeight"], ci["outWidth"], out_c]
+    total = int(np.prod(out_shape, dtype=np.int64))
+    lib = load_library()
+    bufs = []
+    try:
+        dx, dw1, dw2, dw3 = (DeviceBuffer.from_numpy(a) for a in (x, w1, w2, w3))
+        dw1t, dw3t, dy = DeviceBuffer(w1.nbytes), DeviceBuffer(w3.nbytes), DeviceBuffer(max(1, total) * 4)
+        bufs += [dx, dw1, dw2, dw3, dw1t, dw3t, dy]
+        opt = [DeviceBuffer.from_numpy(a) if a is not None else None for a in (b1, b2, b3, res)]
+        bufs += [b for b in opt if b is not None]
+        check(lib.tfhip_transpose2d(dw1.ptr, dw1t.ptr, cin, mid))
+        check(lib.tfhip_transpose2d(dw3.ptr, dw3t.ptr, mid, out_c))
+        ptr = lambda b: b.ptr if b is not None else None
+        check(lib.tfhip_fused_inverted_residual(
+            dx.ptr, dw1t.ptr, ptr(opt[0]), ACTIVATIONS[activation], dw2.ptr, ptr(opt[1]), dw3t.ptr, ptr(opt[2]),
+            ptr(opt[3]), dy.ptr, x.shape[0], x.shape[1], x.shape[2], cin, mid, out_c, ci["strideHeight"],
+            ci["padInfo"]["top"], ci["padInfo"]["left"], ci["outHeight"], ci["outWidth"]))
+        return dy.download(np.float32, total).reshape(out_shape)
+    finally:
+        for buf in bufs:
+            buf.free()
+
+
 def fused_conv2d_depthwise(x, filter, dw_filter, strides=1, pad="same", dw_strides=1, dw_pad="same", bias=None,
                            dw_bias=None, activation="relu6"):
     """Convolution over few input channels + depthwise 3x3 convolution (NHWC, the same activation

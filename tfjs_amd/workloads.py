@@ -225,7 +225,7 @@ class DeviceMobileNetV2:
     load (quantized shard uploaded once, one dequant kernel per tensor) and every
     activation stays in pooled device buffers between kernels."""
 
-    def __init__(self, model_dir, batch, fuse_residual_add=True, fuse_expand_depthwise=True):
+    def __init__(self, model_dir, batch, fuse_residual_add=True, fuse_expand_depthwise=True, fuse_blocks=True):
         from . import pyhost
         from .capi import ACTIVATIONS, DeviceBuffer, check, i64_array, load_library
         from .conv_util import compute_conv2d_info
@@ -236,10 +236,21 @@ class DeviceMobileNetV2:
         self.ops, self.shapes = mobilenet_v2_graph()
         if fuse_residual_add:
             self.ops = self._fuse_residual_adds(self.ops)
+        if fuse_blocks and fuse_residual_add and fuse_expand_depthwise:
+            self.ops = self._fuse_blocks(self.ops, self.shapes, batch, self._lib)
         if fuse_expand_depthwise:
             self.ops = self._fuse_expand_depthwise(self.ops, self.shapes, batch, self._lib)
         buf, specs = read_model(model_dir)
         self.weights = pyhost.decode_weights_to_device(buf, specs)   # name -> (DeviceBuffer, shape)
+        # the 1x1 filters of the blocks that run as one kernel, transposed once (k-contiguous rows)
+        self.transposed = {}
+        for op in self.ops:
+            if op["kind"] == "block":
+                for key in ("w", "w3"):
+                    src, shape = self.weights[op[key]]
+                    dst = DeviceBuffer(int(np.prod(shape)) * 4)
+                    check(self._lib.tfhip_transpose2d(src.ptr, dst.ptr, shape[2], shape[3]))
+                    self.transposed[op[key]] = dst
         self.input = DeviceBuffer(batch * 224 * 224 * 3 * 4)
         # static plan: shapes, conv geometry and last use of every tensor
         self.plan, shape = [], {"input": (batch, 224, 224, 3)}
@@ -268,6 +279,14 @@ class DeviceMobileNetV2:
                 geom = [c1["batchSize"], c1["inHeight"], c1["inWidth"], cin, fh, fw, mid, op["conv_stride"],
                         c1["padInfo"]["top"], c1["padInfo"]["left"], c1["outHeight"], c1["outWidth"], op["stride"],
                         c2["padInfo"]["top"], c2["padInfo"]["left"], c2["outHeight"], c2["outWidth"]]
+                self.plan.append((op, geom))
+            elif k == "block":
+                n, h, w, cin = shape[op["src"][0] if isinstance(op["src"], tuple) else op["src"]]
+                mid, cout = self.shapes[op["w"]][3], self.shapes[op["w3"]][3]
+                ci = compute_conv2d_info((n, h, w, mid), self.shapes[op["w2"]], op["stride"], 1, "same", None, True)
+                shape[op["out"]] = (n, ci["outHeight"], ci["outWidth"], cout)
+                geom = [n, h, w, cin, mid, cout, op["stride"], ci["padInfo"]["top"], ci["padInfo"]["left"],
+                        ci["outHeight"], ci["outWidth"]]
                 self.plan.append((op, geom))
             elif k == "pwdw":
                 n, h, w, _ = shape[src]
@@ -313,6 +332,52 @@ class DeviceMobileNetV2:
         return fused
 
     @staticmethod
+    def _fuse_blocks(ops, shapes, batch, lib):
+        """A 1x1 convolution, the depthwise 3x3 convolution that is its only reader and the linear 1x1
+        convolution (with or without the Add of a skip connection) that is that one's only reader
+        become one op where the whole-block kernel takes the shape and is expected to pay (what the
+        graph model does at load)."""
+        readers, size = {}, {"input": 224}
+        for op in ops:
+            for s in (op["src"] if isinstance(op["src"], tuple) else (op["src"],)):
+                readers[s] = readers.get(s, 0) + 1
+        fused, skip = [], set()
+        for i, op in enumerate(ops):
+            src = op["src"][0] if isinstance(op["src"], tuple) else op["src"]
+            if op["kind"] in ("conv", "dw"):
+                size[op["out"]] = (size[src] + op["stride"] - 1) // op["stride"]
+            elif op["kind"] == "add":
+                size[op["out"]] = size[src]
+            if i in skip:
+                continue
+            dw = ops[i + 1] if i + 1 < len(ops) else None
+            pr = ops[i + 2] if i + 2 < len(ops) else None
+            if (op["kind"] == "conv" and "residual" not in op and dw is not None and pr is not None
+                    and dw["kind"] == "dw" and dw["src"] == op["out"] and readers.get(op["out"]) == 1
+                    and pr["kind"] == "conv" and readers.get(dw["out"]) == 1 and pr["act"] == "linear"
+                    and (pr["src"][0] if isinstance(pr["src"], tuple) else pr["src"]) == dw["out"]
+                    and shapes[op["w"]][:2] == (1, 1) and shapes[pr["w"]][:2] == (1, 1) and op["stride"] == 1
+                    and pr["stride"] == 1 and op["act"] == dw["act"]):
+                cin, mid = shapes[op["w"]][2:]
+                cout = shapes[pr["w"]][3]
+                in_size = size[src]
+                out_size = (in_size + dw["stride"] - 1) // dw["stride"]
+                if lib.tfhip_inverted_residual_pays(batch, in_size, in_size, cin, mid, cout, dw["stride"], out_size,
+                                                    out_size) == 1:
+                    block = dict(kind="block", src=src, out=pr["out"], w=op["w"], b=op["b"], act=op["act"], w2=dw["w"],
+                                 b2=dw["b"], w3=pr["w"], b3=pr["b"], stride=dw["stride"])
+                    if "residual" in pr:
+                        block["residual"] = pr["residual"]
+                        block["src"] = (src, pr["residual"]) if pr["residual"] != src else (src,)
+                    fused.append(block)
+                    size[dw["out"]] = out_size
+                    size[pr["out"]] = out_size
+                    skip.update((i + 1, i + 2))
+                    continue
+            fused.append(op)
+        return fused
+
+    @staticmethod
     def _fuse_expand_depthwise(ops, shapes, batch, lib):
         """A 1x1 convolution whose only reader is the depthwise 3x3 convolution that
         follows it becomes one op, where the fused kernel takes the shape (what the
@@ -324,7 +389,7 @@ class DeviceMobileNetV2:
         fused, skip = [], set()
         for i, op in enumerate(ops):
             src = op["src"][0] if isinstance(op["src"], tuple) else op["src"]
-            if op["kind"] in ("conv", "dw"):
+            if op["kind"] in ("conv", "dw", "block"):
                 size[op["out"]] = (size[src] + op["stride"] - 1) // op["stride"]
             elif op["kind"] == "add":
                 size[op["out"]] = size[src]
@@ -362,8 +427,16 @@ class DeviceMobileNetV2:
         n_out = int(np.prod(self.shape[op["out"]]))
         srcs = op["src"] if isinstance(op["src"], tuple) else (op["src"],)
         n_in = sum(int(np.prod(self.shape[s])) for s in srcs)
-        n_w = sum(int(np.prod(self.shapes[op[key]])) for key in ("w", "b", "w2", "b2") if key in op)
-        if k == "cvdw":
+        n_w = sum(int(np.prod(self.shapes[op[key]])) for key in ("w", "b", "w2", "b2", "w3", "b3") if key in op)
+        if k == "block":
+            geom = self.plan[i][1]
+            cin, mid, cout = geom[3], geom[4], geom[5]
+            n_mid = geom[0] * geom[1] * geom[2] * mid
+            flops = 2 * n_mid * cin + 2 * 9 * geom[0] * geom[9] * geom[10] * mid + 2 * n_out * mid
+            n_in = int(np.prod(self.shape[op["src"][0] if isinstance(op["src"], tuple) else op["src"]]))
+            if "residual" in op:
+                n_in += n_out
+        elif k == "cvdw":
             fh, fw, cin, mid = self.shapes[op["w"]]
             geom = self.plan[i][1]
             n_mid = geom[0] * geom[10] * geom[11] * mid
@@ -402,6 +475,12 @@ class DeviceMobileNetV2:
                 check(lib.tfhip_fused_conv2d(t[op["src"]].ptr, self.weights[op["w"]][0].ptr, out.ptr, *geom, 0,
                                              self.weights[op["b"]][0].ptr, self.strides_c, self._ACT[op["act"]],
                                              None, self.zero4, 0.2))
+            elif k == "block":
+                x_name = op["src"][0] if isinstance(op["src"], tuple) else op["src"]
+                check(lib.tfhip_fused_inverted_residual(
+                    t[x_name].ptr, self.transposed[op["w"]].ptr, self.weights[op["b"]][0].ptr, self._ACT[op["act"]],
+                    self.weights[op["w2"]][0].ptr, self.weights[op["b2"]][0].ptr, self.transposed[op["w3"]].ptr,
+                    self.weights[op["b3"]][0].ptr, t[op["residual"]].ptr if "residual" in op else None, out.ptr, *geom))
             elif k == "cvdw":
                 check(lib.tfhip_fused_conv2d_depthwise(
                     t[op["src"]].ptr, self.weights[op["w"]][0].ptr, self.weights[op["b"]][0].ptr, self._ACT[op["act"]],
@@ -442,6 +521,9 @@ class DeviceMobileNetV2:
 
     def close(self):
         self.input.free()
+        for buf in self.transposed.values():
+            buf.free()
+        self.transposed = {}
         for buf, _ in self.weights.values():
             buf.free()
         self.weights = {}
