@@ -350,6 +350,30 @@ int tfhip_add(const float *a, const int64_t *a_strides, const float *b,
               int rank);
 int tfhip_mean_hw(const float *x, float *y, int64_t batch, int64_t h, int64_t w,
                   int64_t c);
+/* The other element-wise and pooling kernels a converted MobileNetV2 graph holds
+ * between its fused nodes (tfjs-converter's executors arithmetic_executor.ts:30-70,
+ * basic_math_executor.ts:150-160, convolution_executor.ts:219-232,
+ * transformation_executor.ts:28-36):
+ * tfhip_binary: op 0 Add, 1 Sub (tfjs-backend-cpu/src/kernels/Sub.ts), 2 Multiply
+ *   (Multiply.ts), operands addressed as in tfhip_add.
+ * tfhip_unary: the stand-alone activation kernels Relu.ts, Relu6.ts, LeakyRelu.ts,
+ *   Sigmoid.ts, Elu.ts (activation codes as above; prelu and linear are not unary).
+ * tfhip_avg_pool: AvgPool, NHWC (AvgPool.ts:25-58 over utils/pool_utils.ts:20-87):
+ *   y = fround(sum of the window's elements inside the image, in a double / their
+ *   count). The caller passes what computePool2DInfo (conv_util.ts:119-140) gave.
+ * tfhip_cast: Cast.ts:28-46 between float32 (dtype 0), int32 (1) and bool (2, one
+ *   byte per element): to int32 as Int32Array.from (truncate, wrap modulo 2^32, NaN
+ *   and infinities 0), to bool as x != 0. */
+int tfhip_binary(int op, const float *a, const int64_t *a_strides, const float *b,
+                 const int64_t *b_strides, float *out, const int64_t *out_shape,
+                 int rank);
+int tfhip_unary(int activation, const float *x, float *y, int64_t n,
+                double leakyrelu_alpha);
+int tfhip_avg_pool(const float *x, float *y, int64_t batch, int64_t in_h,
+                   int64_t in_w, int64_t c, int64_t f_h, int64_t f_w,
+                   int64_t stride_h, int64_t stride_w, int64_t pad_top,
+                   int64_t pad_left, int64_t out_h, int64_t out_w);
+int tfhip_cast(const void *x, int from_dtype, void *y, int to_dtype, int64_t n);
 
 #ifdef __cplusplus
 }

@@ -150,6 +150,9 @@ static int broadcast_dims(const int64_t *in, int inRank, const int64_t *out,
 
 static inline float binary_apply(int op, float x, float y) {
   if (op == 0) return (float)((double)x + (double)y);
+  /* Sub.ts: (a, b) => a - b; Multiply.ts: (a, b) => a * b */
+  if (op == 2) return (float)((double)x - (double)y);
+  if (op == 3) return (float)((double)x * (double)y);
   /* prelu: xValue < 0 ? aValue * xValue : xValue */
   return x < 0 ? (float)((double)y * (double)x) : x;
 }
@@ -677,4 +680,76 @@ void orc_mean_hw(const float *x, float *y, int64_t batch, int64_t H, int64_t W,
       y[b * C + c] = (float)sum;
     }
   }
+}
+
+/* AvgPool, NHWC: tfjs-backend-cpu/src/kernels/AvgPool.ts:25-58 over
+ * utils/pool_utils.ts:20-87 with poolType 'avg' and dilation 1: the window's
+ * elements inside the image are summed in a double, row by row, and divided by
+ * their count; the store rounds to float32. */
+void orc_avg_pool(const float *xValues, float *outputVals, int64_t batchSize,
+                  int64_t inHeight, int64_t inWidth, int64_t inChannels,
+                  int64_t effectiveFilterHeight, int64_t effectiveFilterWidth,
+                  int64_t strideHeight, int64_t strideWidth, int64_t padTop,
+                  int64_t padLeft, int64_t outHeight, int64_t outWidth) {
+  const int64_t s0 = inHeight * inWidth * inChannels, s1 = inWidth * inChannels,
+                s2 = inChannels;
+  const int64_t outputBatchStrides = outHeight * outWidth * inChannels;
+  const int64_t outputRowStrides = outWidth * inChannels;
+  const int64_t outputColStrides = inChannels;
+#pragma omp parallel for collapse(2)
+  for (int64_t b = 0; b < batchSize; ++b) {
+    for (int64_t d = 0; d < inChannels; ++d) {
+      const int64_t outputBatchOffset = b * outputBatchStrides;
+      const int64_t inputBatchOffset = b * s0;
+      for (int64_t yR = 0; yR < outHeight; ++yR) {
+        const int64_t xRCorner = yR * strideHeight - padTop;
+        const int64_t xRMin = xRCorner > 0 ? xRCorner : 0;
+        const int64_t xRMax = inHeight < effectiveFilterHeight + xRCorner
+                                  ? inHeight
+                                  : effectiveFilterHeight + xRCorner;
+        const int64_t outputRowOffset = outputBatchOffset + yR * outputRowStrides;
+        for (int64_t yC = 0; yC < outWidth; ++yC) {
+          const int64_t xCCorner = yC * strideWidth - padLeft;
+          const int64_t xCMin = xCCorner > 0 ? xCCorner : 0;
+          const int64_t xCMax = inWidth < effectiveFilterWidth + xCCorner
+                                    ? inWidth
+                                    : effectiveFilterWidth + xCCorner;
+          double avgValue = 0;
+          int64_t count = 0;
+          for (int64_t xR = xRMin; xR < xRMax; xR += 1) {
+            const int64_t xROffset = inputBatchOffset + xR * s1;
+            for (int64_t xC = xCMin; xC < xCMax; xC += 1) {
+              const int64_t xCOffset = xROffset + xC * s2;
+              avgValue += (double)xValues[xCOffset + d];
+              count++;
+            }
+          }
+          const int64_t outputOffset = outputRowOffset + yC * outputColStrides + d;
+          outputVals[outputOffset] = (float)(avgValue / (double)count);
+        }
+      }
+    }
+  }
+}
+
+/* Cast: tfjs-backend-cpu/src/kernels/Cast.ts:28-46.
+ *   to int32: Int32Array.from(values) stores ECMAScript ToInt32(v) (js_to_int32
+ *     above): NaN and the infinities become 0; any other value is truncated toward
+ *     zero and taken modulo 2^32 into [-2^31, 2^31);
+ *   to bool: (a !== b) ? 1 : 0 against zero (NaN !== 0 is true);
+ *   to float32 from int32 / bool (no encoding loss path): Float32Array store. */
+void orc_cast_f32_to_i32(const float *x, int32_t *y, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) y[i] = js_to_int32((double)x[i]);
+}
+
+void orc_cast_f32_to_bool(const float *x, uint8_t *y, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) y[i] = (x[i] != 0.0f) ? 1 : 0;
+}
+
+void orc_cast_i32_to_bool(const int32_t *x, uint8_t *y, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) y[i] = (x[i] != 0) ? 1 : 0;
+}
+
+void orc_cast_i32_to_f32(const int32_t *x, float *y, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) y[i] = (float)(double)x[i];
 }

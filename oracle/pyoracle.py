@@ -266,6 +266,70 @@ def add(a, b):
     return out
 
 
+def _binary(op, a, b):
+    a, b = _f32(a), _f32(b)
+    shape = broadcast_shape(list(a.shape), list(b.shape))
+    out = np.empty(shape, dtype=np.float32)
+    out_shape = (ctypes.c_int64 * 8)()
+    rc = lib().orc_binary_broadcast(op, _p(a), _shape_arr(a.shape), a.ndim, _p(b),
+                                    _shape_arr(b.shape), b.ndim, _p(out), out_shape)
+    assert rc == len(shape)
+    return out
+
+
+def sub(a, b):
+    """Broadcasting Sub, tfjs-backend-cpu/src/kernels/Sub.ts."""
+    return _binary(2, a, b)
+
+
+def mul(a, b):
+    """Broadcasting Multiply, tfjs-backend-cpu/src/kernels/Multiply.ts."""
+    return _binary(3, a, b)
+
+
+def avg_pool(x, filter_size, strides, pad, dim_rounding_mode=None):
+    """AvgPool on an NHWC tensor (tfjs-backend-cpu/src/kernels/AvgPool.ts:25-58):
+    computePool2DInfo (conv_util.ts:119-140) is computeConv2DInfo with a filter of
+    [fh, fw, C, C]."""
+    x = _f32(x)
+    fh, fw = (filter_size, filter_size) if isinstance(filter_size, int) else filter_size
+    info = conv2d_info(x.shape, (fh, fw, x.shape[3], x.shape[3]), strides, 1, pad, dim_rounding_mode)
+    n, oh, ow, c = info["outShape"]
+    y = np.empty((n, oh, ow, c), dtype=np.float32)
+    sh, sw = (strides, strides) if isinstance(strides, int) else strides
+    lib().orc_avg_pool(_p(x), _p(y), _i64(n), _i64(x.shape[1]), _i64(x.shape[2]), _i64(c), _i64(fh), _i64(fw),
+                       _i64(sh), _i64(sw), _i64(info["padInfo"]["top"]), _i64(info["padInfo"]["left"]),
+                       _i64(oh), _i64(ow))
+    return y
+
+
+def cast(x, dtype):
+    """Cast between float32, int32 and bool (tfjs-backend-cpu/src/kernels/Cast.ts:28-88)."""
+    x = np.ascontiguousarray(x)
+    src = {"float32": "float32", "int32": "int32", "bool": "bool", "uint8": "bool"}[x.dtype.name]
+    n = _i64(x.size)
+    if dtype == src:
+        return x.copy()
+    if dtype == "int32":
+        if src == "bool":
+            return x.astype(np.int32)
+        y = np.empty(x.shape, dtype=np.int32)
+        lib().orc_cast_f32_to_i32(_p(x), y.ctypes.data_as(ctypes.c_void_p), n)
+        return y
+    if dtype == "bool":
+        y = np.empty(x.shape, dtype=np.uint8)
+        fn = lib().orc_cast_f32_to_bool if src == "float32" else lib().orc_cast_i32_to_bool
+        fn(x.ctypes.data_as(ctypes.c_void_p), y.ctypes.data_as(ctypes.c_void_p), n)
+        return y.astype(bool)
+    if dtype == "float32":
+        if src == "bool":
+            return x.astype(np.float32)
+        y = np.empty(x.shape, dtype=np.float32)
+        lib().orc_cast_i32_to_f32(x.ctypes.data_as(ctypes.c_void_p), _p(y), n)
+        return y
+    raise ValueError("Error in Cast: failed to cast %s to %s" % (src, dtype))
+
+
 def mean_hw(x):
     """Mean over axes [1, 2] of an NHWC tensor (global average pool)."""
     x = _f32(x)

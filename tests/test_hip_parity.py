@@ -151,6 +151,67 @@ def test_config5_bert_matmuls(hip, orc, name):
     assert_parity(hip.fused_matmul(**c), orc.fused_matmul(**c))
 
 
+# ------------------------------------ element-wise, pooling, cast and mean kernels
+
+from test_oracle_golden import _glue_cases, check_glue_case, run_glue_case  # noqa: E402
+
+
+@pytest.mark.parametrize("c", _glue_cases(), ids=lambda c: "%s@%s" % (c["op"], c["source"].split(":")[-1].split(" ")[0]))
+def test_glue_ops_golden(hip, orc, c):
+    out = run_glue_case(hip, c)
+    check_glue_case(out, c)
+    want = run_glue_case(orc, c)
+    if c["op"] == "cast":
+        np.testing.assert_array_equal(out, want)
+    else:
+        assert_parity(out, want, 1e-6)
+
+
+@pytest.mark.parametrize("op", ["sub", "mul"])
+@pytest.mark.parametrize("sa,sb", [((3, 5, 8), (3, 5, 8)), ((2, 1, 7), (4, 1)), ((6,), ()), ((1, 9, 1, 3), (5, 1, 4, 1)),
+                                   ((32, 7, 7, 16), (16,)), ((2, 3, 1, 2, 1, 2), (3, 1, 2, 1))])
+def test_binary_ops_bit_exact(hip, orc, op, sa, sb):
+    rng = np.random.default_rng(len(sa) * 7 + len(sb))
+    a = rng.uniform(-3, 3, sa).astype(np.float32)
+    b = rng.uniform(-3, 3, sb).astype(np.float32)
+    a.flat[0] = np.nan
+    got, want = getattr(hip, op)(a, b), getattr(orc, op)(a, b)
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))    # one IEEE operation each
+
+
+@pytest.mark.parametrize("act", ["relu", "relu6", "leakyrelu", "sigmoid", "elu"])
+def test_standalone_activations(hip, orc, act):
+    rng = np.random.default_rng(9)
+    x = rng.uniform(-8, 8, (3, 1001)).astype(np.float32)
+    x.flat[:4] = [np.nan, -0.0, 0.0, 6.0]
+    got, want = hip.activation(x, act, 0.3), orc.activation(x, act, 0.3)
+    assert_parity(got, want, 1e-6)
+    if act in ("relu", "relu6"):
+        np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("xs,f,s,pad", [((2, 7, 7, 1280), 7, 1, "valid"), ((3, 9, 8, 5), (3, 2), (2, 1), "same"),
+                                       ((1, 14, 14, 32), 2, 2, "valid"), ((2, 5, 5, 4), 3, 1, [[0, 0], [2, 1], [0, 2], [0, 0]]),
+                                       ((2, 6, 6, 3), 1, 1, 0)])
+def test_avg_pool_shapes(hip, orc, xs, f, s, pad):
+    rng = np.random.default_rng(sum(xs))
+    x = rng.uniform(-2, 2, xs).astype(np.float32)
+    got, want = hip.avg_pool(x, f, s, pad), orc.avg_pool(x, f, s, pad)
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_cast_every_pair_bit_exact(hip, orc):
+    rng = np.random.default_rng(2)
+    f = rng.uniform(-5, 5, 4099).astype(np.float32)
+    f[:12] = [0.0, -0.0, 0.5, -0.5, np.nan, np.inf, -np.inf, 2147483648.0, -2147483904.0, 4294967296.0, 1e20, -3.99]
+    i = rng.integers(-2 ** 31, 2 ** 31 - 1, 4099, dtype=np.int64).astype(np.int32)
+    i[:3] = [0, 16777217, -16777217]              # not representable as float32: rounds to even
+    b = rng.integers(0, 2, 4099).astype(bool)
+    for src in (f, i, b):
+        for dtype in ("float32", "int32", "bool"):
+            np.testing.assert_array_equal(hip.cast(src, dtype), orc.cast(src, dtype), err_msg="%s -> %s" % (src.dtype, dtype))
+
+
 # ------------------------------------------------------------------ shape sweeps
 
 @pytest.mark.parametrize("m,n,k", [(1, 1, 1), (5, 3, 7), (47, 49, 48), (64, 64, 16), (65, 63, 17), (130, 100, 36),

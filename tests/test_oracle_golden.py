@@ -428,3 +428,100 @@ def test_device_model_fuses_skip_connections_and_expansion_pairs():
             assert s in produced, "%s is read before it is produced" % s
         produced.add(op["out"])
     assert "logits" in produced
+
+
+# ------------------------------------------------ element-wise, pooling, cast, mean (reference specs)
+
+def _glue_cases():
+    import json
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "glue_ops.json")
+    return json.load(open(path))["cases"]
+
+
+def _num(values):
+    return np.array([np.nan if v == "NaN" else v for v in values], dtype=np.float64)
+
+
+def run_glue_case(mod, c):
+    """Runs one glue_ops.json case with the kernels of `mod` (the oracle or the HIP host)."""
+    op = c["op"]
+    if op in ("relu", "relu6"):
+        return mod.activation(_num(c["x"]).astype(np.float32).reshape(c["shape"]), op)
+    if op in ("mul", "sub"):
+        a = _num(c["a"]).astype(np.float32).reshape(c["a_shape"])
+        b = _num(c["b"]).astype(np.float32).reshape(c["b_shape"])
+        return getattr(mod, op)(a, b)
+    if op == "avg_pool":
+        return mod.avg_pool(_num(c["x"]).astype(np.float32).reshape(c["x_shape"]), c["filter"], c["strides"], c["pad"])
+    if op == "cast":
+        np_dtype = {"float32": np.float32, "int32": np.int32, "bool": bool}[c["x_dtype"]]
+        return mod.cast(np.array(c["x"]).astype(np_dtype), c["dtype"])
+    if op == "mean_hw":
+        return mod.mean_hw(_num(c["x"]).astype(np.float32).reshape(c["x_shape"]))
+    raise AssertionError(op)
+
+
+def check_glue_case(out, c):
+    want = _num(c["expected"])
+    if "shape" in c:
+        assert list(out.shape) == c["shape"]
+    got = np.asarray(out, dtype=np.float64).reshape(-1)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    if c["op"] == "cast":
+        np.testing.assert_array_equal(got, want)             # expectArraysEqual in the reference
+    else:
+        np.testing.assert_allclose(np.nan_to_num(got), np.nan_to_num(want), rtol=0, atol=1e-3)
+
+
+@pytest.mark.parametrize("c", _glue_cases(), ids=lambda c: "%s@%s" % (c["op"], c["source"].split(":")[-1].split(" ")[0]))
+def test_oracle_glue_ops_against_reference_specs(c):
+    check_glue_case(run_glue_case(orc, c), c)
+
+
+def test_oracle_mean_hw_against_the_true_mean_and_its_rounding_rule():
+    # against the exact mean (rational arithmetic) within float32 rounding of 49 terms, and the rule that
+    # distinguishes the reference from a plain sum / n: every term is divided first, in float32
+    from fractions import Fraction
+    rng = np.random.default_rng(12)
+    x = rng.uniform(-3, 3, (2, 7, 7, 5)).astype(np.float32)
+    got = orc.mean_hw(x)
+    for n in range(2):
+        for c in range(5):
+            exact = sum(Fraction(float(v)) for v in x[n, :, :, c].reshape(-1)) / 49
+            assert abs(Fraction(float(got[n, c])) - exact) <= Fraction(1, 10 ** 6)
+    terms = (x.astype(np.float64) / np.float64(np.float32(49))).astype(np.float32)    # Mean.ts:41-48
+    np.testing.assert_array_equal(got, terms.astype(np.float64).sum(axis=(1, 2)).astype(np.float32))
+    # a case where dividing first differs from dividing last
+    y = np.full((1, 3, 1, 1), np.float32(1e-45))       # the smallest subnormal: a third of it rounds to zero
+    assert orc.mean_hw(y)[0, 0] == 0.0
+
+
+def test_oracle_cast_to_int32_is_ecmascript_toint32():
+    x = np.array([0.5, -0.5, 2147483648.0, -2147483649.0, 4294967296.0 + 7, np.nan, np.inf, -np.inf, 1e20, -7.9],
+                 dtype=np.float32)
+    want = []
+    for v in x.astype(np.float64):
+        if not np.isfinite(v):
+            want.append(0)
+            continue
+        t = int(v)                          # truncation toward zero, exact for a float
+        t %= 1 << 32
+        want.append(t - (1 << 32) if t >= 1 << 31 else t)
+    np.testing.assert_array_equal(orc.cast(x, "int32"), np.array(want, dtype=np.int64).astype(np.int32))
+    np.testing.assert_array_equal(orc.cast(x, "bool"), np.array([v != 0 for v in x]))
+
+
+def test_oracle_avg_pool_against_brute_force():
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-1, 1, (2, 7, 6, 3)).astype(np.float32)
+    got = orc.avg_pool(x, (3, 2), (2, 1), "same")
+    info = orc.conv2d_info(x.shape, (3, 2, 3, 3), (2, 1), 1, "same")
+    top, left = info["padInfo"]["top"], info["padInfo"]["left"]
+    assert list(got.shape) == info["outShape"]
+    for n in range(2):
+        for r in range(got.shape[1]):
+            for c in range(got.shape[2]):
+                rows = [i for i in range(r * 2 - top, r * 2 - top + 3) if 0 <= i < 7]
+                cols = [j for j in range(c - left, c - left + 2) if 0 <= j < 6]
+                window = x[n][np.ix_(rows, cols)].astype(np.float64)
+                np.testing.assert_allclose(got[n, r, c], window.mean(axis=(0, 1)), rtol=1e-6)

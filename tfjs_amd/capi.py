@@ -70,6 +70,10 @@ SIGNATURES = {
     "tfhip_dequant_f16": [ctypes.c_void_p, c_i64, ctypes.c_void_p],
     "tfhip_add": [c_f32p, c_i64p, c_f32p, c_i64p, c_f32p, c_i64p, ctypes.c_int],
     "tfhip_mean_hw": [c_f32p, c_f32p, c_i64, c_i64, c_i64, c_i64],
+    "tfhip_binary": [ctypes.c_int, c_f32p, c_i64p, c_f32p, c_i64p, c_f32p, c_i64p, ctypes.c_int],
+    "tfhip_unary": [ctypes.c_int, c_f32p, c_f32p, c_i64, ctypes.c_double],
+    "tfhip_avg_pool": [c_f32p, c_f32p] + [c_i64] * 12,
+    "tfhip_cast": [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, c_i64],
 }
 
 

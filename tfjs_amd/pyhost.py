@@ -311,6 +311,69 @@ def add(a, b):
         return do.download(np.float32, total).reshape(shape)
 
 
+def _binary(op, a, b):
+    init()
+    a, b = _f32(a), _f32(b)
+    shape = broadcast_shape(list(a.shape), list(b.shape))
+    total = int(np.prod(shape, dtype=np.int64))
+    with DeviceBuffer.from_numpy(a) as da, DeviceBuffer.from_numpy(b) as db, DeviceBuffer(max(1, total) * 4) as do:
+        check(load_library().tfhip_binary(op, da.ptr, i64_array(broadcast_strides(list(a.shape), shape)), db.ptr,
+                                          i64_array(broadcast_strides(list(b.shape), shape)), do.ptr,
+                                          i64_array(shape), len(shape)))
+        return do.download(np.float32, total).reshape(shape)
+
+
+def sub(a, b):
+    """Broadcasting Sub (tfjs-backend-cpu/src/kernels/Sub.ts)."""
+    return _binary(1, a, b)
+
+
+def mul(a, b):
+    """Broadcasting Multiply (tfjs-backend-cpu/src/kernels/Multiply.ts)."""
+    return _binary(2, a, b)
+
+
+def activation(x, act, leakyrelu_alpha=0.2):
+    """A stand-alone activation kernel: relu, relu6, leakyrelu, sigmoid or elu."""
+    init()
+    x = _f32(x)
+    with DeviceBuffer.from_numpy(x) as dx, DeviceBuffer(max(1, x.size) * 4) as dy:
+        check(load_library().tfhip_unary(ACTIVATIONS[act], dx.ptr, dy.ptr, x.size, float(leakyrelu_alpha)))
+        return dy.download(np.float32, x.size).reshape(x.shape)
+
+
+def avg_pool(x, filter_size, strides, pad, dim_rounding_mode=None):
+    """AvgPool on an NHWC tensor (tfjs-backend-cpu/src/kernels/AvgPool.ts:25-58): the geometry is
+    computePool2DInfo's, i.e. computeConv2DInfo with a [fh, fw, C, C] filter."""
+    init()
+    x = _f32(x)
+    fh, fw = (filter_size, filter_size) if isinstance(filter_size, int) else filter_size
+    ci = compute_conv2d_info(list(x.shape), [fh, fw, x.shape[3], x.shape[3]], strides, 1, pad, dim_rounding_mode,
+                             False, "channelsLast")
+    n, oh, ow, c = ci["outShape"]
+    total = n * oh * ow * c
+    with DeviceBuffer.from_numpy(x) as dx, DeviceBuffer(max(1, total) * 4) as dy:
+        check(load_library().tfhip_avg_pool(dx.ptr, dy.ptr, n, x.shape[1], x.shape[2], c, fh, fw, ci["strideHeight"],
+                                            ci["strideWidth"], ci["padInfo"]["top"], ci["padInfo"]["left"], oh, ow))
+        return dy.download(np.float32, total).reshape(n, oh, ow, c)
+
+
+_CAST_CODES = {"float32": 0, "int32": 1, "bool": 2}
+_CAST_NUMPY = {"float32": np.float32, "int32": np.int32, "bool": np.uint8}
+
+
+def cast(x, dtype):
+    """Cast between float32, int32 and bool (tfjs-backend-cpu/src/kernels/Cast.ts:28-88)."""
+    init()
+    x = np.ascontiguousarray(x)
+    src = "bool" if x.dtype in (np.bool_, np.uint8) else x.dtype.name
+    x = x.astype(_CAST_NUMPY[src])
+    with DeviceBuffer.from_numpy(x) as dx, DeviceBuffer(max(1, x.size) * 4) as dy:
+        check(load_library().tfhip_cast(dx.ptr, _CAST_CODES[src], dy.ptr, _CAST_CODES[dtype], x.size))
+        out = dy.download(_CAST_NUMPY[dtype], x.size).reshape(x.shape)
+    return out.astype(bool) if dtype == "bool" else out
+
+
 def mean_hw(x):
     init()
     x = _f32(x)
