@@ -441,6 +441,99 @@ function add({inputs, backend}) {
   return addImpl(backend, inputs.a, inputs.b);
 }
 
+const subImpl = binaryKernel((a, b) => a - b);        // Sub.ts
+const multiplyImpl = binaryKernel((a, b) => a * b);   // Multiply.ts
+
+/** AvgPool.ts:25-58 over utils/pool_utils.ts:20-87 ('avg', dilation 1). */
+function avgPool({inputs, backend, attrs}) {
+  const x = inputs.x;
+  const convInfo = shapes.backend_util.computeConv2DInfo(
+      x.shape, (() => {
+        const f = typeof attrs.filterSize === 'number' ? [attrs.filterSize, attrs.filterSize] : attrs.filterSize;
+        return [f[0], f[1], x.shape[3], x.shape[3]];
+      })(), attrs.strides, 1, attrs.pad, attrs.dimRoundingMode, false, 'channelsLast');
+  if (convInfo.filterWidth === 1 && convInfo.filterHeight === 1 &&
+      shapes.util.arraysEqual(convInfo.inShape, convInfo.outShape)) {
+    return identity({inputs: {x}, backend});
+  }
+  const xValues = vals(backend, x);
+  const strides = shapes.util.computeStrides(x.shape);
+  const outputVals = new Float32Array(shapes.util.sizeFromShape(convInfo.outShape));
+  const outputBatchStrides = convInfo.outShape[1] * convInfo.outShape[2] * convInfo.outShape[3];
+  const outputRowStrides = convInfo.outShape[2] * convInfo.outShape[3];
+  const outputColStrides = convInfo.outShape[3];
+  for (let b = 0; b < convInfo.batchSize; ++b) {
+    const outputBatchOffset = b * outputBatchStrides;
+    const inputBatchOffset = b * strides[0];
+    for (let d = 0; d < convInfo.inChannels; ++d) {
+      for (let yR = 0; yR < convInfo.outHeight; ++yR) {
+        const xRCorner = yR * convInfo.strideHeight - convInfo.padInfo.top;
+        const xRMin = Math.max(0, xRCorner);
+        const xRMax = Math.min(convInfo.inHeight, convInfo.effectiveFilterHeight + xRCorner);
+        const outputRowOffset = outputBatchOffset + yR * outputRowStrides;
+        for (let yC = 0; yC < convInfo.outWidth; ++yC) {
+          const xCCorner = yC * convInfo.strideWidth - convInfo.padInfo.left;
+          const xCMin = Math.max(0, xCCorner);
+          const xCMax = Math.min(convInfo.inWidth, convInfo.effectiveFilterWidth + xCCorner);
+          let avgValue = 0;
+          let count = 0;
+          for (let xR = xRMin; xR < xRMax; xR += 1) {
+            const xROffset = inputBatchOffset + xR * strides[1];
+            for (let xC = xCMin; xC < xCMax; xC += 1) {
+              avgValue += xValues[xROffset + xC * strides[2] + d];
+              count++;
+            }
+          }
+          outputVals[outputRowOffset + yC * outputColStrides + d] = avgValue / count;
+        }
+      }
+    }
+  }
+  return backend.makeTensorInfo(convInfo.outShape, 'float32', outputVals);
+}
+
+/** Cast.ts:28-88 for float32 / int32 / bool. */
+function cast({inputs, backend, attrs}) {
+  const x = inputs.x, dtype = attrs.dtype;
+  const lossless = dtype === 'float32' || (dtype === 'int32' && x.dtype !== 'float32') ||
+      (dtype === 'bool' && x.dtype === 'bool');
+  if (lossless) {
+    backend.incRef(x.dataId);
+    return {dataId: x.dataId, shape: x.shape, dtype};
+  }
+  const values = vals(backend, x);
+  if (dtype === 'int32') {
+    return backend.makeTensorInfo(x.shape, 'int32', Int32Array.from(values));
+  }
+  if (dtype === 'bool') {
+    const out = new Uint8Array(values.length);
+    for (let i = 0; i < values.length; ++i) {
+      out[i] = (values[i] !== 0) ? 1 : 0;
+    }
+    return backend.makeTensorInfo(x.shape, 'bool', out);
+  }
+  throw new Error(`Error in Cast: failed to cast ${x.dtype} to ${dtype}`);
+}
+
+/** Transpose.ts / Transpose_impl.ts for rank 2. */
+function transpose({inputs, backend, attrs}) {
+  const x = inputs.x, perm = attrs.perm;
+  if (perm.every((p, i) => p === i)) {
+    return identity({inputs: {x}, backend});
+  }
+  if (x.shape.length !== 2) {
+    throw new Error('oracle Transpose: only rank 2 is restated');
+  }
+  const rows = x.shape[0], cols = x.shape[1], xv = vals(backend, x);
+  const out = new Float32Array(xv.length);
+  for (let r = 0; r < rows; ++r) {
+    for (let c = 0; c < cols; ++c) {
+      out[c * rows + r] = xv[r * cols + c];
+    }
+  }
+  return backend.makeTensorInfo([cols, rows], x.dtype, out);
+}
+
 const kernelFuncs = {
   BatchMatMul: batchMatMul,
   _FusedMatMul: fusedMatMul,
@@ -449,6 +542,16 @@ const kernelFuncs = {
   DepthwiseConv2dNative: depthwiseConv2dNative,
   FusedDepthwiseConv2D: fusedDepthwiseConv2D,
   Add: add,
+  Sub: ({inputs, backend}) => subImpl(backend, inputs.a, inputs.b),
+  Multiply: ({inputs, backend}) => multiplyImpl(backend, inputs.a, inputs.b),
+  Relu: ({inputs, backend}) => reluImpl(backend, inputs.x),
+  Relu6: ({inputs, backend}) => relu6Impl(backend, inputs.x),
+  Elu: ({inputs, backend}) => eluImpl(backend, inputs.x),
+  Sigmoid: ({inputs, backend}) => sigmoidImpl(backend, inputs.x),
+  LeakyRelu: ({inputs, backend, attrs}) => unaryKernel(xi => xi < 0 ? attrs.alpha * xi : xi)(backend, inputs.x),
+  AvgPool: avgPool,
+  Cast: cast,
+  Transpose: transpose,
   Mean: mean,
   Reshape: reshape,
   Identity: identity

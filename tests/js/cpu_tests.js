@@ -36,6 +36,13 @@ golden.FILES.forEach(file => {
   });
 });
 
+h.loadGolden('glue_ops.json').cases.forEach(c => {
+  h.test(`oracle glue_ops.json :: ${c.op} @${c.source.split(':').pop()}`, () => {
+    useBackend('cpu');
+    tf.tidy(() => golden.checkGlueCase(h, golden.runGlueCase(tf, c), c));
+  });
+});
+
 h.loadGolden('conv_util.json').cases.forEach(c => {
   h.test(`standin computeConv2DInfo :: ${c.name} @${c.source.split(':').pop()}`, () => {
     const a = c.args;
@@ -641,6 +648,76 @@ h.test('hip storage: while a recorded graph is alive, released buffers go back t
   v.dispose();
   h.assertEqual(backend.pooledBuffers, 1, 'no graph alive: the free lists serve again');
   backend.releasePool();
+});
+
+// ---- converter-written models that the reference's own tests hold --------------------------------
+const refModels = require('./ref_models');
+
+h.test('reference model load_predict_data/graph_model (old and new format): the expected output of load_predict_test.ts', async () => {
+  useBackend('cpu');
+  const io = {decodeWeights: oracleDecode.decodeWeights};
+  const expected = [0.7567615509033203, -0.18349379301071167, 0.7567615509033203, -0.18349379301071167];
+  for (const json of ['model.json', 'model_new.json']) {
+    const model = hip.loadGraphModel({load: () => refModels.artifacts('load_predict_graph_model', json)}, {}, io);
+    const a = tf.tensor([1, 1, 1, 1], [2, 2]);
+    const result = await model.executeAsync({'Placeholder': a});
+    h.assertEqual(result.shape, [2, 2]);
+    h.assertClose(result.dataSync(), expected);
+    tf.dispose([a, result]);
+    model.dispose();
+  }
+});
+
+h.test('reference model rn59 graph_model (dense layer): MatMul + BiasAdd over the shipped weights', () => {
+  useBackend('cpu');
+  const art = refModels.artifacts('rn59_graph_model', 'model.json');
+  const raw = new Float32Array(art.weightData);            // bias [1], then kernel [10, 1]
+  const model = hip.loadGraphModel({load: () => art}, {}, {decodeWeights: oracleDecode.decodeWeights});
+  const xs = h.rng(4).uniform(30, -2, 2);
+  const x = tf.tensor(xs, [3, 10]);
+  const y = model.predict(x);
+  h.assertEqual(y.shape, [3, 1]);
+  const want = [0, 1, 2].map(r => {
+    let sum = 0;
+    for (let k = 0; k < 10; k++) {
+      sum += xs[r * 10 + k] * raw[1 + k];
+    }
+    return sum + raw[0];
+  });
+  h.assertClose(y.dataSync(), want, 1e-5);
+  tf.dispose([x, y]);
+  model.dispose();
+});
+
+h.test('reference model rn59 sharded_model (MobileNetV2 0.50 as the converter wrote it): every node type runs; the depthwise chains fuse without changing a bit', () => {
+  useBackend('cpu');
+  const io = {decodeWeights: oracleDecode.decodeWeights};
+  const art = refModels.shardedMobileNetArtifacts(5);
+  const ops = {};
+  art.modelTopology.node.forEach(n => ops[n.op] = (ops[n.op] || 0) + 1);
+  h.assertEqual([ops._FusedConv2D, ops.DepthwiseConv2dNative, ops.BiasAdd, ops.Relu6, ops.Add, ops.Mul, ops.Sub, ops.AvgPool, ops.Squeeze],
+                [36, 17, 17, 17, 10, 1, 1, 1, 1]);
+  const x = tf.tensor(h.rng(6).uniform(96 * 96 * 3, 0, 1), [1, 96, 96, 3]);
+  // (the Placeholder says 224x224; the graph is fully convolutional up to its 7x7 AvgPool, so a
+  // CPU-tier run uses the declared size only once, below, and a smaller map for the node-type checks)
+  const model = hip.loadGraphModel({load: () => art}, {}, io);
+  h.assertEqual(Object.keys(model.nodes).filter(n => model.nodes[n].op === 'FusedDepthwiseConv2dNative').length, 17);
+  h.assertEqual(Object.keys(model.nodes).filter(n => /^(DepthwiseConv2dNative|BiasAdd|Relu6)$/.test(model.nodes[n].op)).length, 0);
+  h.assertThrows(() => model.predict(x), /must be \[-1,224,224,3\], but was \[1,96,96,3\]/);
+  const plain = hip.loadGraphModel({load: () => art}, {fuseDepthwiseBiasActivation: false}, io);
+  h.assertEqual(Object.keys(plain.nodes).filter(n => plain.nodes[n].op === 'DepthwiseConv2dNative').length, 17);
+  const full = tf.tensor(h.rng(7).uniform(224 * 224 * 3, 0, 1), [1, 224, 224, 3]);
+  const before = tf.memory().numTensors;
+  const y = model.predict(full), z = plain.predict(full);
+  h.assertEqual(y.shape, [1, 1001]);
+  h.assertBitsEqual(y.dataSync(), z.dataSync());
+  const logits = y.dataSync();
+  h.assert(logits.every(v => Number.isFinite(v)) && Math.max.apply(null, logits) - Math.min.apply(null, logits) > 1e-3,
+           'logits are finite and not constant');
+  h.assertEqual(tf.memory().numTensors, before + 2);
+  tf.dispose([x, full, y, z]);
+  model.dispose();
+  plain.dispose();
 });
 
 h.test('graph model: unsupported nodes and malformed fused nodes throw the reference errors', () => {

@@ -66,6 +66,14 @@ module.exports = {
   dequantF16() { record('dequantF16', arguments); },
   add() { record('add', arguments); },
   meanHW() { record('meanHW', arguments); },
+  binary() { record('binary', arguments); },
+  unary() { record('unary', arguments); },
+  avgPool() { record('avgPool', arguments); },
+  cast() { record('cast', arguments); },
+  transpose2d() { record('transpose2d', arguments); },
+  fusedInvertedResidual() { record('fusedInvertedResidual', arguments); },
+  invertedResidualPays(batch) { return module.exports.blockPaysFromBatch != null && batch >= module.exports.blockPaysFromBatch; },
+  blockPaysFromBatch: null,
   fusedPointwiseDepthwise() { record('fusedPointwiseDepthwise', arguments); },
   pointwiseDepthwisePays(batch) { return module.exports.paysFromBatch != null && batch >= module.exports.paysFromBatch; },
   fusedConv2DDepthwise() { record('fusedConv2DDepthwise', arguments); },

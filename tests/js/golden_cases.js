@@ -36,7 +36,37 @@ function runCase(tf, c) {
   throw new Error(`unknown op ${c.op}`);
 }
 
+/** One case of glue_ops.json (element-wise, pooling, cast, mean specs) through the tf API. */
+function runGlueCase(tf, c) {
+  const num = v => v.map(e => e === 'NaN' ? NaN : e);
+  if (c.op === 'relu' || c.op === 'relu6') {
+    return tf[c.op](tf.tensor(num(c.x), c.shape));
+  } else if (c.op === 'mul' || c.op === 'sub') {
+    return tf[c.op](tf.tensor(num(c.a), c.a_shape), tf.tensor(num(c.b), c.b_shape));
+  } else if (c.op === 'avg_pool') {
+    return tf.avgPool(tf.tensor(num(c.x), c.x_shape), c.filter, c.strides, c.pad);
+  } else if (c.op === 'cast') {
+    return tf.cast(tf.tensor(c.x, [c.x.length], c.x_dtype), c.dtype);
+  } else if (c.op === 'mean_hw') {
+    return tf.mean(tf.tensor(num(c.x), c.x_shape), [1, 2]);
+  }
+  throw new Error(`unknown op ${c.op}`);
+}
+
+function checkGlueCase(h, out, c) {
+  if (c.shape != null) {
+    h.assertEqual(out.shape, c.shape, 'shape');
+  }
+  const want = c.expected.map(e => e === 'NaN' ? NaN : e);
+  if (c.op === 'cast') {
+    h.assertEqual(out.dtype, c.dtype);
+    h.assertEqual(Array.from(out.dataSync()), want);
+  } else {
+    h.assertClose(out.dataSync(), want);
+  }
+}
+
 const FILES = ['fused_mat_mul.json', 'mat_mul.json', 'fused_conv2d.json', 'conv2d.json', 'fused_depthwise_conv2d.json',
                'depthwise_conv2d.json'];
 
-module.exports = {runCase, FILES, toTensor};
+module.exports = {runCase, runGlueCase, checkGlueCase, FILES, toTensor};

@@ -56,6 +56,52 @@ golden.FILES.forEach(file => {
   });
 });
 
+h.loadGolden('glue_ops.json').cases.forEach(c => {
+  h.test(`hip glue_ops.json :: ${c.op} @${c.source.split(':').pop()}`, () => {
+    on('hip', () => {
+      tf.env().set('IS_TEST', true);
+      try {
+        golden.checkGlueCase(h, golden.runGlueCase(tf, c), c);
+      } finally {
+        tf.env().set('IS_TEST', false);
+      }
+    });
+  });
+});
+
+h.test('element-wise, pooling, cast and transpose kernels against the oracle on the same arrays', () => {
+  const r = h.rng(31);
+  const a = r.uniform(2 * 9 * 8 * 6, -3, 3), b = r.uniform(6, -2, 2);
+  a[0] = NaN;
+  for (const op of ['sub', 'mul']) {
+    const [got, want] = both(() => tf[op](tf.tensor(a, [2, 9, 8, 6]), tf.tensor(b, [6])));
+    h.assertBitsEqual(got, want);
+  }
+  for (const op of ['relu', 'relu6', 'elu', 'sigmoid']) {
+    const [got, want] = both(() => tf[op](tf.tensor(a, [2, 9, 8, 6])));
+    h.assertParity(got, want, 1e-6);
+  }
+  let [got, want] = both(() => tf.leakyRelu(tf.tensor(a, [2, 9, 8, 6]), 0.3));
+  h.assertParity(got, want, 1e-6);
+  a[0] = 0.5;
+  [got, want] = both(() => tf.avgPool(tf.tensor(a, [2, 9, 8, 6]), [3, 2], [2, 1], 'same'));
+  h.assertBitsEqual(got, want);
+  [got, want] = both(() => tf.avgPool(tf.tensor(a, [2, 9, 8, 6]), [9, 8], 1, 'valid'));
+  h.assertBitsEqual(got, want);
+  [got, want] = both(() => tf.transpose(tf.tensor(a, [108, 8])));
+  h.assertBitsEqual(got, want);
+  [got, want] = both(() => tf.squeeze(tf.avgPool(tf.tensor(a, [2, 9, 8, 6]), [9, 8], 1, 'valid'), [1, 2]));
+  h.assertBitsEqual(got, want);
+  const f = Float32Array.from([0, -0, 0.5, -0.5, NaN, Infinity, -Infinity, 2147483648, -2147483904, 4294967296, 1e20, -3.99]);
+  on('hip', () => {
+    const asInt = tf.cast(tf.tensor(f, [12]), 'int32');
+    h.assertEqual(Array.from(asInt.dataSync()), Array.from(Int32Array.from(f)));
+    h.assertEqual(Array.from(tf.cast(tf.tensor(f, [12]), 'bool').dataSync()), Array.from(f).map(v => v !== 0 ? 1 : 0));
+    h.assertEqual(Array.from(tf.cast(asInt, 'float32').dataSync()), Array.from(Float32Array.from(Int32Array.from(f))));
+    h.assertEqual(Array.from(tf.cast(tf.tensor([1, 0, 1], [3], 'bool'), 'int32').dataSync()), [1, 0, 1]);
+  });
+});
+
 h.test('config 1: _FusedMatMul [1,256,512] x [1,512,512] + bias, relu', () => {
   const r = h.rng(11);
   const a = r.uniform(256 * 512, -1, 1), b = r.uniform(512 * 512, -1, 1), bias = r.uniform(512, -1, 1);
@@ -350,6 +396,63 @@ h.test('backend: tensors migrate cpu <-> hip with values and refCounts; tf.time 
   h.assertEqual(tf.backend().numDataIds(), ids);
   const info = tf.backend().deviceInfo;
   h.assert(/^gfx950/.test(info.arch), `arch ${info.arch}`);
+});
+
+// ---- converter-written models that the reference's own tests hold --------------------------------
+const refModels = require('./ref_models');
+
+h.test('reference models on the hip backend: load_predict_data/graph_model (both formats) and the rn59 dense model', async () => {
+  h.assert(tf.engine().setBackend('hip') === true);
+  const expected = [0.7567615509033203, -0.18349379301071167, 0.7567615509033203, -0.18349379301071167];
+  for (const json of ['model.json', 'model_new.json']) {
+    const model = hip.loadGraphModel({load: () => refModels.artifacts('load_predict_graph_model', json)}, {},
+                                     {decodeWeights: hip.decodeWeights});
+    const a = tf.tensor([1, 1, 1, 1], [2, 2]);
+    const result = await model.executeAsync({'Placeholder': a});
+    h.assertEqual(result.shape, [2, 2]);
+    h.assertClose(result.dataSync(), expected);
+    tf.dispose([a, result]);
+    model.dispose();
+  }
+  const art = refModels.artifacts('rn59_graph_model', 'model.json');
+  const xs = h.rng(4).uniform(30, -2, 2);
+  const run = (backendName, io) => {
+    h.assert(tf.engine().setBackend(backendName) === true);
+    const model = hip.loadGraphModel({load: () => art}, {}, io);
+    const x = tf.tensor(xs, [3, 10]);
+    const y = model.predict(x);
+    const data = y.dataSync();
+    tf.dispose([x, y]);
+    model.dispose();
+    return data;
+  };
+  h.assertParity(run('hip', {decodeWeights: hip.decodeWeights}), run('cpu', {decodeWeights: oracleDecode.decodeWeights}), 1e-5);
+});
+
+h.test('reference model rn59 sharded_model (MobileNetV2 0.50 as the converter wrote it) on the hip backend against the oracle', () => {
+  const art = refModels.shardedMobileNetArtifacts(5);
+  const xs = h.rng(7).uniform(2 * 224 * 224 * 3, 0, 1);
+  const run = (backendName, io, options) => {
+    h.assert(tf.engine().setBackend(backendName) === true);
+    const model = hip.loadGraphModel({load: () => art}, options, io);
+    const x = tf.tensor(xs, [2, 224, 224, 3]);
+    const before = tf.memory().numTensors;
+    const y = model.predict(x);
+    h.assertEqual(y.shape, [2, 1001]);
+    h.assertEqual(tf.memory().numTensors, before + 1);
+    const data = y.dataSync();
+    tf.dispose([x, y]);
+    model.dispose();
+    return data;
+  };
+  const want = run('cpu', {decodeWeights: oracleDecode.decodeWeights}, {});
+  const got = run('hip', {decodeWeights: hip.decodeWeights}, {});
+  h.assertParity(got, want);
+  // the graph's own nodes, one kernel each: DepthwiseConv2dNative, BiasAdd (Add), Relu6, Mul, Sub, AvgPool, Squeeze
+  const plain = run('hip', {decodeWeights: hip.decodeWeights},
+                    {fuseDepthwiseBiasActivation: false, fuseResidualAdd: false, fusePointwiseDepthwise: false});
+  h.assertParity(plain, want);
+  h.assert(Math.max.apply(null, want) - Math.min.apply(null, want) > 1e-3, 'logits are not constant');
 });
 
 h.test('native errors surface as thrown Errors, not faults', () => {

@@ -109,7 +109,10 @@ def test_addon_loads_and_exports_every_entry_point():
       const a = require('%s/tfjs_amd/lib/tfjs_hip.node');
       const want = ['init','shutdown','deviceInfo','alloc','free','upload','download','sync','memoryInfo','eventRecord',
                     'eventElapsed','setLaunchRepeat','lastKernel','fusedMatMul','fusedConv2D','fusedDepthwiseConv2D',
-                    'dequantAffine','dequantF16','add','meanHW'];
+                    'dequantAffine','dequantF16','add','meanHW','binary','unary','avgPool','cast','transpose2d',
+                    'fusedInvertedResidual','invertedResidualPays','fusedMatMulNoAlloc','fusedPointwiseDepthwise',
+                    'pointwiseDepthwisePays','fusedConv2DDepthwise','conv2dDepthwisePays','copy','captureBegin',
+                    'captureEnd','graphLaunch','graphDestroy','setTuning'];
       const missing = want.filter(n => typeof a[n] !== 'function');
       if (missing.length) { console.log('missing', missing); process.exit(1); }
       console.log('ok', Object.keys(a).length);

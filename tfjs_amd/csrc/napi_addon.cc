@@ -420,6 +420,103 @@ napi_value Add(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+// binary(op, a, aStrides, b, bStrides, out, outShape, rank)   op: 0 add, 1 sub, 2 mul
+napi_value Binary(napi_env env, napi_callback_info info) {
+  Args a(env, info, 8, "binary");
+  const int op = a.i32(0);
+  const uint32_t rank = a.ok ? (uint32_t)a.i32(7) : 0;
+  if (rank > 6) {
+    napi_throw_range_error(env, nullptr, "tfjs_hip.binary: rank above 6");
+    return nullptr;
+  }
+  int64_t as[6] = {0}, bs[6] = {0}, shape[6] = {0};
+  a.ints(2, as, rank);
+  a.ints(4, bs, rank);
+  a.ints(6, shape, rank);
+  const float *pa = (const float *)a.ptr(1), *pb = (const float *)a.ptr(3);
+  float *out = (float *)a.ptr(5);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_binary(op, pa, as, pb, bs, out, shape, (int)rank));
+  return undefined(env);
+}
+
+// unary(activation, x, y, n, leakyreluAlpha)
+napi_value Unary(napi_env env, napi_callback_info info) {
+  Args a(env, info, 5, "unary");
+  const int act = a.i32(0);
+  const float *x = (const float *)a.ptr(1);
+  float *y = (float *)a.ptr(2);
+  const int64_t n = a.i64(3);
+  const double alpha = a.num(4);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_unary(act, x, y, n, alpha));
+  return undefined(env);
+}
+
+// avgPool(x, y, geom[12] = [batch, inH, inW, c, fH, fW, strideH, strideW, padTop, padLeft, outH, outW])
+napi_value AvgPool(napi_env env, napi_callback_info info) {
+  Args a(env, info, 3, "avgPool");
+  int64_t g[12];
+  a.ints(2, g, 12);
+  const float *x = (const float *)a.ptr(0);
+  float *y = (float *)a.ptr(1);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_avg_pool(x, y, g[0], g[1], g[2], g[3], g[4], g[5], g[6], g[7], g[8], g[9], g[10], g[11]));
+  return undefined(env);
+}
+
+// cast(x, fromDtype, y, toDtype, n)   dtypes: 0 float32, 1 int32, 2 bool
+napi_value Cast(napi_env env, napi_callback_info info) {
+  Args a(env, info, 5, "cast");
+  const void *x = a.ptr(0);
+  const int from = a.i32(1);
+  void *y = a.ptr(2);
+  const int to = a.i32(3);
+  const int64_t n = a.i64(4);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_cast(x, from, y, to, n));
+  return undefined(env);
+}
+
+// transpose2d(x, y, rows, cols)
+napi_value Transpose2D(napi_env env, napi_callback_info info) {
+  Args a(env, info, 4, "transpose2d");
+  const float *x = (const float *)a.ptr(0);
+  float *y = (float *)a.ptr(1);
+  const int64_t rows = a.i64(2), cols = a.i64(3);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_transpose2d(x, y, rows, cols));
+  return undefined(env);
+}
+
+// fusedInvertedResidual(x, pwFilterT, pwBias, activation, dwFilter, dwBias, projFilterT, projBias, residual, y,
+//                       geom[11] = [batch, inH, inW, inC, midC, outC, stride, padTop, padLeft, outH, outW])
+napi_value FusedInvertedResidual(napi_env env, napi_callback_info info) {
+  Args a(env, info, 11, "fusedInvertedResidual");
+  int64_t g[11];
+  a.ints(10, g, 11);
+  const float *x = (const float *)a.ptr(0), *w1 = (const float *)a.ptr(1), *b1 = (const float *)a.ptr(2);
+  const int act = a.i32(3);
+  const float *w2 = (const float *)a.ptr(4), *b2 = (const float *)a.ptr(5), *w3 = (const float *)a.ptr(6);
+  const float *b3 = (const float *)a.ptr(7), *res = (const float *)a.ptr(8);
+  float *y = (float *)a.ptr(9);
+  if (!a.ok) return nullptr;
+  HIP_OK(tfhip_fused_inverted_residual(x, w1, b1, act, w2, b2, w3, b3, res, y, g[0], g[1], g[2], g[3], g[4], g[5], g[6],
+                                       g[7], g[8], g[9], g[10]));
+  return undefined(env);
+}
+
+// invertedResidualPays(batch, inH, inW, inC, midC, outC, stride, outH, outW): boolean
+napi_value InvertedResidualPays(napi_env env, napi_callback_info info) {
+  Args a(env, info, 9, "invertedResidualPays");
+  int64_t v[9];
+  for (int i = 0; i < 9; ++i) v[i] = a.i64(i);
+  if (!a.ok) return nullptr;
+  napi_value out;
+  NAPI_OK(napi_get_boolean(env, tfhip_inverted_residual_pays(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8]) == 1, &out));
+  return out;
+}
+
 // meanHW(x, y, batch, h, w, c)
 napi_value MeanHW(napi_env env, napi_callback_info info) {
   Args a(env, info, 6, "meanHW");
@@ -560,6 +657,13 @@ napi_value Register(napi_env env, napi_value exports) {
       FN("dequantF16", DequantF16),
       FN("add", Add),
       FN("meanHW", MeanHW),
+      FN("binary", Binary),
+      FN("unary", Unary),
+      FN("avgPool", AvgPool),
+      FN("cast", Cast),
+      FN("transpose2d", Transpose2D),
+      FN("fusedInvertedResidual", FusedInvertedResidual),
+      FN("invertedResidualPays", InvertedResidualPays),
       FN("fusedPointwiseDepthwise", FusedPointwiseDepthwise),
       FN("pointwiseDepthwisePays", PointwiseDepthwisePays),
       FN("fusedConv2DDepthwise", FusedConv2DDepthwise),

@@ -20,8 +20,9 @@ const graphModel = require('./standin/graph_model');
 const kernelConfigs = [
   matmul.fusedMatMulConfig, matmul.batchMatMulConfig, conv.fusedConv2DConfig,
   conv.fusedConv2DAddConfig, conv.fusedPointwiseDepthwiseConfig, conv.conv2DConfig, conv.fusedDepthwiseConv2DConfig,
-  conv.depthwiseConv2dNativeConfig, glue.addConfig, glue.meanConfig,
-  glue.reshapeConfig, glue.identityConfig, glue.copyConfig
+  conv.depthwiseConv2dNativeConfig, glue.addConfig, glue.subConfig, glue.multiplyConfig, glue.reluConfig,
+  glue.relu6Config, glue.eluConfig, glue.sigmoidConfig, glue.leakyReluConfig, glue.meanConfig, glue.avgPoolConfig,
+  glue.castConfig, glue.transposeConfig, glue.reshapeConfig, glue.identityConfig, glue.copyConfig
 ];
 
 tf.registerBackend('hip', () => new HipBackend(), 3 /* priority */);

@@ -10,8 +10,11 @@
  *   input / output checks         tfjs-converter/src/executor/graph_executor.ts:704-772
  *   attribute decoding            tfjs-converter/src/operations/operation_mapper.ts:437-610
  *   node -> op call               tfjs-converter/src/operations/executors/convolution_executor.ts:28-173,
- *                                 matrices_executor.ts:28-90, arithmetic_executor.ts, reduction_executor.ts,
- *                                 transformation_executor.ts (Reshape), graph_executor.ts (Identity ...)
+ *                                 matrices_executor.ts:28-90, arithmetic_executor.ts (Add, Sub, Mul),
+ *                                 basic_math_executor.ts (Relu, Relu6, Elu, Sigmoid, LeakyRelu),
+ *                                 reduction_executor.ts (Mean), convolution_executor.ts:225-238 (AvgPool),
+ *                                 transformation_executor.ts (Reshape, Squeeze, Cast, Transpose),
+ *                                 graph_executor.ts (Identity ...)
  * The third constructor argument is the io module whose decodeWeights turns the
  * weight bytes into tensors (graph_model.ts:104-107, used at :177): pass
  * {decodeWeights: require('tfjs-backend-hip').decodeWeights} to have quantized
@@ -325,6 +328,41 @@ function compileNode(node) {
     case 'AddV2':
     case 'BiasAdd':
       return inputs => tf.add(inputs[0], inputs[1]);
+    // arithmetic_executor.ts:48-70, basic_math_executor.ts:150-175
+    case 'Sub':
+      return inputs => tf.sub(inputs[0], inputs[1]);
+    case 'Mul':
+      return inputs => tf.mul(inputs[0], inputs[1]);
+    case 'Relu':
+      return inputs => tf.relu(inputs[0]);
+    case 'Relu6':
+      return inputs => tf.relu6(inputs[0]);
+    case 'Elu':
+      return inputs => tf.elu(inputs[0]);
+    case 'Sigmoid':
+      return inputs => tf.sigmoid(inputs[0]);
+    case 'LeakyRelu': {
+      const alpha = getNumberParam(attrs, 'alpha', 0.2);
+      return inputs => tf.leakyRelu(inputs[0], alpha);
+    }
+    // convolution_executor.ts:225-238
+    case 'AvgPool': {
+      const stride = getNumericArrayParam(attrs, 'strides', [1, 1, 1, 1]);
+      const kernelSize = getNumericArrayParam(attrs, 'ksize', [1, 1, 1, 1]);
+      const pad = getPadding(attrs);
+      return inputs => tf.avgPool(inputs[0], [kernelSize[1], kernelSize[2]], [stride[1], stride[2]], pad);
+    }
+    // transformation_executor.ts:28-50
+    case 'Cast': {
+      const dtype = attrs.DstT ? DTYPES[attrs.DstT.type] : undefined;
+      return inputs => tf.cast(inputs[0], dtype);
+    }
+    case 'Squeeze': {
+      const axis = getNumericArrayParam(attrs, 'squeeze_dims', getNumericArrayParam(attrs, 'axis', []));
+      return inputs => tf.squeeze(inputs[0], axis);
+    }
+    case 'Transpose':
+      return inputs => tf.transpose(inputs[0], valuesOf(inputs[1]));
     case 'Mean': {
       const keepDims = getBoolParam(attrs, 'keep_dims', false);
       return inputs => tf.mean(inputs[0], valuesOf(inputs[1]), keepDims);
@@ -385,6 +423,9 @@ class GraphModel {
       this.nodes[node.name] = node;
       this.order.push(node.name);
     });
+    if (this.loadOptions.fuseDepthwiseBiasActivation !== false) {
+      this.rewriteDepthwiseChains();
+    }
     this.placeholders = this.order.filter(n => this.nodes[n].op.startsWith('Placeholder'));
     const consumed = new Set();
     this.order.forEach(n => (this.nodes[n].input || []).forEach(i => consumed.add(parseNodeName(i)[0])));
@@ -395,6 +436,53 @@ class GraphModel {
         this.order.filter(n => !consumed.has(n) && this.nodes[n].op !== 'Const' && this.nodes[n].op !== 'NoOp');
     this.weightMap = this.io.decodeWeights(artifacts.weightData, artifacts.weightSpecs);
     return true;
+  }
+
+  /**
+   * DepthwiseConv2dNative -> BiasAdd [-> Relu | Relu6 | Elu] chains, each link read by the next one
+   * only, become one FusedDepthwiseConv2dNative node named after the chain's last node: the rewrite
+   * the converter's own grappler pass makes
+   * (tfjs-converter/python/tensorflowjs/converters/fuse_depthwise_conv2d.py), for models converted
+   * without it. The fused kernel rounds as the three kernels do, so values do not change;
+   * {fuseDepthwiseBiasActivation: false} in the load options keeps the graph's nodes.
+   */
+  rewriteDepthwiseChains() {
+    const readers = {};
+    this.order.forEach(n => (this.nodes[n].input || []).forEach(i => {
+      const src = parseNodeName(i)[0];
+      (readers[src] = readers[src] || []).push(n);
+    }));
+    const data = node => (node.input || []).filter(i => i[0] !== '^');
+    const onlyReader = name => (readers[name] || []).length === 1 ? this.nodes[readers[name][0]] : null;
+    const activations = {Relu: 'Relu', Relu6: 'Relu6', Elu: 'Elu'};
+    const gone = new Set();
+    this.order.forEach(n => {
+      const dw = this.nodes[n];
+      if (dw.op !== 'DepthwiseConv2dNative' || data(dw).length !== 2 || (dw.input || []).length !== 2) {
+        return;
+      }
+      const bias = onlyReader(n);
+      if (bias == null || bias.op !== 'BiasAdd' || (bias.input || []).length !== 2 || parseNodeName(bias.input[0])[0] !== n ||
+          getStringParam(bias.attr || {}, 'data_format', 'NHWC').toUpperCase() !== 'NHWC' ||
+          getStringParam(dw.attr || {}, 'data_format', 'NHWC').toUpperCase() !== 'NHWC') {
+        return;
+      }
+      const act = onlyReader(bias.name);
+      const withAct = act != null && activations[act.op] != null && (act.input || []).length === 1;
+      const last = withAct ? act : bias;
+      const fusedOps = ['BiasAdd'].concat(withAct ? [activations[act.op]] : []);
+      const attr = Object.assign({}, dw.attr, {
+        fused_ops: {list: {s: fusedOps.map(f => Buffer.from(f).toString('base64'))}},
+        num_args: {i: '1'}
+      });
+      this.nodes[last.name] = {name: last.name, op: 'FusedDepthwiseConv2dNative', input: [dw.input[0], dw.input[1], bias.input[1]], attr};
+      gone.add(n);
+      if (withAct) {
+        gone.add(bias.name);
+      }
+    });
+    gone.forEach(n => delete this.nodes[n]);
+    this.order = this.order.filter(n => !gone.has(n));
   }
 
   get weights() {
@@ -434,6 +522,11 @@ class GraphModel {
 
   predict(inputs, config) {
     return this.execute(inputs, this.outputNodes);
+  }
+
+  /** graph_model.ts:455-470: a Promise of execute (no graph of this path has control flow to wait for). */
+  executeAsync(inputs, outputs) {
+    return new Promise(resolve => resolve(this.execute(inputs, outputs)));
   }
 
   execute(inputs, outputs) {

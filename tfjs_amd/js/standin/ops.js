@@ -2,7 +2,8 @@
 /**
  * Offline stand-in for the op wrappers that call the hot path
  * (tfjs-core/src/ops/fused/{mat_mul,conv2d,depthwise_conv2d}.ts,
- * ops/{mat_mul,conv2d,depthwise_conv2d,add,mean,reshape}.ts): argument
+ * ops/{mat_mul,conv2d,depthwise_conv2d,add,sub,mul,relu,relu6,elu,sigmoid,leaky_relu,
+ * avg_pool,cast,squeeze,transpose,mean,reshape}.ts): argument
  * defaults, the reshapes to the rank the kernels are handed, the validation
  * that throws before any backend is reached, and ENGINE.runKernel with the
  * kernel names and attribute objects of tfjs-core/src/kernel_names.ts.
@@ -93,6 +94,79 @@ function add(a, b) {
   const $a = convertToTensor(a, 'a', 'add');
   const $b = convertToTensor(b, 'b', 'add');
   return ENGINE.runKernel('Add', {a: $a, b: $b});
+}
+
+function binaryOp(kernelName, opName) {
+  return (a, b) => {
+    const $a = convertToTensor(a, 'a', opName);
+    const $b = convertToTensor(b, 'b', opName);
+    return ENGINE.runKernel(kernelName, {a: $a, b: $b});
+  };
+}
+
+function unaryOp(kernelName, opName) {
+  return x => ENGINE.runKernel(kernelName, {x: convertToTensor(x, 'x', opName)});
+}
+
+function leakyRelu(x, alpha) {
+  return ENGINE.runKernel('LeakyRelu', {x: convertToTensor(x, 'x', 'leakyRelu')}, {alpha: alpha == null ? 0.2 : alpha});
+}
+
+/** tfjs-core/src/ops/cast.ts */
+function cast(x, dtype) {
+  const $x = convertToTensor(x, 'x', 'cast');
+  if (['float32', 'int32', 'bool', 'complex64', 'string'].indexOf(dtype) < 0) {
+    throw new Error(`Failed to cast to unknown dtype ${dtype}`);
+  }
+  if ((dtype === 'string') !== ($x.dtype === 'string')) {
+    throw new Error('Only strings can be casted to strings');
+  }
+  return ENGINE.runKernel('Cast', {x: $x}, {dtype});
+}
+
+/** tfjs-core/src/ops/avg_pool.ts:54-95 */
+function avgPool(x, filterSize, strides, pad, dimRoundingMode) {
+  const $x = convertToTensor(x, 'x', 'avgPool', 'float32');
+  util.assert(
+      backend_util.eitherStridesOrDilationsAreOne(strides, 1),
+      () => `Error in avgPool: Either strides or dilations must be 1. Got strides ${strides} and dilations '1'`);
+  assertFloat32($x, 'x', 'avgPool');
+  return ENGINE.tidy(() => {
+    const x4D = $x.rank === 3 ? reshape($x, [1, $x.shape[0], $x.shape[1], $x.shape[2]]) : $x;
+    util.assert(x4D.rank === 4, () => `Error in avgPool: x must be rank 4 but got rank ${x4D.rank}.`);
+    backend_util.checkPadOnDimRoundingMode('avgPool', pad, dimRoundingMode);
+    const res = ENGINE.runKernel('AvgPool', {x: x4D}, {filterSize, strides, pad, dimRoundingMode});
+    return $x.rank === 3 ? reshape(res, [res.shape[1], res.shape[2], res.shape[3]]) : res;
+  });
+}
+
+/** tfjs-core/src/ops/squeeze.ts over util.squeezeShape: size-1 axes (all, or the listed ones) go. */
+function squeeze(x, axis) {
+  const $x = convertToTensor(x, 'x', 'squeeze');
+  const listed = axis == null || (Array.isArray(axis) && axis.length === 0) ?
+      null : util.parseAxisParam(axis, $x.shape);
+  const newShape = [];
+  $x.shape.forEach((d, i) => {
+    if (listed != null && listed.indexOf(i) >= 0) {
+      if (d !== 1) {
+        throw new Error(`Can't squeeze axis ${i} since its dim '${d}' is not 1`);
+      }
+    } else if (d !== 1 || listed != null) {
+      newShape.push(d);
+    }
+  });
+  return reshape($x, newShape);
+}
+
+/** tfjs-core/src/ops/transpose.ts (no conjugation: real tensors only) */
+function transpose(x, perm) {
+  const $x = convertToTensor(x, 'x', 'transpose');
+  const $perm = perm == null ? $x.shape.map((_, i) => i).reverse() : perm;
+  util.assert($x.rank === $perm.length,
+              () => `Error in transpose: rank of input ${$x.rank} must match length of perm ${$perm}.`);
+  $perm.forEach(axis => util.assert(axis >= 0 && axis < $x.rank,
+                                    () => `All entries in 'perm' must be between 0 and ${$x.rank - 1} but got ${$perm}`));
+  return ENGINE.runKernel('Transpose', {x: $x}, {perm: $perm});
 }
 
 function mean(x, axis, keepDims) {
@@ -289,6 +363,17 @@ module.exports = {
   tensor4d: (v, shape, dtype) => tensor(v, shape, dtype),
   reshape,
   add,
+  sub: binaryOp('Sub', 'sub'),
+  mul: binaryOp('Multiply', 'mul'),
+  relu: unaryOp('Relu', 'relu'),
+  relu6: unaryOp('Relu6', 'relu6'),
+  elu: unaryOp('Elu', 'elu'),
+  sigmoid: unaryOp('Sigmoid', 'sigmoid'),
+  leakyRelu,
+  cast,
+  avgPool,
+  squeeze,
+  transpose,
   mean,
   matMul,
   conv2d,

@@ -272,6 +272,14 @@ function computeConv2DInfo(inShape, filterShape, strides, dilations, pad, roundi
   };
 }
 
+/** Pooling geometry: a convolution's, with a [fh, fw, C, C] filter (conv_util.ts:119-140). */
+function computePool2DInfo(inShape, filterSize, strides, dilations, pad, roundingMode, dataFormat) {
+  dataFormat = dataFormat || 'channelsLast';
+  const [fh, fw] = tuple3(filterSize);
+  const channels = inShape[dataFormat === 'channelsLast' ? 3 : 1];
+  return computeConv2DInfo(inShape, [fh, fw, channels, channels], strides, dilations, pad, roundingMode, false, dataFormat);
+}
+
 /** A dimRoundingMode only makes sense with whole-number padding (conv_util.ts:607-631). */
 function checkPadOnDimRoundingMode(opDesc, pad, dimRoundingMode) {
   if (dimRoundingMode == null) return;
@@ -301,7 +309,7 @@ module.exports = {
   },
   broadcast_util: {getBroadcastDims, assertAndGetBroadcastShape},
   backend_util: {
-    computeConv2DInfo, convertConv2DDataFormat, eitherStridesOrDilationsAreOne, tupleValuesAreOne,
+    computeConv2DInfo, computePool2DInfo, convertConv2DDataFormat, eitherStridesOrDilationsAreOne, tupleValuesAreOne,
     checkPadOnDimRoundingMode, getBroadcastDims, assertAndGetBroadcastShape
   }
 };
