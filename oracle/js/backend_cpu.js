@@ -214,7 +214,9 @@ function batchMatMul({inputs, backend, attrs}) {
   const aBatch = aS[0], aOuterStep = transposeA ? 1 : aS[1], aInnerStep = transposeA ? aS[1] : 1;
   const bInnerStep = transposeB ? 1 : bS[1], bOuterStep = transposeB ? bS[1] : 1, bBatch = bS[0];
   const size = leftDim * rightDim;
-  const resVals = new Float32Array(batchDim * size);
+  // the product takes a's dtype (BatchMatMul.ts:90): int32 operands accumulate into an Int32Array
+  const resVals = a.dtype === 'int32' ? new Int32Array(batchDim * size) :
+      a.dtype === 'bool' ? new Uint8Array(batchDim * size) : new Float32Array(batchDim * size);
   const blockSize = backend.blockSize;
   for (let bi = 0; bi < batchDim; bi++) {
     const batchIndexA = bi % batchDimA;
@@ -239,7 +241,7 @@ function batchMatMul({inputs, backend, attrs}) {
       }
     }
   }
-  return backend.makeTensorInfo(outShape, 'float32', resVals);
+  return backend.makeTensorInfo(outShape, a.dtype, resVals);
 }
 
 /** The bias-add and activation passes shared by the three fused kernels

@@ -526,8 +526,10 @@ def main():
                        "depthwise_conv2d.json", {"depthwiseConv2d"}, grad)
     harvest_conv_info("tfjs-core/src/ops/conv_util_test.ts", "conv_util.json")
     with open(os.path.join(OUT, "SKIPPED.txt"), "w") as f:
-        f.write("Specs of the reference's test files that make_fixtures.py did not "
-                "transcribe, with the reason.\n")
+        f.write("Specs of the reference's test files that make_fixtures.py's parser did not read, with the "
+                "parser's reason (line = start of the match, which may sit a blank line above the `it(`). "
+                "Where each of them is carried instead (hand_transcribed.json, tests/js/hand_specs.js, "
+                "tests/js/error_specs.js) or why it is out of scope (gradient, other-op) is in spec_manifest.json.\n")
         f.write("\n".join(skipped) + "\n")
 
 

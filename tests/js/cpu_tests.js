@@ -650,6 +650,28 @@ h.test('hip storage: while a recorded graph is alive, released buffers go back t
   backend.releasePool();
 });
 
+// ---- the error-path specs of the reference's op tests, through the op layer ------------------------------
+require('./error_specs').specs(tf).forEach(spec => {
+  ['cpu', 'hip'].forEach(backendName => {
+    h.test(`error spec @${spec.at} on ${backendName}`, () => {
+      useBackend(backendName);
+      tf.tidy(() => h.assertThrows(spec.fn, spec.message || /./));
+    });
+  });
+});
+
+// ---- specs that test a form of call rather than values: chained ops, composed ops, tensor counts -----------
+require('./hand_specs').specs(tf, h).forEach(spec => {
+  h.test(`hand spec @${spec.at} on cpu`, () => {
+    useBackend('cpu');
+    if (spec.untidied) {
+      spec.fn();
+    } else {
+      tf.tidy(spec.fn);
+    }
+  });
+});
+
 // ---- converter-written models that the reference's own tests hold --------------------------------
 const refModels = require('./ref_models');
 

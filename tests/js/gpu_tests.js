@@ -69,6 +69,21 @@ h.loadGolden('glue_ops.json').cases.forEach(c => {
   });
 });
 
+require('./hand_specs').specs(tf, h).forEach(spec => {
+  h.test(`hip hand spec @${spec.at}`, () => {
+    h.assert(tf.engine().setBackend('hip') === true, 'setBackend(hip)');
+    if (spec.untidied) {
+      spec.fn();
+    } else {
+      tf.tidy(spec.fn);
+    }
+  });
+});
+
+require('./error_specs').specs(tf).forEach(spec => {
+  h.test(`hip error spec @${spec.at}`, () => on('hip', () => h.assertThrows(spec.fn, spec.message || /./)));
+});
+
 h.test('element-wise, pooling, cast and transpose kernels against the oracle on the same arrays', () => {
   const r = h.rng(31);
   const a = r.uniform(2 * 9 * 8 * 6, -3, 3), b = r.uniform(6, -2, 2);

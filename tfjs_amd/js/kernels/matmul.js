@@ -8,6 +8,7 @@
  */
 const tf = require('../core');
 const {activationCode, broadcastStrides, requireFloat32, addon} = require('./fused_util');
+const {castConfig} = require('./glue');
 
 const biasScratch = new Float64Array(3);
 const preluScratch = new Float64Array(3);
@@ -96,9 +97,25 @@ function fusedMatMul(args) {
       '_FusedMatMul');
 }
 
+/**
+ * BatchMatMul. The cpu kernel accumulates in JavaScript numbers and writes a buffer of a's dtype
+ * (BatchMatMul.ts:90), so int32 operands give an int32 product. Here int32 (and bool) operands are
+ * converted to float32 on the device, multiplied by the same GEMM, and the product converted back:
+ * exact while every dot product stays below 2^24 in magnitude, which is also what the reference's
+ * GPU backends offer, whose int32 tensors live in float textures.
+ */
 function batchMatMul(args) {
   const {a, b} = args.inputs;
   const {transposeA, transposeB} = args.attrs;
+  if (a.dtype !== 'float32' && a.dtype === b.dtype && (a.dtype === 'int32' || a.dtype === 'bool')) {
+    const backend = args.backend;
+    const castTo = (x, dtype) => castConfig.kernelFunc({inputs: {x}, attrs: {dtype}, backend});
+    const aFloat = castTo(a, 'float32'), bFloat = castTo(b, 'float32');
+    const product = matMulImpl(backend, aFloat, bFloat, !!transposeA, !!transposeB, null, 'linear', null, 0.2, 'BatchMatMul');
+    const out = castTo(product, a.dtype);
+    [aFloat, bFloat, product].forEach(t => backend.disposeData(t.dataId));
+    return out;
+  }
   return matMulImpl(
       args.backend, a, b, !!transposeA, !!transposeB, null, 'linear', null, 0.2,
       'BatchMatMul');

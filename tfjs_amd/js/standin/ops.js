@@ -65,24 +65,66 @@ function tensor(values, shape, dtype) {
   return ENGINE.makeTensor(data, shape, dtype);
 }
 
+/** What dtype a plain JavaScript value would become as a tensor: strings stay strings, booleans bool, the rest float32. */
+function dtypeOfValues(values) {
+  let v = values;
+  while (Array.isArray(v)) {
+    v = v[0];
+  }
+  if (v instanceof Float32Array) {
+    return 'float32';
+  } else if (v instanceof Int32Array || v instanceof Uint8Array || v instanceof Uint8ClampedArray) {
+    return 'int32';
+  } else if (typeof v === 'string') {
+    return 'string';
+  } else if (typeof v === 'boolean') {
+    return 'bool';
+  }
+  return 'float32';
+}
+
+function checkArgumentDtype(expected, actual, argName, opName) {
+  const wrong = expected === 'numeric' ? actual === 'string' :
+                                         expected !== 'string_or_numeric' && expected !== actual;
+  if (wrong) {
+    throw new Error(
+        `Argument '${argName}' passed to '${opName}' must be ${expected} tensor, but got ${actual} tensor`);
+  }
+}
+
+/**
+ * An op argument as a Tensor (tfjs-core/src/tensor_util_env.ts:98-131): a Tensor goes through once
+ * its dtype fits `dtype` ('numeric' = anything but string, the default); a number, boolean, string,
+ * nested array or typed array becomes one, numbers taking `dtype` when it names a concrete type;
+ * anything else is refused by its constructor's name.
+ */
 function convertToTensor(x, argName, opName, dtype) {
+  const expected = dtype || 'numeric';
   if (x instanceof Tensor) {
+    checkArgumentDtype(expected, x.dtype, argName, opName);
     return x;
   }
-  if (x == null) {
-    throw new Error(
-        `Argument '${argName}' passed to '${opName}' must be a Tensor ` +
-        `or TensorLike, but got 'null'`);
+  let inferred = dtypeOfValues(x);
+  if (inferred !== 'string' && (expected === 'bool' || expected === 'int32' || expected === 'float32')) {
+    inferred = expected;
   }
-  return tensor(x, null, dtype || 'float32');
+  checkArgumentDtype(expected, inferred, argName, opName);
+  const plain = x != null && (ArrayBuffer.isView(x) || Array.isArray(x) || typeof x === 'number' ||
+                              typeof x === 'boolean' || typeof x === 'string');
+  if (!plain) {
+    throw new Error(
+        `Argument '${argName}' passed to '${opName}' must be a Tensor or TensorLike, but got ` +
+        `'${x == null ? 'null' : x.constructor.name}'`);
+  }
+  if (inferred === 'string') {
+    const flat = Array.isArray(x) ? flatten(x, []) : [x];
+    return ENGINE.makeTensor(flat, Array.isArray(x) ? inferShape(x) : [], 'string');
+  }
+  return tensor(x, null, inferred);
 }
 
 function assertFloat32(t, argName, opName) {
-  if (t.dtype !== 'float32') {
-    throw new Error(
-        `Argument '${argName}' passed to '${opName}' must be float32 ` +
-        `tensor, but got ${t.dtype} tensor`);
-  }
+  checkArgumentDtype('float32', t.dtype, argName, opName);
 }
 
 function reshape(x, shape) {
@@ -175,13 +217,28 @@ function mean(x, axis, keepDims) {
       'Mean', {x: $x}, {axis: axis == null ? null : axis, keepDims: !!keepDims});
 }
 
+/**
+ * Operands of two dtypes both become the wider one (tfjs-core/src/tensor_util.ts:23-29 over
+ * types.ts:97-128): bool < int32 < float32 < complex64.
+ */
+function makeTypesMatch(a, b) {
+  if (a.dtype === b.dtype) {
+    return [a, b];
+  }
+  const order = ['bool', 'int32', 'float32', 'complex64'];
+  if (order.indexOf(a.dtype) < 0 || order.indexOf(b.dtype) < 0) {
+    throw new Error(`Can not upcast ${a.dtype} with ${b.dtype}`);
+  }
+  const wider = order[Math.max(order.indexOf(a.dtype), order.indexOf(b.dtype))];
+  return [cast(a, wider), cast(b, wider)];
+}
+
 /** tfjs-core/src/ops/mat_mul.ts:44-57 */
 function matMul(a, b, transposeA, transposeB) {
-  const $a = convertToTensor(a, 'a', 'matMul');
-  const $b = convertToTensor(b, 'b', 'matMul');
-  return ENGINE.runKernel(
-      'BatchMatMul', {a: $a, b: $b},
-      {transposeA: !!transposeA, transposeB: !!transposeB});
+  return ENGINE.tidy(() => {
+    const [$a, $b] = makeTypesMatch(convertToTensor(a, 'a', 'matMul'), convertToTensor(b, 'b', 'matMul'));
+    return ENGINE.runKernel('BatchMatMul', {a: $a, b: $b}, {transposeA: !!transposeA, transposeB: !!transposeB});
+  });
 }
 
 /** tfjs-core/src/ops/fused/mat_mul.ts:58-211 */
@@ -318,44 +375,85 @@ function fusedDepthwiseConv2d(args) {
   return convCommon('depthwiseConv2d', 'FusedDepthwiseConv2D', args, true);
 }
 
-/** tfjs-core/src/ops/conv2d.ts (unfused) */
+/** The checks conv2d and depthwiseConv2d share before the kernel is reached; returns x as rank 4. */
+function convOperands(opName, x, filter, pad, dataFormat, dimRoundingMode, depthMessage) {
+  const $x = convertToTensor(x, 'x', opName, 'float32');
+  const $filter = convertToTensor(filter, 'filter', opName, 'float32');
+  const x4D = $x.rank === 3 ? reshape($x, [1, $x.shape[0], $x.shape[1], $x.shape[2]]) : $x;
+  util.assert(x4D.rank === 4, () => `Error in ${opName}: input must be rank 4, but got rank ${x4D.rank}.`);
+  util.assert($filter.rank === 4, () => `Error in ${opName}: filter must be rank 4, but got rank ${$filter.rank}.`);
+  backend_util.checkPadOnDimRoundingMode(opName, pad, dimRoundingMode);
+  const depth = dataFormat === 'NHWC' ? x4D.shape[3] : x4D.shape[1];
+  util.assert(depth === $filter.shape[2], () => depthMessage(depth, $filter.shape[2]));
+  return {$x, x4D, $filter};
+}
+
+const allPositive = v => (Array.isArray(v) ? v : [v]).every(e => e > 0);
+
+/** tfjs-core/src/ops/conv2d.ts:62-117 (unfused) */
 function conv2d(x, filter, strides, pad, dataFormat, dilations, dimRoundingMode) {
-  const $x = convertToTensor(x, 'x', 'conv2d', 'float32');
-  const $filter = convertToTensor(filter, 'filter', 'conv2d', 'float32');
+  dataFormat = dataFormat || 'NHWC';
+  dilations = dilations == null ? [1, 1] : dilations;
   return ENGINE.tidy(() => {
-    const x4D = $x.rank === 3 ?
-        reshape($x, [1, $x.shape[0], $x.shape[1], $x.shape[2]]) : $x;
-    const res = ENGINE.runKernel('Conv2D', {x: x4D, filter: $filter}, {
-      strides,
-      pad,
-      dataFormat: dataFormat || 'NHWC',
-      dilations: dilations == null ? [1, 1] : dilations,
-      dimRoundingMode
-    });
+    const {$x, x4D, $filter} = convOperands(
+        'conv2d', x, filter, pad, dataFormat, dimRoundingMode,
+        (got, want) => `Error in conv2d: depth of input (${got}) must match input depth for filter ${want}.`);
+    util.assert(
+        backend_util.eitherStridesOrDilationsAreOne(strides, dilations),
+        () => `Error in conv2D: Either strides or dilations must be 1. Got strides ${strides} and dilations '${dilations}'`);
+    util.assert(allPositive(dilations), () => 'Error in conv2D: Dilated rates should be larger than 0.');
+    util.assert(allPositive(strides), () => 'Error in conv2D: Strides should be larger than 0.');
+    const res = ENGINE.runKernel('Conv2D', {x: x4D, filter: $filter}, {strides, pad, dataFormat, dilations, dimRoundingMode});
     return $x.rank === 3 ? reshape(res, res.shape.slice(1)) : res;
   });
 }
 
-/** tfjs-core/src/ops/depthwise_conv2d.ts (unfused) */
+/** tfjs-core/src/ops/depthwise_conv2d.ts:75-121 (unfused) */
 function depthwiseConv2d(x, filter, strides, pad, dataFormat, dilations, dimRoundingMode) {
-  const $x = convertToTensor(x, 'x', 'depthwiseConv2d', 'float32');
-  const $filter = convertToTensor(filter, 'filter', 'depthwiseConv2d', 'float32');
+  dataFormat = dataFormat || 'NHWC';
+  dilations = dilations == null ? [1, 1] : dilations;
   return ENGINE.tidy(() => {
-    const x4D = $x.rank === 3 ?
-        reshape($x, [1, $x.shape[0], $x.shape[1], $x.shape[2]]) : $x;
-    const res = ENGINE.runKernel('DepthwiseConv2dNative', {x: x4D, filter: $filter}, {
-      strides,
-      pad,
-      dataFormat: dataFormat || 'NHWC',
-      dilations: dilations == null ? [1, 1] : dilations,
-      dimRoundingMode
-    });
+    const {$x, x4D, $filter} = convOperands(
+        'depthwiseConv2d', x, filter, pad, dataFormat, dimRoundingMode,
+        (got, want) => `Error in depthwiseConv2d: number of input channels (${got}) must match the inChannels ` +
+            `dimension in filter ${want}.`);
+    const res = ENGINE.runKernel(
+        'DepthwiseConv2dNative', {x: x4D, filter: $filter}, {strides, pad, dataFormat, dilations, dimRoundingMode});
     return $x.rank === 3 ? reshape(res, res.shape.slice(1)) : res;
   });
 }
+
+/** new tensor of one value (tfjs-core/src/ops/{zeros,ones,fill}.ts) */
+function fill(shape, value, dtype) {
+  dtype = dtype || 'float32';
+  const data = util.getTypedArrayFromDType(dtype, util.sizeFromShape(shape));
+  if (value !== 0) {
+    data.fill(value);
+  }
+  return ENGINE.makeTensor(data, shape, dtype);
+}
+
+/**
+ * The chained forms of the ops above (tfjs-core/src/public/chained_ops/*.ts): `a.matMul(b)` is
+ * `matMul(a, b)`, and so on, after a check that the tensor has not been disposed.
+ */
+function chain(method, op) {
+  Tensor.prototype[method] = function(...rest) {
+    this.throwIfDisposed();
+    return op(this, ...rest);
+  };
+}
+[['reshape', reshape], ['add', add], ['sub', binaryOp('Sub', 'sub')], ['mul', binaryOp('Multiply', 'mul')],
+ ['relu', unaryOp('Relu', 'relu')], ['relu6', unaryOp('Relu6', 'relu6')], ['elu', unaryOp('Elu', 'elu')],
+ ['sigmoid', unaryOp('Sigmoid', 'sigmoid')], ['leakyRelu', leakyRelu], ['cast', cast], ['avgPool', avgPool],
+ ['squeeze', squeeze], ['transpose', transpose], ['mean', mean], ['matMul', matMul], ['conv2d', conv2d],
+ ['depthwiseConv2d', depthwiseConv2d]].forEach(([method, op]) => chain(method, op));
 
 module.exports = {
   tensor,
+  zeros: (shape, dtype) => fill(shape, 0, dtype),
+  ones: (shape, dtype) => fill(shape, 1, dtype),
+  fill,
   scalar: (v, dtype) => tensor([v], [], dtype),
   tensor1d: (v, dtype) => tensor(v, null, dtype),
   tensor2d: (v, shape, dtype) => tensor(v, shape, dtype),
