@@ -16,8 +16,12 @@ Besides `value` (images/s) the line carries
                 flops) of its launches in one step / their summed duration
   kernels       the same figure for each benchmark configuration's own kernel
                 (fused matmul, stem and pointwise conv, depthwise, BERT matmuls,
-                dequant), each launched back to back between two events
-  cpu_baseline  the same graph at batch 1 on one host thread, timed beside it
+                dequant): `frac` with the operands coming from memory (a rotation
+                of operand sets larger than the memory-side cache), `frac_warm`
+                launched back to back on one set
+  b1            the same model at batch 1 (the reference's own benchmark setting)
+  unfused_plan  batch 32 with the cross-node fusions of the graph model turned off
+  cpu_baseline  the same graph on one host thread, timed beside it
 
 Other modes:  --kernels-only (skip the model), --no-kernels, --no-cpu-baseline,
 --copy-yardstick MIB (adds copies of known size for hardware-counter runs).
@@ -42,29 +46,15 @@ MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
 RIDGE = MFMA_FP32_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
 BATCH = 32
 
-# HBM bytes per launch (reads + writes), averaged over a symbol's launches in one
-# MobileNetV2 b32 inference: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each
-# scaled by its reading for a 256 MiB copy kernel
-# (profiles/mobilenet_v2_b32_hbm_traffic.md holds the runs). Hardware counters
-# cannot be read from inside this script, so the table is refreshed by hand when a
-# kernel changes; a symbol that is not listed reports null.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "expand_dw_3x3<1, 0, false, 2, 7>": 86256647,
-    "skinny_gemm_regs<1, 2, false>": 77140638,
-    "expand_dw_3x3<2, 1, false, 2, 0>": 75139599,
-    "skinny_gemm<2, 4>": 64073078,
-    "expand_dw_3x3<1, 1, true, 2, 0>": 77991477,
-    "expand_dw_3x3<2, 1, true, 2, 0>": 28900751,
-    "gemm_kernel<32, 32, 32, 2, 2, 0, 1>": 17343859,
-    "gemm_kernel<64, 64, 16, 2, 2, 0, 1>": 18570635,
-    "depthwise_3x3_rows<1, false>": 36289941,
-    "depthwise_3x3_flat<2, false>": 22006225,
-    "depthwise_3x3_flat<1, false>": 17923350,
-    "gemm_kernel<32, 64, 32, 2, 2, 0, 1>": 12344521,
-    "mean_hw_vec": 8295736,
-    "gemm_finish": 896442,
-    "copy_to_host": 277490,
-}
+COLD_BYTES = 512 << 20         # operand sets a cold-cache measurement rotates through: twice the 256 MB memory-side cache
+
+
+def measured_traffic():
+    """HBM bytes per launch by kernel symbol, from profiles/traffic.json (written by
+    `python -m tfjs_amd.traffic` from two hardware-counter runs of this script), and whether the
+    kernel sources have changed since those runs: (table, stale)."""
+    from tfjs_amd import traffic
+    return traffic.load(os.path.join(ROOT, "profiles", "traffic.json"))
 
 
 def roofline_entry(flops, nbytes, seconds):
@@ -127,6 +117,76 @@ def time_launches(lib, check, ev, fn, repeat=50, rounds=3, settle_ms=None):
             best = ms if best is None else min(best, ms)
     finally:
         check(lib.tfhip_set_launch_repeat(1))
+    return best * 1e-3
+
+
+class Slab:
+    """`count` copies of one operand in one device buffer, 256 bytes apart at least: set i of a
+    cold-cache measurement reads or writes copy i."""
+
+    class View:
+        def __init__(self, ptr):
+            self.ptr = ptr
+
+    def __init__(self, source, count):
+        from tfjs_amd.capi import DeviceBuffer
+        host = None if isinstance(source, int) else np.ascontiguousarray(source)
+        nbytes = source if host is None else host.nbytes
+        self.stride = (nbytes + 255) // 256 * 256
+        self.buffer = DeviceBuffer(self.stride * count)
+        if host is not None:
+            for i in range(count):
+                self.buffer.upload(host, i * self.stride)
+
+    def __getitem__(self, i):
+        return Slab.View(self.buffer.ptr + i * self.stride)
+
+    def free(self):
+        self.buffer.free()
+
+
+def sets_for(set_bytes):
+    """How many operand sets of this size make the rotation exceed COLD_BYTES."""
+    return max(2, int(-(-COLD_BYTES // max(1, int(set_bytes)))))
+
+
+def time_launches_cold(lib, check, ev, launch, n_sets, rounds=3, settle_ms=None):
+    """Average duration in seconds of one launch when its operands come from memory: `launch(i)`
+    enqueues the kernel on operand set i, the n_sets sets together exceed the memory-side cache
+    twice over and are visited in turn, so no launch finds what an earlier one left behind. The
+    rotation is recorded once into a HIP graph and replayed between two events (no host work
+    between the launches), best of `rounds`."""
+    graph_id, nodes = ctypes.c_int(), ctypes.c_int()
+    launch(0)
+    check(lib.tfhip_sync())
+    check(lib.tfhip_capture_begin())
+    try:
+        for i in range(n_sets):
+            launch(i)
+    except Exception:
+        lib.tfhip_capture_end(None, ctypes.byref(nodes))
+        raise
+    check(lib.tfhip_capture_end(ctypes.byref(graph_id), ctypes.byref(nodes)))
+    try:
+        settle_ms = SETTLE_MS if settle_ms is None else settle_ms
+        settled, one_ms = 0.0, None
+        while one_ms is None or settled < settle_ms:
+            ev.record(0)
+            check(lib.tfhip_graph_launch(graph_id.value))
+            ev.record(1)
+            one_ms = max(ev.elapsed_ms(0, 1), 0.01)
+            settled += one_ms
+        replays = max(1, int(5.0 / one_ms))
+        best = None
+        for _ in range(rounds):
+            ev.record(0)
+            for _ in range(replays):
+                check(lib.tfhip_graph_launch(graph_id.value))
+            ev.record(1)
+            ms = ev.elapsed_ms(0, 1) / (replays * n_sets)
+            best = ms if best is None else min(best, ms)
+    finally:
+        check(lib.tfhip_graph_destroy(graph_id.value))
     return best * 1e-3
 
 
@@ -200,28 +260,29 @@ def bench_model(model_dir, steps, warmup):
     dominant = max(by_symbol, key=lambda k: by_symbol[k]["seconds"])
     d = by_symbol[dominant]
     roof = roofline_entry(d["flops"], d["bytes"], d["seconds"])
+    traffic_table, traffic_stale = measured_traffic()
     roof.update(kernel=dominant, launches_per_step=d["launches"],
                 avg_launch_us=round(d["seconds"] / d["launches"] * 1e6, 2),
                 share_of_kernel_time=round(d["seconds"] / kernel_seconds, 3),
                 algorithmic_bytes_per_launch=round(d["bytes"] / d["launches"]),
-                traffic=MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(dominant))
+                traffic=traffic_table.get(dominant), traffic_stale=traffic_stale)
     symbols = {k: dict(us_per_step=round(v["seconds"] * 1e6, 1), launches=v["launches"],
                        **roofline_entry(v["flops"], v["bytes"], v["seconds"])) for k, v in by_symbol.items()}
     return dict(ms_per_step=seconds / steps * 1e3, kernel_ms_per_step=kernel_seconds * 1e3, roofline=roof,
-                symbols=symbols, ops=ops, marker_us=marker_ms * 1e3)
+                symbols=symbols, ops=ops, marker_us=marker_ms * 1e3, plan_kernels=[names[i] for i in range(n_ops)])
 
 
-def bench_model_node(model_dir, steps, warmup, prime):
-    """The headline measurement: MobileNetV2 through the tfjs API in Node on the
-    hip backend (KernelBackend + kernel configs + N-API addon). Returns the
-    script's JSON, or None when Node or the addon is not available."""
+def bench_model_node(model_dir, steps, warmup, prime, batch=BATCH, record=False, options=None):
+    """MobileNetV2 through the tfjs API in Node on the hip backend (KernelBackend + kernel configs +
+    N-API addon): the headline measurement at batch 32. Returns the script's JSON, or None when Node
+    or the addon is not available."""
     node = shutil.which("node")
     script = os.path.join(ROOT, "tfjs_amd", "js", "bench", "mobilenet_bench.js")
     addon = os.path.join(ROOT, "tfjs_amd", "lib", "tfjs_hip.node")
     if not (node and os.path.exists(addon)):
         return None
-    proc = subprocess.run([node, script, model_dir, str(BATCH), str(steps), str(warmup), str(prime)], stdout=subprocess.PIPE,
-                          stderr=subprocess.PIPE, text=True, timeout=900)
+    proc = subprocess.run([node, script, model_dir, str(batch), str(steps), str(warmup), str(prime), "1" if record else "0",
+                           json.dumps(options or {})], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=900)
     if proc.returncode != 0:
         raise RuntimeError("node benchmark failed:\n%s" % proc.stderr[-3000:])
     return json.loads(proc.stdout.strip().splitlines()[-1])
@@ -239,55 +300,66 @@ def bench_kernels():
     ev = Events(lib, check)
     out = []
 
+    def row(name, flops, nbytes, warm_s, cold_s):
+        """One configuration's line: `frac` (and us, achieved) are the cold-cache launch, operands from
+        memory; `frac_warm` / `us_warm` the same kernel launched back to back on one operand set, which a
+        working set below the 256 MB memory-side cache flatters."""
+        cold, warm = roofline_entry(flops, nbytes, cold_s), roofline_entry(flops, nbytes, warm_s)
+        out.append(dict(config=name, kernel=last_kernel(lib), us=round(cold_s * 1e6, 2), us_warm=round(warm_s * 1e6, 2),
+                        flops=flops, bytes=nbytes, frac_warm=warm["frac"], achieved_warm=warm["achieved"],
+                        operand_sets=sets_for(nbytes), **cold))
+
     def matmul(name, a, b, bias, activation, transpose_b=False, **_):
         bA, bB, m, n, k, _shape = pyhost.matmul_dims(a.shape, b.shape, False, transpose_b)
-        bufs = [DeviceBuffer.from_numpy(a), DeviceBuffer.from_numpy(b), DeviceBuffer(max(bA, bB) * m * n * 4)]
-        if bias is not None:
-            bufs.append(DeviceBuffer.from_numpy(bias))
-        fn = lambda: pyhost.device_fused_matmul(bufs[0], bufs[1], bufs[2], bA, bB, m, n, k, False, transpose_b,
-                                                bufs[3] if bias is not None else None, [0, 0, 1], activation)
-        sec = time_launches(lib, check, ev, fn)
         flops = 2.0 * max(bA, bB) * m * n * k
         nbytes = 4.0 * (a.size + b.size + max(bA, bB) * m * n + (bias.size if bias is not None else 0))
-        out.append(dict(config=name, kernel=last_kernel(lib), us=round(sec * 1e6, 2), flops=flops, bytes=nbytes,
-                        **roofline_entry(flops, nbytes, sec)))
-        for buf in bufs:
-            buf.free()
+        sets = sets_for(nbytes)
+        slabs = [Slab(a, sets), Slab(b, sets), Slab(max(bA, bB) * m * n * 4, sets)]
+        if bias is not None:
+            slabs.append(Slab(bias, sets))
+        launch = lambda i: pyhost.device_fused_matmul(slabs[0][i], slabs[1][i], slabs[2][i], bA, bB, m, n, k, False,
+                                                      transpose_b, slabs[3][i] if bias is not None else None, [0, 0, 1],
+                                                      activation)
+        warm = time_launches(lib, check, ev, lambda: launch(0))
+        row(name, flops, nbytes, warm, time_launches_cold(lib, check, ev, launch, sets))
+        for slab in slabs:
+            slab.free()
 
     def conv(name, x, w, bias, strides, pad, activation, depthwise=False):
         ci = compute_conv2d_info(x.shape, w.shape, strides, 1, pad, None, depthwise)
         n_out = int(np.prod(ci["outShape"]))
-        bufs = [DeviceBuffer.from_numpy(x), DeviceBuffer.from_numpy(w), DeviceBuffer(n_out * 4),
-                DeviceBuffer.from_numpy(bias)]
+        nbytes = 4.0 * (x.size + w.size + bias.size + n_out)
+        sets = sets_for(nbytes)
+        slabs = [Slab(x, sets), Slab(w, sets), Slab(n_out * 4, sets), Slab(bias, sets)]
         geom = [ci["batchSize"], ci["inHeight"], ci["inWidth"], ci["inChannels"], ci["filterHeight"],
                 ci["filterWidth"], w.shape[3], ci["strideHeight"], ci["strideWidth"], 1, 1, ci["padInfo"]["top"],
                 ci["padInfo"]["left"], ci["outHeight"], ci["outWidth"]]
-        epi = [bufs[3].ptr, i64_array([0, 0, 0, 1]), ACTIVATIONS[activation], None, i64_array([0] * 4), 0.2]
+        epi = lambda i: [slabs[3][i].ptr, i64_array([0, 0, 0, 1]), ACTIVATIONS[activation], None, i64_array([0] * 4), 0.2]
         if depthwise:
-            fn = lambda: check(lib.tfhip_fused_depthwise_conv2d(bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, *geom, *epi))
+            launch = lambda i: check(lib.tfhip_fused_depthwise_conv2d(slabs[0][i].ptr, slabs[1][i].ptr, slabs[2][i].ptr,
+                                                                      *geom, *epi(i)))
             flops = 2.0 * n_out * w.shape[0] * w.shape[1]
         else:
-            fn = lambda: check(lib.tfhip_fused_conv2d(bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, *geom, 0, *epi))
+            launch = lambda i: check(lib.tfhip_fused_conv2d(slabs[0][i].ptr, slabs[1][i].ptr, slabs[2][i].ptr, *geom, 0,
+                                                            *epi(i)))
             flops = 2.0 * n_out * w.shape[0] * w.shape[1] * w.shape[2]
-        sec = time_launches(lib, check, ev, fn)
-        nbytes = 4.0 * (x.size + w.size + bias.size + n_out)
-        out.append(dict(config=name, kernel=last_kernel(lib), us=round(sec * 1e6, 2), flops=flops, bytes=nbytes,
-                        **roofline_entry(flops, nbytes, sec)))
-        for buf in bufs:
-            buf.free()
+        warm = time_launches(lib, check, ev, lambda: launch(0))
+        row(name, flops, nbytes, warm, time_launches_cold(lib, check, ev, launch, sets))
+        for slab in slabs:
+            slab.free()
 
     def dequant(name, n, kind):
         item = 1 if kind == "uint8" else 2
-        q = DeviceBuffer.from_numpy(np.random.default_rng(0).integers(0, 255, n * item, dtype=np.uint8))
-        o = DeviceBuffer(n * 4)
-        if kind == "float16":
-            fn = lambda: check(lib.tfhip_dequant_f16(q.ptr, n, o.ptr))
-        else:
-            fn = lambda: check(lib.tfhip_dequant_affine(q.ptr, item * 8, n, 0.0123, -1.5, o.ptr, 0))
-        sec = time_launches(lib, check, ev, fn)
         nbytes = float(n * (item + 4))
-        out.append(dict(config=name, kernel=last_kernel(lib), us=round(sec * 1e6, 2), flops=0.0, bytes=nbytes,
-                        **roofline_entry(0.0, nbytes, sec)))
+        sets = sets_for(nbytes)
+        q = Slab(np.random.default_rng(0).integers(0, 255, n * item, dtype=np.uint8), sets)
+        o = Slab(n * 4, sets)
+        if kind == "float16":
+            launch = lambda i: check(lib.tfhip_dequant_f16(q[i].ptr, n, o[i].ptr))
+        else:
+            launch = lambda i: check(lib.tfhip_dequant_affine(q[i].ptr, item * 8, n, 0.0123, -1.5, o[i].ptr, 0))
+        warm = time_launches(lib, check, ev, lambda: launch(0))
+        row(name, 0.0, nbytes, warm, time_launches_cold(lib, check, ev, launch, sets))
         q.free()
         o.free()
 
@@ -419,6 +491,25 @@ def main():
         workloads.write_graph_model(model_dir, workloads.mobilenet_v2_weights(seed=3), np.uint8)
         js = bench_model_node(model_dir, args.steps, args.warmup, args.jit_prime)
         m = bench_model(model_dir, args.steps, args.warmup)
+        b1 = unfused = None
+        if js:
+            # the two hosts must have planned the same launches, or the roofline below (measured through
+            # the Python host) would describe another program than the headline (measured through Node)
+            if js["plan_kernels"] != m["plan_kernels"]:
+                raise RuntimeError("the Node graph model and the Python mirror launch different kernels:\n node:   %s\n python: %s"
+                                   % (js["plan_kernels"], m["plan_kernels"]))
+            # batch 1, the reference's own benchmark setting: node by node, and as a recorded launch sequence
+            runs = [bench_model_node(model_dir, max(args.steps, 50), max(args.warmup, 10), args.jit_prime, batch=1, record=r)
+                    for r in (False, True)]
+            best = min(runs, key=lambda r: r["ms_per_step"])
+            b1 = dict(images_per_s=round(1e3 / best["ms_per_step"], 1), ms_per_step=round(best["ms_per_step"], 4),
+                      record_launches=best["record_launches"],
+                      ms_per_step_node_by_node=round(runs[0]["ms_per_step"], 4),
+                      ms_per_step_recorded=round(runs[1]["ms_per_step"], 4))
+            plain = bench_model_node(model_dir, args.steps, args.warmup, args.jit_prime,
+                                     options={"fuseResidualAdd": False, "fusePointwiseDepthwise": False})
+            unfused = dict(images_per_s=round(BATCH / (plain["ms_per_step"] * 1e-3), 1), ms_per_step=round(plain["ms_per_step"], 4),
+                           launches=len(plain["plan_kernels"]), launches_fused=len(js["plan_kernels"]))
         cpu = None if args.no_cpu_baseline else cpu_baseline(model_dir)
     finally:
         shutil.rmtree(model_dir, ignore_errors=True)
@@ -447,6 +538,9 @@ def main():
         "config": {"workload": "MobileNetV2 1.0/224, batch 32, NHWC fp32, uint8-quantized random-init weights "
                                "dequantized on load (benchmark configuration 4)", "batch": BATCH,
                    "jit_priming_batch1_inferences": js["prime"] if js else 0, "host": host, "device": info["arch"], "cus": info["cus"]},
+        "b1": b1,
+        "unfused_plan_images_per_s": unfused["images_per_s"] if unfused else None,
+        "unfused_plan": unfused,
         "weights_load_ms": round(js["load_ms"], 2) if js else None,
         "python_host_ms_per_step": round(m["ms_per_step"], 4),
         "kernel_ms_per_step": round(m["kernel_ms_per_step"], 4),

@@ -53,13 +53,29 @@ class OracleBackendCPU extends tf.KernelBackend {
     return Promise.resolve(this.readSync(dataId));
   }
   readSync(dataId) {
-    return this.data.get(dataId).values;
+    const entry = this.data.get(dataId);
+    if (entry.dtype === 'complex64' && entry.complexTensorInfos != null) {   // backend_cpu.ts:133-141
+      const real = this.readSync(entry.complexTensorInfos.real.dataId);
+      const imag = this.readSync(entry.complexTensorInfos.imag.dataId);
+      const merged = new Float32Array(real.length * 2);
+      for (let i = 0; i < real.length; i++) {
+        merged[2 * i] = real[i];
+        merged[2 * i + 1] = imag[i];
+      }
+      return merged;
+    }
+    return entry.values;
   }
   disposeData(dataId, force) {
     if (this.data.has(dataId)) {
       this.data.get(dataId).refCount--;
       if (!force && this.data.get(dataId).refCount > 0) {
         return false;
+      }
+      const parts = this.data.get(dataId).complexTensorInfos;   // backend_cpu.ts:183-188
+      if (parts != null) {
+        this.disposeData(parts.real.dataId, true);
+        this.disposeData(parts.imag.dataId, true);
       }
       this.data.delete(dataId);
     }
@@ -536,7 +552,28 @@ function transpose({inputs, backend, attrs}) {
   return backend.makeTensorInfo([cols, rows], x.dtype, out);
 }
 
+// ---- Complex.ts:22-44, Real.ts:22-35, Imag.ts: a complex64 tensor owns copies of its two parts ----
+function complex({inputs, backend}) {
+  const {real, imag} = inputs;
+  const info = backend.makeTensorInfo(real.shape, 'complex64', null);
+  backend.data.get(info.dataId).complexTensorInfos = {
+    real: backend.makeTensorInfo(real.shape, 'float32', vals(backend, real)),
+    imag: backend.makeTensorInfo(imag.shape, 'float32', vals(backend, imag))
+  };
+  return info;
+}
+
+function complexPart(part) {
+  return ({inputs, backend}) => {
+    const piece = backend.data.get(inputs.input.dataId).complexTensorInfos[part];
+    return backend.makeTensorInfo(piece.shape, piece.dtype, vals(backend, piece));
+  };
+}
+
 const kernelFuncs = {
+  Complex: complex,
+  Real: complexPart('real'),
+  Imag: complexPart('imag'),
   BatchMatMul: batchMatMul,
   _FusedMatMul: fusedMatMul,
   Conv2D: conv2D,

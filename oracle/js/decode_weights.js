@@ -1,7 +1,7 @@
 'use strict';
 /**
  * JavaScript restatement of decodeWeights / decodeWeight and the float16
- * decoder (tfjs-core/src/io/io_utils.ts:119-292, :645-741) for numeric dtypes.
+ * decoder (tfjs-core/src/io/io_utils.ts:119-292, :645-741).
  * TEST INFRASTRUCTURE: the bit-exact checker of the GPU dequantize-on-load path
  * on the JavaScript side, and part of what the cpu_baseline leg times.
  */
@@ -133,13 +133,33 @@ function decodeWeightValues(spec, byteBuffer) {
   return values;
 }
 
-/** Returns {name: TypedArray}; `toTensors` wraps them as tensors of the active backend. */
+/**
+ * Returns {name: TypedArray}; `toTensors` wraps them as tensors of the active backend. A string entry
+ * gives an array of Uint8Array (io_utils.ts:252-264: a uint32 byte count in front of every element), a
+ * complex64 entry its interleaved (real, imaginary) float32 pairs (io_utils.ts:273-286 splits them).
+ */
 function decodeWeightsToArrays(weightData, specs) {
   const bytes = new Uint8Array(weightData);
   const out = {};
   let offset = 0;
   specs.forEach(spec => {
     const size = tf.util.sizeFromShape(spec.shape);
+    if (spec.dtype === 'string' && !('quantization' in spec)) {
+      const values = [];
+      for (let i = 0; i < size; i++) {
+        const byteLength = new Uint32Array(bytes.slice(offset, offset + 4).buffer)[0];
+        offset += 4;
+        values.push(bytes.slice(offset, offset + byteLength));
+        offset += byteLength;
+      }
+      out[spec.name] = values;
+      return;
+    }
+    if (spec.dtype === 'complex64' && !('quantization' in spec)) {
+      out[spec.name] = new Float32Array(bytes.slice(offset, offset + size * 8).buffer);
+      offset += size * 8;
+      return;
+    }
     const per = 'quantization' in spec ? DTYPE_VALUE_SIZE_MAP[spec.quantization.dtype] : DTYPE_VALUE_SIZE_MAP[spec.dtype];
     // CompositeArrayBuffer.slice copies, so uint16 data is aligned (io_utils.ts:128-131)
     const slice = bytes.slice(offset, offset + size * per).buffer;
@@ -153,7 +173,22 @@ function decodeWeights(weightData, specs) {
   const arrays = decodeWeightsToArrays(weightData, specs);
   const out = {};
   specs.forEach(spec => {
-    out[spec.name] = tf.tensor(arrays[spec.name], spec.shape, spec.dtype);
+    if (spec.dtype === 'string') {
+      out[spec.name] = tf.engine().makeTensor(arrays[spec.name], spec.shape, 'string');
+    } else if (spec.dtype === 'complex64' && !('quantization' in spec)) {
+      const pairs = arrays[spec.name], n = pairs.length / 2;
+      const real = new Float32Array(n), imag = new Float32Array(n);
+      for (let i = 0; i < n; i++) {
+        real[i] = pairs[2 * i];
+        imag[i] = pairs[2 * i + 1];
+      }
+      const realTensor = tf.tensor(real, spec.shape, 'float32'), imagTensor = tf.tensor(imag, spec.shape, 'float32');
+      out[spec.name] = tf.complex(realTensor, imagTensor);
+      realTensor.dispose();
+      imagTensor.dispose();
+    } else {
+      out[spec.name] = tf.tensor(arrays[spec.name], spec.shape, spec.dtype);
+    }
   });
   return out;
 }

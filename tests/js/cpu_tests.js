@@ -313,6 +313,26 @@ h.test('hip decodeWeights: reference error messages, plain entries pass through'
   h.assertThrows(() => hip.decodeWeights(new ArrayBuffer(0), []), /needs the 'hip' backend to be active/);
 });
 
+const {referenceStringAndComplexShard, checkStringAndComplexWeights} = require('./string_complex_weights')(tf, h);
+
+h.test('decodeWeights: string and complex64 entries in the layout of io_utils_test.ts, oracle and hip decoders', () => {
+  const {shard, specs, strings} = referenceStringAndComplexShard();
+  useBackend('cpu');
+  const before = tf.memory().numTensors;
+  let out = oracleDecode.decodeWeights(shard, specs);
+  checkStringAndComplexWeights(tf.tidy(() => { checkStringAndComplexWeights(out, strings); return out; }), strings);
+  tf.dispose(out);
+  useBackend('hip');
+  out = hip.decodeWeights(shard, specs);
+  tf.tidy(() => checkStringAndComplexWeights(out, strings));
+  const ids = tf.backend().numDataIds();
+  tf.dispose(out);
+  h.assertEqual(tf.backend().numDataIds(), ids - 9 - 6);   // nine tensors, and the two parts of each complex one
+  h.assertThrows(() => hip.decodeWeights(shard.slice(0, 30), specs), /ends inside string weight 'x3'/);
+  useBackend('cpu');
+  h.assert(tf.memory().numTensors >= before);
+});
+
 // ---- graph model stand-in over the JavaScript oracle backend ------------------------
 const b64 = t => Buffer.from(t).toString('base64');
 function tinyGraphArtifacts() {

@@ -79,7 +79,11 @@ module.exports = {
   fusedConv2DDepthwise() { record('fusedConv2DDepthwise', arguments); },
   conv2dDepthwisePays(batch) { return module.exports.paysFromBatch != null && batch >= module.exports.paysFromBatch; },
   paysFromBatch: null,   // tests set the batch size from which the fused kernel "pays"
-  copy() { record('copy', arguments); },
+  copy(dst, src, bytes) {   // data movement, like upload and download: carried out (within the blocks' sizes)
+    record('copy', arguments);
+    const to = need(dst), from = need(src);
+    to.set(from.subarray(0, Math.min(bytes, from.byteLength, to.byteLength)));
+  },
   captureBegin() { record('captureBegin', arguments); },
   captureEnd(keep) { record('captureEnd', arguments); return {id: keep ? 1 : 0, nodes: 0}; },
   graphLaunch() { record('graphLaunch', arguments); },

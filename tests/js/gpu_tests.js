@@ -189,6 +189,17 @@ h.test('decodeWeights on the GPU is bit-identical to the JavaScript decoder (uin
   });
 });
 
+h.test('decodeWeights: string and complex64 entries in the layout of io_utils_test.ts', () => {
+  const cases = require('./string_complex_weights')(tf, h);
+  const {shard, specs, strings} = cases.referenceStringAndComplexShard();
+  h.assert(tf.engine().setBackend('hip') === true, 'setBackend(hip)');
+  const ids = tf.backend().numDataIds();
+  const out = hip.decodeWeights(shard, specs);
+  tf.tidy(() => cases.checkStringAndComplexWeights(out, strings));
+  tf.dispose(out);
+  h.assertEqual(tf.backend().numDataIds(), ids);
+});
+
 h.test('float16 decode: all 65536 bit patterns', () => {
   const all = new Uint16Array(65536);
   for (let i = 0; i < 65536; i++) {

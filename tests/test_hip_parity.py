@@ -581,6 +581,38 @@ def test_dequant_large_bit_exact(hip, orc, kind):
         assert np.abs(got - data).max() <= meta["scale"] * 0.5001
 
 
+@pytest.mark.parametrize("bits,to_int", [(8, 0), (8, 1), (16, 0), (16, 1), ("f16", 0)])
+def test_dequant_every_source_offset_and_ragged_length(hip, orc, bits, to_int):
+    """Through the C ABI at every byte offset of the codes inside a 16-byte line and lengths that leave a
+    head before and a tail after the stretch the 16-byte kernel takes, including lengths shorter than
+    the head: bit-exact, and nothing is written past the last element."""
+    from tfjs_amd import capi
+    lib = capi.load_library()
+    bytes_per = 1 if bits == 8 else 2
+    rng = np.random.default_rng(21)
+    scale, min_ = 0.0123, -1.5
+    for offset in range(0, 18):
+        for n in (1, 3, 5, 15, 16, 17, 63, 64, 65, 1000, 4099, 70001):
+            if bytes_per == 2:
+                codes = rng.integers(0, 65536, n).astype(np.uint16)
+            else:
+                codes = rng.integers(0, 256, n).astype(np.uint8)
+            spec = [{"name": "w", "dtype": "int32" if to_int else "float32", "shape": [n],
+                     "quantization": {"dtype": "float16"} if bits == "f16" else
+                     {"dtype": "uint%d" % bits, "scale": scale, "min": min_}}]
+            want = orc.decode_weights(codes.tobytes(), spec)["w"].view(np.uint32)
+            with capi.DeviceBuffer(offset + n * bytes_per + 64) as src, capi.DeviceBuffer((n + 8) * 4) as dst:
+                src.upload(np.frombuffer(codes.tobytes(), np.uint8), offset)
+                dst.upload(np.full(n + 8, 0xdeadbeef, np.uint32))
+                if bits == "f16":
+                    capi.check(lib.tfhip_dequant_f16(src.ptr + offset, n, dst.ptr))
+                else:
+                    capi.check(lib.tfhip_dequant_affine(src.ptr + offset, bits, n, scale, min_, dst.ptr, to_int))
+                got = dst.download(np.uint32, n + 8)
+            np.testing.assert_array_equal(got[:n], want, err_msg="offset %d n %d" % (offset, n))
+            assert (got[n:] == 0xdeadbeef).all(), "offset %d n %d wrote past the end" % (offset, n)
+
+
 def test_decode_weights_errors(hip):
     with pytest.raises(ValueError, match="doesn't have corresponding metadata min and scale"):
         hip.decode_weights(b"\0", [{"name": "w", "dtype": "float32", "shape": [1],

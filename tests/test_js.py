@@ -128,3 +128,59 @@ def test_node_gpu_tier(tmp_path):
     proc = run_node("tests/js/gpu_tests.js", env={"TFJS_HIP_TEST_MODEL_DIR": str(tmp_path)})
     assert proc.returncode == 0, proc.stdout[-4000:]
     assert " 0 failed" in proc.stdout
+
+
+@pytest.mark.gpu
+@needs_node
+def test_graph_model_predict_batch32_matches_the_c_oracle(tmp_path):
+    """The headline's own path, end to end: a converter-format MobileNetV2 (uint8 weights, dequantized on
+    the GPU at load) through loadGraphModel + GraphModel.predict in Node at batch 32, against the C oracle
+    run layer by layer on the same decoded weights and the same input. Tolerance: the float32 bound of the
+    build, |got - want| <= 1e-3 * max(1, |want|) on every logit (tfjs's float32 test epsilon); the
+    observed error is about 2e-5."""
+    from oracle import pyoracle as orc
+    from tfjs_amd import workloads
+    model_dir = tmp_path / "model"
+    model_dir.mkdir()
+    workloads.write_graph_model(str(model_dir), workloads.mobilenet_v2_weights(seed=3), np.uint8)
+    buf, specs = workloads.read_model(str(model_dir))
+    decoded = orc.decode_weights(buf, specs)
+    x = workloads.mobilenet_v2_input(32)
+    ops, _ = workloads.mobilenet_v2_graph()
+    want = workloads.run_graph(orc, ops, decoded, x)
+    x.astype("<f4").tofile(str(tmp_path / "x.bin"))
+    script = """
+      const fs = require('fs');
+      const hip = require('%s/tfjs_amd/js/index');
+      const tf = hip.tf;
+      (async () => {
+        await tf.setBackend('hip');
+        const raw = fs.readFileSync(process.argv[3]);
+        const x = tf.tensor(new Float32Array(raw.buffer, raw.byteOffset, raw.length / 4), [32, 224, 224, 3]);
+        const out = {};
+        for (const record of [false, true]) {
+          const model = hip.loadGraphModel(process.argv[2], {recordLaunches: record}, {decodeWeights: hip.decodeWeights});
+          let y = null;
+          for (let i = 0; i < 3; i++) {     // the third call of the recording model is a replay
+            if (y) y.dispose();
+            y = model.predict(x);
+          }
+          out[record ? 'recorded' : 'plain'] = Array.from(y.dataSync());
+          out.shape = y.shape;
+          y.dispose();
+          model.dispose();
+        }
+        fs.writeFileSync(process.argv[4], JSON.stringify(out));
+      })().catch(e => { console.error(e.stack); process.exit(1); });
+    """ % ROOT
+    (tmp_path / "run.js").write_text(script)
+    proc = subprocess.run([NODE, str(tmp_path / "run.js"), str(model_dir), str(tmp_path / "x.bin"), str(tmp_path / "out.json")],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stdout[-3000:]
+    got = json.loads((tmp_path / "out.json").read_text())
+    assert got["shape"] == list(want.shape)
+    plain = np.array(got["plain"], dtype=np.float32).reshape(want.shape)
+    err = np.abs(plain.astype(np.float64) - want) / np.maximum(1.0, np.abs(want))
+    assert err.max() <= 1e-3, err.max()
+    # a replay runs the recorded kernels on the same operands: the same bits
+    np.testing.assert_array_equal(np.array(got["recorded"], dtype=np.float32).reshape(want.shape), plain)

@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void conv_few_channels(FewChannelsArgs g) {
         if (g.activation == TFHIP_RELU6 && q[k] > 6.f) q[k] = 6.f;
       }
     }
-    *reinterpret_cast<float4 *>(y + o) = make_float4(q[0], q[1], q[2], q[3]);
+    store_result4(y + o, make_float4(q[0], q[1], q[2], q[3]));
   }
 }
 

@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256) void depthwise_3x3_halo(DwParams p, Epilogue e
     o.y = finish(e, acc.y, 0, 0, c + 1, n, oh, ow);
     o.z = finish(e, acc.z, 0, 0, c + 2, n, oh, ow);
     o.w = finish(e, acc.w, 0, 0, c + 3, n, oh, ow);
-    y4[(((long long)n * p.out_h + oh) * p.out_w + ow) * c4_total + cq0 + c4] = o;
+    store_result4(reinterpret_cast<float *>(y4 + (((long long)n * p.out_h + oh) * p.out_w + ow) * c4_total + cq0 + c4), o);
   }
 }
 
@@ -182,7 +182,7 @@ __device__ __forceinline__ float4 dw_load4(__amdgpu_buffer_rsrc_t r, unsigned of
 __device__ __forceinline__ void dw_store4(__amdgpu_buffer_rsrc_t r, unsigned off, float4 v) {
   dw_uint4 u;
   u.x = __float_as_uint(v.x); u.y = __float_as_uint(v.y); u.z = __float_as_uint(v.z); u.w = __float_as_uint(v.w);
-  __builtin_amdgcn_raw_buffer_store_b128(u, r, (int)off, 0, 0);
+  __builtin_amdgcn_raw_buffer_store_b128(u, r, (int)off, 0, TFHIP_NT_OUT ? 2 : 0);
 }
 
 // Bias + activation of four channels. The common case (per-channel operands,

@@ -104,6 +104,21 @@ __device__ __forceinline__ float finish(const Epilogue &e, float v, long long ba
   return activate(v, e.activation, alpha, e.leaky_alpha);
 }
 
+// The float4 store every kernel writes its results with. TFHIP_NT_OUT (a build-time switch for
+// measurement) makes it a streaming store.
+#ifndef TFHIP_NT_OUT
+#define TFHIP_NT_OUT 0
+#endif
+__device__ __forceinline__ void store_result4(float *p, float4 v) {
+#if TFHIP_NT_OUT
+  typedef float result4_t __attribute__((ext_vector_type(4)));
+  const result4_t t = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(t, reinterpret_cast<result4_t *>(p));
+#else
+  *reinterpret_cast<float4 *>(p) = v;
+#endif
+}
+
 // Workgroup barrier that orders LDS traffic only. __syncthreads() also fences
 // global memory, which makes every wave wait for all of its outstanding global
 // loads (vmcnt(0)) at each barrier and so drains the prefetch ring once per k

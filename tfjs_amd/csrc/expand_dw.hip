@@ -293,7 +293,7 @@ __global__ __launch_bounds__(256) void expand_dw_3x3(ExpandDwArgs g, StemTaps ta
         out.y = relu_like<ACT>(acc.y + b2q.y);
         out.z = relu_like<ACT>(acc.z + b2q.z);
         out.w = relu_like<ACT>(acc.w + b2q.w);
-        *reinterpret_cast<float4 *>(g.y + (((long long)n * g.out_h + oh) * g.out_w + ow0 + q) * g.c + 4 * c4) = out;
+        store_result4(g.y + (((long long)n * g.out_h + oh) * g.out_w + ow0 + q) * g.c + 4 * c4, out);
       }
     }
     if (more) expand_rows(first, S, new_slot);

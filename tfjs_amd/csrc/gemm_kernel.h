@@ -555,7 +555,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
             const float4 r4 = *reinterpret_cast<const float4 *>(R + base + col);
             out[0] += r4.x; out[1] += r4.y; out[2] += r4.z; out[3] += r4.w;
           }
-          *reinterpret_cast<float4 *>(C + base + col) = make_float4(out[0], out[1], out[2], out[3]);
+          store_result4(C + base + col, make_float4(out[0], out[1], out[2], out[3]));
         } else {
 #pragma unroll
           for (int q = 0; q < 4; ++q) {

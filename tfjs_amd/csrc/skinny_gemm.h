@@ -175,7 +175,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
             const float4 r4 = *reinterpret_cast<const float4 *>(g.residual + (long long)row * g.N + col);
             out[0] += r4.x; out[1] += r4.y; out[2] += r4.z; out[3] += r4.w;
           }
-          *reinterpret_cast<float4 *>(g.c + (long long)row * g.N + col) = make_float4(out[0], out[1], out[2], out[3]);
+          store_result4(g.c + (long long)row * g.N + col, make_float4(out[0], out[1], out[2], out[3]));
         }
 #pragma unroll
         for (int h = 0; h < NA; ++h) acc[h][n] = (float4_t){0.f, 0.f, 0.f, 0.f};
@@ -289,7 +289,7 @@ __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
         out[k] = v;
       }
       if (row < g.M && col < g.N)
-        *reinterpret_cast<float4 *>(g.c + (long long)row * g.N + col) = make_float4(out[0], out[1], out[2], out[3]);
+        store_result4(g.c + (long long)row * g.N + col, make_float4(out[0], out[1], out[2], out[3]));
     }
     cur = nxt;
   }

@@ -184,7 +184,7 @@ __global__ __launch_bounds__(256) void small_k_gemm(SmallKArgs g) {
         }
         out[q] = v;
       }
-      *reinterpret_cast<float4 *>(C + (long long)row * g.N + col) = make_float4(out[0], out[1], out[2], out[3]);
+      store_result4(C + (long long)row * g.N + col, make_float4(out[0], out[1], out[2], out[3]));
     }
   }
 }

@@ -165,6 +165,16 @@ class HipBackend extends tf.KernelBackend {
   /** Device buffer of `size` elements of `dtype`; registers a new dataId. */
   allocate(shape, dtype, dataId) {
     const size = tf.util.sizeFromShape(shape);
+    if (dtype === 'string' || dtype === 'complex64') {
+      // Neither has a device buffer of its own. A string tensor's values (one Uint8Array per
+      // element) stay on the host, as in every backend of the reference; a complex64 tensor owns
+      // two float32 tensors, its real and imaginary parts (tfjs-backend-cpu/src/backend_cpu.ts:28-31),
+      // attached by the Complex kernel.
+      dataId = dataId || this.nextDataId();
+      this.data.set(dataId, {ptr: null, bytes: 0, dtype, shape: shape.slice(), refCount: 1, values: null,
+                             complexTensorInfos: null});
+      return dataId;
+    }
     if (!(dtype in BYTES)) {
       throw new Error(`tfjs-backend-hip does not support dtype ${dtype}`);
     }
@@ -185,6 +195,24 @@ class HipBackend extends tf.KernelBackend {
 
   uploadValues(dataId, values) {
     const info = this.data.get(dataId);
+    if (info.dtype === 'string') {
+      info.values = values;
+      return;
+    }
+    if (info.dtype === 'complex64') {
+      // interleaved (real, imaginary) pairs, the layout readSync returns
+      const n = values.length / 2;
+      const real = new Float32Array(n), imag = new Float32Array(n);
+      for (let i = 0; i < n; i++) {
+        real[i] = values[2 * i];
+        imag[i] = values[2 * i + 1];
+      }
+      info.complexTensorInfos = {
+        real: {dataId: this.write(real, info.shape, 'float32'), shape: info.shape, dtype: 'float32'},
+        imag: {dataId: this.write(imag, info.shape, 'float32'), shape: info.shape, dtype: 'float32'}
+      };
+      return;
+    }
     let typed = values;
     if (!ArrayBuffer.isView(values) ||
         values.BYTES_PER_ELEMENT !== BYTES[info.dtype] ||
@@ -218,7 +246,12 @@ class HipBackend extends tf.KernelBackend {
   }
 
   ptr(dataId) {
-    return this.data.get(dataId).ptr;
+    const info = this.data.get(dataId);
+    if (info.ptr == null) {
+      throw new Error(`tfjs-backend-hip: a ${info.dtype} tensor has no device buffer of its own; ` +
+                      `this kernel takes float32, int32 or bool tensors`);
+    }
+    return info.ptr;
   }
 
   refCount(dataId) {
@@ -244,6 +277,19 @@ class HipBackend extends tf.KernelBackend {
 
   readSync(dataId) {
     const info = this.data.get(dataId);
+    if (info.dtype === 'string') {
+      return info.values;
+    }
+    if (info.dtype === 'complex64') {
+      const real = this.readSync(info.complexTensorInfos.real.dataId);
+      const imag = this.readSync(info.complexTensorInfos.imag.dataId);
+      const merged = new Float32Array(real.length * 2);
+      for (let i = 0; i < real.length; i++) {
+        merged[2 * i] = real[i];
+        merged[2 * i + 1] = imag[i];
+      }
+      return merged;
+    }
     const out = typedArrayFor(info.dtype, info.bytes / BYTES[info.dtype]);
     if (info.bytes > 0) {
       addon.download(info.ptr, 0, out);
@@ -262,7 +308,13 @@ class HipBackend extends tf.KernelBackend {
       if (!force && info.refCount > 0) {
         return false;
       }
-      this.release(info.ptr, Math.max(info.bytes, 1));
+      if (info.complexTensorInfos != null) {
+        this.disposeData(info.complexTensorInfos.real.dataId, true);
+        this.disposeData(info.complexTensorInfos.imag.dataId, true);
+      }
+      if (info.ptr != null) {
+        this.release(info.ptr, Math.max(info.bytes, 1));
+      }
       this.data.delete(dataId);
     }
     return true;

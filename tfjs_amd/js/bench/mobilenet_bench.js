@@ -2,14 +2,18 @@
 /**
  * MobileNetV2 through the tfjs API on the hip backend, timed the reference's way
  * (predict plus download of the result, e2e/benchmarks/benchmark_util.js:246-286).
- *   node tfjs_amd/js/bench/mobilenet_bench.js MODEL_DIR BATCH STEPS WARMUP [PRIME [RECORD]]
+ *   node tfjs_amd/js/bench/mobilenet_bench.js MODEL_DIR BATCH STEPS WARMUP [PRIME [RECORD [OPTIONS]]]
  * PRIME (default 0) batch-1 inferences run first, outside warm-up and timing, so
  * that V8 has compiled the host path before a short measurement starts. RECORD 1
  * loads the graph model with {recordLaunches: true}: the kernels of an inference
- * are recorded into a HIP graph once and replayed from then on.
+ * are recorded into a HIP graph once and replayed from then on. OPTIONS is a JSON
+ * object of further load options of the graph model, e.g.
+ * {"fuseResidualAdd":false,"fusePointwiseDepthwise":false} for the plan without the
+ * cross-node fusions.
  * Prints one JSON line: ms_per_step (wall clock around STEPS steps, stream
  * drained on both sides), load_ms (read + upload + GPU dequant of the weights),
- * kernel_ms_per_step (device time between two events around the same steps).
+ * device_ms_per_step (device time between two events around the same steps),
+ * plan_kernels (the kernel symbol each launching node of one inference chose, in order).
  */
 const fs = require('fs');
 const path = require('path');
@@ -26,15 +30,16 @@ async function main() {
   const warmup = parseInt(process.argv[5] || '5', 10);
   const prime = parseInt(process.argv[6] || '0', 10);
   const record = parseInt(process.argv[7] || '0', 10) === 1;
+  const options = Object.assign({}, JSON.parse(process.argv[8] || '{}'), {recordLaunches: record});
   await tf.setBackend('hip');
   const t0 = tf.util.now();
   // A converter-format model.json runs as a graph model (model.predict, what a
   // tfjs user of a converted network calls); a bare weights manifest through the
   // same ops called directly.
   const asGraph = fs.existsSync(path.join(modelDir, 'model.json'));
-  let predict;
+  let predict, graph = null;
   if (asGraph) {
-    const graph = hip.loadGraphModel(modelDir, {recordLaunches: record}, {decodeWeights: hip.decodeWeights});
+    graph = hip.loadGraphModel(modelDir, options, {decodeWeights: hip.decodeWeights});
     predict = x => graph.predict(x);
   } else {
     const m = model.readModel(modelDir);
@@ -75,6 +80,22 @@ async function main() {
   const wallMs = tf.util.now() - start;
   addon.eventRecord(1);
   const deviceMs = addon.eventElapsed(0, 1);
+  // One more inference, node by node, asking the library after every node which kernel it chose.
+  // Nodes that launch nothing (Reshape, Squeeze, Identity share their input's buffer) are left out.
+  let planKernels = null;
+  if (graph != null) {
+    const probe = hip.loadGraphModel(modelDir, Object.assign({}, options, {recordLaunches: false}),
+                                     {decodeWeights: hip.decodeWeights});
+    planKernels = [];
+    probe.afterNode = (step, node) => {
+      if (node == null || ['Reshape', 'Squeeze', 'Identity'].indexOf(node.op) < 0) {
+        planKernels.push(addon.lastKernel());
+      }
+    };
+    probe.predict(x).dispose();
+    probe.dispose();
+    addon.sync();
+  }
   const mem = tf.memory();
   console.log(JSON.stringify({
     ms_per_step: wallMs / steps,
@@ -85,6 +106,8 @@ async function main() {
     warmup,
     prime,
     record_launches: record && asGraph,
+    options,
+    plan_kernels: planKernels,
     checksum,
     node: process.version,
     core: tf.usingStandin ? 'standin' : '@tensorflow/tfjs-core',

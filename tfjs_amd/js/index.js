@@ -22,7 +22,8 @@ const kernelConfigs = [
   conv.fusedConv2DAddConfig, conv.fusedPointwiseDepthwiseConfig, conv.conv2DConfig, conv.fusedDepthwiseConv2DConfig,
   conv.depthwiseConv2dNativeConfig, glue.addConfig, glue.subConfig, glue.multiplyConfig, glue.reluConfig,
   glue.relu6Config, glue.eluConfig, glue.sigmoidConfig, glue.leakyReluConfig, glue.meanConfig, glue.avgPoolConfig,
-  glue.castConfig, glue.transposeConfig, glue.reshapeConfig, glue.identityConfig, glue.copyConfig
+  glue.castConfig, glue.transposeConfig, glue.reshapeConfig, glue.identityConfig, glue.copyConfig,
+  glue.complexConfig, glue.realConfig, glue.imagConfig
 ];
 
 tf.registerBackend('hip', () => new HipBackend(), 3 /* priority */);

@@ -3,9 +3,10 @@
  * decodeWeights with the dequantize step on the GPU.
  *
  * Same signature and results as tfjs-core's decodeWeights
- * (tfjs-core/src/io/io_utils.ts:119-135 over decodeWeight :185-292) for the
- * numeric dtypes: (weightData: ArrayBuffer | ArrayBuffer[], specs:
- * WeightsManifestEntry[]) => NamedTensorMap. Where the reference expands
+ * (tfjs-core/src/io/io_utils.ts:119-135 over decodeWeight :185-292), every
+ * dtype of a weights manifest included (float32, int32, bool, complex64, string):
+ * (weightData: ArrayBuffer | ArrayBuffer[], specs: WeightsManifestEntry[]) =>
+ * NamedTensorMap. Where the reference expands
  * uint8 / uint16 / float16 entries in a JavaScript loop and then uploads
  * float32, this uploads the quantized bytes once and expands every quantized
  * entry with one kernel reading at its byte offset; the tensors it returns are
@@ -74,10 +75,34 @@ function validate(spec) {
     }
     return DTYPE_VALUE_SIZE_MAP[quantization.dtype];
   }
-  if (dtype !== 'float32' && dtype !== 'int32' && dtype !== 'bool') {
+  if (dtype === 'string') {
+    return null;   // length-prefixed elements: the byte length is found by walking them
+  }
+  if (dtype !== 'float32' && dtype !== 'int32' && dtype !== 'bool' && dtype !== 'complex64') {
     throw new Error(`Unsupported dtype in weight '${name}': ${dtype}`);
   }
   return DTYPE_VALUE_SIZE_MAP[dtype];
+}
+
+/** Each element of a string weight: a little-endian uint32 byte count, then the bytes (io_utils.ts:252-264). */
+const NUM_BYTES_STRING_LENGTH = 4;
+
+function readStrings(bytes, offset, count, name) {
+  const values = [];
+  const view = new DataView(bytes.buffer, bytes.byteOffset, bytes.byteLength);
+  for (let i = 0; i < count; i++) {
+    if (offset + NUM_BYTES_STRING_LENGTH > bytes.byteLength) {
+      throw new Error(`decodeWeights: the weight data ends inside string weight '${name}'`);
+    }
+    const byteLength = view.getUint32(offset, true);
+    offset += NUM_BYTES_STRING_LENGTH;
+    if (offset + byteLength > bytes.byteLength) {
+      throw new Error(`decodeWeights: the weight data ends inside string weight '${name}'`);
+    }
+    values.push(bytes.slice(offset, offset + byteLength));
+    offset += byteLength;
+  }
+  return {values, end: offset};
 }
 
 function decodeWeights(weightData, specs) {
@@ -93,7 +118,14 @@ function decodeWeights(weightData, specs) {
   let anyQuantized = false;
   specs.forEach(spec => {
     const size = tf.util.sizeFromShape(spec.shape);
-    const byteLength = size * validate(spec);
+    const elementBytes = validate(spec);
+    if (elementBytes == null) {
+      const strings = readStrings(bytes, offset, size, spec.name);
+      plan.push({spec, size, offset, byteLength: strings.end - offset, strings: strings.values});
+      offset = strings.end;
+      return;
+    }
+    const byteLength = size * elementBytes;
     plan.push({spec, size, offset, byteLength});
     anyQuantized = anyQuantized || 'quantization' in spec;
     offset += byteLength;
@@ -125,6 +157,21 @@ function decodeWeights(weightData, specs) {
           }
         }
         out[spec.name] = tf.engine().makeTensorFromTensorInfo(info, backend);
+      } else if (p.strings != null) {
+        out[spec.name] = tf.engine().makeTensor(p.strings, spec.shape, 'string', backend);
+      } else if (spec.dtype === 'complex64') {
+        // interleaved (real, imaginary) float32 pairs become the two parts of tf.complex (io_utils.ts:273-286)
+        const pairs = new Float32Array(bytes.slice(p.offset, p.offset + p.byteLength).buffer);
+        const real = new Float32Array(p.size), imag = new Float32Array(p.size);
+        for (let i = 0; i < p.size; i++) {
+          real[i] = pairs[2 * i];
+          imag[i] = pairs[2 * i + 1];
+        }
+        const realTensor = tf.engine().makeTensor(real, spec.shape, 'float32', backend);
+        const imagTensor = tf.engine().makeTensor(imag, spec.shape, 'float32', backend);
+        out[spec.name] = tf.complex(realTensor, imagTensor);
+        realTensor.dispose();
+        imagTensor.dispose();
       } else {
         // plain entry: copy out of the (possibly unaligned) byte stream
         const slice = bytes.slice(p.offset, p.offset + p.byteLength);

@@ -6,7 +6,8 @@
  * Elu.ts, Sigmoid.ts, LeakyRelu.ts), Mean over the two spatial axes (Mean.ts:26-56
  * over Sum.ts:30-92), AvgPool (AvgPool.ts:25-58), Cast (Cast.ts:48-88), the rank-2
  * Transpose (Transpose.ts), and the aliasing Reshape / Identity (Reshape.ts:24-52,
- * Identity.ts:22-30), which share the input's buffer and bump its refCount.
+ * Identity.ts:22-30), which share the input's buffer and bump its refCount, and
+ * Complex / Real / Imag, which is all a complex64 weight needs to load.
  * HipCopy (no counterpart in the reference) duplicates a tensor on the device:
  * what moves inputs into and results out of the fixed buffers of a recorded
  * launch sequence.
@@ -201,6 +202,33 @@ function identity(args) {
   return {dataId: x.dataId, shape: x.shape, dtype: x.dtype};
 }
 
+/**
+ * Complex (tfjs-backend-cpu/src/kernels/Complex.ts:22-44): a complex64 tensor that owns copies of its
+ * two float32 parts; Real / Imag (Real.ts:22-35, Imag.ts) hand back a copy of one part, which outlives
+ * the complex tensor.
+ */
+function complex(args) {
+  const {real, imag} = args.inputs;
+  const backend = args.backend;
+  requireFloat32([real, imag], 'Complex');
+  tf.util.assert(tf.util.arraysEqual(real.shape, imag.shape),
+                 () => `real and imag shapes, ${real.shape} and ${imag.shape}, must match in call to tf.complex().`);
+  const out = backend.makeOutput(real.shape, 'complex64');
+  backend.data.get(out.dataId).complexTensorInfos = {real: copy({inputs: {x: real}, backend}), imag: copy({inputs: {x: imag}, backend})};
+  return out;
+}
+
+function complexPart(part) {
+  return args => {
+    const {input} = args.inputs;
+    const info = args.backend.data.get(input.dataId);
+    if (info.complexTensorInfos == null) {
+      throw new Error(`${part === 'real' ? 'Real' : 'Imag'}: the input is not a complex64 tensor (got ${input.dtype})`);
+    }
+    return copy({inputs: {x: info.complexTensorInfos[part]}, backend: args.backend});
+  };
+}
+
 /** A copy of x in a buffer of its own (device to device). */
 function copy(args) {
   const {x} = args.inputs;
@@ -224,5 +252,8 @@ module.exports = {
   transposeConfig: {kernelName: 'Transpose', backendName: 'hip', kernelFunc: transpose},
   meanConfig: {kernelName: 'Mean', backendName: 'hip', kernelFunc: mean},
   reshapeConfig: {kernelName: 'Reshape', backendName: 'hip', kernelFunc: reshape},
-  identityConfig: {kernelName: 'Identity', backendName: 'hip', kernelFunc: identity}
+  identityConfig: {kernelName: 'Identity', backendName: 'hip', kernelFunc: identity},
+  complexConfig: {kernelName: 'Complex', backendName: 'hip', kernelFunc: complex},
+  realConfig: {kernelName: 'Real', backendName: 'hip', kernelFunc: complexPart('real')},
+  imagConfig: {kernelName: 'Imag', backendName: 'hip', kernelFunc: complexPart('imag')}
 };

@@ -623,6 +623,9 @@ class GraphModel {
             this.compiled[key] = run;
           }
           const out = values[name] = run(args);
+          if (this.afterNode != null) {
+            this.afterNode(step, this.nodes[name]);   // a caller's probe: which step just ran
+          }
           // intermediates that nobody reads again can go now
           for (let i = 0; i < step.release.length; i++) {
             const src = step.release[i];

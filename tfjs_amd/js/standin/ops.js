@@ -423,6 +423,23 @@ function depthwiseConv2d(x, filter, strides, pad, dataFormat, dilations, dimRoun
   });
 }
 
+/** tfjs-core/src/ops/complex.ts, real.ts, imag.ts */
+function complex(real, imag) {
+  const $real = convertToTensor(real, 'real', 'complex');
+  const $imag = convertToTensor(imag, 'imag', 'complex');
+  util.assert(util.arraysEqual($real.shape, $imag.shape),
+              () => `real and imag shapes, ${$real.shape} and ${$imag.shape}, must match in call to tf.complex().`);
+  return ENGINE.runKernel('Complex', {real: $real, imag: $imag});
+}
+
+function real(input) {
+  return ENGINE.runKernel('Real', {input: convertToTensor(input, 'input', 'real')});
+}
+
+function imag(input) {
+  return ENGINE.runKernel('Imag', {input: convertToTensor(input, 'input', 'imag')});
+}
+
 /** new tensor of one value (tfjs-core/src/ops/{zeros,ones,fill}.ts) */
 function fill(shape, value, dtype) {
   dtype = dtype || 'float32';
@@ -468,6 +485,9 @@ module.exports = {
   elu: unaryOp('Elu', 'elu'),
   sigmoid: unaryOp('Sigmoid', 'sigmoid'),
   leakyRelu,
+  complex,
+  real,
+  imag,
   cast,
   avgPool,
   squeeze,

@@ -85,7 +85,7 @@ function parseAxisParam(axis, shape) {
   return list.map(a => (a < 0 ? a + rank : a));
 }
 
-const ELEMENT_BYTES = {float32: 4, int32: 4, complex64: 8, bool: 1};
+const ELEMENT_BYTES = {float32: 4, int32: 4, complex64: 8, bool: 1, string: 0};   // (string tensors count their bytes one by one)
 const TYPED_ARRAYS = {float32: Float32Array, int32: Int32Array, bool: Uint8Array};
 
 function bytesPerElement(dtype) {
