@@ -127,7 +127,8 @@ int tfhip_graph_destroy(int graph_id);
  *   pointwise + depthwise kernel where both take a shape), "tile_slice" (32 / 48 /
  *   64 channels per workgroup of the channel-sliced kernel), "tile_chunks" (its row
  *   chunks per image), "block_rows" (output rows per workgroup of the whole-block
- *   kernel), "fuse_block" (tfhip_inverted_residual_pays: 1 always, 0 never). TFHIP_TILE,
+ *   kernel), "fuse_block" (tfhip_inverted_residual_pays: 1 always, 0 never), "k_groups" (1 / 2 / 4
+ *   groups of wavefronts that share a GEMM tile and split its k loop). TFHIP_TILE,
  *   TFHIP_SPLITK, TFHIP_DW_ROWS, TFHIP_DW_HALO, TFHIP_NO_SKINNY, TFHIP_DW_FLAT,
  *   TFHIP_SKINNY_REGS, TFHIP_SMALL_K, TFHIP_FUSE_PW_DW in the environment set them at
  *   tfhip_init(). */

@@ -510,6 +510,38 @@ def test_conv2d_split_k(hip, orc, tuning, fmt):
     assert_parity(hip.fused_conv2d(x, w, **kw), orc.fused_conv2d(x, w, **kw))
 
 
+@pytest.mark.parametrize("tile,groups", [(12, 2), (12, 4), (10, 2)])
+def test_gemm_k_groups(hip, orc, tuning, tile, groups):
+    """Groups of wavefronts that split a tile's k loop and add their sums through LDS: against the
+    oracle for k extents that divide evenly, raggedly, and into fewer tiles than groups (idle groups
+    add zeros), with bias and activation applied once, and through the residual tail of a pointwise
+    convolution."""
+    from tfjs_amd.capi import load_library
+    tuning("tile", tile)
+    tuning("k_groups", groups)
+    tuning("no_skinny", 1)
+    rng = np.random.default_rng(4200 + tile * 10 + groups)
+    name = ctypes.create_string_buffer(256)
+    for m, n, k in [(96, 64, 768), (200, 84, 1000), (37 * 4, 52, 36), (64, 32, 32), (130, 96, 3072 + 20)]:
+        a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+        b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+        kw = dict(bias=rng.uniform(-1, 1, (n,)).astype(np.float32), activation="relu6")
+        assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
+        load_library().tfhip_last_kernel(name, 256)
+        assert name.value.decode().endswith(", 0, 1, %d>" % groups), name.value
+    a = rng.uniform(-1, 1, (3, 70, 260)).astype(np.float32)     # batched, b shared
+    b = rng.uniform(-1, 1, (1, 260, 40)).astype(np.float32)
+    assert_parity(hip.fused_matmul(a, b), orc.fused_matmul(a, b))
+    x = rng.uniform(-1, 1, (2, 7, 7, 960)).astype(np.float32)   # MobileNetV2's last projections, with the skip connection
+    w = rng.normal(0, 0.1, (1, 1, 960, 160)).astype(np.float32)
+    res = rng.uniform(-1, 1, (2, 7, 7, 160)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (160,)).astype(np.float32)
+    want = orc.fused_conv2d(x, w, bias=bias) + res
+    assert_parity(hip.fused_conv2d(x, w, bias=bias, residual=res), want)
+    load_library().tfhip_last_kernel(name, 256)
+    assert name.value.decode().endswith(", 0, 1, %d>" % groups), name.value
+
+
 # ---------------------------------------------------------------------- dequant
 
 @pytest.mark.parametrize("bits", [8, 16])
@@ -812,6 +844,63 @@ def test_pointwise_depthwise_tile_kernel(hip, orc, tuning, case):
     assert_parity(got, want)
 
 
+STREAM_CASES = [
+    # batch, h, w, in_c, mid_c, stride, pad, activation, knobs
+    (2, 56, 56, 24, 144, 1, "same", "relu6", {}),                  # MobileNetV2 block 2: four strips of 14 columns
+    (2, 56, 56, 24, 144, 2, "same", "relu6", {}),                  # stride 2: even and odd column blocks, strips of 15
+    (1, 112, 112, 16, 96, 2, "same", "relu6", {"stream_rows": 7}),  # block 1, eight chunks of seven rows
+    (2, 28, 28, 32, 192, 1, "same", "relu6", {}),
+    (2, 28, 28, 32, 192, 2, "same", "relu6", {}),
+    (2, 14, 14, 64, 384, 1, "same", "relu6", {}),                  # one strip
+    (2, 14, 14, 96, 576, 2, "same", "relu6", {}),
+    (2, 7, 7, 160, 960, 1, "same", "relu", {}),                    # half a strip, ten k groups; relu
+    (1, 9, 23, 16, 96, 1, "valid", "relu6", {}),                   # no padding, ragged last strip
+    (2, 17, 13, 32, 96, 2, "same", "relu", {"stream_rows": 3}),    # odd sizes, ragged last chunk
+    (1, 5, 31, 64, 192, 1, [[0, 0], [2, 0], [1, 2], [0, 0]], "relu6", {"stream_rows": 1}),   # explicit padding, a row per wavefront
+    (1, 6, 33, 8, 48, 2, [[0, 0], [1, 2], [2, 1], [0, 0]], "relu6", {}),                     # eight input channels: the half k group alone
+    (32, 14, 14, 64, 384, 1, "same", "relu6", {}),                 # the full batch
+]
+
+
+@pytest.mark.parametrize("case", STREAM_CASES, ids=[str(i) for i in range(len(STREAM_CASES))])
+def test_pointwise_depthwise_stream_kernel(hip, orc, tuning, case):
+    """The register-streaming fused kernel against the oracle's two convolutions and against the two
+    separate launches (whose instruction order it keeps: the same bits)."""
+    from tfjs_amd import capi
+    n, h, w, cin, mid, stride, pad, act, knobs = case
+    tuning("pw_dw_stream", 1)
+    for k, v in knobs.items():
+        tuning(k, v)
+    rng = np.random.default_rng(n * 19 + h * 5 + w + cin + mid + stride)
+    x = rng.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    w1 = rng.normal(0, 0.4, (1, 1, cin, mid)).astype(np.float32)
+    b1 = rng.uniform(-1, 2, (mid,)).astype(np.float32)       # positive: relu6(bias) is far from the zero padding
+    w2 = rng.normal(0, 0.5, (3, 3, mid, 1)).astype(np.float32)
+    b2 = rng.uniform(-1, 1, (mid,)).astype(np.float32)
+    got = hip.fused_pointwise_depthwise(x, w1, w2, strides=stride, pad=pad, pw_bias=b1, pw_activation=act,
+                                        dw_bias=b2, dw_activation=act)
+    name = ctypes.create_string_buffer(256)
+    capi.load_library().tfhip_last_kernel(name, 256)
+    assert name.value.decode().startswith("expand_dw_stream<%d, " % stride), name.value
+    mid_hip = hip.fused_conv2d(x, w1, bias=b1, activation=act)
+    capi.load_library().tfhip_last_kernel(name, 256)
+    two = hip.fused_depthwise_conv2d(mid_hip, w2, strides=stride, pad=pad, bias=b2, activation=act)
+    if n <= 4:
+        want = orc.fused_depthwise_conv2d(orc.fused_conv2d(x, w1, bias=b1, activation=act), w2, strides=stride, pad=pad,
+                                          bias=b2, activation=act)
+        assert_parity(got, want)
+    first = name.value.decode()
+    if first.startswith("skinny_gemm_regs") or (first.startswith("gemm_kernel") and cin % 16 == 0 and not first.endswith(", 2>")):
+        np.testing.assert_array_equal(got.view(np.uint32), two.view(np.uint32))
+    else:
+        assert_parity(got, two, 1e-5)
+    # without biases
+    got = hip.fused_pointwise_depthwise(x[:1], w1, w2, strides=stride, pad=pad, pw_activation=act, dw_activation=act)
+    want = orc.fused_depthwise_conv2d(orc.fused_conv2d(x[:1], w1, activation=act), w2, strides=stride, pad=pad,
+                                      activation=act)
+    assert_parity(got, want)
+
+
 BLOCK_CASES = [
     # batch, h, w, in_c, mid_c, out_c, stride, pad, activation, residual, block_rows knob
     (2, 14, 14, 64, 384, 64, 1, "same", "relu6", True, None),       # MobileNetV2 b7-b9: two waves per pixel block
@@ -887,8 +976,12 @@ STEM_DW_CASES = [
 
 
 @pytest.mark.parametrize("case", STEM_DW_CASES, ids=[str(i) for i in range(len(STEM_DW_CASES))])
-def test_conv2d_depthwise_fused(hip, orc, case):
+@pytest.mark.parametrize("stream", [0, 1], ids=["ring", "stream"])
+def test_conv2d_depthwise_fused(hip, orc, tuning, case, stream):
+    """Both fused kernels (the row ring through LDS, and the register-streaming one)."""
+    from tfjs_amd import capi
     xs, fs, stride, pad, dw_stride, dw_pad, act = case
+    tuning("pw_dw_stream", stream)
     rng = np.random.default_rng(sum(xs) + sum(fs))
     x = rng.uniform(-1, 1, xs).astype(np.float32)
     w1 = rng.normal(0, 0.5, fs).astype(np.float32)
@@ -897,6 +990,9 @@ def test_conv2d_depthwise_fused(hip, orc, case):
     b2 = rng.uniform(-1, 1, (fs[3],)).astype(np.float32)
     got = hip.fused_conv2d_depthwise(x, w1, w2, strides=stride, pad=pad, dw_strides=dw_stride, dw_pad=dw_pad, bias=b1,
                                      dw_bias=b2, activation=act)
+    name = ctypes.create_string_buffer(256)
+    capi.load_library().tfhip_last_kernel(name, 256)
+    assert name.value.decode().startswith("expand_dw_stream<" if stream else "expand_dw_3x3<"), name.value
     mid = hip.fused_conv2d(x, w1, strides=stride, pad=pad, bias=b1, activation=act)
     two = hip.fused_depthwise_conv2d(mid, w2, strides=dw_stride, pad=dw_pad, bias=b2, activation=act)
     want = orc.fused_depthwise_conv2d(orc.fused_conv2d(x, w1, strides=stride, pad=pad, bias=b1, activation=act), w2,

@@ -17,7 +17,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libtfjs_hip.so")
 ADDON = os.path.join(LIB_DIR, "tfjs_hip.node")
 
-HIP_SOURCES = ["runtime.hip", "dequant.hip", "depthwise.hip", "gemm.hip", "conv2d.hip", "glue.hip", "expand_dw.hip", "expand_dw_tile.hip", "block_fused.hip"]
+HIP_SOURCES = ["runtime.hip", "dequant.hip", "depthwise.hip", "gemm.hip", "conv2d.hip", "glue.hip", "expand_dw.hip", "expand_dw_tile.hip", "expand_dw_stream.hip", "block_fused.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops off: the compiler must not form packed FP32 instructions
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=on",

@@ -26,6 +26,7 @@
 //                the depthwise stage pads with), not activation(bias)
 #include "common.h"
 #include "epilogue.h"
+#include "expand_dw_stream.h"
 #include "expand_dw_tile.h"
 
 namespace tfhip {
@@ -45,14 +46,6 @@ struct ExpandDwArgs {
   // first stage a convolution over few input channels instead of a 1x1 one (TAPS > 0): x is
   // [batch, xh, xw, xc], the "expanded" tensor [batch, in_h, in_w, c] is its output
   int xh, xw, xc, conv_stride, conv_pad_top, conv_pad_left, k;
-};
-
-// Tap k = (fr * f_w + fs) * xc + ch of the first-stage filter: row / column relative to a
-// window's top-left input element, and byte offset from it (rows beyond K: a row no image has).
-constexpr int kMaxStemTaps = 36;
-struct StemTaps {
-  int dh[kMaxStemTaps], dw[kMaxStemTaps];
-  unsigned off_bytes[kMaxStemTaps];
 };
 
 template <int ACT>
@@ -442,6 +435,27 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
                        (pw_bias == nullptr || reinterpret_cast<uintptr_t>(pw_bias) % 16 == 0) &&
                        plan_expand_dw_tile(t, &tile_lds_bytes);
 
+  // the register-streaming kernel (a wavefront per strip and block of 16 channels, no LDS)
+  ExpandDwStreamArgs st = {};
+  st.x = x; st.w1 = pw_filter; st.b1 = pw_bias; st.w2 = dw_filter; st.b2 = dw_bias; st.y = y;
+  st.batch = (int)batch; st.in_h = (int)in_h; st.in_w = (int)in_w; st.cin = (int)in_c; st.c = (int)mid_c;
+  st.stride = (int)stride; st.pad_top = (int)pad_top; st.pad_left = (int)pad_left; st.out_h = (int)out_h; st.out_w = (int)out_w;
+  st.cap = t.cap;
+  st.x_bytes = g.x_bytes;
+  const bool stream_ok = aligned && same_relu &&
+                         (pw_bias == nullptr || reinterpret_cast<uintptr_t>(pw_bias) % 16 == 0) &&
+                         plan_expand_dw_stream(st);
+  {
+    // Measured at batch 32 with operands from memory (streaming against the better of the other two):
+    // 112x112 16 -> 96 stride 2: 34 against 47 us; 56x56 24 -> 144: 38 against 55 (stride 1), 21
+    // against 29 (stride 2); 28x28 32 -> 192 stride 1: 14.2 against 15.5. On the smaller maps, whose
+    // many input channels every wavefront would hold in registers, the tile kernel stays ahead.
+    const int knob = tuning(kTunePwDwStream);
+    const bool wide = out_w * stride >= 56 || (stride == 1 && out_w * stride >= 28 && in_c <= 32);
+    const bool other_forced = tuning(kTunePwDwTile) >= 0 && (tile_ok || ring_ok);   // that knob names one of the other two
+    if (stream_ok && (knob >= 0 ? knob > 0 : ((wide && !other_forced) || (!tile_ok && !ring_ok)))) return launch_expand_dw_stream(st);
+  }
+
   bool use_tile = tile_ok && !ring_ok;
   if (tile_ok && ring_ok) {
     const int knob = tuning(kTunePwDwTile);
@@ -558,6 +572,19 @@ extern "C" int tfhip_fused_conv2d_depthwise(const float *x, const float *filter,
     taps.dh[k] = k < K ? fr : (1 << 28);
     taps.dw[k] = fs;
     taps.off_bytes[k] = (unsigned)((((long long)fr * in_w + fs) * in_c + ch) * 4);
+  }
+  if (tuning(kTunePwDwStream) != 0) {   // (224x224x3 -> 112x112x32 at batch 32: 40 against 52 us with operands from memory)
+    ExpandDwStreamArgs st = {};
+    st.x = x; st.w1 = filter; st.b1 = bias; st.w2 = dw_filter; st.b2 = dw_bias; st.y = y;
+    st.batch = (int)batch; st.in_h = (int)mid_h; st.in_w = (int)mid_w; st.cin = (int)in_c; st.c = (int)mid_c;
+    st.stride = (int)dw_stride; st.pad_top = (int)dw_pad_top; st.pad_left = (int)dw_pad_left;
+    st.out_h = (int)out_h; st.out_w = (int)out_w;
+    st.cap = activation == TFHIP_RELU6 ? 6.f : __builtin_inff();
+    st.x_bytes = g.x_bytes;
+    st.xh = g.xh; st.xw = g.xw; st.xc = g.xc; st.conv_stride = g.conv_stride; st.conv_pad_top = g.conv_pad_top;
+    st.conv_pad_left = g.conv_pad_left; st.k = g.k; st.k_steps = k_steps;
+    if ((bias == nullptr || reinterpret_cast<uintptr_t>(bias) % 16 == 0) && plan_expand_dw_stream(st))
+      return launch_stem_dw_stream(st, taps);
   }
   const int key = (int)dw_stride * 10 + k_steps;
   switch (key) {

@@ -1,0 +1,348 @@
+// Pointwise expansion + depthwise 3x3 stage in one launch, everything in registers.
+//
+//   y = act(depthwise3x3(act(x * W1 + b1), W2) + b2)        act = relu or relu6 for both
+//
+// One wavefront owns a block of 16 expanded channels of a strip of the map and walks down its
+// rows. An expanded row of the strip is one 16 x 16 block of MFMA results: lane (grp, r) ends up
+// with the four channels 4 grp .. 4 grp + 3 of pixel r. The depthwise stage needs that pixel's
+// left and right neighbours, which are the neighbouring lanes of the same 16-lane row (one DPP
+// row shift each), and the rows above and below, which the wavefront still holds from the steps
+// before. So the expanded tensor never leaves the registers: no LDS, no barrier, and the
+// wavefronts of a workgroup (the channel blocks of one strip, which read the same input) do
+// not wait for one another.
+//
+// The strip is 16 expanded pixels wide. At stride 1 they give 14 output columns (the two outer
+// pixels are halo); at stride 2 the wavefront computes two blocks per expanded row, the even and
+// the odd columns, and needs one shifted copy of the even ones: 15 output columns.
+//
+// Products and sums are formed in the order of the separate kernels (k ascending inside the MFMA
+// chain starting from the bias; the nine taps row by row from zero, then the bias), so the result
+// has the bits of FusedConv2D followed by FusedDepthwiseConv2D.
+#include <type_traits>
+
+#include "common.h"
+#include "epilogue.h"
+#include "expand_dw_stream.h"
+
+namespace tfhip {
+namespace {
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+constexpr unsigned kNoOff = 0xffffffffu;   // an offset no buffer descriptor covers: loads return 0
+
+__device__ __forceinline__ float relu_cap(float v, float cap) {
+  const float t = (v > 0.f || v != v) ? v : 0.f;     // Math.max(0, x): NaN stays, -0 becomes +0
+  return t > cap ? cap : t;                          // cap = 6 for relu6, +inf for relu
+}
+
+// The value of the lane below (r - 1) / above (r + 1) in the 16-lane row; 0 at the row's end.
+__device__ __forceinline__ float from_lane_below(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x111, 0xf, 0xf, true));   // row_shr:1
+}
+__device__ __forceinline__ float from_lane_above(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x101, 0xf, 0xf, true));   // row_shl:1
+}
+__device__ __forceinline__ float4 from_lane_below(const float4 &v) {
+  return make_float4(from_lane_below(v.x), from_lane_below(v.y), from_lane_below(v.z), from_lane_below(v.w));
+}
+__device__ __forceinline__ float4 from_lane_above(const float4 &v) {
+  return make_float4(from_lane_above(v.x), from_lane_above(v.y), from_lane_above(v.z), from_lane_above(v.w));
+}
+
+// The three horizontal taps of one expanded row at this lane's output column.
+struct Taps {
+  float4 t0, t1, t2;
+};
+
+// S: stride of the depthwise stage. K = 16 KF + (HALF ? 8 : 0) input channels.
+// TAPS > 0: the first stage is a convolution of at most 4 TAPS taps (filter height x width x input
+// channels, a network stem) gathered element by element with the lane layout and instruction
+// order of the few-taps convolution kernel (lane (grp, r) feeds tap 4 t + grp in k step t); KF and
+// HALF are then unused.
+template <int S, int KF, bool HALF, int TAPS>
+__global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, StemTaps taps) {
+  constexpr int K = 16 * KF + (HALF ? 8 : 0);
+  const int lane = threadIdx.x & 63;
+  const int grp = lane >> 4, r = lane & 15;
+  // everything derived from the wavefront's index is the same in all its lanes: pinned to scalar
+  // registers, so that row addresses, loop bounds and the in-image tests of a row cost no vector
+  // instruction
+  long long w = (long long)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  if (w >= g.waves) return;   // (whole wavefronts: nothing below synchronises across them)
+  const int cb = (int)(w % g.cblocks);
+  w /= g.cblocks;
+  const int strip = (int)(w % g.strips);
+  w /= g.strips;
+  const int chunk = (int)(w % g.chunks_h), n = (int)(w / g.chunks_h);
+  const int oh0 = chunk * g.rows, ow0 = strip * g.strip_w;
+  const int rows = oh0 + g.rows <= g.out_h ? g.rows : g.out_h - oh0;
+  const int e0 = oh0 * S - g.pad_top;               // first expanded row this wavefront needs
+  const int ch = 16 * cb + 4 * grp;                 // this lane's four channels
+  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)g.x, 0, (int)g.x_bytes, 0x00020000);
+
+  // expansion weights of channel 16 cb + r at k = 16 t + 4 grp .. + 3 (the MFMA's first operand), bias
+  float4 wq[KF > 0 ? KF : 1];
+  float2 wh = make_float2(0.f, 0.f);
+  float wt[TAPS > 0 ? TAPS : 1];
+  int tap_dh[TAPS > 0 ? TAPS : 1], tap_dw[TAPS > 0 ? TAPS : 1];
+  unsigned tap_off[TAPS > 0 ? TAPS : 1];
+  if (TAPS > 0) {
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t) {
+      const int k = 4 * t + grp;
+      wt[t] = k < g.k ? g.w1[(long long)k * g.c + 16 * cb + r] : 0.f;   // taps beyond the filter multiply zeros
+      tap_dh[t] = taps.dh[k];
+      tap_dw[t] = taps.dw[k];
+      tap_off[t] = taps.off_bytes[k];
+    }
+  } else {
+    const float *col = g.w1 + 16 * cb + r;
+#pragma unroll
+    for (int t = 0; t < KF; ++t) {
+      const int k = 16 * t + 4 * grp;
+      wq[t] = make_float4(col[(long long)k * g.c], col[(long long)(k + 1) * g.c], col[(long long)(k + 2) * g.c],
+                          col[(long long)(k + 3) * g.c]);
+    }
+    if (HALF) {
+      const int k = 16 * KF + 2 * grp;
+      wh = make_float2(col[(long long)k * g.c], col[(long long)(k + 1) * g.c]);
+    }
+  }
+  float4_t b1q = {0.f, 0.f, 0.f, 0.f};
+  if (g.b1) b1q = *reinterpret_cast<const float4_t *>(g.b1 + ch);
+  float4 w2q[9], b2q = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int t = 0; t < 9; ++t) w2q[t] = *reinterpret_cast<const float4 *>(g.w2 + (long long)t * g.c + ch);
+  if (g.b2) b2q = *reinterpret_cast<const float4 *>(g.b2 + ch);
+
+  // This lane's expanded column in block b (S == 1: one block; S == 2: even and odd columns),
+  // whether it lies in the image, and its byte offset inside a row of x (1x1 first stage: the k
+  // group of this lane included) or the column of its window's first element (few-taps first stage).
+  int ecol[S];
+  bool col_ok[S];
+  unsigned col_off[S];
+#pragma unroll
+  for (int b = 0; b < S; ++b) {
+    ecol[b] = S == 1 ? ow0 - g.pad_left + r : 2 * (ow0 + r) - g.pad_left + b;
+    col_ok[b] = ecol[b] >= 0 && ecol[b] < g.in_w;
+    col_off[b] = TAPS > 0 ? 0u : (unsigned)(ecol[b] * K * 4 + (HALF && KF == 0 ? 2 : 4) * grp * 4);
+  }
+  const unsigned row_bytes = TAPS > 0 ? 0u : (unsigned)(g.in_w * K * 4);
+  const unsigned image_off = TAPS > 0 ? 0u : (unsigned)((long long)n * g.in_h * g.in_w * K * 4);
+
+  struct AFrag {
+    float4 full[KF > 0 ? KF : 1];
+    float2 half;
+    float tap[TAPS > 0 ? TAPS : 1];
+  };
+  // The inputs of expanded row e: one fragment per block. 1x1 first stage: the loads of a position
+  // outside the image may return anything (a neighbouring row, or zero past the tensor's end; the
+  // descriptor keeps them inside the tensor): expand() discards what is computed from them.
+  auto load_row = [&](AFrag (&a)[S], int e) __attribute__((always_inline)) {
+#pragma unroll
+    for (int b = 0; b < S; ++b) {
+      if (TAPS > 0) {
+        // the window of first-stage output pixel (e, ecol); its top-left element may lie before the
+        // image, the sum with an inside tap's offset is exact modulo 2^32
+        const bool inside = e >= 0 && e < g.in_h && col_ok[b];
+        const int xh0 = e * g.conv_stride - g.conv_pad_top, xw0 = ecol[b] * g.conv_stride - g.conv_pad_left;
+        const unsigned base = (unsigned)((((long long)n * g.xh + xh0) * g.xw + xw0) * g.xc * 4);
+#pragma unroll
+        for (int t = 0; t < TAPS; ++t) {
+          const bool ok = inside && (unsigned)(xh0 + tap_dh[t]) < (unsigned)g.xh && (unsigned)(xw0 + tap_dw[t]) < (unsigned)g.xw;
+          a[b].tap[t] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rx, (int)(ok ? base + tap_off[t] : kNoOff), 0, 0));
+        }
+        continue;
+      }
+      const unsigned base = image_off + (unsigned)e * row_bytes + col_off[b];
+#pragma unroll
+      for (int t = 0; t < KF; ++t) {
+        const auto v = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)(base + 64 * t), 0, 0);
+        a[b].full[t] = make_float4(__uint_as_float(v[0]), __uint_as_float(v[1]), __uint_as_float(v[2]), __uint_as_float(v[3]));
+      }
+      if (HALF) {
+        // (the lane's k group is two wide here: col_off holds 16 grp bytes when KF > 0, 8 grp when the half group is alone)
+        const auto v = __builtin_amdgcn_raw_buffer_load_b64(rx, (int)(base + 64 * KF - (KF > 0 ? 8 * grp : 0)), 0, 0);
+        a[b].half = make_float2(__uint_as_float(v[0]), __uint_as_float(v[1]));
+      }
+    }
+  };
+  // expanded row e of block b: activation applied, zero outside the image (the depthwise stage's padding)
+  auto expand = [&](const AFrag &a, int e, int b) __attribute__((always_inline)) {
+    float4_t acc = b1q;
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wt[t], a.tap[t], acc, 0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < (TAPS > 0 ? 0 : KF); ++t) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[t].x, a.full[t].x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[t].y, a.full[t].y, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[t].z, a.full[t].z, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[t].w, a.full[t].w, acc, 0, 0, 0);
+    }
+    if (HALF && TAPS == 0) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wh.x, a.half.x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wh.y, a.half.y, acc, 0, 0, 0);
+    }
+    // relu and the padding in one select: the value stays where it is positive (or NaN) and inside
+    const bool inside = e >= 0 && e < g.in_h && col_ok[b];
+    float4 out;
+    float *o4 = &out.x;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float v = acc[q];
+      const float t = (inside && (v > 0.f || v != v)) ? v : 0.f;
+      o4[q] = t > g.cap ? g.cap : t;
+    }
+    return out;
+  };
+  // S == 1: the output column of lane r is expanded column r's; its taps sit in lanes r - 1, r, r + 1.
+  // S == 2: output column ow0 + r reads even column r, odd column r, even column r + 1.
+  auto taps_of = [&](Taps &t, const AFrag (&a)[S], int e) __attribute__((always_inline)) {
+    if (S == 1) {
+      t.t1 = expand(a[0], e, 0);
+      t.t0 = from_lane_below(t.t1);
+      t.t2 = from_lane_above(t.t1);
+    } else {
+      t.t0 = expand(a[0], e, 0);
+      t.t1 = expand(a[S - 1], e, S - 1);
+      t.t2 = from_lane_above(t.t0);
+    }
+  };
+  const int ocol = S == 1 ? ow0 + r - 1 : ow0 + r;
+  const bool out_lane = (S == 1 ? (r >= 1 && r <= 14) : r <= 14) && ocol < g.out_w && ocol < ow0 + g.strip_w;
+  // this lane's place in an output row, and the rows' distance
+  float *out_ptr = g.y + (((long long)n * g.out_h + oh0) * g.out_w + ocol) * g.c + ch;
+  const long long out_row = (long long)g.out_w * g.c;
+  auto emit = [&](int o, const Taps &r0, const Taps &r1, const Taps &r2) __attribute__((always_inline)) {
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    const Taps *rw[3] = {&r0, &r1, &r2};
+#pragma unroll
+    for (int wr = 0; wr < 3; ++wr) {
+      const float4 e[3] = {rw[wr]->t0, rw[wr]->t1, rw[wr]->t2};
+#pragma unroll
+      for (int wc = 0; wc < 3; ++wc) {
+        const float4 wt4 = w2q[wr * 3 + wc];
+        acc.x = fmaf(e[wc].x, wt4.x, acc.x);
+        acc.y = fmaf(e[wc].y, wt4.y, acc.y);
+        acc.z = fmaf(e[wc].z, wt4.z, acc.z);
+        acc.w = fmaf(e[wc].w, wt4.w, acc.w);
+      }
+    }
+    if (out_lane) {
+      const float4 out = make_float4(relu_cap(acc.x + b2q.x, g.cap), relu_cap(acc.y + b2q.y, g.cap),
+                                     relu_cap(acc.z + b2q.z, g.cap), relu_cap(acc.w + b2q.w, g.cap));
+      store_result4(out_ptr + o * out_row, out);
+    }
+  };
+
+  // The inputs of a row are fetched while the two rows before it are worked on: two fragment sets
+  // used in turn. The three expanded rows a depthwise output reads move through three register sets.
+  AFrag fa[2][S];
+  Taps r0, r1, r2;
+  if (S == 1) {
+    load_row(fa[0], e0);
+    load_row(fa[1], e0 + 1);
+    taps_of(r0, fa[0], e0);
+    load_row(fa[0], e0 + 2);
+    taps_of(r1, fa[1], e0 + 1);
+    load_row(fa[1], e0 + 3);
+    for (int o = 0; o < rows; o += 2) {
+      taps_of(r2, fa[0], e0 + o + 2);
+      load_row(fa[0], e0 + o + 4);
+      emit(o, r0, r1, r2);
+      r0 = r1;
+      r1 = r2;
+      if (o + 1 < rows) {
+        taps_of(r2, fa[1], e0 + o + 3);
+        load_row(fa[1], e0 + o + 5);
+        emit(o + 1, r0, r1, r2);
+        r0 = r1;
+        r1 = r2;
+      }
+    }
+  } else {
+    load_row(fa[1], e0);
+    load_row(fa[0], e0 + 1);
+    taps_of(r0, fa[1], e0);
+    load_row(fa[1], e0 + 2);
+    for (int o = 0; o < rows; ++o) {
+      taps_of(r1, fa[0], e0 + 2 * o + 1);
+      load_row(fa[0], e0 + 2 * o + 3);
+      taps_of(r2, fa[1], e0 + 2 * o + 2);
+      load_row(fa[1], e0 + 2 * o + 4);
+      emit(o, r0, r1, r2);
+      r0 = r2;
+    }
+  }
+}
+
+template <int S, int KF, bool HALF, int TAPS>
+int launch_stream(const ExpandDwStreamArgs &g, const StemTaps &taps) {
+  const long long blocks = (g.waves + 3) / 4;
+  if (blocks > 0x7fffffffLL) return fail(kBadArgument, "expand_dw_stream: %lld workgroups exceed the grid limit", blocks);
+  note_kernel("expand_dw_stream<%d, %d, %s, %d>", S, KF, HALF ? "true" : "false", TAPS);
+  TFHIP_LAUNCH((expand_dw_stream<S, KF, HALF, TAPS><<<dim3((unsigned)blocks), dim3(256), 0, stream()>>>(g, taps)));
+  return kOk;
+}
+
+template <int S>
+int launch_stream_k(const ExpandDwStreamArgs &g) {
+  const StemTaps none = {};
+  switch (g.cin) {
+    case 8: return launch_stream<S, 0, true, 0>(g, none);
+    case 16: return launch_stream<S, 1, false, 0>(g, none);
+    case 24: return launch_stream<S, 1, true, 0>(g, none);
+    case 32: return launch_stream<S, 2, false, 0>(g, none);
+    case 64: return launch_stream<S, 4, false, 0>(g, none);
+    case 96: return launch_stream<S, 6, false, 0>(g, none);
+    case 160: return launch_stream<S, 10, false, 0>(g, none);
+    default: return fail(kBadArgument, "expand_dw_stream: %d input channels not instantiated", g.cin);
+  }
+}
+
+template <int S>
+int launch_stream_taps(const ExpandDwStreamArgs &g, const StemTaps &taps) {
+  switch (g.k_steps) {
+    case 3: return launch_stream<S, 0, false, 3>(g, taps);
+    case 7: return launch_stream<S, 0, false, 7>(g, taps);
+    case 9: return launch_stream<S, 0, false, 9>(g, taps);
+    default: return fail(kBadArgument, "expand_dw_stream: %d k steps of filter taps not instantiated", g.k_steps);
+  }
+}
+
+}  // namespace
+
+bool expand_dw_stream_takes_k(int cin) {
+  return cin == 8 || cin == 16 || cin == 24 || cin == 32 || cin == 64 || cin == 96 || cin == 160;
+}
+
+// Fills the tiling of `g`; false when the shape is one the kernel does not take.
+bool plan_expand_dw_stream(ExpandDwStreamArgs &g) {
+  if (g.c % 16 != 0 || (g.stride != 1 && g.stride != 2)) return false;
+  if (g.k_steps > 0 ? (g.k_steps != 3 && g.k_steps != 7 && g.k_steps != 9) : !expand_dw_stream_takes_k(g.cin)) return false;
+  g.strip_w = g.stride == 1 ? 14 : 15;
+  g.strips = (g.out_w + g.strip_w - 1) / g.strip_w;
+  g.cblocks = g.c / 16;
+  // Output rows per wavefront: every chunk computes two expanded rows of halo again, so as many
+  // rows as still give every SIMD two wavefronts to switch between (measured at batch 32 on
+  // MobileNetV2's first blocks: more, shorter wavefronts were slower or no faster).
+  const long long want = 2LL * 4 * num_cus();
+  const int forced = tuning(kTuneStreamRows);
+  int rows = g.out_h;
+  while (rows > 7 && (long long)g.batch * ((g.out_h + rows - 1) / rows) * g.strips * g.cblocks < want) rows = (rows + 1) / 2;
+  if (forced > 0) rows = forced < g.out_h ? forced : g.out_h;
+  g.rows = rows;
+  g.chunks_h = (g.out_h + rows - 1) / rows;
+  g.waves = (long long)g.batch * g.chunks_h * g.strips * g.cblocks;
+  return true;
+}
+
+int launch_expand_dw_stream(const ExpandDwStreamArgs &g) {
+  return g.stride == 1 ? launch_stream_k<1>(g) : launch_stream_k<2>(g);
+}
+
+int launch_stem_dw_stream(const ExpandDwStreamArgs &g, const StemTaps &taps) {
+  return g.stride == 1 ? launch_stream_taps<1>(g, taps) : launch_stream_taps<2>(g, taps);
+}
+
+}  // namespace tfhip

@@ -52,6 +52,14 @@ inline int choose_tile_shape(long long M, long long N, long long K, long long ba
   // Very large products: the 128x128 tile with several workgroups per compute unit
   // runs the k loop at 85% of the matrix-core rate, the small tiles at 78%.
   if (((M + 127) / 128) * ((N + 127) / 128) * batch >= 3LL * cus && K >= 512) return 0;
+  // One 64 x 48 tile on (nearly) every compute unit and a long k: that tile with two groups of
+  // wavefronts sharing it (choose_k_groups) beats the 32 x 32 tile the estimate below prefers
+  // (1024 x 768 x 3072: 43.9 against 47.0 us back to back, 45.4 against 55.2 us with operands from
+  // memory; 1024 x 768 x 768: 15.5 against 15.7, 16.9 against 18.1).
+  {
+    const long long tiles = ((M + 63) / 64) * ((N + 47) / 48) * batch;
+    if (tiles <= cus && tiles * 4 >= 3LL * cus && K >= 768) return 10;
+  }
   int best = 0;
   double best_us = 0;
   for (int i = 0; i < kNumTileShapes; ++i) {
@@ -64,9 +72,9 @@ inline int choose_tile_shape(long long M, long long N, long long K, long long ba
   return best;
 }
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int A_KIND, int B_KIND>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int A_KIND, int B_KIND, int KG = 1>
 inline int launch_gemm(GemmParams &p) {
-  using T = GemmTile<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>;
+  using T = GemmTile<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND, KG>;
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const long long tiles = (long long)p.tiles_m * p.tiles_n * p.batch;
@@ -125,39 +133,64 @@ inline int launch_gemm(GemmParams &p) {
     p.group_m = g > p.tiles_m ? p.tiles_m : g;
   }
   if (grid > 0x7fffffffLL) return fail(kBadArgument, "gemm: %lld tiles exceed the grid limit", grid);
-  if (T::LDS_FLOATS * sizeof(float) > 64 * 1024) {
+  if (T::LDS_FLOATS * sizeof(float) > 64 * 1024) {   // (also with KG groups of buffers)
     // dynamic LDS above the default limit: the attribute once per instantiation and device set-up
     static int raised = 0;
     if (raised != init_count()) {
       TFHIP_CHECK_HIP(hipFuncSetAttribute(
-          reinterpret_cast<const void *>(gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>),
+          reinterpret_cast<const void *>(gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND, KG>),
           hipFuncAttributeMaxDynamicSharedMemorySize, (int)(T::LDS_FLOATS * sizeof(float))));
       raised = init_count();
     }
   }
-  note_kernel("gemm_kernel<%d, %d, %d, %d, %d, %d, %d>", BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND);
+  if (KG > 1) note_kernel("gemm_kernel<%d, %d, %d, %d, %d, %d, %d, %d>", BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND, KG);
+  else note_kernel("gemm_kernel<%d, %d, %d, %d, %d, %d, %d>", BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND);
   // The fused epilogue covers per-column operands with a relu-family activation;
   // anything else leaves raw sums for gemm_finish.
   const Epilogue &e = p.epi;
   p.inline_epilogue = p.splits == 1 && e.channel_operands && (e.activation <= TFHIP_LEAKYRELU);
   if (p.inline_epilogue) {
-    TFHIP_LAUNCH((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>
-                  <<<dim3((unsigned)grid), dim3(256), T::LDS_FLOATS * sizeof(float), stream()>>>(p)));
+    TFHIP_LAUNCH((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND, KG>
+                  <<<dim3((unsigned)grid), dim3(256 * KG), T::LDS_FLOATS * sizeof(float), stream()>>>(p)));
   } else {
     const long long total = (long long)p.M * p.N * p.batch;
     long long blocks = (total + 255) / 256;
     const long long cap = (long long)num_cus() * 16;
     if (blocks > cap) blocks = cap;
-    TFHIP_LAUNCH((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>
-                  <<<dim3((unsigned)grid), dim3(256), T::LDS_FLOATS * sizeof(float), stream()>>>(p),
+    TFHIP_LAUNCH((gemm_kernel<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND, KG>
+                  <<<dim3((unsigned)grid), dim3(256 * KG), T::LDS_FLOATS * sizeof(float), stream()>>>(p),
                   gemm_finish<<<dim3((unsigned)blocks), dim3(256), 0, stream()>>>(p)));
   }
   return kOk;
 }
 
+// Groups of wavefronts that share a tile and split its k loop (GemmTile's KG), for the two small
+// tiles with row-major operands. Measured over BERT-base and MobileNetV2 products: two groups gain
+// 5-8% when every compute unit holds at most one tile and k spans 24 tiles or more (1024 x 768 x
+// 3072 on the 64 x 48 tile: 47.0 -> 43.9 us; 1568 x 160 x 960 on the 32 x 32 tile: 10.5 -> 9.7 us);
+// with more tiles per compute unit or a shorter k the extra barrier traffic and the final sum cost
+// more than the shorter loop saves, and four groups never won. The "k_groups" tuning knob overrides
+// (1, 2 or 4; 4 on the 32 x 32 tile only).
+inline int choose_k_groups(int shape, const GemmParams &p, int cus) {
+  const TileShape &t = kTileShapes[shape];
+  const long long tiles = ((p.M + t.bm - 1) / t.bm) * ((p.N + t.bn - 1) / t.bn) * (long long)p.batch;
+  const int k_tiles = (p.K + t.bk - 1) / t.bk;
+  const int forced = tuning(kTuneKGroups);
+  if (forced > 0) return forced >= 4 ? (shape == 12 ? 4 : 2) : (forced >= 2 ? 2 : 1);
+  return (tiles <= cus && k_tiles >= 24) ? 2 : 1;
+}
+
 // Dispatch over the instantiated tile shapes for one loader combination.
 template <int A_KIND, int B_KIND>
 inline int launch_gemm_shape(int shape, GemmParams &p) {
+  if constexpr (A_KIND == kLoadKVec && B_KIND == kLoadXVec) {
+    if (shape == 10 || shape == 12) {
+      const int kg = choose_k_groups(shape, p, num_cus());
+      if (kg == 4) return launch_gemm<32, 32, 32, 2, 2, A_KIND, B_KIND, 4>(p);
+      if (kg == 2 && shape == 10) return launch_gemm<64, 48, 32, 4, 1, A_KIND, B_KIND, 2>(p);
+      if (kg == 2) return launch_gemm<32, 32, 32, 2, 2, A_KIND, B_KIND, 2>(p);
+    }
+  }
   switch (shape) {
     case 0: return launch_gemm<128, 128, 16, 2, 2, A_KIND, B_KIND>(p);
     case 1: return launch_gemm<128, 96, 16, 2, 2, A_KIND, B_KIND>(p);

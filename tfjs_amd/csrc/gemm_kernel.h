@@ -93,9 +93,13 @@ typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
 
 constexpr unsigned kNoOffset = 0xffffffffu;  // a buffer offset no descriptor covers: loads return 0
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int A_KIND, int B_KIND>
+// KG: groups of four wavefronts per workgroup. Every group runs the whole pipeline below on its own
+// slice of k, with LDS buffers of its own, and the groups' sums are added through LDS at the end: a
+// product with few tiles and a long k then has KG times the wavefronts per compute unit to hide the
+// latencies of a k step behind, and a k loop KG times shorter.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int A_KIND, int B_KIND, int KG = 1>
 struct GemmTile {
-  static constexpr int kThreads = 256;
+  static constexpr int kThreads = 256;   // per group
   static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per workgroup");
   static_assert(BK == 16 || BK == 32, "k step of the tile");
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -109,7 +113,9 @@ struct GemmTile {
   static constexpr int A_BUF = BM * PITCH, B_BUF = BN * PITCH;
   // three tiles in flight between global memory and LDS, three LDS buffers
   static constexpr int PREFETCH = 3;
-  static constexpr int LDS_FLOATS = 3 * (A_BUF + B_BUF);
+  static constexpr int GROUP_LDS_FLOATS = 3 * (A_BUF + B_BUF);
+  static constexpr int LDS_FLOATS = KG * GROUP_LDS_FLOATS;
+  static_assert(KG == 1 || (KG - 1) * kThreads * TM * TN * 4 <= LDS_FLOATS, "the groups' sums fit the tile buffers");
 };
 
 __device__ __forceinline__ const float *uniform_pointer(const float *ptr) {
@@ -277,12 +283,14 @@ __device__ __forceinline__ float quad_element(const float4 &v, int j) {
   return j == 0 ? v.x : (j == 1 ? v.y : (j == 2 ? v.z : v.w));
 }
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int A_KIND, int B_KIND>
-__global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
-  using T = GemmTile<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND>;
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int A_KIND, int B_KIND, int KG = 1>
+__global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
+  using T = GemmTile<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND, KG>;
   extern __shared__ float lds[];
-  float *lds_a = lds;                   // [3][BM][PITCH]
-  float *lds_b = lds + 3 * T::A_BUF;    // [3][BN][PITCH]
+  // this wavefront's group, and its thread index inside the group
+  const int kgroup = KG > 1 ? __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8) : 0;
+  float *lds_a = lds + kgroup * T::GROUP_LDS_FLOATS;   // [3][BM][PITCH]
+  float *lds_b = lds_a + 3 * T::A_BUF;                 // [3][BN][PITCH]
 
   // Workgroup id -> (batch, tile_m, tile_n). Ids i, i+8, i+16, ... share an XCD;
   // give each XCD one contiguous band of the tile sequence.
@@ -296,8 +304,19 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   id -= split * tiles_per_batch * p.batch;
   const int bz = id / tiles_per_batch;
   const int t = id - bz * tiles_per_batch;
-  const int k_begin = split * p.k_per_split;
-  const int k_end = k_begin + p.k_per_split < p.K ? k_begin + p.k_per_split : p.K;
+  int k_begin = split * p.k_per_split;
+  int k_end = k_begin + p.k_per_split < p.K ? k_begin + p.k_per_split : p.K;
+  // the groups cut this range into KG runs of whole k tiles, all of the same tile count (a run that
+  // starts beyond the range reads zeros), so that every group reaches every barrier
+  int group_k_tiles = 0;
+  if (KG > 1) {
+    const int all_tiles = (k_end - k_begin + BK - 1) / BK;
+    group_k_tiles = (all_tiles + KG - 1) / KG;
+    k_begin += kgroup * group_k_tiles * BK;
+    const int run_end = k_begin + group_k_tiles * BK;
+    k_end = run_end < k_end ? run_end : k_end;
+    if (k_end < k_begin) k_end = k_begin;
+  }
   // Tiles are numbered in panels of group_m tile rows, column by column inside a
   // panel, so that the run of consecutive ids that is resident on one XCD covers
   // a near-square block of C: the rows of A and columns of B it needs per k tile
@@ -318,7 +337,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)A, 0, (int)p.a_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void *)B, 0, (int)p.b_bytes, 0x00020000);
 
-  const int tid = threadIdx.x;
+  const int tid = KG > 1 ? (int)threadIdx.x & 255 : (int)threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave / WAVES_N) * T::WM, wn0 = (wave % WAVES_N) * T::WN;
@@ -342,7 +361,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   float4_t acc[T::TM][T::TN];
   {
     const int lane_col = n0 + wn0 + (lane >> 4) * 4;
-    const bool with_bias = fused && e.bias != nullptr;
+    const bool with_bias = fused && e.bias != nullptr && kgroup == 0;
 #pragma unroll
     for (int j = 0; j < T::TN; ++j) {
       float4_t b4 = {0.f, 0.f, 0.f, 0.f};
@@ -368,7 +387,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   //    every wave finished before it reached the barrier inside tile t-2.
   constexpr int D = T::PREFETCH;
   float4 ra[D][T::A_VECS], rb[D][T::B_VECS];
-  const int k_tiles = (k_end - k_begin + BK - 1) / BK;
+  const int k_tiles = KG > 1 ? group_k_tiles : (k_end - k_begin + BK - 1) / BK;
 
   // Every fetch is unconditional: a tile past K reads as zeros through the buffer
   // descriptor at no memory cost, and with no branch around a load the compiler
@@ -494,6 +513,27 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   }
   if (kt < k_tiles) tile_step(kt, std::integral_constant<int, 0>());
   if (kt + 1 < k_tiles) tile_step(kt + 1, std::integral_constant<int, 1>());
+
+  // ---- the groups' sums into group 0, through LDS (the tile buffers are free once every
+  // wavefront is past its last fragment read)
+  if (KG > 1) {
+    lds_barrier();
+    float4_t *sums = reinterpret_cast<float4_t *>(lds);   // [KG - 1][TM * TN][256]
+    if (kgroup > 0) {
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) sums[((kgroup - 1) * T::TM * T::TN + i * T::TN + j) * 256 + tid] = acc[i][j];
+    }
+    lds_barrier();
+    if (kgroup > 0) return;
+#pragma unroll
+    for (int gk = 1; gk < KG; ++gk)
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) acc[i][j] += sums[((gk - 1) * T::TM * T::TN + i * T::TN + j) * 256 + tid];
+  }
 
   // ---- epilogue: registers -> global. Lane l of a 16x16 block holds row l % 16,
   // columns 4 * (l / 16) .. +3 (the operands went into the MFMA swapped).
