@@ -24,8 +24,9 @@ struct ExpandDwStreamArgs {
   // tiling (plan_expand_dw_stream)
   int strip_w, strips;             // output columns per wavefront, wavefronts along a row
   int rows, chunks_h;              // output rows per wavefront, wavefronts along the rows
-  int cblocks;                     // blocks of 16 expanded channels
-  long long waves;                 // batch x chunks_h x strips x cblocks
+  int ahead;                       // rows ahead of their use the inputs are fetched (2 or 4)
+  int cblocks, ncb;                // blocks of 16 expanded channels, and how many of them a wavefront takes (1 or 2)
+  long long waves;                 // batch x chunks_h x strips x ceil(cblocks / ncb)
   unsigned x_bytes;
   // first stage a convolution over few input channels instead of a 1x1 one (k_steps > 0): x is
   // [batch, xh, xw, xc], the "expanded" tensor [batch, in_h, in_w, c] is its output; k filter taps

@@ -59,7 +59,10 @@ struct Taps {
 // channels, a network stem) gathered element by element with the lane layout and instruction
 // order of the few-taps convolution kernel (lane (grp, r) feeds tap 4 t + grp in k step t); KF and
 // HALF are then unused.
-template <int S, int KF, bool HALF, int TAPS>
+// NCB: blocks of 16 channels per wavefront (1 or 2). Two blocks share every input fragment, and
+// the wavefront's stores cover 128 contiguous bytes of a pixel instead of 64.
+// AHEAD: how many expanded rows ahead of their use the inputs are fetched (2 or 4).
+template <int S, int KF, bool HALF, int TAPS, int NCB, int AHEAD>
 __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, StemTaps taps) {
   constexpr int K = 16 * KF + (HALF ? 8 : 0);
   const int lane = threadIdx.x & 63;
@@ -69,51 +72,69 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
   // instruction
   long long w = (long long)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   if (w >= g.waves) return;   // (whole wavefronts: nothing below synchronises across them)
-  const int cb = (int)(w % g.cblocks);
-  w /= g.cblocks;
+  const int cgroups = (g.cblocks + NCB - 1) / NCB;
+  const int cb0 = (int)(w % cgroups) * NCB;         // first channel block of this wavefront
+  w /= cgroups;
   const int strip = (int)(w % g.strips);
   w /= g.strips;
   const int chunk = (int)(w % g.chunks_h), n = (int)(w / g.chunks_h);
   const int oh0 = chunk * g.rows, ow0 = strip * g.strip_w;
   const int rows = oh0 + g.rows <= g.out_h ? g.rows : g.out_h - oh0;
   const int e0 = oh0 * S - g.pad_top;               // first expanded row this wavefront needs
-  const int ch = 16 * cb + 4 * grp;                 // this lane's four channels
+  // (an odd count of channel blocks: the last wavefront's second block repeats its first and is not stored)
+  int cbs[NCB], ch[NCB];                            // channel blocks, and this lane's four channels in each
+#pragma unroll
+  for (int u = 0; u < NCB; ++u) {
+    cbs[u] = cb0 + u < g.cblocks ? cb0 + u : cb0;
+    ch[u] = 16 * cbs[u] + 4 * grp;
+  }
   const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)g.x, 0, (int)g.x_bytes, 0x00020000);
 
   // expansion weights of channel 16 cb + r at k = 16 t + 4 grp .. + 3 (the MFMA's first operand), bias
-  float4 wq[KF > 0 ? KF : 1];
-  float2 wh = make_float2(0.f, 0.f);
-  float wt[TAPS > 0 ? TAPS : 1];
+  float4 wq[NCB][KF > 0 ? KF : 1];
+  float2 wh[NCB];
+  float wt[NCB][TAPS > 0 ? TAPS : 1];
   int tap_dh[TAPS > 0 ? TAPS : 1], tap_dw[TAPS > 0 ? TAPS : 1];
   unsigned tap_off[TAPS > 0 ? TAPS : 1];
+  float4_t b1q[NCB];
+  float4 w2q[NCB][9], b2q[NCB];
   if (TAPS > 0) {
 #pragma unroll
     for (int t = 0; t < TAPS; ++t) {
-      const int k = 4 * t + grp;
-      wt[t] = k < g.k ? g.w1[(long long)k * g.c + 16 * cb + r] : 0.f;   // taps beyond the filter multiply zeros
-      tap_dh[t] = taps.dh[k];
-      tap_dw[t] = taps.dw[k];
-      tap_off[t] = taps.off_bytes[k];
-    }
-  } else {
-    const float *col = g.w1 + 16 * cb + r;
-#pragma unroll
-    for (int t = 0; t < KF; ++t) {
-      const int k = 16 * t + 4 * grp;
-      wq[t] = make_float4(col[(long long)k * g.c], col[(long long)(k + 1) * g.c], col[(long long)(k + 2) * g.c],
-                          col[(long long)(k + 3) * g.c]);
-    }
-    if (HALF) {
-      const int k = 16 * KF + 2 * grp;
-      wh = make_float2(col[(long long)k * g.c], col[(long long)(k + 1) * g.c]);
+      tap_dh[t] = taps.dh[4 * t + grp];
+      tap_dw[t] = taps.dw[4 * t + grp];
+      tap_off[t] = taps.off_bytes[4 * t + grp];
     }
   }
-  float4_t b1q = {0.f, 0.f, 0.f, 0.f};
-  if (g.b1) b1q = *reinterpret_cast<const float4_t *>(g.b1 + ch);
-  float4 w2q[9], b2q = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-  for (int t = 0; t < 9; ++t) w2q[t] = *reinterpret_cast<const float4 *>(g.w2 + (long long)t * g.c + ch);
-  if (g.b2) b2q = *reinterpret_cast<const float4 *>(g.b2 + ch);
+  for (int u = 0; u < NCB; ++u) {
+    wh[u] = make_float2(0.f, 0.f);
+    if (TAPS > 0) {
+#pragma unroll
+      for (int t = 0; t < TAPS; ++t) {
+        const int k = 4 * t + grp;
+        wt[u][t] = k < g.k ? g.w1[(long long)k * g.c + 16 * cbs[u] + r] : 0.f;   // taps beyond the filter multiply zeros
+      }
+    } else {
+      const float *col = g.w1 + 16 * cbs[u] + r;
+#pragma unroll
+      for (int t = 0; t < KF; ++t) {
+        const int k = 16 * t + 4 * grp;
+        wq[u][t] = make_float4(col[(long long)k * g.c], col[(long long)(k + 1) * g.c], col[(long long)(k + 2) * g.c],
+                               col[(long long)(k + 3) * g.c]);
+      }
+      if (HALF) {
+        const int k = 16 * KF + 2 * grp;
+        wh[u] = make_float2(col[(long long)k * g.c], col[(long long)(k + 1) * g.c]);
+      }
+    }
+    b1q[u] = float4_t{0.f, 0.f, 0.f, 0.f};
+    if (g.b1) b1q[u] = *reinterpret_cast<const float4_t *>(g.b1 + ch[u]);
+    b2q[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int t = 0; t < 9; ++t) w2q[u][t] = *reinterpret_cast<const float4 *>(g.w2 + (long long)t * g.c + ch[u]);
+    if (g.b2) b2q[u] = *reinterpret_cast<const float4 *>(g.b2 + ch[u]);
+  }
 
   // This lane's expanded column in block b (S == 1: one block; S == 2: even and odd columns),
   // whether it lies in the image, and its byte offset inside a row of x (1x1 first stage: the k
@@ -167,21 +188,22 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
       }
     }
   };
-  // expanded row e of block b: activation applied, zero outside the image (the depthwise stage's padding)
-  auto expand = [&](const AFrag &a, int e, int b) __attribute__((always_inline)) {
-    float4_t acc = b1q;
+  // expanded row e of block b, channel block u: activation applied, zero outside the image (the
+  // depthwise stage's padding)
+  auto expand = [&](const AFrag &a, int e, int b, int u) __attribute__((always_inline)) {
+    float4_t acc = b1q[u];
 #pragma unroll
-    for (int t = 0; t < TAPS; ++t) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wt[t], a.tap[t], acc, 0, 0, 0);
+    for (int t = 0; t < TAPS; ++t) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wt[u][t], a.tap[t], acc, 0, 0, 0);
 #pragma unroll
     for (int t = 0; t < (TAPS > 0 ? 0 : KF); ++t) {
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[t].x, a.full[t].x, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[t].y, a.full[t].y, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[t].z, a.full[t].z, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[t].w, a.full[t].w, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[u][t].x, a.full[t].x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[u][t].y, a.full[t].y, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[u][t].z, a.full[t].z, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wq[u][t].w, a.full[t].w, acc, 0, 0, 0);
     }
     if (HALF && TAPS == 0) {
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wh.x, a.half.x, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wh.y, a.half.y, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wh[u].x, a.half.x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wh[u].y, a.half.y, acc, 0, 0, 0);
     }
     // relu and the padding in one select: the value stays where it is positive (or NaN) and inside
     const bool inside = e >= 0 && e < g.in_h && col_ok[b];
@@ -197,92 +219,130 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
   };
   // S == 1: the output column of lane r is expanded column r's; its taps sit in lanes r - 1, r, r + 1.
   // S == 2: output column ow0 + r reads even column r, odd column r, even column r + 1.
-  auto taps_of = [&](Taps &t, const AFrag (&a)[S], int e) __attribute__((always_inline)) {
-    if (S == 1) {
-      t.t1 = expand(a[0], e, 0);
-      t.t0 = from_lane_below(t.t1);
-      t.t2 = from_lane_above(t.t1);
-    } else {
-      t.t0 = expand(a[0], e, 0);
-      t.t1 = expand(a[S - 1], e, S - 1);
-      t.t2 = from_lane_above(t.t0);
+  auto taps_of = [&](Taps (&t)[NCB], const AFrag (&a)[S], int e) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < NCB; ++u) {
+      if (S == 1) {
+        t[u].t1 = expand(a[0], e, 0, u);
+        t[u].t0 = from_lane_below(t[u].t1);
+        t[u].t2 = from_lane_above(t[u].t1);
+      } else {
+        t[u].t0 = expand(a[0], e, 0, u);
+        t[u].t1 = expand(a[S - 1], e, S - 1, u);
+        t[u].t2 = from_lane_above(t[u].t0);
+      }
     }
   };
   const int ocol = S == 1 ? ow0 + r - 1 : ow0 + r;
   const bool out_lane = (S == 1 ? (r >= 1 && r <= 14) : r <= 14) && ocol < g.out_w && ocol < ow0 + g.strip_w;
-  // this lane's place in an output row, and the rows' distance
-  float *out_ptr = g.y + (((long long)n * g.out_h + oh0) * g.out_w + ocol) * g.c + ch;
+  // this lane's place in an output row (channel block 0 of the wavefront), and the rows' distance
+  float *out_ptr = g.y + (((long long)n * g.out_h + oh0) * g.out_w + ocol) * g.c + ch[0];
   const long long out_row = (long long)g.out_w * g.c;
-  auto emit = [&](int o, const Taps &r0, const Taps &r1, const Taps &r2) __attribute__((always_inline)) {
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    const Taps *rw[3] = {&r0, &r1, &r2};
+  auto emit = [&](int o, const Taps (&r0)[NCB], const Taps (&r1)[NCB], const Taps (&r2)[NCB]) __attribute__((always_inline)) {
 #pragma unroll
-    for (int wr = 0; wr < 3; ++wr) {
-      const float4 e[3] = {rw[wr]->t0, rw[wr]->t1, rw[wr]->t2};
+    for (int u = 0; u < NCB; ++u) {
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      const Taps *rw[3] = {&r0[u], &r1[u], &r2[u]};
 #pragma unroll
-      for (int wc = 0; wc < 3; ++wc) {
-        const float4 wt4 = w2q[wr * 3 + wc];
-        acc.x = fmaf(e[wc].x, wt4.x, acc.x);
-        acc.y = fmaf(e[wc].y, wt4.y, acc.y);
-        acc.z = fmaf(e[wc].z, wt4.z, acc.z);
-        acc.w = fmaf(e[wc].w, wt4.w, acc.w);
+      for (int wr = 0; wr < 3; ++wr) {
+        const float4 e[3] = {rw[wr]->t0, rw[wr]->t1, rw[wr]->t2};
+#pragma unroll
+        for (int wc = 0; wc < 3; ++wc) {
+          const float4 wt4 = w2q[u][wr * 3 + wc];
+          acc.x = fmaf(e[wc].x, wt4.x, acc.x);
+          acc.y = fmaf(e[wc].y, wt4.y, acc.y);
+          acc.z = fmaf(e[wc].z, wt4.z, acc.z);
+          acc.w = fmaf(e[wc].w, wt4.w, acc.w);
+        }
       }
-    }
-    if (out_lane) {
-      const float4 out = make_float4(relu_cap(acc.x + b2q.x, g.cap), relu_cap(acc.y + b2q.y, g.cap),
-                                     relu_cap(acc.z + b2q.z, g.cap), relu_cap(acc.w + b2q.w, g.cap));
-      store_result4(out_ptr + o * out_row, out);
+      if (out_lane && (u == 0 || cb0 + u < g.cblocks)) {
+        const float4 out = make_float4(relu_cap(acc.x + b2q[u].x, g.cap), relu_cap(acc.y + b2q[u].y, g.cap),
+                                       relu_cap(acc.z + b2q[u].z, g.cap), relu_cap(acc.w + b2q[u].w, g.cap));
+        store_result4(out_ptr + o * out_row + 16 * u, out);
+      }
     }
   };
 
-  // The inputs of a row are fetched while the two rows before it are worked on: two fragment sets
-  // used in turn. The three expanded rows a depthwise output reads move through three register sets.
-  AFrag fa[2][S];
-  Taps r0, r1, r2;
+  // The inputs of a row are fetched kAhead rows before they are used (two; four where the planner
+  // expects them to come from memory rather than cache, a round trip that outlasts two rows of
+  // work), into kAhead fragment sets used in turn; the loops are unrolled over one turn so that each set
+  // stays in fixed registers. The three expanded rows a depthwise output reads move through three
+  // register sets.
+  constexpr int kAhead = AHEAD;
+  AFrag fa[kAhead][S];
+  Taps r0[NCB], r1[NCB], r2[NCB];
+  auto move = [&](Taps (&dst)[NCB], const Taps (&src)[NCB]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < NCB; ++u) dst[u] = src[u];
+  };
+  // expanded row e0 + i lives in fragment set i % kAhead
+#pragma unroll
+  for (int i = 0; i < kAhead; ++i) load_row(fa[i], e0 + i);
   if (S == 1) {
-    load_row(fa[0], e0);
-    load_row(fa[1], e0 + 1);
     taps_of(r0, fa[0], e0);
-    load_row(fa[0], e0 + 2);
-    taps_of(r1, fa[1], e0 + 1);
-    load_row(fa[1], e0 + 3);
-    for (int o = 0; o < rows; o += 2) {
-      taps_of(r2, fa[0], e0 + o + 2);
-      load_row(fa[0], e0 + o + 4);
+    load_row(fa[0], e0 + kAhead);
+    taps_of(r1, fa[1 % kAhead], e0 + 1);
+    load_row(fa[1 % kAhead], e0 + 1 + kAhead);
+    // output row o: the new expanded row is e0 + o + 2
+    auto step = [&](auto phase, int o) __attribute__((always_inline)) {
+      constexpr int F = (decltype(phase)::value + 2) % kAhead;
+      taps_of(r2, fa[F], e0 + o + 2);
+      load_row(fa[F], e0 + o + 2 + kAhead);
       emit(o, r0, r1, r2);
-      r0 = r1;
-      r1 = r2;
-      if (o + 1 < rows) {
-        taps_of(r2, fa[1], e0 + o + 3);
-        load_row(fa[1], e0 + o + 5);
-        emit(o + 1, r0, r1, r2);
-        r0 = r1;
-        r1 = r2;
-      }
+      move(r0, r1);
+      move(r1, r2);
+    };
+    for (int o = 0; o < rows; o += 4) {
+      step(std::integral_constant<int, 0>(), o);
+      if (o + 1 < rows) step(std::integral_constant<int, 1>(), o + 1);
+      if (o + 2 < rows) step(std::integral_constant<int, 2>(), o + 2);
+      if (o + 3 < rows) step(std::integral_constant<int, 3>(), o + 3);
     }
   } else {
-    load_row(fa[1], e0);
-    load_row(fa[0], e0 + 1);
-    taps_of(r0, fa[1], e0);
-    load_row(fa[1], e0 + 2);
-    for (int o = 0; o < rows; ++o) {
-      taps_of(r1, fa[0], e0 + 2 * o + 1);
-      load_row(fa[0], e0 + 2 * o + 3);
-      taps_of(r2, fa[1], e0 + 2 * o + 2);
-      load_row(fa[1], e0 + 2 * o + 4);
+    taps_of(r0, fa[0], e0);
+    load_row(fa[0], e0 + kAhead);
+    // output row o reads expanded rows e0 + 2 o .. + 2: the first is the last of the row before
+    auto step = [&](auto phase, int o) __attribute__((always_inline)) {
+      constexpr int F1 = (2 * decltype(phase)::value + 1) % kAhead, F2 = (2 * decltype(phase)::value + 2) % kAhead;
+      taps_of(r1, fa[F1], e0 + 2 * o + 1);
+      load_row(fa[F1], e0 + 2 * o + 1 + kAhead);
+      taps_of(r2, fa[F2], e0 + 2 * o + 2);
+      load_row(fa[F2], e0 + 2 * o + 2 + kAhead);
       emit(o, r0, r1, r2);
-      r0 = r2;
+      move(r0, r2);
+    };
+    for (int o = 0; o < rows; o += 2) {
+      step(std::integral_constant<int, 0>(), o);
+      if (o + 1 < rows) step(std::integral_constant<int, 1>(), o + 1);
     }
   }
 }
 
-template <int S, int KF, bool HALF, int TAPS>
-int launch_stream(const ExpandDwStreamArgs &g, const StemTaps &taps) {
+template <int S, int KF, bool HALF, int TAPS, int NCB, int AHEAD>
+int launch_stream_ahead(const ExpandDwStreamArgs &g, const StemTaps &taps) {
   const long long blocks = (g.waves + 3) / 4;
   if (blocks > 0x7fffffffLL) return fail(kBadArgument, "expand_dw_stream: %lld workgroups exceed the grid limit", blocks);
-  note_kernel("expand_dw_stream<%d, %d, %s, %d>", S, KF, HALF ? "true" : "false", TAPS);
-  TFHIP_LAUNCH((expand_dw_stream<S, KF, HALF, TAPS><<<dim3((unsigned)blocks), dim3(256), 0, stream()>>>(g, taps)));
+  note_kernel("expand_dw_stream<%d, %d, %s, %d, %d, %d>", S, KF, HALF ? "true" : "false", TAPS, NCB, AHEAD);
+  TFHIP_LAUNCH((expand_dw_stream<S, KF, HALF, TAPS, NCB, AHEAD><<<dim3((unsigned)blocks), dim3(256), 0, stream()>>>(g, taps)));
   return kOk;
+}
+
+template <int S, int KF, bool HALF, int TAPS, int NCB>
+int launch_stream_ncb(const ExpandDwStreamArgs &g, const StemTaps &taps) {
+  if constexpr (TAPS == 0 && NCB == 1 && KF <= 2) {
+    if (g.ahead == 4) return launch_stream_ahead<S, KF, HALF, TAPS, NCB, 4>(g, taps);
+  }
+  return launch_stream_ahead<S, KF, HALF, TAPS, NCB, 2>(g, taps);
+}
+
+// Two channel blocks per wavefront where the input fragments are short enough for the registers
+// to hold both blocks' rows and weights.
+template <int S, int KF, bool HALF, int TAPS>
+int launch_stream(const ExpandDwStreamArgs &g, const StemTaps &taps) {
+  if constexpr (KF <= 2 && TAPS <= 7) {
+    if (g.ncb == 2) return launch_stream_ncb<S, KF, HALF, TAPS, 2>(g, taps);
+  }
+  return launch_stream_ncb<S, KF, HALF, TAPS, 1>(g, taps);
 }
 
 template <int S>
@@ -323,17 +383,30 @@ bool plan_expand_dw_stream(ExpandDwStreamArgs &g) {
   g.strip_w = g.stride == 1 ? 14 : 15;
   g.strips = (g.out_w + g.strip_w - 1) / g.strip_w;
   g.cblocks = g.c / 16;
+  {
+    const int forced = tuning(kTuneStreamBlocks);
+    const bool short_k = g.k_steps > 0 ? g.k_steps <= 7 : g.cin <= 32;
+    // Off unless the "stream_blocks" knob asks for it. Measured at batch 32: two blocks lose 1 - 4 us on
+    // every 1x1 first stage; on MobileNetV2's stem they gain when the kernel is launched alone with its
+    // operands from memory (39 -> 34 us) and lose inside an inference (42 -> 49 us).
+    g.ncb = forced >= 2 && g.cblocks >= 2 && short_k ? 2 : 1;
+  }
+  const int cgroups = (g.cblocks + g.ncb - 1) / g.ncb;
+  // Inputs four rows ahead on the large maps (measured at batch 32, operands from memory: 112x112
+  // 16 -> 96 stride 2: 33 against 37 us; 56x56 24 -> 144 stride 1: 36 against 41; a loss of 1 us on
+  // 56x56 stride 2 and on 28x28).
+  g.ahead = (g.k_steps == 0 && g.out_w * g.stride >= 56 && (g.stride == 1 || g.cin <= 16)) ? 4 : 2;
   // Output rows per wavefront: every chunk computes two expanded rows of halo again, so as many
   // rows as still give every SIMD two wavefronts to switch between (measured at batch 32 on
   // MobileNetV2's first blocks: more, shorter wavefronts were slower or no faster).
   const long long want = 2LL * 4 * num_cus();
   const int forced = tuning(kTuneStreamRows);
   int rows = g.out_h;
-  while (rows > 7 && (long long)g.batch * ((g.out_h + rows - 1) / rows) * g.strips * g.cblocks < want) rows = (rows + 1) / 2;
+  while (rows > 7 && (long long)g.batch * ((g.out_h + rows - 1) / rows) * g.strips * cgroups < want) rows = (rows + 1) / 2;
   if (forced > 0) rows = forced < g.out_h ? forced : g.out_h;
   g.rows = rows;
   g.chunks_h = (g.out_h + rows - 1) / rows;
-  g.waves = (long long)g.batch * g.chunks_h * g.strips * g.cblocks;
+  g.waves = (long long)g.batch * g.chunks_h * g.strips * cgroups;
   return true;
 }
 
