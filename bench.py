@@ -150,29 +150,40 @@ def sets_for(set_bytes):
     return max(2, int(-(-COLD_BYTES // max(1, int(set_bytes)))))
 
 
+COLD_THROUGH_GRAPH = True   # --cold-host-launches: a profiler on this image crashes in hipGraphLaunch
+
+
 def time_launches_cold(lib, check, ev, launch, n_sets, rounds=3, settle_ms=None):
     """Average duration in seconds of one launch when its operands come from memory: `launch(i)`
     enqueues the kernel on operand set i, the n_sets sets together exceed the memory-side cache
     twice over and are visited in turn, so no launch finds what an earlier one left behind. The
     rotation is recorded once into a HIP graph and replayed between two events (no host work
-    between the launches), best of `rounds`."""
+    between the launches), best of `rounds`. With COLD_THROUGH_GRAPH off the host enqueues every
+    launch of the rotation itself: the same memory behaviour for a counter-collecting profiler,
+    durations that include the host's pace."""
     graph_id, nodes = ctypes.c_int(), ctypes.c_int()
     launch(0)
     check(lib.tfhip_sync())
-    check(lib.tfhip_capture_begin())
-    try:
-        for i in range(n_sets):
-            launch(i)
-    except Exception:
-        lib.tfhip_capture_end(None, ctypes.byref(nodes))
-        raise
-    check(lib.tfhip_capture_end(ctypes.byref(graph_id), ctypes.byref(nodes)))
+    if COLD_THROUGH_GRAPH:
+        check(lib.tfhip_capture_begin())
+        try:
+            for i in range(n_sets):
+                launch(i)
+        except Exception:
+            lib.tfhip_capture_end(None, ctypes.byref(nodes))
+            raise
+        check(lib.tfhip_capture_end(ctypes.byref(graph_id), ctypes.byref(nodes)))
+        rotation = lambda: check(lib.tfhip_graph_launch(graph_id.value))
+    else:
+        def rotation():
+            for i in range(n_sets):
+                launch(i)
     try:
         settle_ms = SETTLE_MS if settle_ms is None else settle_ms
         settled, one_ms = 0.0, None
         while one_ms is None or settled < settle_ms:
             ev.record(0)
-            check(lib.tfhip_graph_launch(graph_id.value))
+            rotation()
             ev.record(1)
             one_ms = max(ev.elapsed_ms(0, 1), 0.01)
             settled += one_ms
@@ -181,12 +192,13 @@ def time_launches_cold(lib, check, ev, launch, n_sets, rounds=3, settle_ms=None)
         for _ in range(rounds):
             ev.record(0)
             for _ in range(replays):
-                check(lib.tfhip_graph_launch(graph_id.value))
+                rotation()
             ev.record(1)
             ms = ev.elapsed_ms(0, 1) / (replays * n_sets)
             best = ms if best is None else min(best, ms)
     finally:
-        check(lib.tfhip_graph_destroy(graph_id.value))
+        if COLD_THROUGH_GRAPH:
+            check(lib.tfhip_graph_destroy(graph_id.value))
     return best * 1e-3
 
 
@@ -288,7 +300,7 @@ def bench_model_node(model_dir, steps, warmup, prime, batch=BATCH, record=False,
     return json.loads(proc.stdout.strip().splitlines()[-1])
 
 
-def bench_kernels():
+def bench_kernels(cold=True):
     """One line per benchmark configuration: its kernel at its shape."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import synth
@@ -321,7 +333,7 @@ def bench_kernels():
                                                       transpose_b, slabs[3][i] if bias is not None else None, [0, 0, 1],
                                                       activation)
         warm = time_launches(lib, check, ev, lambda: launch(0))
-        row(name, flops, nbytes, warm, time_launches_cold(lib, check, ev, launch, sets))
+        row(name, flops, nbytes, warm, time_launches_cold(lib, check, ev, launch, sets) if cold else warm)
         for slab in slabs:
             slab.free()
 
@@ -344,7 +356,7 @@ def bench_kernels():
                                                             *epi(i)))
             flops = 2.0 * n_out * w.shape[0] * w.shape[1] * w.shape[2]
         warm = time_launches(lib, check, ev, lambda: launch(0))
-        row(name, flops, nbytes, warm, time_launches_cold(lib, check, ev, launch, sets))
+        row(name, flops, nbytes, warm, time_launches_cold(lib, check, ev, launch, sets) if cold else warm)
         for slab in slabs:
             slab.free()
 
@@ -457,6 +469,15 @@ def main():
     ap.add_argument("--kernels-only", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the batch-1 and unfused-plan legs (three more Node processes); for profiler runs, which "
+                         "are about the Python process's kernels")
+    ap.add_argument("--cold-host-launches", action="store_true",
+                    help="kernel rows: the host enqueues every launch of the cold-cache rotation instead of replaying "
+                         "a recorded HIP graph (for profiler runs; durations then include the host's pace)")
+    ap.add_argument("--no-cold", action="store_true",
+                    help="kernel rows: skip the cold-cache rotation (a recorded HIP graph) and report the back-to-back "
+                         "timing as both")
     ap.add_argument("--cpu-baseline-child", metavar="MODEL_DIR")
     ap.add_argument("--jit-prime", type=int, default=200, metavar="N",
                     help="batch-1 inferences the Node process runs before the warm-up steps (outside the timed "
@@ -472,6 +493,7 @@ def main():
                          "of this command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     globals()["SETTLE_MS"] = args.settle_ms
+    globals()["COLD_THROUGH_GRAPH"] = not args.cold_host_launches
     if args.cpu_baseline_child:
         cpu_baseline_child(args.cpu_baseline_child)
         return
@@ -480,7 +502,8 @@ def main():
                          "(the path shards by batch with no exchange step)\n" % args.gpus)
         sys.exit(2)
     if args.kernels_only:
-        print(json.dumps(dict(kernels=bench_kernels())))
+        kernels = bench_kernels(not args.no_cold)
+        print(json.dumps(dict(kernels=kernels, copy_yardstick_gbs=copy_yardstick(args.copy_yardstick) if args.copy_yardstick else None)))
         return
 
     from tfjs_amd import pyhost, workloads
@@ -492,12 +515,12 @@ def main():
         js = bench_model_node(model_dir, args.steps, args.warmup, args.jit_prime)
         m = bench_model(model_dir, args.steps, args.warmup)
         b1 = unfused = None
-        if js:
-            # the two hosts must have planned the same launches, or the roofline below (measured through
-            # the Python host) would describe another program than the headline (measured through Node)
-            if js["plan_kernels"] != m["plan_kernels"]:
-                raise RuntimeError("the Node graph model and the Python mirror launch different kernels:\n node:   %s\n python: %s"
-                                   % (js["plan_kernels"], m["plan_kernels"]))
+        # the two hosts must have planned the same launches, or the roofline below (measured through
+        # the Python host) would describe another program than the headline (measured through Node)
+        if js and js["plan_kernels"] != m["plan_kernels"]:
+            raise RuntimeError("the Node graph model and the Python mirror launch different kernels:\n node:   %s\n python: %s"
+                               % (js["plan_kernels"], m["plan_kernels"]))
+        if js and not args.no_extras:
             # batch 1, the reference's own benchmark setting: node by node, and as a recorded launch sequence
             runs = [bench_model_node(model_dir, max(args.steps, 50), max(args.warmup, 10), args.jit_prime, batch=1, record=r)
                     for r in (False, True)]
@@ -516,7 +539,7 @@ def main():
     if args.per_op:
         with open(args.per_op, "w") as f:
             json.dump(m["ops"], f, indent=0)
-    kernels = None if args.no_kernels else bench_kernels()
+    kernels = None if args.no_kernels else bench_kernels(not args.no_cold)
     copy_gbs = copy_yardstick(args.copy_yardstick) if args.copy_yardstick else None
     ms_per_step = js["ms_per_step"] if js else m["ms_per_step"]
     host = ("node %s, %s -> tfjs API -> KernelBackend 'hip' -> N-API addon -> C ABI (tfjs-core: %s)"

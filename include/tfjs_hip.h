@@ -110,7 +110,7 @@ int tfhip_graph_destroy(int graph_id);
  *   around one call times n launches without n trips through the caller's
  *   language. n = 1 is normal operation.
  * tfhip_last_kernel: symbol of the kernel the last entry point chose, spelled as
- *   a profiler demangles it, e.g. "gemm_kernel<128, 128, 16, 2, 2, 0, 1>".
+ *   a profiler demangles it, e.g. "gemm_kernel<128, 128, 16, 2, 2, 0, 1, 1>".
  * tfhip_copy: a plain device-to-device copy kernel ("copy_f4": reads `bytes`,
  *   writes `bytes`; both pointers 16-byte aligned, bytes a multiple of 16): the
  *   yardstick that a kernel's bandwidth and a profiler's traffic counters are

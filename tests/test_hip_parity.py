@@ -487,7 +487,7 @@ def test_every_gemm_tile_shape_with_every_loader(hip, orc, tuning, tile):
     kw = dict(pad="same", strides=2, bias=rng.uniform(-1, 1, (20,)).astype(np.float32), activation="relu6")
     assert_parity(hip.fused_conv2d(x, w, **kw), orc.fused_conv2d(x, w, **kw))
     load_library().tfhip_last_kernel(name, 256)
-    assert name.value.decode().endswith("3, 1>"), name.value      # vector im2col A, row-major B
+    assert name.value.decode().endswith("3, 1, 1>"), name.value   # vector im2col A, row-major B, one group of wavefronts
     # odd extents: the scalar loaders (their tile shape is fixed, the knob must not break them)
     a = rng.uniform(-1, 1, (37, 23)).astype(np.float32)
     b = rng.uniform(-1, 1, (23, 19)).astype(np.float32)
@@ -890,7 +890,7 @@ def test_pointwise_depthwise_stream_kernel(hip, orc, tuning, case):
                                           bias=b2, activation=act)
         assert_parity(got, want)
     first = name.value.decode()
-    if first.startswith("skinny_gemm_regs") or (first.startswith("gemm_kernel") and cin % 16 == 0 and not first.endswith(", 2>")):
+    if first.startswith("skinny_gemm_regs") or (first.startswith("gemm_kernel") and cin % 16 == 0 and first.endswith(", 1>")):
         np.testing.assert_array_equal(got.view(np.uint32), two.view(np.uint32))
     else:
         assert_parity(got, two, 1e-5)

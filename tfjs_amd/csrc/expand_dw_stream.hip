@@ -70,7 +70,15 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
   // everything derived from the wavefront's index is the same in all its lanes: pinned to scalar
   // registers, so that row addresses, loop bounds and the in-image tests of a row cost no vector
   // instruction
-  long long w = (long long)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  // Workgroup ids i, i + 8, i + 16, ... share an XCD and its L2: each XCD takes one contiguous band
+  // of the wavefront sequence, so that the channel blocks of a strip, which read the same input
+  // rows, find them in one L2 instead of fetching them into all eight.
+  long long block = blockIdx.x;
+  {
+    const long long per_xcd = gridDim.x / 8;
+    if (per_xcd > 0 && block < per_xcd * 8) block = (block % 8) * per_xcd + block / 8;
+  }
+  long long w = block * 4 + __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   if (w >= g.waves) return;   // (whole wavefronts: nothing below synchronises across them)
   const int cgroups = (g.cblocks + NCB - 1) / NCB;
   const int cb0 = (int)(w % cgroups) * NCB;         // first channel block of this wavefront

@@ -143,8 +143,7 @@ inline int launch_gemm(GemmParams &p) {
       raised = init_count();
     }
   }
-  if (KG > 1) note_kernel("gemm_kernel<%d, %d, %d, %d, %d, %d, %d, %d>", BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND, KG);
-  else note_kernel("gemm_kernel<%d, %d, %d, %d, %d, %d, %d>", BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND);
+  note_kernel("gemm_kernel<%d, %d, %d, %d, %d, %d, %d, %d>", BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND, KG);
   // The fused epilogue covers per-column operands with a relu-family activation;
   // anything else leaves raw sums for gemm_finish.
   const Epilogue &e = p.epi;

@@ -52,15 +52,19 @@ def symbol(kernel_name):
     return head.split("::")[-1] + tail.replace("tfhip::", "").replace("(anonymous namespace)::", "")
 
 
-def read_counter(path, counter):
+def read_counter(path, counter, by_grid=False):
     """{symbol: [value per dispatch]} for one counter; the values of one dispatch (one row per
-    XCD or shader engine in some rocprofv3 versions) are summed."""
+    XCD or shader engine in some rocprofv3 versions) are summed. by_grid: a symbol's launches are
+    told apart by their grid size (one template serves several shapes)."""
     per_dispatch = {}
     with open(path, newline="") as f:
         for row in csv.DictReader(f):
             if row["Counter_Name"] != counter:
                 continue
-            key = (row["Dispatch_Id"], symbol(row["Kernel_Name"]))
+            name = symbol(row["Kernel_Name"])
+            if by_grid and name != "copy_f4":
+                name += " grid " + row["Grid_Size"]
+            key = (row["Dispatch_Id"], name)
             per_dispatch[key] = per_dispatch.get(key, 0.0) + float(row["Counter_Value"])
     out = {}
     for (_, name), value in per_dispatch.items():
@@ -68,8 +72,8 @@ def read_counter(path, counter):
     return out
 
 
-def summarise(fetch_csv, write_csv, copy_bytes):
-    fetch, write = read_counter(fetch_csv, "FETCH_SIZE"), read_counter(write_csv, "WRITE_SIZE")
+def summarise(fetch_csv, write_csv, copy_bytes, by_grid=False):
+    fetch, write = read_counter(fetch_csv, "FETCH_SIZE", by_grid), read_counter(write_csv, "WRITE_SIZE", by_grid)
     if "copy_f4" not in fetch or "copy_f4" not in write:
         raise SystemExit("the profiled command launched no copy_f4 kernel: nothing to scale the counters by")
     mean = lambda v: sum(v) / len(v)
@@ -112,9 +116,10 @@ def main():
     ap.add_argument("--json", help="write the bytes-per-launch table here (bench.py reads profiles/traffic.json)")
     ap.add_argument("--md", help="write a readable summary here")
     ap.add_argument("--command", default="", help="the profiled command, quoted into the summary")
+    ap.add_argument("--by-grid", action="store_true", help="one row per symbol and grid size")
     ap.add_argument("--title", default="HBM traffic per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
-    rows, fs, ws, fcopy, wcopy = summarise(args.fetch_csv, args.write_csv, args.copy_mib << 20)
+    rows, fs, ws, fcopy, wcopy = summarise(args.fetch_csv, args.write_csv, args.copy_mib << 20, args.by_grid)
     head, digest = git_head(), source_hash()
     if args.json:
         with open(args.json, "w") as f:
