@@ -58,6 +58,8 @@ export interface HipGraphModelOptions {
   fusePointwiseDepthwise?: boolean;
   /** default false: record the kernels of an execution into a HIP graph and replay it for the same input shapes */
   recordLaunches?: boolean;
+  /** default true: DepthwiseConv2dNative -> BiasAdd -> Relu | Relu6 | Elu chains run as one FusedDepthwiseConv2dNative step */
+  fuseDepthwiseBiasActivation?: boolean;
 }
 
 /** decodeWeights with the dequantize step on the GPU; inject as GraphModel's tfio. */
@@ -79,6 +81,9 @@ export declare class GraphModel {
   load(): boolean | Promise<boolean>;
   predict(inputs: Tensor | Tensor[] | {[name: string]: Tensor}, config?: object): Tensor | Tensor[];
   execute(inputs: Tensor | Tensor[] | {[name: string]: Tensor}, outputs?: string | string[]): Tensor | Tensor[];
+  executeAsync(inputs: Tensor | Tensor[] | {[name: string]: Tensor}, outputs?: string | string[]): Promise<Tensor | Tensor[]>;
+  /** a caller's probe: called after every launching step of an execution with the plan step and its graph node */
+  afterNode?: (step: object, node: object) => void;
   dispose(): void;
   readonly inputs: Array<{name: string, shape?: number[], dtype?: string}>;
   readonly outputs: Array<{name: string}>;
