@@ -92,3 +92,68 @@ export declare class GraphModel {
 export declare function loadGraphModel(
     modelUrl: string | ModelArtifactsHandler, options?: HipGraphModelOptions, tfio?: IoWithDecodeWeights): GraphModel | Promise<GraphModel>;
 export declare function fileSystem(path: string): ModelArtifactsHandler;
+
+/** A device pointer as the addon hands it out: a JavaScript number below 2^53. */
+export type DevicePtr = number;
+
+/**
+ * The N-API addon (tfjs_hip.node), one method per C entry point of include/tfjs_hip.h
+ * (the pattern of tfjs-node/src/tfjs_binding.ts:32-87). Every method throws an Error that
+ * carries tfhip_last_error() when the native call fails.
+ */
+export interface HipBinding {
+  init(device: number): void;
+  shutdown(): void;
+  deviceInfo(): {name: string, arch: string, cus: number, clockKhz: number, hbmBytes: number};
+  alloc(bytes: number): DevicePtr;
+  free(ptr: DevicePtr): void;
+  upload(ptr: DevicePtr, offset: number, data: ArrayBufferView): void;
+  download(ptr: DevicePtr, offset: number, out: ArrayBufferView): ArrayBufferView;
+  sync(): void;
+  memoryInfo(): {live: number, liveBytes: number, pooledBytes: number};
+  eventRecord(slot: number): void;
+  eventElapsed(startSlot: number, endSlot: number): number;
+  setLaunchRepeat(n: number): void;
+  lastKernel(): string;
+  setTuning(name: string, value: number): void;
+  copy(dst: DevicePtr, src: DevicePtr, bytes: number): void;
+  fusedMatMul(a: DevicePtr, b: DevicePtr, out: DevicePtr, batchA: number, batchB: number, m: number, n: number, k: number,
+              transposeA: number, transposeB: number, bias: DevicePtr|null, biasStrides: Float64Array|null,
+              activation: number, prelu: DevicePtr|null, preluStrides: Float64Array|null, leakyreluAlpha: number): void;
+  fusedMatMulNoAlloc(a: DevicePtr, b: DevicePtr, out: DevicePtr, batchA: number, batchB: number, m: number, n: number,
+                     k: number, transposeA: number, transposeB: number, bias: DevicePtr|null,
+                     biasStrides: Float64Array|null, activation: number, prelu: DevicePtr|null,
+                     preluStrides: Float64Array|null, leakyreluAlpha: number): void;
+  fusedConv2D(x: DevicePtr, filter: DevicePtr, y: DevicePtr, geometry: Float64Array, nchw: number, bias: DevicePtr|null,
+              biasStrides: Float64Array|null, activation: number, prelu: DevicePtr|null,
+              preluStrides: Float64Array|null, leakyreluAlpha: number, residual?: DevicePtr|null): void;
+  fusedDepthwiseConv2D(x: DevicePtr, filter: DevicePtr, y: DevicePtr, geometry: Float64Array, bias: DevicePtr|null,
+                       biasStrides: Float64Array|null, activation: number, prelu: DevicePtr|null,
+                       preluStrides: Float64Array|null, leakyreluAlpha: number): void;
+  fusedPointwiseDepthwise(x: DevicePtr, pwFilter: DevicePtr, pwBias: DevicePtr|null, pwActivation: number,
+                          dwFilter: DevicePtr, dwBias: DevicePtr|null, dwActivation: number, y: DevicePtr,
+                          geometry: Float64Array): void;
+  pointwiseDepthwisePays(batch: number, inC: number, midC: number, stride: number, outH: number, outW: number): boolean;
+  fusedConv2DDepthwise(x: DevicePtr, filter: DevicePtr, bias: DevicePtr|null, activation: number, dwFilter: DevicePtr,
+                       dwBias: DevicePtr|null, dwActivation: number, y: DevicePtr, geometry: Float64Array): void;
+  conv2dDepthwisePays(batch: number, inC: number, fH: number, fW: number, midC: number, midH: number, midW: number,
+                      dwStride: number, outH: number, outW: number): boolean;
+  invertedResidualPays(batch: number, inH: number, inW: number, inC: number, midC: number, outC: number, stride: number,
+                       outH: number, outW: number): boolean;
+  dequantAffine(q: DevicePtr, byteOffset: number, bits: 8|16, n: number, scale: number, min: number, out: DevicePtr,
+                toInt32: number): void;
+  dequantF16(q: DevicePtr, byteOffset: number, n: number, out: DevicePtr): void;
+  add(a: DevicePtr, aStrides: Float64Array, b: DevicePtr, bStrides: Float64Array, out: DevicePtr, outShape: Float64Array,
+      rank?: number): void;
+  binary(op: number, a: DevicePtr, aStrides: Float64Array, b: DevicePtr, bStrides: Float64Array, out: DevicePtr,
+         outShape: Float64Array, rank: number): void;
+  unary(activation: number, x: DevicePtr, y: DevicePtr, n: number, alpha: number): void;
+  meanHW(x: DevicePtr, y: DevicePtr, batch: number, h: number, w: number, c: number): void;
+  avgPool(x: DevicePtr, y: DevicePtr, geometry: Float64Array): void;
+  cast(x: DevicePtr, fromDtype: number, y: DevicePtr, toDtype: number, n: number): void;
+  transpose2d(x: DevicePtr, y: DevicePtr, rows: number, cols: number): void;
+  captureBegin(): void;
+  captureEnd(keep: boolean): {id: number, nodes: number};
+  graphLaunch(id: number): void;
+  graphDestroy(id: number): void;
+}
