@@ -175,7 +175,10 @@ struct DwRowsState {
 };
 
 __device__ __forceinline__ float4 dw_load4(__amdgpu_buffer_rsrc_t r, unsigned off) {
-  const dw_uint4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+#ifndef TFHIP_DW_LOAD_AUX
+#define TFHIP_DW_LOAD_AUX 0
+#endif
+  const dw_uint4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, TFHIP_DW_LOAD_AUX);
   return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
 }
 

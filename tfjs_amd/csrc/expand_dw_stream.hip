@@ -6,8 +6,8 @@
 // rows. An expanded row of the strip is one 16 x 16 block of MFMA results: lane (grp, r) ends up
 // with the four channels 4 grp .. 4 grp + 3 of pixel r. The depthwise stage needs that pixel's
 // left and right neighbours, which are the neighbouring lanes of the same 16-lane row (one DPP
-// row shift each), and the rows above and below, which the wavefront still holds from the steps
-// before. So the expanded tensor never leaves the registers: no LDS, no barrier, and the
+// row shift each), and the rows above and below, which the wavefront has already added into the
+// running sums of the output rows they belong to. So the expanded tensor never leaves the registers: no LDS, no barrier, and the
 // wavefronts of a workgroup (the channel blocks of one strip, which read the same input) do
 // not wait for one another.
 //
@@ -30,9 +30,13 @@ namespace {
 typedef float float4_t __attribute__((ext_vector_type(4)));
 constexpr unsigned kNoOff = 0xffffffffu;   // an offset no buffer descriptor covers: loads return 0
 
-__device__ __forceinline__ float relu_cap(float v, float cap) {
-  const float t = (v > 0.f || v != v) ? v : 0.f;     // Math.max(0, x): NaN stays, -0 becomes +0
-  return t > cap ? cap : t;                          // cap = 6 for relu6, +inf for relu
+// min(max(0, v), cap) as Math.max / Math.min form it: NaN stays NaN (cap = 6 for relu6, +inf for
+// relu). The median of (v, 0, cap) is the answer for every v that is a number; `nan_classes` names
+// the classes of v that are handed through instead (both kinds of NaN).
+constexpr int kNanClasses = 0x3;
+__device__ __forceinline__ float relu_cap(float v, float cap, int nan_classes = kNanClasses) {
+  const float t = __builtin_amdgcn_fmed3f(v, 0.f, cap);
+  return __builtin_amdgcn_classf(v, nan_classes) ? v : t;
 }
 
 // The value of the lane below (r - 1) / above (r + 1) in the 16-lane row; 0 at the row's end.
@@ -62,8 +66,12 @@ struct Taps {
 // NCB: blocks of 16 channels per wavefront (1 or 2). Two blocks share every input fragment, and
 // the wavefront's stores cover 128 contiguous bytes of a pixel instead of 64.
 // AHEAD: how many expanded rows ahead of their use the inputs are fetched (2 or 4).
+// (Two wavefronts per SIMD asked for wherever the registers allow: with at most 256 registers per
+// lane the matrix instructions keep their results in ordinary vector registers, where the
+// activation reads them, instead of the accumulation registers they would have to be copied out of.)
 template <int S, int KF, bool HALF, int TAPS, int NCB, int AHEAD>
-__global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, StemTaps taps) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((S * KF * NCB >= 16 || (S == 2 && TAPS >= 7)) ? 1 : 2)))
+void expand_dw_stream(ExpandDwStreamArgs g, StemTaps taps) {
   constexpr int K = 16 * KF + (HALF ? 8 : 0);
   const int lane = threadIdx.x & 63;
   const int grp = lane >> 4, r = lane & 15;
@@ -73,19 +81,19 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
   // Workgroup ids i, i + 8, i + 16, ... share an XCD and its L2: each XCD takes one contiguous band
   // of the wavefront sequence, so that the channel blocks of a strip, which read the same input
   // rows, find them in one L2 instead of fetching them into all eight.
-  long long block = blockIdx.x;
+  unsigned block = blockIdx.x;
   {
-    const long long per_xcd = gridDim.x / 8;
+    const unsigned per_xcd = gridDim.x / 8;
     if (per_xcd > 0 && block < per_xcd * 8) block = (block % 8) * per_xcd + block / 8;
   }
-  long long w = block * 4 + __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
-  if (w >= g.waves) return;   // (whole wavefronts: nothing below synchronises across them)
-  const int cgroups = (g.cblocks + NCB - 1) / NCB;
+  unsigned w = block * 4 + (unsigned)__builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  if (w >= (unsigned)g.waves) return;   // (whole wavefronts: nothing below synchronises across them)
+  const unsigned cgroups = (unsigned)(g.cblocks + NCB - 1) / NCB;
   const int cb0 = (int)(w % cgroups) * NCB;         // first channel block of this wavefront
   w /= cgroups;
-  const int strip = (int)(w % g.strips);
-  w /= g.strips;
-  const int chunk = (int)(w % g.chunks_h), n = (int)(w / g.chunks_h);
+  const int strip = (int)(w % (unsigned)g.strips);
+  w /= (unsigned)g.strips;
+  const int chunk = (int)(w % (unsigned)g.chunks_h), n = (int)(w / (unsigned)g.chunks_h);
   const int oh0 = chunk * g.rows, ow0 = strip * g.strip_w;
   const int rows = oh0 + g.rows <= g.out_h ? g.rows : g.out_h - oh0;
   const int e0 = oh0 * S - g.pad_top;               // first expanded row this wavefront needs
@@ -104,6 +112,8 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
   float wt[NCB][TAPS > 0 ? TAPS : 1];
   int tap_dh[TAPS > 0 ? TAPS : 1], tap_dw[TAPS > 0 ? TAPS : 1];
   unsigned tap_off[TAPS > 0 ? TAPS : 1];
+  int tap_row[S][TAPS > 0 ? TAPS : 1];        // filled below, once this lane's columns are known
+  unsigned tap_col_off[S][TAPS > 0 ? TAPS : 1];
   float4_t b1q[NCB];
   float4 w2q[NCB][9], b2q[NCB];
   if (TAPS > 0) {
@@ -156,6 +166,32 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
     col_ok[b] = ecol[b] >= 0 && ecol[b] < g.in_w;
     col_off[b] = TAPS > 0 ? 0u : (unsigned)(ecol[b] * K * 4 + (HALF && KF == 0 ? 2 : 4) * grp * 4);
   }
+  // The expanded tensor's padding folded into the activation: a column outside the map gets the
+  // cap 0 and no NaN handed through, so whatever was computed for it comes out as 0.
+  float cap_col[S];
+  int nan_col[S];
+#pragma unroll
+  for (int b = 0; b < S; ++b) {
+    cap_col[b] = col_ok[b] ? g.cap : 0.f;
+    nan_col[b] = col_ok[b] ? kNanClasses : 0;
+  }
+  if (TAPS > 0) {
+    // Few-taps first stage: whether a tap's column lies in the image does not change from row to
+    // row, so it is folded into the tap's row offset once: a tap whose column (or whose pixel's
+    // column) is outside gets a row offset no image reaches, and the one test a row then needs per
+    // tap, "is the tap's row inside", fails for it as well. The byte offset of the tap from the
+    // first element of the window's row 0 takes the window's column along.
+#pragma unroll
+    for (int b = 0; b < S; ++b) {
+      const int xw0 = ecol[b] * g.conv_stride - g.conv_pad_left;
+#pragma unroll
+      for (int t = 0; t < TAPS; ++t) {
+        const bool col_in = col_ok[b] & ((unsigned)(xw0 + tap_dw[t]) < (unsigned)g.xw);
+        tap_row[b][t] = col_in ? tap_dh[t] : 0x40000000;
+        tap_col_off[b][t] = (unsigned)(xw0 * g.xc * 4) + tap_off[t];   // (exact modulo 2^32 for a tap inside)
+      }
+    }
+  }
   const unsigned row_bytes = TAPS > 0 ? 0u : (unsigned)(g.in_w * K * 4);
   const unsigned image_off = TAPS > 0 ? 0u : (unsigned)((long long)n * g.in_h * g.in_w * K * 4);
 
@@ -171,15 +207,17 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
 #pragma unroll
     for (int b = 0; b < S; ++b) {
       if (TAPS > 0) {
-        // the window of first-stage output pixel (e, ecol); its top-left element may lie before the
-        // image, the sum with an inside tap's offset is exact modulo 2^32
-        const bool inside = e >= 0 && e < g.in_h && col_ok[b];
-        const int xh0 = e * g.conv_stride - g.conv_pad_top, xw0 = ecol[b] * g.conv_stride - g.conv_pad_left;
-        const unsigned base = (unsigned)((((long long)n * g.xh + xh0) * g.xw + xw0) * g.xc * 4);
+        // the window of first-stage output pixel (e, ecol): its first row may lie before the image,
+        // the sum with an inside tap's offset is exact modulo 2^32. Row number, row limit and the
+        // row's byte offset are the same in every lane (scalar); a row outside the expanded map
+        // gets the limit 0, which no tap passes.
+        const int xh0 = e * g.conv_stride - g.conv_pad_top;
+        const unsigned limit = (e >= 0 && e < g.in_h) ? (unsigned)g.xh : 0u;
+        const unsigned base = (unsigned)((((long long)n * g.xh + xh0) * g.xw) * g.xc * 4);
 #pragma unroll
         for (int t = 0; t < TAPS; ++t) {
-          const bool ok = inside && (unsigned)(xh0 + tap_dh[t]) < (unsigned)g.xh && (unsigned)(xw0 + tap_dw[t]) < (unsigned)g.xw;
-          a[b].tap[t] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rx, (int)(ok ? base + tap_off[t] : kNoOff), 0, 0));
+          const bool ok = (unsigned)(xh0 + tap_row[b][t]) < limit;
+          a[b].tap[t] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rx, (int)(ok ? base + tap_col_off[b][t] : kNoOff), 0, 0));
         }
         continue;
       }
@@ -196,7 +234,7 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
       }
     }
   };
-  // expanded row e of block b, channel block u: activation applied, zero outside the image (the
+  // expanded row e of block b, channel block u: activation applied, zero outside the map (the
   // depthwise stage's padding)
   auto expand = [&](const AFrag &a, int e, int b, int u) __attribute__((always_inline)) {
     float4_t acc = b1q[u];
@@ -213,17 +251,12 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
       acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wh[u].x, a.half.x, acc, 0, 0, 0);
       acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wh[u].y, a.half.y, acc, 0, 0, 0);
     }
-    // relu and the padding in one select: the value stays where it is positive (or NaN) and inside
-    const bool inside = e >= 0 && e < g.in_h && col_ok[b];
-    float4 out;
-    float *o4 = &out.x;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float v = acc[q];
-      const float t = (inside && (v > 0.f || v != v)) ? v : 0.f;
-      o4[q] = t > g.cap ? g.cap : t;
-    }
-    return out;
+    // (a row outside the map, the same test in every lane: like a column outside)
+    const bool row_in = e >= 0 && e < g.in_h;
+    const float cap = row_in ? cap_col[b] : 0.f;
+    const int nan = row_in ? nan_col[b] : 0;
+    return make_float4(relu_cap(acc[0], cap, nan), relu_cap(acc[1], cap, nan), relu_cap(acc[2], cap, nan),
+                       relu_cap(acc[3], cap, nan));
   };
   // S == 1: the output column of lane r is expanded column r's; its taps sit in lanes r - 1, r, r + 1.
   // S == 2: output column ow0 + r reads even column r, odd column r, even column r + 1.
@@ -246,59 +279,67 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
   // this lane's place in an output row (channel block 0 of the wavefront), and the rows' distance
   float *out_ptr = g.y + (((long long)n * g.out_h + oh0) * g.out_w + ocol) * g.c + ch[0];
   const long long out_row = (long long)g.out_w * g.c;
-  auto emit = [&](int o, const Taps (&r0)[NCB], const Taps (&r1)[NCB], const Taps (&r2)[NCB]) __attribute__((always_inline)) {
+  // One expanded row's share of a depthwise sum: the three taps of filter row wr, left to right.
+  auto add_row = [&](const float4 &sum, const Taps &t, int wr, int u) __attribute__((always_inline)) {
+    float4 acc = sum;
+    const float4 e[3] = {t.t0, t.t1, t.t2};
 #pragma unroll
-    for (int u = 0; u < NCB; ++u) {
-      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-      const Taps *rw[3] = {&r0[u], &r1[u], &r2[u]};
-#pragma unroll
-      for (int wr = 0; wr < 3; ++wr) {
-        const float4 e[3] = {rw[wr]->t0, rw[wr]->t1, rw[wr]->t2};
-#pragma unroll
-        for (int wc = 0; wc < 3; ++wc) {
-          const float4 wt4 = w2q[u][wr * 3 + wc];
-          acc.x = fmaf(e[wc].x, wt4.x, acc.x);
-          acc.y = fmaf(e[wc].y, wt4.y, acc.y);
-          acc.z = fmaf(e[wc].z, wt4.z, acc.z);
-          acc.w = fmaf(e[wc].w, wt4.w, acc.w);
-        }
-      }
-      if (out_lane && (u == 0 || cb0 + u < g.cblocks)) {
-        const float4 out = make_float4(relu_cap(acc.x + b2q[u].x, g.cap), relu_cap(acc.y + b2q[u].y, g.cap),
-                                       relu_cap(acc.z + b2q[u].z, g.cap), relu_cap(acc.w + b2q[u].w, g.cap));
-        store_result4(out_ptr + o * out_row + 16 * u, out);
-      }
+    for (int wc = 0; wc < 3; ++wc) {
+      const float4 wt4 = w2q[u][wr * 3 + wc];
+      acc.x = fmaf(e[wc].x, wt4.x, acc.x);
+      acc.y = fmaf(e[wc].y, wt4.y, acc.y);
+      acc.z = fmaf(e[wc].z, wt4.z, acc.z);
+      acc.w = fmaf(e[wc].w, wt4.w, acc.w);
+    }
+    return acc;
+  };
+  auto store_row = [&](int o, int u, const float4 &acc) __attribute__((always_inline)) {
+    if (out_lane && (u == 0 || cb0 + u < g.cblocks)) {
+      const float4 out = make_float4(relu_cap(acc.x + b2q[u].x, g.cap), relu_cap(acc.y + b2q[u].y, g.cap),
+                                     relu_cap(acc.z + b2q[u].z, g.cap), relu_cap(acc.w + b2q[u].w, g.cap));
+      store_result4(out_ptr + o * out_row + 16 * u, out);
     }
   };
 
   // The inputs of a row are fetched kAhead rows before they are used (two; four where the planner
   // expects them to come from memory rather than cache, a round trip that outlasts two rows of
   // work), into kAhead fragment sets used in turn; the loops are unrolled over one turn so that each set
-  // stays in fixed registers. The three expanded rows a depthwise output reads move through three
-  // register sets.
+  // stays in fixed registers.
+  // An expanded row is used the moment it exists and then dropped: it adds filter row 2 to the
+  // output row that it completes, filter row 1 to the next (stride 1) and starts the one after with
+  // filter row 0. The sums of the output rows in progress are all the wavefront keeps, each still
+  // formed tap by tap in filter order from zero.
   constexpr int kAhead = AHEAD;
   AFrag fa[kAhead][S];
-  Taps r0[NCB], r1[NCB], r2[NCB];
-  auto move = [&](Taps (&dst)[NCB], const Taps (&src)[NCB]) __attribute__((always_inline)) {
-#pragma unroll
-    for (int u = 0; u < NCB; ++u) dst[u] = src[u];
-  };
+  Taps t[NCB];
+  float4 sum0[NCB], sum1[NCB];   // the output row two (stride 2: one or two) expanded rows in, and the one with one row in
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
   // expanded row e0 + i lives in fragment set i % kAhead
 #pragma unroll
   for (int i = 0; i < kAhead; ++i) load_row(fa[i], e0 + i);
   if (S == 1) {
-    taps_of(r0, fa[0], e0);
+    taps_of(t, fa[0], e0);
     load_row(fa[0], e0 + kAhead);
-    taps_of(r1, fa[1 % kAhead], e0 + 1);
+#pragma unroll
+    for (int u = 0; u < NCB; ++u) sum0[u] = add_row(zero, t[u], 0, u);
+    taps_of(t, fa[1 % kAhead], e0 + 1);
     load_row(fa[1 % kAhead], e0 + 1 + kAhead);
+#pragma unroll
+    for (int u = 0; u < NCB; ++u) {
+      sum0[u] = add_row(sum0[u], t[u], 1, u);
+      sum1[u] = add_row(zero, t[u], 0, u);
+    }
     // output row o: the new expanded row is e0 + o + 2
     auto step = [&](auto phase, int o) __attribute__((always_inline)) {
       constexpr int F = (decltype(phase)::value + 2) % kAhead;
-      taps_of(r2, fa[F], e0 + o + 2);
+      taps_of(t, fa[F], e0 + o + 2);
       load_row(fa[F], e0 + o + 2 + kAhead);
-      emit(o, r0, r1, r2);
-      move(r0, r1);
-      move(r1, r2);
+#pragma unroll
+      for (int u = 0; u < NCB; ++u) {
+        store_row(o, u, add_row(sum0[u], t[u], 2, u));
+        sum0[u] = add_row(sum1[u], t[u], 1, u);
+        sum1[u] = add_row(zero, t[u], 0, u);
+      }
     };
     for (int o = 0; o < rows; o += 4) {
       step(std::integral_constant<int, 0>(), o);
@@ -307,17 +348,24 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
       if (o + 3 < rows) step(std::integral_constant<int, 3>(), o + 3);
     }
   } else {
-    taps_of(r0, fa[0], e0);
+    taps_of(t, fa[0], e0);
     load_row(fa[0], e0 + kAhead);
-    // output row o reads expanded rows e0 + 2 o .. + 2: the first is the last of the row before
+#pragma unroll
+    for (int u = 0; u < NCB; ++u) sum0[u] = add_row(zero, t[u], 0, u);
+    // output row o reads expanded rows e0 + 2 o .. + 2: the last is the first of the row after
     auto step = [&](auto phase, int o) __attribute__((always_inline)) {
       constexpr int F1 = (2 * decltype(phase)::value + 1) % kAhead, F2 = (2 * decltype(phase)::value + 2) % kAhead;
-      taps_of(r1, fa[F1], e0 + 2 * o + 1);
+      taps_of(t, fa[F1], e0 + 2 * o + 1);
       load_row(fa[F1], e0 + 2 * o + 1 + kAhead);
-      taps_of(r2, fa[F2], e0 + 2 * o + 2);
+#pragma unroll
+      for (int u = 0; u < NCB; ++u) sum0[u] = add_row(sum0[u], t[u], 1, u);
+      taps_of(t, fa[F2], e0 + 2 * o + 2);
       load_row(fa[F2], e0 + 2 * o + 2 + kAhead);
-      emit(o, r0, r1, r2);
-      move(r0, r2);
+#pragma unroll
+      for (int u = 0; u < NCB; ++u) {
+        store_row(o, u, add_row(sum0[u], t[u], 2, u));
+        sum0[u] = add_row(zero, t[u], 0, u);
+      }
     };
     for (int o = 0; o < rows; o += 2) {
       step(std::integral_constant<int, 0>(), o);
@@ -329,7 +377,7 @@ __global__ __launch_bounds__(256) void expand_dw_stream(ExpandDwStreamArgs g, St
 template <int S, int KF, bool HALF, int TAPS, int NCB, int AHEAD>
 int launch_stream_ahead(const ExpandDwStreamArgs &g, const StemTaps &taps) {
   const long long blocks = (g.waves + 3) / 4;
-  if (blocks > 0x7fffffffLL) return fail(kBadArgument, "expand_dw_stream: %lld workgroups exceed the grid limit", blocks);
+  if (blocks > 0x3fffffffLL) return fail(kBadArgument, "expand_dw_stream: %lld workgroups exceed the limit of 2^30", blocks);   // (the kernel counts wavefronts in 32 bits)
   note_kernel("expand_dw_stream<%d, %d, %s, %d, %d, %d>", S, KF, HALF ? "true" : "false", TAPS, NCB, AHEAD);
   TFHIP_LAUNCH((expand_dw_stream<S, KF, HALF, TAPS, NCB, AHEAD><<<dim3((unsigned)blocks), dim3(256), 0, stream()>>>(g, taps)));
   return kOk;
@@ -394,10 +442,12 @@ bool plan_expand_dw_stream(ExpandDwStreamArgs &g) {
   {
     const int forced = tuning(kTuneStreamBlocks);
     const bool short_k = g.k_steps > 0 ? g.k_steps <= 7 : g.cin <= 32;
-    // Off unless the "stream_blocks" knob asks for it. Measured at batch 32: two blocks lose 1 - 4 us on
-    // every 1x1 first stage; on MobileNetV2's stem they gain when the kernel is launched alone with its
-    // operands from memory (39 -> 34 us) and lose inside an inference (42 -> 49 us).
-    g.ncb = forced >= 2 && g.cblocks >= 2 && short_k ? 2 : 1;
+    // Two blocks per wavefront on a few-taps first stage, whose gathered input fragments are the
+    // costly part of a row and are shared by the two blocks (MobileNetV2's stem at batch 32, inside an
+    // inference: 38.8 -> 33.3 us). On a 1x1 first stage they lose 1 - 4 us on every shape measured
+    // and stay off unless the "stream_blocks" knob asks (2: on, 1: off everywhere).
+    const bool two = forced >= 0 ? forced >= 2 : g.k_steps > 0;
+    g.ncb = two && g.cblocks >= 2 && short_k ? 2 : 1;
   }
   const int cgroups = (g.cblocks + g.ncb - 1) / g.ncb;
   // Inputs four rows ahead on the large maps (measured at batch 32, operands from memory: 112x112

@@ -165,8 +165,9 @@ inline int launch_gemm(GemmParams &p) {
 
 // Groups of wavefronts that share a tile and split its k loop (GemmTile's KG), for the two small
 // tiles with row-major operands. Measured over BERT-base and MobileNetV2 products: two groups gain
-// 5-8% when every compute unit holds at most one tile and k spans 24 tiles or more (1024 x 768 x
-// 3072 on the 64 x 48 tile: 47.0 -> 43.9 us; 1568 x 160 x 960 on the 32 x 32 tile: 10.5 -> 9.7 us);
+// 5-8% when every compute unit holds at most one tile, at least half of them hold one, and k spans
+// 18 tiles or more (1024 x 768 x 3072 on the 64 x 48 tile: 47.0 -> 43.9 us; on the 32 x 32 tile
+// 1568 x 160 x 960: 10.5 -> 9.7 us, 1568 x 160 x 576: 9.1 -> 8.6 us with operands from memory);
 // with more tiles per compute unit or a shorter k the extra barrier traffic and the final sum cost
 // more than the shorter loop saves, and four groups never won. The "k_groups" tuning knob overrides
 // (1, 2 or 4; 4 on the 32 x 32 tile only).
@@ -176,7 +177,7 @@ inline int choose_k_groups(int shape, const GemmParams &p, int cus) {
   const int k_tiles = (p.K + t.bk - 1) / t.bk;
   const int forced = tuning(kTuneKGroups);
   if (forced > 0) return forced >= 4 ? (shape == 12 ? 4 : 2) : (forced >= 2 ? 2 : 1);
-  return (tiles <= cus && k_tiles >= 24) ? 2 : 1;
+  return (tiles <= cus && tiles * 2 >= cus && k_tiles >= 18) ? 2 : 1;   // (a handful of tiles, like a batch-32 classifier: 9.8 us with one group, 10.5 with two)
 }
 
 // Dispatch over the instantiated tile shapes for one loader combination.
