@@ -102,41 +102,46 @@ __global__ __launch_bounds__(256) void expand_dw_tile(ExpandDwTileArgs g) {
     }
   };
 
-  // first pixel block of this wave: its fetch travels together with the weights'
+  // ---- prologue: every operand fetch is issued before anything waits for one of them, so that the
+  // workgroup pays one memory round trip, with the LDS set-up done while it is under way. (Issued
+  // one after the other, each behind a wait for the one before - the weights, then this wave's
+  // first pixels, then the depthwise operands behind the barrier's full wait - they cost three.)
+  // The slice of the expansion's weights: w1 is [K][c], 16-byte loads along the channels.
+  constexpr int quads = CS / 4, total = quads * K, NV = (total + 255) / 256;
+  float4 wv[NV];
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int i = tid + u * 256;
+    const int ii = i < total ? i : total - 1;
+    const int k = ii / quads, col = 4 * (ii - k * quads);
+    wv[u] = *reinterpret_cast<const float4 *>(g.w1 + (long long)k * g.c + c0 + col);
+  }
+  // first pixel block of this wave
   AFrag a_cur, a_next;
   unsigned off_cur = kNoOff, off_next = kNoOff;
   int pos_cur = -1, pos_next = -1;
-  if (wave < mblocks) {
-    locate(wave, off_cur, pos_cur);
-    load_a(a_cur, off_cur);
-  }
-
-  // the slice of the expansion's weights, transposed: w1 is [K][c], 16-byte loads along the
-  // channels, up to eight of a lane in flight
-  {
-    constexpr int quads = CS / 4, total = quads * K;
-    for (int i0 = tid; i0 < total; i0 += 256 * 8) {
-      float4 v[8];
+  if (wave < mblocks) locate(wave, off_cur, pos_cur);
+  load_a(a_cur, off_cur);   // (no block: every offset is out of range, nothing is read)
+  // this lane's biases of the expansion: channels 16 cb + 4 grp .. +3 of the slice
+  float4_t bias1[NCB];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int i = i0 + u * 256;
-        const int ii = i < total ? i : total - 1;
-        const int k = ii / quads, col = 4 * (ii - k * quads);
-        v[u] = *reinterpret_cast<const float4 *>(g.w1 + (long long)k * g.c + c0 + col);
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int i = i0 + u * 256;
-        if (i < total) {
-          const int k = i / quads, col = 4 * (i - k * quads);
-          w1t[(col + 0) * KP + k] = v[u].x;
-          w1t[(col + 1) * KP + k] = v[u].y;
-          w1t[(col + 2) * KP + k] = v[u].z;
-          w1t[(col + 3) * KP + k] = v[u].w;
-        }
-      }
+  for (int cb = 0; cb < NCB; ++cb) {
+    bias1[cb] = {0.f, 0.f, 0.f, 0.f};
+    if (g.b1) {
+      const float4 b = *reinterpret_cast<const float4 *>(g.b1 + c0 + 16 * cb + 4 * grp);
+      bias1[cb] = {b.x, b.y, b.z, b.w};
     }
   }
+  // depthwise stage: this lane's four channels, its weights and bias (the lanes left over when the
+  // channel quads do not divide 256 fetch like the others and sit the phase out)
+  constexpr int CQ = CS / 4, SLOTS = 256 / CQ;   // lanes along the channels, output pixels served at once
+  const int c4 = tid % CQ, slot = tid / CQ;
+  const bool dw_lane = slot < SLOTS;
+  float4 w2q[9], b2q = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int t = 0; t < 9; ++t) w2q[t] = *reinterpret_cast<const float4 *>(g.w2 + (long long)t * g.c + c0 + 4 * c4);
+  if (g.b2) b2q = *reinterpret_cast<const float4 *>(g.b2 + c0 + 4 * c4);
+
   // tile positions outside the image: the zero padding of the depthwise stage
   {
     const int positions = erows * g.ecols;
@@ -150,28 +155,19 @@ __global__ __launch_bounds__(256) void expand_dw_tile(ExpandDwTileArgs g) {
       }
     }
   }
-  // this lane's biases of the expansion: channels 16 cb + 4 grp .. +3 of the slice
-  float4_t bias1[NCB];
+  // the weights, transposed, into LDS (they were fetched first: the wait leaves the later fetches in flight)
 #pragma unroll
-  for (int cb = 0; cb < NCB; ++cb) {
-    bias1[cb] = {0.f, 0.f, 0.f, 0.f};
-    if (g.b1) {
-      const float4 b = *reinterpret_cast<const float4 *>(g.b1 + c0 + 16 * cb + 4 * grp);
-      bias1[cb] = {b.x, b.y, b.z, b.w};
+  for (int u = 0; u < NV; ++u) {
+    const int i = tid + u * 256;
+    if (i < total) {
+      const int k = i / quads, col = 4 * (i - k * quads);
+      w1t[(col + 0) * KP + k] = wv[u].x;
+      w1t[(col + 1) * KP + k] = wv[u].y;
+      w1t[(col + 2) * KP + k] = wv[u].z;
+      w1t[(col + 3) * KP + k] = wv[u].w;
     }
   }
-  // depthwise stage: this lane's four channels, its weights and bias
-  constexpr int CQ = CS / 4, SLOTS = 256 / CQ;   // lanes along the channels, output pixels served at once
-  const int c4 = tid % CQ, slot = tid / CQ;
-  const bool dw_lane = slot < SLOTS;
-  float4 w2q[9], b2q = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-  for (int t = 0; t < 9; ++t) {
-    w2q[t] = dw_lane ? *reinterpret_cast<const float4 *>(g.w2 + (long long)t * g.c + c0 + 4 * c4) : b2q;
-  }
-  if (dw_lane && g.b2) b2q = *reinterpret_cast<const float4 *>(g.b2 + c0 + 4 * c4);
-
-  __syncthreads();   // w1t
+  lds_barrier();   // w1t and the zeros; nobody waits for a fetch here
 
   // ---- phase 1: the expanded tile
   const float *wcol = w1t + r * KP + 4 * grp;
