@@ -48,6 +48,7 @@
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "epilogue.h"
 
@@ -111,7 +112,10 @@ struct GemmTile {
   static constexpr int A_VECS = (BM * BK / 4 + kThreads - 1) / kThreads;
   static constexpr int B_VECS = (BN * BK / 4 + kThreads - 1) / kThreads;
   static constexpr int A_BUF = BM * PITCH, B_BUF = BN * PITCH;
-  // three tiles in flight between global memory and LDS, three LDS buffers
+  // Three LDS buffers, and three tiles in flight between global memory and LDS (the ring of register
+  // slots in gemm_kernel takes any depth; six slots on the 32 x 32 x 32 and 64 x 64 x 16 tiles were
+  // slower on every MobileNetV2 projection, by 0.5 - 1.5 us of 7 - 15: the k loop of these
+  // launches is not waiting for a fetch that three tiles in flight fail to cover)
   static constexpr int PREFETCH = 3;
   static constexpr int GROUP_LDS_FLOATS = 3 * (A_BUF + B_BUF);
   static constexpr int LDS_FLOATS = KG * GROUP_LDS_FLOATS;
@@ -279,6 +283,12 @@ __device__ __forceinline__ void load_fragment(float4 (&frag)[NT], const float *l
     frag[t] = *reinterpret_cast<const float4 *>(lane_base + buf_off + t * 16 * PITCH + quad * 16);
 }
 
+// f(integral_constant<int, I>) for every I of the sequence, in order.
+template <int... I, typename F>
+__device__ __forceinline__ void static_for(std::integer_sequence<int, I...>, F &&f) {
+  (f(std::integral_constant<int, I>()), ...);
+}
+
 __device__ __forceinline__ float quad_element(const float4 &v, int j) {
   return j == 0 ? v.x : (j == 1 ? v.y : (j == 2 ? v.z : v.w));
 }
@@ -300,9 +310,12 @@ __global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
     if (per_xcd > 0 && id < per_xcd * 8) id = (id % 8) * per_xcd + id / 8;
   }
   const int tiles_per_batch = p.tiles_m * p.tiles_n;
-  const int split = id / (tiles_per_batch * p.batch);
-  id -= split * tiles_per_batch * p.batch;
-  const int bz = id / tiles_per_batch;
+  int split = 0, bz = 0;
+  if (p.splits * p.batch > 1) {   // (most launches: one product, not split; no division for them)
+    split = id / (tiles_per_batch * p.batch);
+    id -= split * tiles_per_batch * p.batch;
+    bz = id / tiles_per_batch;
+  }
   const int t = id - bz * tiles_per_batch;
   int k_begin = split * p.k_per_split;
   int k_end = k_begin + p.k_per_split < p.K ? k_begin + p.k_per_split : p.K;
@@ -352,34 +365,13 @@ __global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
   const float *a_lane = lds_a + (wm0 + (lane & 15)) * T::PITCH + (lane >> 4) * 4;
   const float *b_lane = lds_b + (wn0 + (lane & 15)) * T::PITCH + (lane >> 4) * 4;
 
-  // The accumulators start from the bias (lane l of a 16x16 block ends up with
-  // columns 4 * (l / 16) .. +3 of its row, see the epilogue): its fetch overlaps
-  // the first tiles' instead of following the k loop, and it costs no register
-  // past this point. A product that is completed by gemm_finish starts from zero.
   const Epilogue &e = p.epi;
   const bool fused = p.inline_epilogue != 0;
   float4_t acc[T::TM][T::TN];
-  {
-    const int lane_col = n0 + wn0 + (lane >> 4) * 4;
-    const bool with_bias = fused && e.bias != nullptr && kgroup == 0;
-#pragma unroll
-    for (int j = 0; j < T::TN; ++j) {
-      float4_t b4 = {0.f, 0.f, 0.f, 0.f};
-      if (with_bias) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int col = lane_col + j * 16 + q;
-          b4[q] = e.bias[(long long)(col < p.N ? col : p.N - 1) * e.bias_s[3]];
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < T::TM; ++i) acc[i][j] = b4;
-    }
-  }
 
-  // Software pipeline over k tiles, three deep at both levels:
-  //  * registers: tile t lives in ring slot t % 3 from its global fetch (issued
-  //    while tile t-4 computes) until it is stored to LDS (while tile t-1 computes)
+  // Software pipeline over k tiles, D (three or six) deep in registers, three deep in LDS:
+  //  * registers: tile t lives in ring slot t % D from its global fetch (issued
+  //    while tile t-D-1 computes) until it is stored to LDS (while tile t-1 computes)
   //  * LDS: tile t lives in buffer t % 3. It is written during the first k steps of
   //    tile t-1, ONE barrier in the middle of tile t-1 publishes it, and the last k
   //    step of tile t-1 already fetches its first fragments, so no wave ever waits
@@ -399,6 +391,28 @@ __global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
                                          p.conv);
     load_tile<BN, BK, B_KIND, T::B_VECS>(rb[d], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0, k_begin + d * BK, tid,
                                          p.conv);
+  }
+  // The accumulators start from the bias (lane l of a 16x16 block ends up with
+  // columns 4 * (l / 16) .. +3 of its row, see the epilogue): its fetch is issued
+  // behind the first tiles' and shares their round trip, instead of costing one of
+  // its own before them or after the k loop. A product that is completed by
+  // gemm_finish starts from zero.
+  {
+    const int lane_col = n0 + wn0 + (lane >> 4) * 4;
+    const bool with_bias = fused && e.bias != nullptr && kgroup == 0;
+#pragma unroll
+    for (int j = 0; j < T::TN; ++j) {
+      float4_t b4 = {0.f, 0.f, 0.f, 0.f};
+      if (with_bias) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int col = lane_col + j * 16 + q;
+          b4[q] = e.bias[(long long)(col < p.N ? col : p.N - 1) * e.bias_s[3]];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i) acc[i][j] = b4;
+    }
   }
   store_tile<BM, BK, T::PITCH, A_KIND, T::A_VECS>(lds_a, ra[0], tid);
   store_tile<BN, BK, T::PITCH, B_KIND, T::B_VECS>(lds_b, rb[0], tid);
@@ -436,10 +450,12 @@ __global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
   constexpr int kBarrierGroup = (kStores - 1) / kPerGroup;   // the group that holds the last store
   static_assert(kBarrierGroup <= 4 * (Q - 1) + 1, "fragments of the next tile are read after the barrier");
 
-  // One k tile: tile kt sits in LDS buffer u = kt % 3, tile kt+1 in ring slot (u+1) % 3.
-  auto tile_step = [&](int kt, auto u_tag) __attribute__((always_inline)) {
-    constexpr int u = decltype(u_tag)::value;
+  // One k tile: tile kt = L * n + i sits in LDS buffer u = i % 3, tile kt+1 in ring slot (i+1) % D and
+  // goes to LDS buffer (u+1) % 3.
+  auto tile_step = [&](int kt, auto i_tag) __attribute__((always_inline)) {
+    constexpr int u = decltype(i_tag)::value % 3;
     constexpr int nb = (u + 1) % 3;
+    constexpr int slot = (decltype(i_tag)::value + 1) % D;
     const int a_off = u * T::A_BUF, b_off = u * T::B_BUF;
 #pragma unroll
     for (int quad = 0; quad < Q; ++quad) {
@@ -460,15 +476,15 @@ __global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
 #pragma unroll
         for (int piece = group * kPerGroup; piece < (group + 1) * kPerGroup && piece < kPieces; ++piece) {
           if (piece < T::A_VECS) {
-            store_tile<BM, BK, T::PITCH, A_KIND, T::A_VECS>(lds_a + nb * T::A_BUF, ra[nb], tid, piece, piece + 1);
+            store_tile<BM, BK, T::PITCH, A_KIND, T::A_VECS>(lds_a + nb * T::A_BUF, ra[slot], tid, piece, piece + 1);
           } else if (piece < kStores) {
-            store_tile<BN, BK, T::PITCH, B_KIND, T::B_VECS>(lds_b + nb * T::B_BUF, rb[nb], tid, piece - T::A_VECS,
+            store_tile<BN, BK, T::PITCH, B_KIND, T::B_VECS>(lds_b + nb * T::B_BUF, rb[slot], tid, piece - T::A_VECS,
                                                             piece - T::A_VECS + 1);
           } else if (piece == kStores) {
-            load_tile<BM, BK, A_KIND, T::A_VECS>(ra[nb], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0,
+            load_tile<BM, BK, A_KIND, T::A_VECS>(ra[slot], sa, rsrc_a, A, p.a_sx, p.a_sk, p.M, k_end, m0,
                                                  k_begin + (kt + 1 + D) * BK, tid, p.conv);
           } else {
-            load_tile<BN, BK, B_KIND, T::B_VECS>(rb[nb], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0,
+            load_tile<BN, BK, B_KIND, T::B_VECS>(rb[slot], sb, rsrc_b, B, p.b_sx, p.b_sk, p.N, k_end, n0,
                                                  k_begin + (kt + 1 + D) * BK, tid, p.conv);
           }
         }
@@ -503,16 +519,15 @@ __global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
     }
   };
 
-  // Full groups of three tiles run without a branch between them; the remainder
-  // (one or two tiles) follows with one check per tile.
+  // Full turns of the two rings (L tiles: both ring positions are then constants) run without a
+  // branch between them; the remainder follows with one check per tile.
+  constexpr int L = D % 3 == 0 ? D : 3 * D;
   int kt = 0;
-  for (; kt + 3 <= k_tiles; kt += 3) {
-    tile_step(kt, std::integral_constant<int, 0>());
-    tile_step(kt + 1, std::integral_constant<int, 1>());
-    tile_step(kt + 2, std::integral_constant<int, 2>());
-  }
-  if (kt < k_tiles) tile_step(kt, std::integral_constant<int, 0>());
-  if (kt + 1 < k_tiles) tile_step(kt + 1, std::integral_constant<int, 1>());
+  for (; kt + L <= k_tiles; kt += L)
+    static_for(std::make_integer_sequence<int, L>(), [&](auto i) __attribute__((always_inline)) { tile_step(kt + decltype(i)::value, i); });
+  static_for(std::make_integer_sequence<int, L - 1>(), [&](auto i) __attribute__((always_inline)) {
+    if (kt + decltype(i)::value < k_tiles) tile_step(kt + decltype(i)::value, i);
+  });
 
   // ---- the groups' sums into group 0, through LDS (the tile buffers are free once every
   // wavefront is past its last fragment read)
