@@ -106,16 +106,10 @@ void expand_dw_stream(ExpandDwStreamArgs g, StemTaps taps) {
   }
   const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)g.x, 0, (int)g.x_bytes, 0x00020000);
 
-  // expansion weights of channel 16 cb + r at k = 16 t + 4 grp .. + 3 (the MFMA's first operand), bias
-  float4 wq[NCB][KF > 0 ? KF : 1];
-  float2 wh[NCB];
-  float wt[NCB][TAPS > 0 ? TAPS : 1];
   int tap_dh[TAPS > 0 ? TAPS : 1], tap_dw[TAPS > 0 ? TAPS : 1];
   unsigned tap_off[TAPS > 0 ? TAPS : 1];
   int tap_row[S][TAPS > 0 ? TAPS : 1];        // filled below, once this lane's columns are known
   unsigned tap_col_off[S][TAPS > 0 ? TAPS : 1];
-  float4_t b1q[NCB];
-  float4 w2q[NCB][9], b2q[NCB];
   if (TAPS > 0) {
 #pragma unroll
     for (int t = 0; t < TAPS; ++t) {
@@ -124,36 +118,6 @@ void expand_dw_stream(ExpandDwStreamArgs g, StemTaps taps) {
       tap_off[t] = taps.off_bytes[4 * t + grp];
     }
   }
-#pragma unroll
-  for (int u = 0; u < NCB; ++u) {
-    wh[u] = make_float2(0.f, 0.f);
-    if (TAPS > 0) {
-#pragma unroll
-      for (int t = 0; t < TAPS; ++t) {
-        const int k = 4 * t + grp;
-        wt[u][t] = k < g.k ? g.w1[(long long)k * g.c + 16 * cbs[u] + r] : 0.f;   // taps beyond the filter multiply zeros
-      }
-    } else {
-      const float *col = g.w1 + 16 * cbs[u] + r;
-#pragma unroll
-      for (int t = 0; t < KF; ++t) {
-        const int k = 16 * t + 4 * grp;
-        wq[u][t] = make_float4(col[(long long)k * g.c], col[(long long)(k + 1) * g.c], col[(long long)(k + 2) * g.c],
-                               col[(long long)(k + 3) * g.c]);
-      }
-      if (HALF) {
-        const int k = 16 * KF + 2 * grp;
-        wh[u] = make_float2(col[(long long)k * g.c], col[(long long)(k + 1) * g.c]);
-      }
-    }
-    b1q[u] = float4_t{0.f, 0.f, 0.f, 0.f};
-    if (g.b1) b1q[u] = *reinterpret_cast<const float4_t *>(g.b1 + ch[u]);
-    b2q[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-    for (int t = 0; t < 9; ++t) w2q[u][t] = *reinterpret_cast<const float4 *>(g.w2 + (long long)t * g.c + ch[u]);
-    if (g.b2) b2q[u] = *reinterpret_cast<const float4 *>(g.b2 + ch[u]);
-  }
-
   // This lane's expanded column in block b (S == 1: one block; S == 2: even and odd columns),
   // whether it lies in the image, and its byte offset inside a row of x (1x1 first stage: the k
   // group of this lane included) or the column of its window's first element (few-taps first stage).
@@ -234,6 +198,55 @@ void expand_dw_stream(ExpandDwStreamArgs g, StemTaps taps) {
       }
     }
   };
+  // The first rows' inputs are fetched before the weights: everything the wavefront needs before its
+  // first matrix instruction is then in flight together, one memory round trip instead of two.
+  // Expanded row e0 + i lives in fragment set i % AHEAD.
+  AFrag fa[AHEAD][S];
+#pragma unroll
+  for (int i = 0; i < AHEAD; ++i) load_row(fa[i], e0 + i);
+
+  // expansion weights of channel 16 cb + r at k = 16 t + 4 grp .. + 3 (the MFMA's first operand), bias
+  float4 wq[NCB][KF > 0 ? KF : 1];
+  float2 wh[NCB];
+  float wt[NCB][TAPS > 0 ? TAPS : 1];
+  float4_t b1q[NCB];
+  float4 w2q[NCB][9], b2q[NCB];
+#pragma unroll
+  for (int u = 0; u < NCB; ++u) {
+    wh[u] = make_float2(0.f, 0.f);
+    if (TAPS > 0) {
+#pragma unroll
+      for (int t = 0; t < TAPS; ++t) {
+        const int k = 4 * t + grp;
+        wt[u][t] = k < g.k ? g.w1[(long long)k * g.c + 16 * cbs[u] + r] : 0.f;   // taps beyond the filter multiply zeros
+      }
+    } else {
+      const float *col = g.w1 + 16 * cbs[u] + r;
+#pragma unroll
+      for (int t = 0; t < KF; ++t) {
+        const int k = 16 * t + 4 * grp;
+        wq[u][t] = make_float4(col[(long long)k * g.c], col[(long long)(k + 1) * g.c], col[(long long)(k + 2) * g.c],
+                               col[(long long)(k + 3) * g.c]);
+      }
+      if (HALF) {
+        const int k = 16 * KF + 2 * grp;
+        wh[u] = make_float2(col[(long long)k * g.c], col[(long long)(k + 1) * g.c]);
+      }
+    }
+    // (a missing bias: the fetch goes to the depthwise weights instead and is dropped; a branch around a
+    // load would make the wavefront wait at its end for every fetch in flight)
+    {
+      const float4_t v = *reinterpret_cast<const float4_t *>((g.b1 ? g.b1 : g.w2) + ch[u]);
+      b1q[u] = g.b1 ? v : float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int t = 0; t < 9; ++t) w2q[u][t] = *reinterpret_cast<const float4 *>(g.w2 + (long long)t * g.c + ch[u]);
+    {
+      const float4 v = *reinterpret_cast<const float4 *>((g.b2 ? g.b2 : g.w2) + ch[u]);
+      b2q[u] = g.b2 ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  }
+
   // expanded row e of block b, channel block u: activation applied, zero outside the map (the
   // depthwise stage's padding)
   auto expand = [&](const AFrag &a, int e, int b, int u) __attribute__((always_inline)) {
@@ -310,13 +323,9 @@ void expand_dw_stream(ExpandDwStreamArgs g, StemTaps taps) {
   // filter row 0. The sums of the output rows in progress are all the wavefront keeps, each still
   // formed tap by tap in filter order from zero.
   constexpr int kAhead = AHEAD;
-  AFrag fa[kAhead][S];
   Taps t[NCB];
   float4 sum0[NCB], sum1[NCB];   // the output row two (stride 2: one or two) expanded rows in, and the one with one row in
   const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-  // expanded row e0 + i lives in fragment set i % kAhead
-#pragma unroll
-  for (int i = 0; i < kAhead; ++i) load_row(fa[i], e0 + i);
   if (S == 1) {
     taps_of(t, fa[0], e0);
     load_row(fa[0], e0 + kAhead);
@@ -454,13 +463,31 @@ bool plan_expand_dw_stream(ExpandDwStreamArgs &g) {
   // 16 -> 96 stride 2: 33 against 37 us; 56x56 24 -> 144 stride 1: 36 against 41; a loss of 1 us on
   // 56x56 stride 2 and on 28x28).
   g.ahead = (g.k_steps == 0 && g.out_w * g.stride >= 56 && (g.stride == 1 || g.cin <= 16)) ? 4 : 2;
-  // Output rows per wavefront: every chunk computes two expanded rows of halo again, so as many
-  // rows as still give every SIMD two wavefronts to switch between (measured at batch 32 on
-  // MobileNetV2's first blocks: more, shorter wavefronts were slower or no faster).
-  const long long want = 2LL * 4 * num_cus();
+  // Output rows per wavefront. The launch is bound by its arithmetic, which the wavefronts of a compute
+  // unit share, so it lasts as long as the compute unit with the most workgroups needs for them: the
+  // number of workgroups per compute unit, rounded up, times the row steps of a wavefront (its rows,
+  // the two rows of halo a stride-1 chunk computes again, and about a step and a half of set-up). A
+  // single wavefront per SIMD has nobody to hide its waits behind and is priced a quarter higher.
+  // The row count with the lowest price wins, the larger one on a tie. (Measured at batch 32 on
+  // MobileNetV2's shapes, this order of the candidates is the measured one: 56x56 / 144 channels,
+  // stride 1: 14 rows 22.1 us, 28 rows 24.2, 7 rows 23.4; stride 2: 6 rows 16.8, 7 rows 18.4, 14 rows 21.6.)
   const int forced = tuning(kTuneStreamRows);
   int rows = g.out_h;
-  while (rows > 7 && (long long)g.batch * ((g.out_h + rows - 1) / rows) * g.strips * cgroups < want) rows = (rows + 1) / 2;
+  {
+    const long long cus = num_cus();
+    double best = 0;
+    for (int cand = g.out_h < 4 ? g.out_h : 4; cand <= g.out_h; ++cand) {
+      const long long chunks = (g.out_h + cand - 1) / cand;
+      const long long groups = ((long long)g.batch * chunks * g.strips * cgroups + 3) / 4;
+      const long long per_cu = (groups + cus - 1) / cus;
+      const double steps = cand + (g.stride == 1 ? 2.0 : 0.5) + 1.5;
+      const double price = (double)per_cu * steps * (per_cu < 2 ? 1.25 : 1.0);
+      if (cand == (g.out_h < 4 ? g.out_h : 4) || price <= best) {
+        best = price;
+        rows = cand;
+      }
+    }
+  }
   if (forced > 0) rows = forced < g.out_h ? forced : g.out_h;
   g.rows = rows;
   g.chunks_h = (g.out_h + rows - 1) / rows;
