@@ -480,8 +480,8 @@ def main():
                          "timing as both")
     ap.add_argument("--cpu-baseline-child", metavar="MODEL_DIR")
     ap.add_argument("--jit-prime", type=int, default=200, metavar="N",
-                    help="batch-1 inferences the Node process runs before the warm-up steps (outside the timed "
-                         "region) so that V8 has compiled the host path; 0 disables")
+                    help="inferences the Node process runs before the warm-up steps (outside the timed region, at "
+                         "the measured batch size) so that V8 has compiled the host path; 0 disables")
     ap.add_argument("--settle-ms", type=float, default=SETTLE_MS, metavar="MS",
                     help="untimed run of each configuration's kernel before its timed launches (default 20: the GPU "
                          "reaches its sustained clock); small under a counter-collecting profiler, where only "
@@ -560,7 +560,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "MobileNetV2 1.0/224, batch 32, NHWC fp32, uint8-quantized random-init weights "
                                "dequantized on load (benchmark configuration 4)", "batch": BATCH,
-                   "jit_priming_batch1_inferences": js["prime"] if js else 0, "host": host, "device": info["arch"], "cus": info["cus"]},
+                   "jit_priming_inferences": js["prime"] if js else 0, "host": host, "device": info["arch"], "cus": info["cus"]},
         "b1": b1,
         "unfused_plan_images_per_s": unfused["images_per_s"] if unfused else None,
         "unfused_plan": unfused,

@@ -55,17 +55,19 @@ async function main() {
     checksum = data[0];
     y.dispose();
   };
+  // Priming, outside the timed region and at the batch size that is measured: V8 compiles the host
+  // path from the types and branches it has seen, and a function that meets a new branch at another
+  // batch size (the kernels chosen differ) falls back to the interpreter and is compiled again some
+  // twenty calls later, 2 ms on the main thread, which would land inside a short timed run.
   if (prime > 0) {
-    const x1 = tf.tensor(model.syntheticInput(1, 3), [1, 224, 224, 3]);
     for (let i = 0; i < prime; i++) {
-      const y = predict(x1);
+      const y = predict(x);
       if (i % 16 === 15) {
         y.dataSync();  // keeps the host at most 16 inferences ahead of the stream
       }
       y.dispose();
     }
     addon.sync();
-    x1.dispose();
   }
   for (let i = 0; i < warmup; i++) {
     step();
@@ -73,11 +75,15 @@ async function main() {
   addon.sync();
   addon.eventRecord(0);
   const start = tf.util.now();
+  const stepEnds = new Float64Array(steps);
   for (let i = 0; i < steps; i++) {
     step();
+    stepEnds[i] = tf.util.now();
   }
   addon.sync();
   const wallMs = tf.util.now() - start;
+  // (every step ends in a dataSync, so the differences are whole steps: a host pause shows as one long step)
+  const stepMs = Array.from(stepEnds, (t, i) => t - (i === 0 ? start : stepEnds[i - 1])).sort((a, b) => a - b);
   addon.eventRecord(1);
   const deviceMs = addon.eventElapsed(0, 1);
   // One more inference, node by node, asking the library after every node which kernel it chose.
@@ -99,6 +105,8 @@ async function main() {
   const mem = tf.memory();
   console.log(JSON.stringify({
     ms_per_step: wallMs / steps,
+    step_ms_median: stepMs[stepMs.length >> 1],
+    step_ms_max: stepMs[stepMs.length - 1],
     device_ms_per_step: deviceMs / steps,
     load_ms: loadMs,
     batch,
