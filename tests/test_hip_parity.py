@@ -901,6 +901,43 @@ def test_pointwise_depthwise_stream_kernel(hip, orc, tuning, case):
     assert_parity(got, want)
 
 
+@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("act", ["relu", "relu6"])
+def test_pointwise_depthwise_stream_kernel_non_finite(hip, orc, tuning, stride, act):
+    """NaN and the infinities through the streaming kernel's clamps (a median instruction plus a class
+    test): NaN stays NaN, +Inf becomes the cap (or stays, for relu), -Inf becomes 0, as Math.max /
+    Math.min give them in the reference (Relu.ts:22, Relu6.ts:22-23), also next to the padding."""
+    tuning("pw_dw_stream", 1)
+    rng = np.random.default_rng(41 + stride)
+    n, h, w, cin, mid = 2, 12, 19, 16, 48
+    x = rng.uniform(-1, 1, (n, h, w, cin)).astype(np.float32)
+    x[0, 0, 0, 3] = np.nan            # a corner: its window reaches into the padding
+    x[0, 5, 7, 1] = np.inf
+    x[0, 6, 18, 2] = -np.inf          # the last column
+    x[1, 11, 9, 0] = np.nan           # the last row
+    x[1, 3, 4, 5] = np.inf
+    x[1, 3, 4, 6] = -np.inf           # Inf - Inf in one pixel's sums
+    w1 = rng.normal(0, 0.4, (1, 1, cin, mid)).astype(np.float32)
+    b1 = rng.uniform(-1, 2, (mid,)).astype(np.float32)
+    w2 = rng.normal(0, 0.5, (3, 3, mid, 1)).astype(np.float32)
+    b2 = rng.uniform(-1, 1, (mid,)).astype(np.float32)
+    got = hip.fused_pointwise_depthwise(x, w1, w2, strides=stride, pad="same", pw_bias=b1, pw_activation=act,
+                                        dw_bias=b2, dw_activation=act)
+    want = orc.fused_depthwise_conv2d(orc.fused_conv2d(x, w1, bias=b1, activation=act), w2, strides=stride, pad="same",
+                                      bias=b2, activation=act)
+    assert np.isnan(want).any() and np.isfinite(want).any()
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+    np.testing.assert_array_equal(np.isposinf(got), np.isposinf(want))
+    np.testing.assert_array_equal(np.isneginf(got), np.isneginf(want))
+    finite = np.isfinite(want)
+    assert_parity(got[finite], want[finite])
+    two = hip.fused_depthwise_conv2d(hip.fused_conv2d(x, w1, bias=b1, activation=act), w2, strides=stride, pad="same",
+                                     bias=b2, activation=act)
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(two))
+    ok = ~np.isnan(got)
+    np.testing.assert_array_equal(got[ok].view(np.uint32), two[ok].view(np.uint32))
+
+
 BLOCK_CASES = [
     # batch, h, w, in_c, mid_c, out_c, stride, pad, activation, residual, block_rows knob
     (2, 14, 14, 64, 384, 64, 1, "same", "relu6", True, None),       # MobileNetV2 b7-b9: two waves per pixel block
@@ -972,6 +1009,7 @@ STEM_DW_CASES = [
     ((2, 20, 30, 1), (3, 3, 1, 16), 1, "valid", 1, "same", "relu6"),       # 9 taps: three k steps, one channel block
     ((1, 18, 18, 4), (3, 3, 4, 48), 1, "same", 1, "valid", "relu6"),       # 36 taps: nine k steps
     ((2, 24, 40, 2), (1, 7, 2, 64), 1, [[0, 0], [0, 0], [3, 3], [0, 0]], 2, "same", "relu6"),   # 1x7 filter, explicit padding
+    ((2, 20, 22, 3), (3, 3, 3, 48), 2, "same", 1, "same", "relu"),         # three channel blocks: the streaming kernel's last wavefront has one
 ]
 
 
@@ -1000,6 +1038,14 @@ def test_conv2d_depthwise_fused(hip, orc, tuning, case, stream):
     assert_parity(got, want)
     # the separate stem kernels feed the matrix cores in the same order: the same bits
     np.testing.assert_array_equal(got.view(np.uint32), two.view(np.uint32))
+    if stream:
+        # one channel block per wavefront (the default for a few-taps first stage is two)
+        tuning("stream_blocks", 1)
+        one = hip.fused_conv2d_depthwise(x, w1, w2, strides=stride, pad=pad, dw_strides=dw_stride, dw_pad=dw_pad, bias=b1,
+                                         dw_bias=b2, activation=act)
+        capi.load_library().tfhip_last_kernel(name, 256)
+        assert ", 1, 2>" in name.value.decode(), name.value
+        np.testing.assert_array_equal(got.view(np.uint32), one.view(np.uint32))
 
 
 def test_pointwise_depthwise_without_biases_and_unsupported_shapes(hip, orc):
