@@ -60,16 +60,6 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
   const int my_blocks = first < blocks ? (blocks - first + step - 1) / step : 0;
   const int total = my_blocks * chunks;
 
-  // per-lane epilogue operands: four consecutive columns of each 16-column group
-  float bias_q[TN][4];
-#pragma unroll
-  for (int n = 0; n < TN; ++n)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int col = n * 16 + grp * 4 + q;
-      bias_q[n][q] = (g.bias && col < g.N) ? g.bias[(long long)col * g.bias_stride] : 0.f;
-    }
-
   // loads of one step: k = c * 64 + 16 t + 4 grp .. +3 of row b * 16 + r
   auto issue = [&](float4 (&dst)[4], int b, int c) __attribute__((always_inline)) {
     const int row = b * 16 + r;
@@ -90,40 +80,64 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
 #pragma unroll
     for (int n = 0; n < TN; ++n) acc[h][n] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-  // the first fetch of A is issued before B is staged, so the two overlap
+  // ---- prologue: the first fetch of A, the whole of B and the bias are issued before anything
+  // waits, so the three share one memory round trip (a fetch behind a branch, or the bias in front
+  // of A, costs a round trip of its own: 3.4 us of an 11 us launch went into them, measured with
+  // timestamps inside the kernel).
   float4 cur[4], nxt[4];
-  if (total > 0) issue(cur, first, 0);
+  issue(cur, total > 0 ? first : blocks, 0);   // (no row block: every offset is out of range, nothing is read)
 
   // B -> LDS, transposed. Columns >= N and rows >= K read as zero; rows beyond
   // the last 16-row group that holds real data are never read. Consecutive lanes
   // take consecutive k (conflict-free LDS stores; B itself is small and cached),
-  // and eight fetches are issued before the first is stored, so the fill costs
-  // one or two memory round trips instead of one per element.
-  {
-    const int kk = ((g.K + 15) / 16) * 16;
-    const int items = kk * (16 * TN / 4);
-    for (int i0 = tid; i0 < items; i0 += kThreads * 8) {
-      float4 v[8];
+  // and a thread's fetches of a pass are all issued before the first is stored.
+  const int kk = ((g.K + 15) / 16) * 16;
+  const int items = kk * (16 * TN / 4);
+  constexpr int kFill = 8;   // fetches per thread and pass
+  float4 v[kFill];
+  auto fetch_b = [&](int i0) __attribute__((always_inline)) {
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int i = i0 + u * kThreads;
-        const int c = (i / kk) * 4, k = i - (i / kk) * kk;
-        v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (i < items && k < g.K && c < g.N) v[u] = *reinterpret_cast<const float4 *>(g.b + (long long)k * g.N + c);
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int i = i0 + u * kThreads;
-        if (i >= items) continue;
-        const int c = (i / kk) * 4, k = i - (i / kk) * kk;
-        lds_bt[(c + 0) * pitch + k] = v[u].x;
-        lds_bt[(c + 1) * pitch + k] = v[u].y;
-        lds_bt[(c + 2) * pitch + k] = v[u].z;
-        lds_bt[(c + 3) * pitch + k] = v[u].w;
-      }
+    for (int u = 0; u < kFill; ++u) {
+      const int i = i0 + u * kThreads;
+      const int c = (i / kk) * 4, k = i - (i / kk) * kk;
+      const bool real = i < items && k < g.K && c < g.N;
+      const float4 w = *reinterpret_cast<const float4 *>(g.b + (real ? (long long)k * g.N + c : 0));
+      v[u] = real ? w : make_float4(0.f, 0.f, 0.f, 0.f);
     }
+  };
+  auto store_b = [&](int i0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < kFill; ++u) {
+      const int i = i0 + u * kThreads;
+      if (i >= items) continue;
+      const int c = (i / kk) * 4, k = i - (i / kk) * kk;
+      lds_bt[(c + 0) * pitch + k] = v[u].x;
+      lds_bt[(c + 1) * pitch + k] = v[u].y;
+      lds_bt[(c + 2) * pitch + k] = v[u].z;
+      lds_bt[(c + 3) * pitch + k] = v[u].w;
+    }
+  };
+  fetch_b(tid);
+
+  // per-lane epilogue operands: four consecutive columns of each 16-column group (a missing
+  // bias or a column beyond N: the fetch goes to B's first element and is dropped)
+  float bias_q[TN][4];
+#pragma unroll
+  for (int n = 0; n < TN; ++n)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int col = n * 16 + grp * 4 + q;
+      const bool real = g.bias != nullptr && col < g.N;
+      const float w = real ? g.bias[(long long)col * g.bias_stride] : g.b[0];
+      bias_q[n][q] = real ? w : 0.f;
+    }
+
+  store_b(tid);
+  for (int i0 = tid + kThreads * kFill; i0 < items; i0 += kThreads * kFill) {
+    fetch_b(i0);
+    store_b(i0);
   }
-  __syncthreads();
+  lds_barrier();   // B is in LDS; nobody waits for a fetch here
 
   int b = first, c = 0;
   for (int q = 0; q < total; ++q) {
