@@ -297,6 +297,13 @@ template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int A_KIND, int B_KI
 __global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
   using T = GemmTile<BM, BN, BK, WAVES_M, WAVES_N, A_KIND, B_KIND, KG>;
   extern __shared__ float lds[];
+  // Every kernel argument the prologue reads, asked for here in one piece: the compiler fetches an
+  // argument where it is first used, and the prologue's branches and divisions would otherwise cut
+  // those fetches into three or four batches, each waiting a scalar-cache miss of its own.
+  asm volatile("" ::"s"(p.a), "s"(p.b), "s"(p.c), "s"(p.M), "s"(p.N), "s"(p.K), "s"(p.batch), "s"(p.a_sx), "s"(p.a_sk),
+               "s"(p.b_sx), "s"(p.b_sk), "s"(p.ldc), "s"(p.a_bytes), "s"(p.b_bytes), "s"(p.tiles_m), "s"(p.tiles_n),
+               "s"(p.group_m), "s"(p.splits), "s"(p.k_per_split), "s"(p.vec_store), "s"(p.inline_epilogue),
+               "s"(p.epi.bias), "s"(p.epi.bias_s[3]), "s"(p.epi.activation), "s"(p.epi.residual), "s"(p.epi.addressing));
   // this wavefront's group, and its thread index inside the group
   const int kgroup = KG > 1 ? __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8) : 0;
   float *lds_a = lds + kgroup * T::GROUP_LDS_FLOATS;   // [3][BM][PITCH]
