@@ -243,7 +243,6 @@ int launch_few_taps_k(const GemmParams &p, int f_h) {
 
 template <int OC>
 int launch_few_channels(const GemmParams &p, int f_h) {
-  const ConvGeom &c = p.conv;
   FewChannelsArgs g;
   fill_few_channels_args(g, p, f_h);
   dim3 grid((unsigned)((p.M + 255) / 256), (unsigned)(p.N / OC), 1);
