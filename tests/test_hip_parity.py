@@ -1066,8 +1066,9 @@ def test_pointwise_depthwise_without_biases_and_unsupported_shapes(hip, orc):
     assert lib.tfhip_pointwise_depthwise_pays(32, 32, 192, 1, 28, 28) == 1     # the channel-sliced kernel
     assert lib.tfhip_pointwise_depthwise_pays(32, 64, 384, 1, 14, 14) == 1
     assert lib.tfhip_pointwise_depthwise_pays(32, 160, 960, 1, 7, 7) == 1
-    assert lib.tfhip_pointwise_depthwise_pays(1, 16, 96, 2, 56, 56) == 0       # one image: the expanded tensor is small
-    assert lib.tfhip_pointwise_depthwise_pays(1, 64, 384, 1, 14, 14) == 0      # ... and too few workgroups to fill the chip
+    assert lib.tfhip_pointwise_depthwise_pays(1, 16, 96, 2, 56, 56) == 1       # one image: one launch instead of two
+    assert lib.tfhip_pointwise_depthwise_pays(1, 64, 384, 1, 14, 14) == 1
+    assert lib.tfhip_pointwise_depthwise_pays(1, 16, 80, 1, 20, 20) == 0       # only the row-ring kernel takes it: from 48 MB
     assert lib.tfhip_pointwise_depthwise_pays(32, 128, 384, 1, 14, 14) == 0    # a count of input channels neither kernel has
     assert lib.tfhip_pointwise_depthwise_pays(64, 16, 40, 2, 112, 112) == 0    # channels no multiple of 16
     assert lib.tfhip_pointwise_depthwise_pays(64, 16, 96, 3, 112, 112) == 0    # stride 3
@@ -1197,7 +1198,8 @@ def test_config4_mobilenet_v2_batch1_vs_oracle(hip, orc, tmp_path):
     # the ten skip connections as Add kernels of their own, expansions and depthwise stages as two kernels
     plain = workloads.DeviceMobileNetV2(str(tmp_path), 2, fuse_residual_add=False, fuse_expand_depthwise=False)
     try:
-        fused_pairs = sum(1 for op, _ in model.plan if op["kind"] == "pwdw")   # none at this small batch
+        fused_pairs = sum(1 for op, _ in model.plan if op["kind"] in ("pwdw", "cvdw"))   # all 17, at every batch size
+        assert fused_pairs == 17
         assert len(plain.plan) == len(model.plan) + 10 + fused_pairs
         plain.set_input(x)
         # (at this small batch the separate expansions run on the tiled kernel, whose k order differs)

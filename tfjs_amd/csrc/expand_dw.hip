@@ -482,13 +482,16 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
   }
 }
 
-// 1 when tfhip_fused_pointwise_depthwise takes this shape and is expected to beat the two
-// kernels, else 0. Measured at batch 32 in sequence, where the expanded tensor really goes to
-// memory and back (fused against expansion + depthwise stage): 16 -> 96 channels at 112x112,
-// stride 2: 43 us against 38 + 55; 24 -> 144 at 56x56, stride 2: 27 against 19 + 18, stride 1:
-// 49 against 19 + 36; 32 -> 192 at 28x28, where the expanded tensor (19 MB) stays in cache:
-// 24 and 27 against 27 and 25 at stride 1, 38 against 21 at stride 2. So: an expanded
-// tensor of at least 48 MB.
+// 1 when tfhip_fused_pointwise_depthwise takes this shape and is expected to beat the two kernels,
+// else 0. The streaming kernel and the channel-sliced one pay at every batch size: at batch 32 the
+// expanded tensor no longer goes to memory and back, and at small batches, where both separate
+// launches are all latency, one launch replaces two (MobileNetV2 through the graph model as a
+// recorded launch sequence, all 17 pairs fused against the two kernels each: 0.284 against 0.296
+// ms at batch 1, 0.298 against 0.331 at batch 4, 0.407 against 0.424 at batch 16). The row-ring
+// kernel, which is what is left for shapes neither of them takes, pays from an expanded tensor of
+// 48 MB (measured at batch 32 in sequence: 16 -> 96 channels at 112x112, stride 2: 43 us against
+// 38 + 55; 32 -> 192 at 28x28, where the expanded tensor of 19 MB stays in cache: 38 against 21
+// at stride 2).
 extern "C" int tfhip_pointwise_depthwise_pays(int64_t batch, int64_t in_c, int64_t mid_c, int64_t stride,
                                               int64_t out_h, int64_t out_w) {
   if (!initialised() || batch <= 0 || out_h <= 0 || out_w <= 0 || mid_c <= 0 || mid_c > 0x7fffffff || in_c <= 0 ||
@@ -503,12 +506,17 @@ extern "C" int tfhip_pointwise_depthwise_pays(int64_t batch, int64_t in_c, int64
   ExpandDwTileArgs t = {};
   t.batch = (int)batch; t.cin = (int)in_c; t.c = (int)mid_c; t.stride = (int)stride; t.out_h = (int)out_h; t.out_w = (int)out_w;
   const bool tile_ok = plan_expand_dw_tile(t, &lds_bytes);
-  if (!ring_ok && !tile_ok) return 0;
+  ExpandDwStreamArgs st = {};
+  st.batch = (int)batch; st.cin = (int)in_c; st.c = (int)mid_c; st.stride = (int)stride; st.out_h = (int)out_h; st.out_w = (int)out_w;
+  const bool stream_ok = tuning(kTunePwDwStream) != 0 && plan_expand_dw_stream(st);
+  if (!ring_ok && !tile_ok && !stream_ok) return 0;
   if (tuning(kTuneFusePwDw) >= 0) return tuning(kTuneFusePwDw) > 0 ? 1 : 0;   // knob: always / never
+  // (the maps on which the entry point runs the streaming kernel by choice; elsewhere it is only the
+  // fallback for a channel count the channel-sliced kernel does not divide, and priced like the ring)
+  const bool wide = out_w * stride >= 56 || (stride == 1 && out_w * stride >= 28 && in_c <= 32);
+  if (tile_ok || (stream_ok && wide)) return 1;
   const int64_t expanded_bytes = batch * out_h * stride * out_w * stride * mid_c * 4;
-  if (ring_ok && expanded_bytes >= 48LL * 1000 * 1000) return 1;
-  // the tile kernel: one launch instead of two once the launch has enough workgroups to fill the chip
-  return tile_ok && (long long)t.batch * t.chunks_h * t.slices >= num_cus() / 2 ? 1 : 0;
+  return expanded_bytes >= 48LL * 1000 * 1000 ? 1 : 0;
 }
 
 namespace {
@@ -597,8 +605,9 @@ extern "C" int tfhip_fused_conv2d_depthwise(const float *x, const float *filter,
   }
 }
 
-// 1 when tfhip_fused_conv2d_depthwise takes this shape and is expected to beat the two kernels (the
-// tensor between the stages of at least 48 MB, as for the pointwise first stage), else 0.
+// 1 when tfhip_fused_conv2d_depthwise takes this shape and is expected to beat the two kernels, else
+// 0: always where the streaming kernel takes it, from a tensor of 48 MB between the stages where
+// only the row-ring kernel does (as for the pointwise first stage).
 extern "C" int tfhip_conv2d_depthwise_pays(int64_t batch, int64_t in_c, int64_t f_h, int64_t f_w, int64_t mid_c,
                                            int64_t mid_h, int64_t mid_w, int64_t dw_stride, int64_t out_h,
                                            int64_t out_w) {
@@ -612,5 +621,9 @@ extern "C" int tfhip_conv2d_depthwise_pays(int64_t batch, int64_t in_c, int64_t 
   size_t lds_bytes = 0;
   if (!plan_expand_dw(g, (int)dw_stride, 4 * stem_k_steps(f_h * f_w * in_c), &lds_bytes)) return 0;
   if (tuning(kTuneFusePwDw) >= 0) return tuning(kTuneFusePwDw) > 0 ? 1 : 0;
+  ExpandDwStreamArgs st = {};
+  st.batch = (int)batch; st.cin = (int)in_c; st.c = (int)mid_c; st.stride = (int)dw_stride; st.out_h = (int)out_h; st.out_w = (int)out_w;
+  st.k_steps = stem_k_steps(f_h * f_w * in_c);
+  if (tuning(kTunePwDwStream) != 0 && plan_expand_dw_stream(st)) return 1;
   return batch * mid_h * mid_w * mid_c * 4 >= 48LL * 1000 * 1000 ? 1 : 0;
 }
