@@ -104,16 +104,26 @@ __device__ __forceinline__ float finish(const Epilogue &e, float v, long long ba
   return activate(v, e.activation, alpha, e.leaky_alpha);
 }
 
-// The float4 store every kernel writes its results with. TFHIP_NT_OUT (a build-time switch for
-// measurement) makes it a streaming store.
+// The float4 stores the kernels write their results with. The streaming form (a non-temporal
+// store: the line is not kept in the cache) is for outputs whose next reader gains nothing from
+// finding them there and whose stores are pieces of cache lines, which the cache would otherwise
+// collect: the fused expansion + depthwise kernels on the small maps, where a lane writes 16
+// bytes of a pixel's 1.5 - 4 KB of channels (MobileNetV2 at batch 32, in sequence: the eleven tile-
+// kernel launches 177 -> 154 us, the projections that read those outputs unchanged). The outputs of
+// the GEMMs stay cached: the streaming kernels that read them lose 2 - 5 us each when they come
+// from memory. TFHIP_NT_OUT is a build-time switch for measurement that makes every result store a
+// streaming one.
 #ifndef TFHIP_NT_OUT
 #define TFHIP_NT_OUT 0
 #endif
-__device__ __forceinline__ void store_result4(float *p, float4 v) {
-#if TFHIP_NT_OUT
+__device__ __forceinline__ void store_result4_streaming(float *p, float4 v) {
   typedef float result4_t __attribute__((ext_vector_type(4)));
   const result4_t t = {v.x, v.y, v.z, v.w};
   __builtin_nontemporal_store(t, reinterpret_cast<result4_t *>(p));
+}
+__device__ __forceinline__ void store_result4(float *p, float4 v) {
+#if TFHIP_NT_OUT
+  store_result4_streaming(p, v);
 #else
   *reinterpret_cast<float4 *>(p) = v;
 #endif

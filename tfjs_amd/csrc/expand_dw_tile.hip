@@ -247,7 +247,7 @@ __global__ __launch_bounds__(256) void expand_dw_tile(ExpandDwTileArgs g) {
       out.y = relu_cap(acc.y + b2q.y, g.cap);
       out.z = relu_cap(acc.z + b2q.z, g.cap);
       out.w = relu_cap(acc.w + b2q.w, g.cap);
-      store_result4(g.y + (((long long)n * g.out_h + oh0 + o) * g.out_w + q) * g.c + c0 + 4 * c4, out);
+      store_result4_streaming(g.y + (((long long)n * g.out_h + oh0 + o) * g.out_w + q) * g.c + c0 + 4 * c4, out);
     }
   }
 }
