@@ -41,8 +41,15 @@ struct SkinnyArgs {
 constexpr int kSkinnyChunk = 64;   // k per pipeline step: four float4 per lane
 constexpr int kSkinnyPad = 8;      // LDS row pitch k_pad + 8: the pitch the 16-byte fragment reads run fastest at
 
-// WAVES wavefronts per workgroup share one copy of B.
-template <int TN, int WAVES>
+// Cache policy of the fetches of A. Every element of A is read once, so a large A (beyond what the L2
+// caches hold together) is fetched non-temporally: it would only push out what later kernels still
+// want to find there - weights, residuals, the network's input (MobileNetV2 at batch 32, in
+// sequence: the three launches here get 5 us slower in total and the rest of the inference 17 us
+// faster).
+constexpr long long kSkinnyStreamBytes = 32LL << 20;
+
+// WAVES wavefronts per workgroup share one copy of B. STREAM_A: see above.
+template <int TN, int WAVES, bool STREAM_A>
 __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
   constexpr int kThreads = WAVES * 64;
   extern __shared__ float lds_bt[];          // [16 * TN][k_pad + kSkinnyPad]: B transposed, zero padded
@@ -67,7 +74,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
     for (int t = 0; t < 4; ++t) {
       const int k = c * kSkinnyChunk + 16 * t + 4 * grp;
       const unsigned off = (row < g.M && k < g.K) ? (unsigned)(((long long)row * g.K + k) * 4) : kNoOffset;
-      dst[t] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
+      dst[t] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, STREAM_A ? 2 : 0));
     }
   };
 
@@ -213,7 +220,7 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
 //   KF    full k groups of 16 (lane takes k = 16 t + 4 g + j, a float4 of A)
 //   HALF  one more group of 8 (lane takes k = 16 KF + 2 g + j, a float2 of A):
 //         K = 24 costs six matrix instructions per block instead of eight
-template <int TN, int KF, bool HALF>
+template <int TN, int KF, bool HALF, bool STREAM_A>
 __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
   constexpr int STEPS = 4 * KF + (HALF ? 2 : 0);
   const int lane = threadIdx.x & 63;
@@ -236,12 +243,12 @@ __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
     for (int t = 0; t < KF; ++t) {
       const int k = 16 * t + 4 * grp;
       const unsigned off = (row_ok && k < g.K) ? (unsigned)(((long long)row * g.K + k) * 4) : kNoOffset;
-      dst.full[t] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
+      dst.full[t] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, STREAM_A ? 2 : 0));
     }
     if (HALF) {
       const int k = 16 * KF + 2 * grp;
       const unsigned off = (row_ok && k < g.K) ? (unsigned)(((long long)row * g.K + k) * 4) : kNoOffset;
-      const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)off, 0, 0);
+      const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)off, 0, STREAM_A ? 2 : 0);
       dst.half = make_float2(__uint_as_float(v[0]), __uint_as_float(v[1]));
     }
   };
@@ -314,7 +321,7 @@ inline int launch_skinny_regs(const SkinnyArgs &g, int column_groups) {
   static int resident = 0;   // workgroups per compute unit at this instantiation's register count
   if (resident == 0) {
     int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_gemm_regs<TN, KF, HALF>, 256, 0) != hipSuccess || n < 1) {
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_gemm_regs<TN, KF, HALF, false>, 256, 0) != hipSuccess || n < 1) {
       (void)hipGetLastError();
       n = 1;
     }
@@ -327,8 +334,13 @@ inline int launch_skinny_regs(const SkinnyArgs &g, int column_groups) {
   if (cap < 1) cap = 1;
   if (grid > cap) grid = cap;
   note_kernel("skinny_gemm_regs<%d, %d, %s>", TN, KF, HALF ? "true" : "false");
-  TFHIP_LAUNCH((skinny_gemm_regs<TN, KF, HALF>
-                <<<dim3((unsigned)grid, (unsigned)column_groups), dim3(256), 0, stream()>>>(g)));
+  if ((long long)g.M * g.K * 4 >= kSkinnyStreamBytes) {
+    TFHIP_LAUNCH((skinny_gemm_regs<TN, KF, HALF, true>
+                  <<<dim3((unsigned)grid, (unsigned)column_groups), dim3(256), 0, stream()>>>(g)));
+  } else {
+    TFHIP_LAUNCH((skinny_gemm_regs<TN, KF, HALF, false>
+                  <<<dim3((unsigned)grid, (unsigned)column_groups), dim3(256), 0, stream()>>>(g)));
+  }
   return kOk;
 }
 
@@ -383,7 +395,11 @@ inline int launch_skinny_tn(const SkinnyArgs &g) {
   const long long cap = (long long)num_cus() * 3;
   if (grid > cap) grid = cap;
   note_kernel("skinny_gemm<%d, %d>", TN, WAVES);
-  TFHIP_LAUNCH((skinny_gemm<TN, WAVES><<<dim3((unsigned)grid), dim3(WAVES * 64), lds, stream()>>>(g)));
+  if ((long long)g.M * g.K * 4 >= kSkinnyStreamBytes) {
+    TFHIP_LAUNCH((skinny_gemm<TN, WAVES, true><<<dim3((unsigned)grid), dim3(WAVES * 64), lds, stream()>>>(g)));
+  } else {
+    TFHIP_LAUNCH((skinny_gemm<TN, WAVES, false><<<dim3((unsigned)grid), dim3(WAVES * 64), lds, stream()>>>(g)));
+  }
   return kOk;
 }
 
