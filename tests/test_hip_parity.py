@@ -351,6 +351,25 @@ def test_depthwise_row_chunks(hip, orc, tuning, rows, stride, pad):
     assert_parity(hip.fused_depthwise_conv2d(x, w, **kw), orc.fused_depthwise_conv2d(x, w, **kw))
 
 
+@pytest.mark.parametrize("stride", [1, 2])
+def test_depthwise_large_result_is_streamed(hip, orc, stride):
+    # a result of 32 MB or more is stored non-temporally: same values, another kernel variant
+    from tfjs_amd.capi import load_library
+    rng = np.random.default_rng(37 + stride)
+    x = rng.uniform(-1, 1, (4, 128 * stride, 129 * stride, 128)).astype(np.float32)
+    w = rng.normal(0, 0.5, (3, 3, 128, 1)).astype(np.float32)
+    kw = dict(pad="same", strides=stride, bias=rng.uniform(-1, 1, (128,)).astype(np.float32), activation="relu6")
+    got = hip.fused_depthwise_conv2d(x, w, **kw)
+    name = ctypes.create_string_buffer(256)
+    load_library().tfhip_last_kernel(name, 256)
+    assert name.value.decode() == "depthwise_3x3_rows<%d, false, true>" % stride, name.value
+    assert_parity(got, orc.fused_depthwise_conv2d(x, w, **kw))
+    small = hip.fused_depthwise_conv2d(x[:3], w, **kw)
+    load_library().tfhip_last_kernel(name, 256)
+    assert name.value.decode() == "depthwise_3x3_rows<%d, false, false>" % stride, name.value
+    assert np.array_equal(small, got[:3])
+
+
 def test_depthwise_linearity_full_size(hip):
     # size-independent property at the benchmark shape: conv(x1 + x2) = conv(x1) + conv(x2)
     c = synth.config3(1)

@@ -149,6 +149,9 @@ constexpr int kRowsPW = 4;   // output columns per lane
 #define DW_WAVES 1
 #endif
 constexpr unsigned kDwNoOffset = 0xffffffffu;
+// Results of at least this many bytes are stored non-temporally: all eight L2
+// caches together hold 32 MB, so such a result cannot wait there for its reader.
+constexpr long long kDwStreamBytes = 32LL << 20;
 typedef unsigned int dw_uint4 __attribute__((ext_vector_type(4)));
 
 struct DwRowsArgs {
@@ -182,10 +185,13 @@ __device__ __forceinline__ float4 dw_load4(__amdgpu_buffer_rsrc_t r, unsigned of
   return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
 }
 
+// STREAM: a non-temporal store, for a result too large to still be in the cache
+// when its reader starts (it would only push out what the reader does find there).
+template <bool STREAM>
 __device__ __forceinline__ void dw_store4(__amdgpu_buffer_rsrc_t r, unsigned off, float4 v) {
   dw_uint4 u;
   u.x = __float_as_uint(v.x); u.y = __float_as_uint(v.y); u.z = __float_as_uint(v.z); u.w = __float_as_uint(v.w);
-  __builtin_amdgcn_raw_buffer_store_b128(u, r, (int)off, 0, TFHIP_NT_OUT ? 2 : 0);
+  __builtin_amdgcn_raw_buffer_store_b128(u, r, (int)off, 0, (STREAM || TFHIP_NT_OUT) ? 2 : 0);
 }
 
 // Bias + activation of four channels. The common case (per-channel operands,
@@ -235,7 +241,7 @@ __device__ __forceinline__ void dw_load_row(const DwRowsState<S> &st, __amdgpu_b
 
 // Scatters input row i into the output rows it is a tap row of; PHASE is i
 // modulo the rotation period of the accumulators, so slots are compile-time.
-template <int S, int PHASE, bool GENERAL>
+template <int S, int PHASE, bool GENERAL, bool STREAM>
 __device__ __forceinline__ void dw_compute_row(DwRowsState<S> &st, const Epilogue &e, __amdgpu_buffer_rsrc_t ry,
                                                int i, const float4 (&in)[DwRowsState<S>::NIN]) {
   using St = DwRowsState<S>;
@@ -270,25 +276,25 @@ __device__ __forceinline__ void dw_compute_row(DwRowsState<S> &st, const Epilogu
 #pragma unroll
       for (int x = 0; x < kRowsPW; ++x) {
         const unsigned off = (row_ok && st.y_col[x] != kDwNoOffset) ? row_off + st.y_col[x] : kDwNoOffset;
-        dw_store4(ry, off, dw_finish4<GENERAL>(e, st.acc[slot][x], st.bias4, st.c, st.n, oh, st.ow0 + x));
+        dw_store4<STREAM>(ry, off, dw_finish4<GENERAL>(e, st.acc[slot][x], st.bias4, st.c, st.n, oh, st.ow0 + x));
       }
     }
   }
 }
 
 // One pipeline step: `a` holds input row i0+K, `b` receives row i0+K+1.
-template <int S, int K, bool GENERAL>
+template <int S, int K, bool GENERAL, bool STREAM>
 __device__ __forceinline__ void dw_step(DwRowsState<S> &st, const Epilogue &e, __amdgpu_buffer_rsrc_t rx,
                                         __amdgpu_buffer_rsrc_t ry, int i0, const float4 (&a)[DwRowsState<S>::NIN],
                                         float4 (&b)[DwRowsState<S>::NIN]) {
   constexpr int PERIOD = S * DwRowsState<S>::NSLOT;
   if (i0 + K >= st.rows_in) return;
   dw_load_row<S>(st, rx, i0 + K + 1, b);
-  dw_compute_row<S, K % PERIOD, GENERAL>(st, e, ry, i0 + K, a);
+  dw_compute_row<S, K % PERIOD, GENERAL, STREAM>(st, e, ry, i0 + K, a);
 }
 
 // GENERAL = false: per-channel bias and a relu-family activation, all inline.
-template <int S, bool GENERAL>
+template <int S, bool GENERAL, bool STREAM>
 __global__ __launch_bounds__(256, DW_WAVES) void depthwise_3x3_rows(DwParams p, Epilogue e, DwRowsArgs g) {
   using St = DwRowsState<S>;
   const int c4 = blockIdx.y * kCQ + (threadIdx.x % kCQ);
@@ -343,13 +349,13 @@ __global__ __launch_bounds__(256, DW_WAVES) void depthwise_3x3_rows(DwParams p, 
   float4 cur[St::NIN], nxt[St::NIN];
   dw_load_row<S>(st, rx, 0, cur);
   for (int i0 = 0; i0 < st.rows_in; i0 += UNROLL) {
-    dw_step<S, 0, GENERAL>(st, e, rx, ry, i0, cur, nxt);
-    dw_step<S, 1, GENERAL>(st, e, rx, ry, i0, nxt, cur);
-    dw_step<S, 2, GENERAL>(st, e, rx, ry, i0, cur, nxt);
-    dw_step<S, 3, GENERAL>(st, e, rx, ry, i0, nxt, cur);
+    dw_step<S, 0, GENERAL, STREAM>(st, e, rx, ry, i0, cur, nxt);
+    dw_step<S, 1, GENERAL, STREAM>(st, e, rx, ry, i0, nxt, cur);
+    dw_step<S, 2, GENERAL, STREAM>(st, e, rx, ry, i0, cur, nxt);
+    dw_step<S, 3, GENERAL, STREAM>(st, e, rx, ry, i0, nxt, cur);
     if (UNROLL > 4) {
-      dw_step<S, 4, GENERAL>(st, e, rx, ry, i0, cur, nxt);
-      dw_step<S, 5, GENERAL>(st, e, rx, ry, i0, nxt, cur);
+      dw_step<S, 4, GENERAL, STREAM>(st, e, rx, ry, i0, cur, nxt);
+      dw_step<S, 5, GENERAL, STREAM>(st, e, rx, ry, i0, nxt, cur);
     }
   }
 }
@@ -409,9 +415,9 @@ __global__ __launch_bounds__(256) void depthwise_3x3_flat(DwParams p, Epilogue e
     st.bias4 = make_float4(e.bias[(st.c + 0) * bs], e.bias[(st.c + 1) * bs], e.bias[(st.c + 2) * bs],
                            e.bias[(st.c + 3) * bs]);
   }
-  dw_compute_row<S, 0, GENERAL>(st, e, ry, 0, r0);
-  dw_compute_row<S, 1, GENERAL>(st, e, ry, 1, r1);
-  dw_compute_row<S, 2, GENERAL>(st, e, ry, 2, r2);
+  dw_compute_row<S, 0, GENERAL, false>(st, e, ry, 0, r0);
+  dw_compute_row<S, 1, GENERAL, false>(st, e, ry, 1, r1);
+  dw_compute_row<S, 2, GENERAL, false>(st, e, ry, 2, r2);
 }
 
 int balanced_tile(int extent, int max_tile) {
@@ -588,15 +594,20 @@ extern "C" int tfhip_fused_depthwise_conv2d(
     if (blocks_x <= 0x7fffffffLL) {
       dim3 grid((unsigned)blocks_x, (g.c4_total + kCQ - 1) / kCQ, 1);
       const bool general = !(e.addressing == kChannel && activation <= TFHIP_RELU6);
-      note_kernel("depthwise_3x3_rows<%d, %s>", S, general ? "true" : "false");
-      if (S == 1 && !general)
-        TFHIP_LAUNCH((depthwise_3x3_rows<1, false><<<grid, 256, 0, stream()>>>(p, e, g)));
+      const bool streamed = !general && total * 4 >= kDwStreamBytes;
+      note_kernel("depthwise_3x3_rows<%d, %s, %s>", S, general ? "true" : "false", streamed ? "true" : "false");
+      if (S == 1 && streamed)
+        TFHIP_LAUNCH((depthwise_3x3_rows<1, false, true><<<grid, 256, 0, stream()>>>(p, e, g)));
+      else if (S == 1 && !general)
+        TFHIP_LAUNCH((depthwise_3x3_rows<1, false, false><<<grid, 256, 0, stream()>>>(p, e, g)));
       else if (S == 1)
-        TFHIP_LAUNCH((depthwise_3x3_rows<1, true><<<grid, 256, 0, stream()>>>(p, e, g)));
+        TFHIP_LAUNCH((depthwise_3x3_rows<1, true, false><<<grid, 256, 0, stream()>>>(p, e, g)));
+      else if (streamed)
+        TFHIP_LAUNCH((depthwise_3x3_rows<2, false, true><<<grid, 256, 0, stream()>>>(p, e, g)));
       else if (!general)
-        TFHIP_LAUNCH((depthwise_3x3_rows<2, false><<<grid, 256, 0, stream()>>>(p, e, g)));
+        TFHIP_LAUNCH((depthwise_3x3_rows<2, false, false><<<grid, 256, 0, stream()>>>(p, e, g)));
       else
-        TFHIP_LAUNCH((depthwise_3x3_rows<2, true><<<grid, 256, 0, stream()>>>(p, e, g)));
+        TFHIP_LAUNCH((depthwise_3x3_rows<2, true, false><<<grid, 256, 0, stream()>>>(p, e, g)));
       return kOk;
     }
   }
