@@ -396,7 +396,7 @@ def test_matmul_tall_small_b(hip, orc, m, n, k, act):
 @pytest.mark.parametrize("regs", [0, 1])
 @pytest.mark.parametrize("m,n,k,act", [(65537, 16, 8, "relu"), (66000, 32, 12, "linear"), (65700, 48, 20, "relu6"),
                                         (65600, 64, 28, "leakyrelu"), (65536, 96, 32, "relu6"), (98400, 144, 16, "relu"),
-                                        (98310, 136, 24, "relu6")])
+                                        (98310, 136, 24, "relu6"), (270001, 16, 32, "relu6"), (1100000, 24, 8, "relu")])
 def test_matmul_tall_tiny_k(hip, orc, tuning, m, n, k, act, regs):
     # K <= 32: B lives in registers (every column-group count, full and half k groups), or in LDS when told so
     tuning("skinny_regs", regs)
@@ -405,6 +405,12 @@ def test_matmul_tall_tiny_k(hip, orc, tuning, m, n, k, act, regs):
     b = rng.normal(0, 0.3, (k, n)).astype(np.float32)
     kw = dict(bias=rng.uniform(-1, 1, (n,)).astype(np.float32), activation=act, leakyrelu_alpha=0.1)
     assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
+    # an A of 32 MB or more is fetched non-temporally: the variant shows in the symbol
+    from tfjs_amd.capi import load_library
+    name = ctypes.create_string_buffer(256)
+    load_library().tfhip_last_kernel(name, 256)
+    assert name.value.decode().startswith("skinny_gemm")
+    assert name.value.decode().endswith("true>" if m * k * 4 >= 32 << 20 else "false>"), name.value
 
 
 @pytest.mark.parametrize("rows", [32, 64])

@@ -333,8 +333,9 @@ inline int launch_skinny_regs(const SkinnyArgs &g, int column_groups) {
   long long cap = (long long)num_cus() * resident / column_groups;
   if (cap < 1) cap = 1;
   if (grid > cap) grid = cap;
-  note_kernel("skinny_gemm_regs<%d, %d, %s>", TN, KF, HALF ? "true" : "false");
-  if ((long long)g.M * g.K * 4 >= kSkinnyStreamBytes) {
+  const bool stream_a = (long long)g.M * g.K * 4 >= kSkinnyStreamBytes;
+  note_kernel("skinny_gemm_regs<%d, %d, %s, %s>", TN, KF, HALF ? "true" : "false", stream_a ? "true" : "false");
+  if (stream_a) {
     TFHIP_LAUNCH((skinny_gemm_regs<TN, KF, HALF, true>
                   <<<dim3((unsigned)grid, (unsigned)column_groups), dim3(256), 0, stream()>>>(g)));
   } else {
@@ -394,8 +395,9 @@ inline int launch_skinny_tn(const SkinnyArgs &g) {
   long long grid = (blocks + WAVES - 1) / WAVES;
   const long long cap = (long long)num_cus() * 3;
   if (grid > cap) grid = cap;
-  note_kernel("skinny_gemm<%d, %d>", TN, WAVES);
-  if ((long long)g.M * g.K * 4 >= kSkinnyStreamBytes) {
+  const bool stream_a = (long long)g.M * g.K * 4 >= kSkinnyStreamBytes;
+  note_kernel("skinny_gemm<%d, %d, %s>", TN, WAVES, stream_a ? "true" : "false");
+  if (stream_a) {
     TFHIP_LAUNCH((skinny_gemm<TN, WAVES, true><<<dim3((unsigned)grid), dim3(WAVES * 64), lds, stream()>>>(g)));
   } else {
     TFHIP_LAUNCH((skinny_gemm<TN, WAVES, false><<<dim3((unsigned)grid), dim3(WAVES * 64), lds, stream()>>>(g)));
