@@ -1102,6 +1102,20 @@ def test_pointwise_depthwise_without_biases_and_unsupported_shapes(hip, orc):
                                       rng.normal(0, 1, (1, 1, 12, 32)).astype(np.float32), w2)
 
 
+def test_fused_pairs_refuse_sizes_that_overflow(hip):
+    # dimensions whose product does not fit 64 bits are refused before anything is computed with them
+    from tfjs_amd import capi
+    lib = capi.load_library()
+    big = 1 << 40
+    with capi.DeviceBuffer(64) as buf:
+        p = buf.ptr
+        rc = lib.tfhip_fused_pointwise_depthwise(p, p, None, 1, p, None, 1, p, big, big, big, 16, 32, 1, 0, 0, big, big)
+        assert rc != 0 and "supported range" in lib.tfhip_last_error().decode()
+        rc = lib.tfhip_fused_conv2d_depthwise(p, p, None, 1, p, None, 1, p, big, big, big, 3, 3, 3, 32, 2, 0, 0, big, big,
+                                              1, 1, 1, big, big)
+        assert rc != 0 and "supported range" in lib.tfhip_last_error().decode()
+
+
 # -------------------------------------------------- recorded launch sequences
 
 def test_recorded_graph_replays(hip, orc):

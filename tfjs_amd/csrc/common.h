@@ -1,6 +1,7 @@
 // Internal declarations shared by the translation units of libtfjs_hip.so.
 #pragma once
 
+#include <initializer_list>
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdint.h>
@@ -45,6 +46,18 @@ int setup_static_scratch(int device);
 
 // True when [p, p + bytes) lies inside one live block (own or external).
 bool range_is_live(const void *p, size_t bytes);
+// True when the product of the non-negative factors is below `limit`, decided
+// without forming a product that could overflow 64 bits.
+inline bool product_below(int64_t limit, std::initializer_list<int64_t> factors) {
+  int64_t p = 1;
+  for (const int64_t f : factors) {
+    if (f < 0) return false;
+    if (f == 0) return limit > 0;
+    if (p > (limit - 1) / f) return false;
+    p *= f;
+  }
+  return p < limit;
+}
 // True between tfhip_capture_begin and tfhip_capture_end.
 bool capturing();
 

@@ -391,7 +391,8 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
                       pad_top >= 0 && pad_left >= 0,
                   "tfhip_fused_pointwise_depthwise: bad dimension");
   const int64_t lim = 0x7fffffff;
-  TFHIP_CHECK_ARG(batch * in_h * in_w * (in_c > mid_c ? in_c : mid_c) < lim && batch * out_h * out_w * mid_c < lim,
+  TFHIP_CHECK_ARG(product_below(lim, {batch, in_h, in_w, in_c > mid_c ? in_c : mid_c}) &&
+                      product_below(lim, {batch, out_h, out_w, mid_c}) && stride < lim && pad_top < lim && pad_left < lim,
                   "tfhip_fused_pointwise_depthwise: tensor exceeds the supported range");
   TFHIP_CHECK_ARG(batch * in_h * in_w * in_c * 4 <= 0xfffffffeLL,
                   "tfhip_fused_pointwise_depthwise: x exceeds the 4 GiB one buffer descriptor addresses");
@@ -538,7 +539,10 @@ extern "C" int tfhip_fused_conv2d_depthwise(const float *x, const float *filter,
                       pad_left >= 0 && dw_pad_top >= 0 && dw_pad_left >= 0,
                   "tfhip_fused_conv2d_depthwise: bad dimension");
   const int64_t lim = 0x7fffffff;
-  TFHIP_CHECK_ARG(batch * in_h * in_w * in_c < lim && batch * mid_h * mid_w * mid_c < lim && batch * out_h * out_w * mid_c < lim,
+  TFHIP_CHECK_ARG(product_below(lim, {batch, in_h, in_w, in_c}) && product_below(lim, {batch, mid_h, mid_w, mid_c}) &&
+                      product_below(lim, {batch, out_h, out_w, mid_c}) && product_below(lim, {f_h, f_w, in_c, mid_c}) &&
+                      stride < lim && dw_stride < lim && pad_top < lim && pad_left < lim && dw_pad_top < lim &&
+                      dw_pad_left < lim,
                   "tfhip_fused_conv2d_depthwise: tensor exceeds the supported range");
   TFHIP_CHECK_ARG(activation >= TFHIP_LINEAR && activation <= TFHIP_ELU && dw_activation >= TFHIP_LINEAR &&
                       dw_activation <= TFHIP_ELU,
