@@ -443,19 +443,29 @@ __global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
   //   pieces A_VECS .. A_VECS+B_VECS-1  the same for B
   //   then the global fetches of tile kt+4 into the ring slot just drained, A and
   //   B as one piece each.
-  // The next quad's fragments are fetched in group 2 of each quad; for the last
-  // quad of a tile they come from tile kt+1, so its stores and the barrier must
-  // be over by group 1 of that quad.
+  // The next quad's fragments are fetched in group 2 of each quad (group 0 for the smallest
+  // wave tiles, below); for the last quad of a tile they come from tile kt+1, so its stores and
+  // the barrier must be over by the group before.
+  // A wavefront with a single block has groups of one matrix instruction: two groups are 64
+  // cycles, less than an LDS read takes, and every quad then began with a wait for its
+  // fragments. There the next quad's fragments are fetched in group 0, a whole quad ahead, and
+  // the barrier comes as late as that allows, so that the tile stores in front of it have the
+  // longest time to complete (256 x 512 x 512 on the 32 x 32 x 32 tile: 7.0 -> 6.55 us back to
+  // back; the fifteen MobileNetV2 projections on that tile 0.1 - 0.5 us each).
   constexpr int Q = T::QUADS;
+  constexpr bool kFewBlocks = T::TM * T::TN == 1 && Q >= 2;
+  constexpr int kFetchGroup = kFewBlocks ? 0 : 2;   // group of a quad that fetches the next quad's fragments
   constexpr int kGroups = 4 * Q;
   constexpr int kStores = T::A_VECS + T::B_VECS;
   constexpr int kPieces = kStores + 2;
   constexpr int kEven = (kPieces + kGroups - 1) / kGroups;
-  constexpr int kStoreGroups = 4 * (Q - 1) + 2;
+  constexpr int kStoreGroups = 4 * (Q - 1) + kFetchGroup;   // groups in front of the fetch from tile kt+1
   constexpr int kForStores = (kStores + kStoreGroups - 1) / kStoreGroups;
   constexpr int kPerGroup = kEven > kForStores ? kEven : kForStores;
-  constexpr int kBarrierGroup = (kStores - 1) / kPerGroup;   // the group that holds the last store
-  static_assert(kBarrierGroup <= 4 * (Q - 1) + 1, "fragments of the next tile are read after the barrier");
+  constexpr int kLastStoreGroup = (kStores - 1) / kPerGroup;
+  constexpr int kBarrierGroup = kFewBlocks ? kStoreGroups - 1 : kLastStoreGroup;
+  static_assert(kLastStoreGroup <= kBarrierGroup && kBarrierGroup < kStoreGroups,
+                "the barrier follows the last store and precedes the fetch of the next tile's fragments");
 
   // One k tile: tile kt = L * n + i sits in LDS buffer u = i % 3, tile kt+1 in ring slot (i+1) % D and
   // goes to LDS buffer (u+1) % 3.
@@ -471,7 +481,7 @@ __global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
         constexpr int kDummy = 0;
         (void)kDummy;
         const int group = quad * 4 + j;
-        if (j == 2) {
+        if (j == kFetchGroup) {
           if (quad + 1 < Q) {
             load_fragment<T::PITCH, T::TM>(na, a_lane, a_off, quad + 1);
             load_fragment<T::PITCH, T::TN>(nb4, b_lane, b_off, quad + 1);
