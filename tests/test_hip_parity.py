@@ -393,6 +393,28 @@ def test_matmul_tall_small_b(hip, orc, m, n, k, act):
     assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
 
 
+@pytest.mark.parametrize("m,n,k,act", [(90001, 24, 96, "relu6"), (65600, 24, 144, "linear"), (65601, 16, 192, "relu"),
+                                        (70000, 32, 144, "leakyrelu")])
+def test_matmul_tall_a_through_lds(hip, orc, tuning, m, n, k, act):
+    # a streamed A (32 MB or more) with K = 96 / 144 / 192 and at most 32 columns is fetched as whole row
+    # blocks and staged in LDS: same values, bit for bit, as the direct fetch
+    from tfjs_amd.capi import load_library
+    rng = np.random.default_rng(m + n + k)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 0.3, (k, n)).astype(np.float32)
+    kw = dict(bias=rng.uniform(-1, 1, (n,)).astype(np.float32), activation=act, leakyrelu_alpha=0.1)
+    name = ctypes.create_string_buffer(256)
+    got = hip.fused_matmul(a, b, **kw)
+    load_library().tfhip_last_kernel(name, 256)
+    assert name.value.decode() == "skinny_gemm<%d, 4, true, %d>" % ((n + 15) // 16, k // 16), name.value
+    assert_parity(got, orc.fused_matmul(a, b, **kw))
+    tuning("skinny_stage", 0)
+    direct = hip.fused_matmul(a, b, **kw)
+    load_library().tfhip_last_kernel(name, 256)
+    assert name.value.decode() == "skinny_gemm<%d, 4, true>" % ((n + 15) // 16), name.value
+    np.testing.assert_array_equal(got.view(np.uint32), direct.view(np.uint32))
+
+
 @pytest.mark.parametrize("regs", [0, 1])
 @pytest.mark.parametrize("m,n,k,act", [(65537, 16, 8, "relu"), (66000, 32, 12, "linear"), (65700, 48, 20, "relu6"),
                                         (65600, 64, 28, "leakyrelu"), (65536, 96, 32, "relu6"), (98400, 144, 16, "relu"),

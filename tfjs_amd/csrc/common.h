@@ -111,7 +111,7 @@ int launch_repeat();
 
 // Tuning overrides (tfhip_set_tuning, or TFHIP_<NAME> in the environment at
 // tfhip_init): -1 when unset.
-enum TuningKey { kTuneTile = 0, kTuneSplitK, kTuneDwRows, kTuneDwHalo, kTuneNoSkinny, kTuneDwFlat, kTuneSkinnyRegs, kTuneSmallK, kTuneFusePwDw, kTunePwDwTile, kTuneTileSlice, kTuneTileChunks, kTuneBlockRows, kTuneFuseBlock, kTuneKGroups, kTunePwDwStream, kTuneStreamRows, kTuneStreamBlocks, kTuneCount };
+enum TuningKey { kTuneTile = 0, kTuneSplitK, kTuneDwRows, kTuneDwHalo, kTuneNoSkinny, kTuneDwFlat, kTuneSkinnyRegs, kTuneSmallK, kTuneFusePwDw, kTunePwDwTile, kTuneTileSlice, kTuneTileChunks, kTuneBlockRows, kTuneFuseBlock, kTuneKGroups, kTunePwDwStream, kTuneStreamRows, kTuneStreamBlocks, kTuneSkinnyStage, kTuneCount };
 int tuning(int key);
 
 // Enqueues `launch_expr` launch_repeat() times and checks the launch.

@@ -117,7 +117,7 @@ int launch_repeat() { return g_repeat; }
 
 int g_init_count = 0;
 int g_tuning[kTuneCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
-const char *const kTuningNames[kTuneCount] = {"tile", "splitk", "dw_rows", "dw_halo", "no_skinny", "dw_flat", "skinny_regs", "small_k", "fuse_pw_dw", "pw_dw_tile", "tile_slice", "tile_chunks", "block_rows", "fuse_block", "k_groups", "pw_dw_stream", "stream_rows", "stream_blocks"};
+const char *const kTuningNames[kTuneCount] = {"tile", "splitk", "dw_rows", "dw_halo", "no_skinny", "dw_flat", "skinny_regs", "small_k", "fuse_pw_dw", "pw_dw_tile", "tile_slice", "tile_chunks", "block_rows", "fuse_block", "k_groups", "pw_dw_stream", "stream_rows", "stream_blocks", "skinny_stage"};
 int tuning(int key) { return g_tuning[key]; }
 
 void read_tuning_from_environment() {
@@ -126,7 +126,7 @@ void read_tuning_from_environment() {
                                                     "TFHIP_SMALL_K", "TFHIP_FUSE_PW_DW", "TFHIP_PW_DW_TILE",
                                                     "TFHIP_TILE_SLICE", "TFHIP_TILE_CHUNKS", "TFHIP_BLOCK_ROWS",
                                                     "TFHIP_FUSE_BLOCK", "TFHIP_K_GROUPS", "TFHIP_PW_DW_STREAM",
-                                                    "TFHIP_STREAM_ROWS", "TFHIP_STREAM_BLOCKS"};
+                                                    "TFHIP_STREAM_ROWS", "TFHIP_STREAM_BLOCKS", "TFHIP_SKINNY_STAGE"};
   for (int i = 0; i < kTuneCount; ++i) {
     const char *e = getenv(env_names[i]);
     g_tuning[i] = e ? atoi(e) : -1;

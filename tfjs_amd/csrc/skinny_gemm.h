@@ -49,7 +49,12 @@ constexpr int kSkinnyPad = 8;      // LDS row pitch k_pad + 8: the pitch the 16-
 constexpr long long kSkinnyStreamBytes = 32LL << 20;
 
 // WAVES wavefronts per workgroup share one copy of B. STREAM_A: see above.
-template <int TN, int WAVES, bool STREAM_A>
+// SV > 0 (K = 16 SV): A goes through LDS. A 16-row block of A is one contiguous piece of memory, so
+// the wavefront fetches it as such - every instruction 1 KB of whole cache lines instead of 64 bytes
+// of each of 16 rows, whose other halves the next instruction asks for again - parks it in a region
+// of LDS of its own (rows 4 floats apart from a multiple of 16: conflict-free fragment reads) and
+// takes its fragments from there; the registers are free for the next block's fetch at once.
+template <int TN, int WAVES, bool STREAM_A, int SV = 0>
 __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
   constexpr int kThreads = WAVES * 64;
   extern __shared__ float lds_bt[];          // [16 * TN][k_pad + kSkinnyPad]: B transposed, zero padded
@@ -92,7 +97,30 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
   // of A, costs a round trip of its own: 3.4 us of an 11 us launch went into them, measured with
   // timestamps inside the kernel).
   float4 cur[4], nxt[4];
-  issue(cur, total > 0 ? first : blocks, 0);   // (no row block: every offset is out of range, nothing is read)
+  constexpr int NV = SV > 0 ? SV : 1;
+  float4 blk[NV];
+  unsigned park[NV];   // where this lane's fetches of a block go in the wavefront's LDS region (float index)
+  const int a_pitch = g.K + 4;
+  float *stage = lds_bt + 16 * TN * pitch + wave * 16 * a_pitch;
+  auto issue_block = [&](int b) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const long long e = (long long)b * 16 * g.K + 4 * (lane + 64 * i);   // first of this lane's four floats
+      const unsigned off = (b < blocks && e * 4 < (long long)g.a_bytes) ? (unsigned)(e * 4) : kNoOffset;
+      blk[i] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, STREAM_A ? 2 : 0));
+    }
+  };
+  if (SV > 0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e = 4 * (lane + 64 * i);
+      const int row = e / g.K;
+      park[i] = (unsigned)(row * a_pitch + (e - row * g.K));
+    }
+    issue_block(first);
+  } else {
+    issue(cur, total > 0 ? first : blocks, 0);   // (no row block: every offset is out of range, nothing is read)
+  }
 
   // B -> LDS, transposed. Columns >= N and rows >= K read as zero; rows beyond
   // the last 16-row group that holds real data are never read. Consecutive lanes
@@ -146,6 +174,68 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
   }
   lds_barrier();   // B is in LDS; nobody waits for a fetch here
 
+  // bias, activation, residual and store of the finished row block b; the accumulators start over
+  auto finish_block = [&](int b) __attribute__((always_inline)) {
+    // lane holds row b*16 + r, columns n*16 + 4*grp .. +3
+    const int row = b * 16 + r;
+#pragma unroll
+    for (int n = 0; n < TN; ++n) {
+      const int col = n * 16 + grp * 4;
+      float out[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float v = (NA == 2 ? acc[0][n][k] + acc[NA - 1][n][k] : acc[0][n][k]) + bias_q[n][k];
+        switch (g.activation) {
+          case TFHIP_RELU: v = (v > 0.f || v != v) ? v : 0.f; break;
+          case TFHIP_RELU6: v = (v > 0.f || v != v) ? v : 0.f; v = v > 6.f ? 6.f : v; break;
+          case TFHIP_LEAKYRELU: v = v < 0.f ? (float)(g.leaky_alpha * (double)v) : v; break;
+          default: break;
+        }
+        out[k] = v;
+      }
+      if (row < g.M && col < g.N) {
+        if (g.residual) {
+          const float4 r4 = *reinterpret_cast<const float4 *>(g.residual + (long long)row * g.N + col);
+          out[0] += r4.x; out[1] += r4.y; out[2] += r4.z; out[3] += r4.w;
+        }
+        store_result4(g.c + (long long)row * g.N + col, make_float4(out[0], out[1], out[2], out[3]));
+      }
+#pragma unroll
+      for (int h = 0; h < NA; ++h) acc[h][n] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  // the four matrix instructions per column group that one float4 of A feeds
+  auto multiply = [&](const float4 &a, const float *bt) __attribute__((always_inline)) {
+    const float a4[4] = {a.x, a.y, a.z, a.w};
+    float4 b4[TN];
+#pragma unroll
+    for (int n = 0; n < TN; ++n) b4[n] = *reinterpret_cast<const float4 *>(bt + n * 16 * pitch);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int n = 0; n < TN; ++n) {
+        const float bv = j == 0 ? b4[n].x : (j == 1 ? b4[n].y : (j == 2 ? b4[n].z : b4[n].w));
+        acc[j % NA][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(bv, a4[j], acc[j % NA][n], 0, 0, 0);
+      }
+    }
+  };
+
+  if (SV > 0) {
+    for (int b = first; b < blocks; b += step) {
+      // the block in the registers -> LDS (the wavefront's own region: its LDS accesses execute in
+      // order, nobody else reads them), and the registers take the next block's fetch
+#pragma unroll
+      for (int i = 0; i < NV; ++i) *reinterpret_cast<float4 *>(stage + park[i]) = blk[i];
+      issue_block(b + step);   // past the end: every offset is out of range, nothing is read
+      const float *at = stage + r * a_pitch + 4 * grp;
+      const float *bt = lds_bt + r * pitch + 4 * grp;
+#pragma unroll
+      for (int t = 0; t < NV; ++t) multiply(*reinterpret_cast<const float4 *>(at + 16 * t), bt + 16 * t);
+      finish_block(b);
+    }
+    return;
+  }
+
   int b = first, c = 0;
   for (int q = 0; q < total; ++q) {
     int nb = b, nc = c + 1;
@@ -159,49 +249,9 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       if (c * kSkinnyChunk + 16 * t >= g.K) continue;   // nothing but padding (the same for all lanes)
-      const float a4[4] = {cur[t].x, cur[t].y, cur[t].z, cur[t].w};
-      float4 b4[TN];
-#pragma unroll
-      for (int n = 0; n < TN; ++n) b4[n] = *reinterpret_cast<const float4 *>(bt + n * 16 * pitch + 16 * t);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-#pragma unroll
-        for (int n = 0; n < TN; ++n) {
-          const float bv = j == 0 ? b4[n].x : (j == 1 ? b4[n].y : (j == 2 ? b4[n].z : b4[n].w));
-          acc[j % NA][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(bv, a4[j], acc[j % NA][n], 0, 0, 0);
-        }
-      }
+      multiply(cur[t], bt + 16 * t);
     }
-
-    if (c == chunks - 1) {
-      // the row block is complete: lane holds row b*16 + r, columns n*16 + 4*grp .. +3
-      const int row = b * 16 + r;
-#pragma unroll
-      for (int n = 0; n < TN; ++n) {
-        const int col = n * 16 + grp * 4;
-        float out[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          float v = (NA == 2 ? acc[0][n][k] + acc[NA - 1][n][k] : acc[0][n][k]) + bias_q[n][k];
-          switch (g.activation) {
-            case TFHIP_RELU: v = (v > 0.f || v != v) ? v : 0.f; break;
-            case TFHIP_RELU6: v = (v > 0.f || v != v) ? v : 0.f; v = v > 6.f ? 6.f : v; break;
-            case TFHIP_LEAKYRELU: v = v < 0.f ? (float)(g.leaky_alpha * (double)v) : v; break;
-            default: break;
-          }
-          out[k] = v;
-        }
-        if (row < g.M && col < g.N) {
-          if (g.residual) {
-            const float4 r4 = *reinterpret_cast<const float4 *>(g.residual + (long long)row * g.N + col);
-            out[0] += r4.x; out[1] += r4.y; out[2] += r4.z; out[3] += r4.w;
-          }
-          store_result4(g.c + (long long)row * g.N + col, make_float4(out[0], out[1], out[2], out[3]));
-        }
-#pragma unroll
-        for (int h = 0; h < NA; ++h) acc[h][n] = (float4_t){0.f, 0.f, 0.f, 0.f};
-      }
-    }
+    if (c == chunks - 1) finish_block(b);
 #pragma unroll
     for (int t = 0; t < 4; ++t) cur[t] = nxt[t];
     b = nb;
@@ -396,6 +446,23 @@ inline int launch_skinny_tn(const SkinnyArgs &g) {
   const long long cap = (long long)num_cus() * 3;
   if (grid > cap) grid = cap;
   const bool stream_a = (long long)g.M * g.K * 4 >= kSkinnyStreamBytes;
+  if constexpr (TN <= 2) {
+    // A through LDS (instantiated for the k of the wide early projections)
+    const int sv = (stream_a && g.K % 16 == 0 && tuning(kTuneSkinnyStage) != 0) ? g.K / 16 : 0;
+    const size_t lds_staged = lds + (size_t)WAVES * 16 * (g.K + 4) * sizeof(float);
+    if ((sv == 6 || sv == 9 || sv == 12) && lds_staged <= 64 * 1024) {
+      long long per_cu = (long long)(160 * 1024) / (long long)lds_staged;
+      per_cu = per_cu > 3 ? 3 : per_cu;
+      long long staged_grid = (blocks + WAVES - 1) / WAVES;
+      if (staged_grid > num_cus() * per_cu) staged_grid = num_cus() * per_cu;
+      note_kernel("skinny_gemm<%d, %d, true, %d>", TN, WAVES, sv);
+      const dim3 grid3((unsigned)staged_grid), block3(WAVES * 64);
+      if (sv == 6) TFHIP_LAUNCH((skinny_gemm<TN, WAVES, true, 6><<<grid3, block3, lds_staged, stream()>>>(g)));
+      else if (sv == 9) TFHIP_LAUNCH((skinny_gemm<TN, WAVES, true, 9><<<grid3, block3, lds_staged, stream()>>>(g)));
+      else TFHIP_LAUNCH((skinny_gemm<TN, WAVES, true, 12><<<grid3, block3, lds_staged, stream()>>>(g)));
+      return kOk;
+    }
+  }
   note_kernel("skinny_gemm<%d, %d, %s>", TN, WAVES, stream_a ? "true" : "false");
   if (stream_a) {
     TFHIP_LAUNCH((skinny_gemm<TN, WAVES, true><<<dim3((unsigned)grid), dim3(WAVES * 64), lds, stream()>>>(g)));
