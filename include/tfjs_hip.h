@@ -128,10 +128,12 @@ int tfhip_graph_destroy(int graph_id);
  *   64 channels per workgroup of the channel-sliced kernel), "tile_chunks" (its row
  *   chunks per image), "block_rows" (output rows per workgroup of the whole-block
  *   kernel), "fuse_block" (tfhip_inverted_residual_pays: 1 always, 0 never), "k_groups" (1 / 2 / 4
- *   groups of wavefronts that share a GEMM tile and split its k loop). TFHIP_TILE,
- *   TFHIP_SPLITK, TFHIP_DW_ROWS, TFHIP_DW_HALO, TFHIP_NO_SKINNY, TFHIP_DW_FLAT,
- *   TFHIP_SKINNY_REGS, TFHIP_SMALL_K, TFHIP_FUSE_PW_DW in the environment set them at
- *   tfhip_init(). */
+ *   groups of wavefronts that share a GEMM tile and split its k loop), "pw_dw_stream"
+ *   (1 / 0: the register-streaming pointwise + depthwise kernel wherever it takes the
+ *   shape / never), "stream_rows" (its output rows per wavefront), "stream_blocks" (1 / 2
+ *   blocks of 16 channels per wavefront), "skinny_stage" (0: the streaming GEMM never
+ *   stages A in LDS). The environment variable of a knob is its name in capitals behind
+ *   TFHIP_ (TFHIP_TILE, TFHIP_SPLITK, ... TFHIP_SKINNY_STAGE), read at tfhip_init(). */
 int tfhip_set_launch_repeat(int n);
 int tfhip_last_kernel(char *name, size_t name_len);
 int tfhip_set_tuning(const char *name, int value);
