@@ -433,6 +433,15 @@ def test_matmul_tall_tiny_k(hip, orc, tuning, m, n, k, act, regs):
     load_library().tfhip_last_kernel(name, 256)
     assert name.value.decode().startswith("skinny_gemm")
     assert name.value.decode().endswith("true>" if m * k * 4 >= 32 << 20 else "false>"), name.value
+    if regs and k == 32 and m * k * 4 >= 32 << 20:
+        # ... and with K = 32 as whole row blocks through LDS: the same bits as the direct fetch
+        assert name.value.decode().endswith("true, true>"), name.value
+        got = hip.fused_matmul(a, b, **kw)
+        tuning("skinny_stage", 0)
+        direct = hip.fused_matmul(a, b, **kw)
+        load_library().tfhip_last_kernel(name, 256)
+        assert name.value.decode().endswith("false, true>"), name.value
+        np.testing.assert_array_equal(got.view(np.uint32), direct.view(np.uint32))
 
 
 @pytest.mark.parametrize("rows", [32, 64])

@@ -270,9 +270,15 @@ __global__ __launch_bounds__(WAVES * 64) void skinny_gemm(SkinnyArgs g) {
 //   KF    full k groups of 16 (lane takes k = 16 t + 4 g + j, a float4 of A)
 //   HALF  one more group of 8 (lane takes k = 16 KF + 2 g + j, a float2 of A):
 //         K = 24 costs six matrix instructions per block instead of eight
-template <int TN, int KF, bool HALF, bool STREAM_A>
+//   STAGED  (K = 32, a streamed A) the 2 KB row block is fetched as one contiguous piece, whole
+//         cache lines per instruction, and turned into the fragment layout through a region of
+//         LDS that belongs to the wavefront alone (see skinny_gemm)
+template <int TN, int KF, bool HALF, bool STREAM_A, bool STAGED = false>
 __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
+  static_assert(!STAGED || (KF == 2 && !HALF), "the staged form is the K = 32 one");
   constexpr int STEPS = 4 * KF + (HALF ? 2 : 0);
+  constexpr int kPitch = 36;   // floats per staged row: 16-byte reads of eight rows on different banks
+  __shared__ float staged_rows[STAGED ? 4 * 16 * kPitch : 1];
   const int lane = threadIdx.x & 63;
   const int grp = lane >> 4, r = lane & 15;
   const __amdgpu_buffer_rsrc_t rsrc =
@@ -303,7 +309,18 @@ __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
     }
   };
   ABlock cur, nxt;
-  issue(cur, first);
+  float *stage = staged_rows + (threadIdx.x >> 6) * 16 * kPitch;
+  const int park0 = (lane >> 3) * kPitch + 4 * (lane & 7);   // lane's float4 of the first 1 KB: row lane / 8
+  auto issue_flat = [&](ABlock &dst, int b) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const long long e = (long long)b * 512 + 4 * (lane + 64 * i);
+      const unsigned off = (b < blocks && e * 4 < (long long)g.a_bytes) ? (unsigned)(e * 4) : kNoOffset;
+      dst.full[i < KF ? i : 0] = as_float4(__builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, STREAM_A ? 2 : 0));
+    }
+  };
+  if (STAGED) issue_flat(nxt, first);
+  else issue(cur, first);
 
   // this lane's B values and epilogue operands
   float breg[STEPS][TN];
@@ -326,7 +343,17 @@ __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
     }
 
   for (int b = first; b < blocks; b += waves) {
-    issue(nxt, b + waves);   // past the end: every offset is out of range, nothing is read
+    if (STAGED) {
+      // nxt holds block b as fetched; through LDS into the fragment layout (the wavefront's LDS
+      // accesses execute in order), and nxt takes the next block's fetch
+      *reinterpret_cast<float4 *>(stage + park0) = nxt.full[0];
+      *reinterpret_cast<float4 *>(stage + park0 + 8 * kPitch) = nxt.full[KF > 1 ? 1 : 0];
+      issue_flat(nxt, b + waves);
+      cur.full[0] = *reinterpret_cast<const float4 *>(stage + r * kPitch + 4 * grp);
+      cur.full[KF > 1 ? 1 : 0] = *reinterpret_cast<const float4 *>(stage + r * kPitch + 16 + 4 * grp);
+    } else {
+      issue(nxt, b + waves);   // past the end: every offset is out of range, nothing is read
+    }
     float4_t acc[TN];
 #pragma unroll
     for (int n = 0; n < TN; ++n) acc[n] = bias4[n];
@@ -362,7 +389,7 @@ __global__ __launch_bounds__(256) void skinny_gemm_regs(SkinnyArgs g) {
       if (row < g.M && col < g.N)
         store_result4(g.c + (long long)row * g.N + col, make_float4(out[0], out[1], out[2], out[3]));
     }
-    cur = nxt;
+    if (!STAGED) cur = nxt;
   }
 }
 
@@ -384,6 +411,14 @@ inline int launch_skinny_regs(const SkinnyArgs &g, int column_groups) {
   if (cap < 1) cap = 1;
   if (grid > cap) grid = cap;
   const bool stream_a = (long long)g.M * g.K * 4 >= kSkinnyStreamBytes;
+  if constexpr (KF == 2 && !HALF) {
+    if (stream_a && g.K == 32 && tuning(kTuneSkinnyStage) != 0) {
+      note_kernel("skinny_gemm_regs<%d, 2, false, true, true>", TN);
+      TFHIP_LAUNCH((skinny_gemm_regs<TN, 2, false, true, true>
+                    <<<dim3((unsigned)grid, (unsigned)column_groups), dim3(256), 0, stream()>>>(g)));
+      return kOk;
+    }
+  }
   note_kernel("skinny_gemm_regs<%d, %d, %s, %s>", TN, KF, HALF ? "true" : "false", stream_a ? "true" : "false");
   if (stream_a) {
     TFHIP_LAUNCH((skinny_gemm_regs<TN, KF, HALF, true>
