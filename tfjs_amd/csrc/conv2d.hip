@@ -329,6 +329,7 @@ int fused_conv2d(const float *x, const float *filter, float *y, int64_t batch, i
   const int64_t x_bytes = batch * in_h * in_w * in_c * 4, w_bytes = K * out_c * 4;
   p.a_bytes = (unsigned)(x_bytes <= kMaxBufferBytes ? x_bytes : 0);
   p.b_bytes = (unsigned)(w_bytes <= kMaxBufferBytes ? w_bytes : 0);
+  p.c_bytes = (unsigned)(M * out_c * 4 <= kMaxBufferBytes ? M * out_c * 4 : 0);
   p.vec_store = !nchw && out_c % 4 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
   const bool x16 = reinterpret_cast<uintptr_t>(x) % 16 == 0 && p.a_bytes != 0,
              w16 = reinterpret_cast<uintptr_t>(filter) % 16 == 0 && p.b_bytes != 0;

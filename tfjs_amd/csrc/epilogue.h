@@ -104,15 +104,27 @@ __device__ __forceinline__ float finish(const Epilogue &e, float v, long long ba
   return activate(v, e.activation, alpha, e.leaky_alpha);
 }
 
-// The float4 stores the kernels write their results with. The streaming form (a non-temporal
-// store: the line is not kept in the cache) is for outputs whose next reader gains nothing from
-// finding them there and whose stores are pieces of cache lines, which the cache would otherwise
-// collect: the fused expansion + depthwise kernels on the small maps, where a lane writes 16
-// bytes of a pixel's 1.5 - 4 KB of channels (MobileNetV2 at batch 32, in sequence: the eleven tile-
-// kernel launches 177 -> 154 us, the projections that read those outputs unchanged). The outputs of
-// the GEMMs stay cached: the streaming kernels that read them lose 2 - 5 us each when they come
-// from memory. TFHIP_NT_OUT is a build-time switch for measurement that makes every result store a
-// streaming one.
+// The float4 stores the kernels write their results with, in three cache policies. A result is
+// written once and read by the next launch, on any of the eight XCDs, whose L2 caches do not see
+// each other's dirty lines: what a kernel leaves dirty in its L2 is written back when it ends,
+// and that write-back is part of the launch.
+//  * store_result4_through: write-through (`sc1`), through a buffer descriptor. The line goes to
+//    memory as the store is issued, so nothing is left to write back at the end, and it stays in
+//    the memory-side cache, where the reader finds it. The tiled GEMMs, the register-streaming pair
+//    kernel and the channel-sliced pair kernel's results below 8 MB (MobileNetV2 at batch 32, in
+//    sequence: 473 -> 460 us per inference, writers and readers both faster). It is the
+//    compiler's own buffer store with the scope bit set: the same instruction written as inline
+//    assembly, which the compiler cannot see into, lost a float4 now and then.
+//  * store_result4_streaming: non-temporal. For a result of 8 MB or more that is stored in pieces
+//    of cache lines and read once: the channel-sliced pair kernel on its larger maps, where a lane
+//    writes 16 bytes of a pixel's 1.5 - 2.3 KB of channels (its eleven launches 177 -> 154 us
+//    against cached stores; write-through instead costs those launches 0.7 us each).
+//  * store_result4: a plain cached store. The streaming GEMMs: the pair kernels that read their
+//    results, every channel block once more, lose 23 us per inference when those come from
+//    memory, and write-through costs the larger of them 2 us. Also every result too large for the
+//    32-bit offsets of a descriptor.
+// TFHIP_NT_OUT is a build-time switch for measurement that makes every result store a streaming
+// one.
 #ifndef TFHIP_NT_OUT
 #define TFHIP_NT_OUT 0
 #endif
@@ -120,6 +132,12 @@ __device__ __forceinline__ void store_result4_streaming(float *p, float4 v) {
   typedef float result4_t __attribute__((ext_vector_type(4)));
   const result4_t t = {v.x, v.y, v.z, v.w};
   __builtin_nontemporal_store(t, reinterpret_cast<result4_t *>(p));
+}
+// `byte_offset` is relative to the descriptor's base; an offset beyond its extent drops the store.
+__device__ __forceinline__ void store_result4_through(__amdgpu_buffer_rsrc_t rsrc, unsigned byte_offset, float4 v) {
+  typedef unsigned int result4_bits __attribute__((ext_vector_type(4)));
+  const result4_bits d = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+  __builtin_amdgcn_raw_buffer_store_b128(d, rsrc, (int)byte_offset, 0, TFHIP_NT_OUT ? 2 : 16);
 }
 __device__ __forceinline__ void store_result4(float *p, float4 v) {
 #if TFHIP_NT_OUT

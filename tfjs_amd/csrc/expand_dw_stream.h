@@ -28,6 +28,7 @@ struct ExpandDwStreamArgs {
   int cblocks, ncb;                // blocks of 16 expanded channels, and how many of them a wavefront takes (1 or 2)
   long long waves;                 // batch x chunks_h x strips x ceil(cblocks / ncb)
   unsigned x_bytes;
+  int through;                     // an image of the result fits 32-bit offsets: written through a descriptor
   // first stage a convolution over few input channels instead of a 1x1 one (k_steps > 0): x is
   // [batch, xh, xw, xc], the "expanded" tensor [batch, in_h, in_w, c] is its output; k filter taps
   int xh, xw, xc, conv_stride, conv_pad_top, conv_pad_left, k, k_steps;

@@ -292,6 +292,9 @@ void expand_dw_stream(ExpandDwStreamArgs g, StemTaps taps) {
   // this lane's place in an output row (channel block 0 of the wavefront), and the rows' distance
   float *out_ptr = g.y + (((long long)n * g.out_h + oh0) * g.out_w + ocol) * g.c + ch[0];
   const long long out_row = (long long)g.out_w * g.c;
+  const __amdgpu_buffer_rsrc_t rsrc_y = __builtin_amdgcn_make_buffer_rsrc(
+      (void *)(g.y + (long long)n * g.out_h * g.out_w * g.c), 0, (int)((unsigned)g.out_h * g.out_w * g.c * 4u), 0x00020000);
+  const unsigned out_off = (unsigned)((oh0 * g.out_w + ocol) * g.c + ch[0]) * 4u;   // (meaningful where g.through)
   // One expanded row's share of a depthwise sum: the three taps of filter row wr, left to right.
   auto add_row = [&](const float4 &sum, const Taps &t, int wr, int u) __attribute__((always_inline)) {
     float4 acc = sum;
@@ -310,10 +313,12 @@ void expand_dw_stream(ExpandDwStreamArgs g, StemTaps taps) {
     if (out_lane && (u == 0 || cb0 + u < g.cblocks)) {
       const float4 out = make_float4(relu_cap(acc.x + b2q[u].x, g.cap), relu_cap(acc.y + b2q[u].y, g.cap),
                                      relu_cap(acc.z + b2q[u].z, g.cap), relu_cap(acc.w + b2q[u].w, g.cap));
-      // (streaming stores behind a 1x1 first stage: the four pairs measured 99.6 -> 91.6 us in sequence at
-      // batch 32; behind a few-taps first stage, whose output the next kernel reads at once and whole,
-      // they cost 6 us)
-      if (TAPS == 0) {
+      // (written through: against non-temporal stores behind a 1x1 first stage the GEMMs that read
+      // these 19 - 38 MB maps get 2 us faster per inference, and against cached stores the launch
+      // behind a few-taps first stage 1 - 2 us; an image beyond 32-bit offsets: the stores of before)
+      if (g.through) {
+        store_result4_through(rsrc_y, out_off + (unsigned)(o * (int)out_row + 16 * u) * 4u, out);
+      } else if (TAPS == 0) {
         store_result4_streaming(out_ptr + o * out_row + 16 * u, out);
       } else {
         store_result4(out_ptr + o * out_row + 16 * u, out);
@@ -499,6 +504,7 @@ bool plan_expand_dw_stream(ExpandDwStreamArgs &g) {
   g.rows = rows;
   g.chunks_h = (g.out_h + rows - 1) / rows;
   g.waves = (long long)g.batch * g.chunks_h * g.strips * cgroups;
+  g.through = (long long)g.out_h * g.out_w * g.c * 4 <= 0xfffffff0LL ? 1 : 0;
   return true;
 }
 

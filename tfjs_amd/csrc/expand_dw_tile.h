@@ -17,6 +17,8 @@ struct ExpandDwTileArgs {
   int rows, chunks_h;              // output rows per workgroup, workgroups along the rows
   int erows, ecols;                // expanded tile with halo: rows of the tallest chunk, columns
   unsigned x_bytes;
+  int stream_out;                  // the result leaves as non-temporal stores (8 MB or more in all, or an image
+                                   // beyond 32-bit offsets), else written through
 };
 
 bool expand_dw_tile_takes_k(int cin);

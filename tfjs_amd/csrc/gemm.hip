@@ -130,6 +130,7 @@ static int fused_matmul_impl(const char *who, const float *a, const float *b, fl
   const int64_t kMaxBufferBytes = 0xfffffffeLL;   // one buffer descriptor addresses at most this much
   p.a_bytes = (unsigned)(M * K * 4 <= kMaxBufferBytes ? M * K * 4 : 0);
   p.b_bytes = (unsigned)(K * N * 4 <= kMaxBufferBytes ? K * N * 4 : 0);
+  p.c_bytes = (unsigned)(M * N * 4 <= kMaxBufferBytes ? M * N * 4 : 0);
   p.vec_store = N % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
   const bool a16 = reinterpret_cast<uintptr_t>(a) % 16 == 0 && p.a_bytes != 0,
              b16 = reinterpret_cast<uintptr_t>(b) % 16 == 0 && p.b_bytes != 0;

@@ -77,6 +77,9 @@ struct GemmParams {
   long long ldc;
   // bytes addressable from the (per-batch) base of each operand, for the buffer descriptors
   unsigned a_bytes, b_bytes;
+  // bytes addressable from the (per-batch) base of C, which is also the size of a split-K slab; 0: more
+  // than a descriptor's 32-bit offsets reach (results then leave as plain stores, else written through)
+  unsigned c_bytes;
   int tiles_m, tiles_n;
   int group_m;    // tile rows per panel of the tile numbering
   // split K: the grid holds `splits` copies of the tile set, copy s sums
@@ -576,6 +579,9 @@ __global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
   const long long ldc = to_ws ? p.N : p.ldc;
   const bool conv_addr = !to_ws && e.addressing == kConv;
   const bool vec = to_ws ? p.N % 4 == 0 : p.vec_store != 0;
+  const bool through = p.c_bytes != 0;
+  const __amdgpu_buffer_rsrc_t rsrc_c =
+      __builtin_amdgcn_make_buffer_rsrc((void *)uniform_pointer(C), 0, (int)p.c_bytes, 0x00020000);
   // the residual lies where the output element does
   const float *R = (fused && e.residual) ? e.residual + (long long)bz * p.c_batch_stride : nullptr;
   float alpha_q[T::TN][4];
@@ -627,7 +633,9 @@ __global__ __launch_bounds__(256 * KG) void gemm_kernel(GemmParams p) {
             const float4 r4 = *reinterpret_cast<const float4 *>(R + base + col);
             out[0] += r4.x; out[1] += r4.y; out[2] += r4.z; out[3] += r4.w;
           }
-          store_result4(C + base + col, make_float4(out[0], out[1], out[2], out[3]));
+          const float4 out4 = make_float4(out[0], out[1], out[2], out[3]);
+          if (through) store_result4_through(rsrc_c, (unsigned)((base + col) * 4), out4);
+          else store_result4(C + base + col, out4);
         } else {
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
