@@ -353,7 +353,7 @@ def test_depthwise_row_chunks(hip, orc, tuning, rows, stride, pad):
 
 @pytest.mark.parametrize("stride", [1, 2])
 def test_depthwise_large_result_is_streamed(hip, orc, stride):
-    # a result of 32 MB or more is stored non-temporally: same values, another kernel variant
+    # a result of 8 MB or more is stored non-temporally: same values, another kernel variant
     from tfjs_amd.capi import load_library
     rng = np.random.default_rng(37 + stride)
     x = rng.uniform(-1, 1, (4, 128 * stride, 129 * stride, 128)).astype(np.float32)
@@ -364,10 +364,13 @@ def test_depthwise_large_result_is_streamed(hip, orc, stride):
     load_library().tfhip_last_kernel(name, 256)
     assert name.value.decode() == "depthwise_3x3_rows<%d, false, true>" % stride, name.value
     assert_parity(got, orc.fused_depthwise_conv2d(x, w, **kw))
-    small = hip.fused_depthwise_conv2d(x[:3], w, **kw)
+    # the top 64 output rows of the first image on their own (4 MB): cached stores, and the same
+    # bits wherever the cut does not change the padding
+    small = hip.fused_depthwise_conv2d(x[:1, :64 * stride], w, **kw)
     load_library().tfhip_last_kernel(name, 256)
-    assert name.value.decode() == "depthwise_3x3_rows<%d, false, false>" % stride, name.value
-    assert np.array_equal(small, got[:3])
+    label = name.value.decode()   # (the row pipeline, or the one-row-per-lane kernel: neither streams)
+    assert label.startswith("depthwise_3x3_") and not label.endswith("true>"), label
+    assert np.array_equal(small[:, :62], got[:1, :62])
 
 
 def test_depthwise_linearity_full_size(hip):

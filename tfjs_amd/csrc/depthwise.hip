@@ -149,9 +149,11 @@ constexpr int kRowsPW = 4;   // output columns per lane
 #define DW_WAVES 1
 #endif
 constexpr unsigned kDwNoOffset = 0xffffffffu;
-// Results of at least this many bytes are stored non-temporally: all eight L2
-// caches together hold 32 MB, so such a result cannot wait there for its reader.
-constexpr long long kDwStreamBytes = 32LL << 20;
+// Results of at least this many bytes are stored non-temporally: an L2 holds 4 MB,
+// so such a result cannot wait there for its reader (measured with operands from
+// memory: 51 MB 21.3 -> 20.3 us, 12 MB at stride 2 13.7 -> 12.7 us; written through
+// instead, 21.6 and 13.6 us).
+constexpr long long kDwStreamBytes = 8LL << 20;
 typedef unsigned int dw_uint4 __attribute__((ext_vector_type(4)));
 
 struct DwRowsArgs {
