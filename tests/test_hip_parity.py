@@ -396,6 +396,20 @@ def test_matmul_tall_small_b(hip, orc, m, n, k, act):
     assert_parity(hip.fused_matmul(a, b, **kw), orc.fused_matmul(a, b, **kw))
 
 
+def test_matmul_finishing_pass_reads_every_store(hip, orc):
+    # The finishing pass runs right behind the GEMM whose write-through stores it reads: every float4 of
+    # the raw sums has to be there (a store that arrives late, or not at all, shows as sigmoid(bias)).
+    rng = np.random.default_rng(4711)
+    b = rng.normal(0, 0.3, (144, 24)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (24,)).astype(np.float32)
+    for trip in range(6):
+        a = rng.uniform(-1, 1, (65600, 144)).astype(np.float32)
+        got = hip.fused_matmul(a, b, bias=bias, activation="sigmoid")
+        assert_parity(got, orc.fused_matmul(a, b, bias=bias, activation="sigmoid"))
+        # other work between the trips, so that the pool hands the buffers out again with other contents
+        hip.fused_matmul(a[:4096], b, bias=bias, activation="relu")
+
+
 @pytest.mark.parametrize("m,n,k,act", [(90001, 24, 96, "relu6"), (65600, 24, 144, "linear"), (65601, 16, 192, "relu"),
                                         (70000, 32, 144, "leakyrelu")])
 def test_matmul_tall_a_through_lds(hip, orc, tuning, m, n, k, act):
