@@ -68,6 +68,13 @@ int tfhip_sync(void);
 /* live: blocks handed out and not freed; live_bytes: their total size;
  * pooled_bytes: freed blocks kept for reuse. */
 int tfhip_memory_info(size_t *live, size_t *live_bytes, size_t *pooled_bytes);
+/* The scratch block that kernels needing device memory beyond their operands
+ * share (partial sums of a matmul whose K is cut into slices). It is not a
+ * tensor, so tfhip_memory_info does not count it. bytes: its present size;
+ * allocations: hipMalloc calls made for it since tfhip_init; last_splits: the
+ * number of K slices of the last matmul / convolution launched as a GEMM. For
+ * tests and diagnosis; no counterpart in the reference. */
+int tfhip_workspace_info(size_t *bytes, size_t *allocations, int *last_splits);
 /* Lets kernels accept device memory the caller allocated elsewhere. */
 int tfhip_register_external(void *dptr, size_t bytes);
 int tfhip_unregister_external(void *dptr);
@@ -160,18 +167,23 @@ int tfhip_fused_matmul(const float *a, const float *b, float *out,
 
 /* tfhip_fused_matmul for callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It
- * has no counterpart in the reference. Same arguments, same kernels and the
- * same result bit for bit; the one difference is where a product whose K is
- * cut into slices keeps its partial sums: not in the library's growing
- * workspace but in a static device array of TFHIP_NOALLOC_SCRATCH_BYTES that
- * each GPU holds until the process ends. The call makes no hipMalloc / hipFree.
- * A product whose partial sums (slices x batch x M x N x 4 bytes, with the
- * slices the library chooses: at most 8, and 1 whenever the tiles already
- * fill the GPU or K is short) exceed the array fails with a message that
- * states both sizes, and launches nothing. Every call on a GPU shares that
- * GPU's array: calls that overlap on one GPU (other threads, other streams)
- * race. Nothing is cleared between calls because each call writes every
- * element it later reads. */
+ * has no counterpart in the reference. Same arguments and the same kernels; the
+ * one difference is where a product whose K is cut into slices keeps its
+ * partial sums: not in the library's growing workspace but in a static device
+ * array of TFHIP_NOALLOC_SCRATCH_BYTES that each GPU holds until the process
+ * ends. The call makes no hipMalloc / hipFree. When the slices the library
+ * would choose (at most 8, and 1 whenever the tiles already fill the GPU or K
+ * is short) need more than the array (slices x batch x M x N x 4 bytes), it
+ * takes the largest number of slices that fits, down to one slice, which needs
+ * no scratch: the result then has tfhip_fused_matmul's bits only where the two
+ * slice counts agree, and is within the float32 bound otherwise. A slice count
+ * the caller forced with the "splitk" knob is not reduced: if it does not fit,
+ * the call fails with a message that states both sizes, and launches nothing.
+ * Every call on a GPU shares that GPU's array: calls that overlap on one GPU
+ * (other threads, other streams) race on it. The array belongs to the calling
+ * thread for the length of the call; tfhip_fused_matmul on another thread keeps
+ * the library's workspace. Nothing is cleared between calls because each call
+ * writes every element it later reads. */
 #define TFHIP_NOALLOC_SCRATCH_BYTES (16u << 20)
 int tfhip_fused_matmul_noalloc(const float *a, const float *b, float *out,
                                int64_t batch_a, int64_t batch_b, int64_t M,

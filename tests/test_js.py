@@ -107,7 +107,7 @@ def test_c_abi_library_exports_every_declared_symbol():
 def test_addon_loads_and_exports_every_entry_point():
     proc = subprocess.run([NODE, "-e", """
       const a = require('%s/tfjs_amd/lib/tfjs_hip.node');
-      const want = ['init','shutdown','deviceInfo','alloc','free','upload','download','sync','memoryInfo','eventRecord',
+      const want = ['init','shutdown','deviceInfo','alloc','free','upload','download','sync','memoryInfo','workspaceInfo','eventRecord',
                     'eventElapsed','setLaunchRepeat','lastKernel','fusedMatMul','fusedConv2D','fusedDepthwiseConv2D',
                     'dequantAffine','dequantF16','add','meanHW','binary','unary','avgPool','cast','transpose2d',
                     'fusedInvertedResidual','invertedResidualPays','fusedMatMulNoAlloc','fusedPointwiseDepthwise',

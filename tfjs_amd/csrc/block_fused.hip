@@ -430,8 +430,9 @@ bool dims_in_range(int64_t batch, int64_t in_h, int64_t in_w, int64_t in_c, int6
   const int64_t lim = 0x7fffffff;
   return batch >= 0 && in_h > 0 && in_w > 0 && in_c > 0 && mid_c > 0 && out_c > 0 && stride > 0 && out_h >= 0 && out_w >= 0 &&
          pad_top >= 0 && pad_left >= 0 && pad_top < lim && pad_left < lim && in_c <= 4096 && mid_c <= 65536 && out_c <= 4096 &&
-         batch * in_h * in_w * in_c * 4 <= 0xfffffffeLL && batch * out_h * out_w * out_c < lim && in_h < lim && in_w < lim &&
-         out_h < lim && out_w < lim;
+         in_h < lim && in_w < lim && out_h < lim && out_w < lim && batch < lim &&
+         product_below(0x40000000LL, {batch, in_h, in_w, in_c}) && product_below(lim, {batch, out_h, out_w, out_c}) &&
+         product_below(lim, {batch, out_h, out_w, mid_c});
 }
 
 }  // namespace

@@ -30,15 +30,17 @@ int num_cus();
 int device_index();        // the device tfhip_init was given
 // Device scratch of at least `bytes` (nullptr if it cannot be allocated); valid until the next call.
 void *workspace(size_t bytes);
-// While a FixedWorkspace object lives, workspace() hands out the caller's block
-// instead of the library's growing one and allocates nothing: a request beyond
-// `bytes` returns nullptr, and workspace_is_fixed() tells a launcher to fail
-// rather than fall back.
+// While a FixedWorkspace object lives, workspace() hands the thread that made it
+// the caller's block instead of the library's growing one and allocates nothing:
+// a request beyond `bytes` returns nullptr, and workspace_is_fixed() tells a
+// launcher to fit its request to fixed_workspace_bytes().
 struct FixedWorkspace {
   FixedWorkspace(void *ptr, size_t bytes);
   ~FixedWorkspace();
 };
 bool workspace_is_fixed();
+// Records the number of K slices a GEMM launch was cut into (tfhip_workspace_info reports the last).
+void note_splits(int splits);
 size_t fixed_workspace_bytes();
 // Resolves the device address of gemm.hip's static scratch array for `device`
 // (which must be current). Called by tfhip_init.
@@ -110,8 +112,21 @@ void note_kernel(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 int launch_repeat();
 
 // Tuning overrides (tfhip_set_tuning, or TFHIP_<NAME> in the environment at
-// tfhip_init): -1 when unset.
-enum TuningKey { kTuneTile = 0, kTuneSplitK, kTuneDwRows, kTuneDwHalo, kTuneNoSkinny, kTuneDwFlat, kTuneSkinnyRegs, kTuneSmallK, kTuneFusePwDw, kTunePwDwTile, kTuneTileSlice, kTuneTileChunks, kTuneBlockRows, kTuneFuseBlock, kTuneKGroups, kTunePwDwStream, kTuneStreamRows, kTuneStreamBlocks, kTuneSkinnyStage, kTuneCount };
+// tfhip_init): -1 when unset. One list names every knob: the enumerator, the
+// name tfhip_set_tuning takes, and (in capitals behind TFHIP_) its environment variable.
+#define TFHIP_TUNING_KNOBS(X)                                                                              \
+  X(Tile, "tile") X(SplitK, "splitk") X(DwRows, "dw_rows") X(DwHalo, "dw_halo") X(NoSkinny, "no_skinny")    \
+  X(DwFlat, "dw_flat") X(SkinnyRegs, "skinny_regs") X(SmallK, "small_k") X(FusePwDw, "fuse_pw_dw")          \
+  X(PwDwTile, "pw_dw_tile") X(TileSlice, "tile_slice") X(TileChunks, "tile_chunks")                         \
+  X(FuseBlock, "fuse_block") X(KGroups, "k_groups") X(PwDwStream, "pw_dw_stream")                           \
+  X(StreamRows, "stream_rows") X(StreamBlocks, "stream_blocks") X(SkinnyStage, "skinny_stage")              \
+  X(BlockRows, "block_rows")
+enum TuningKey {
+#define TFHIP_TUNING_ENUM(id, name) kTune##id,
+  TFHIP_TUNING_KNOBS(TFHIP_TUNING_ENUM)
+#undef TFHIP_TUNING_ENUM
+  kTuneCount
+};
 int tuning(int key);
 
 // Enqueues `launch_expr` launch_repeat() times and checks the launch.

@@ -102,6 +102,11 @@ static int fused_matmul_impl(const char *who, const float *a, const float *b, fl
   const int64_t batch = batch_a > batch_b ? batch_a : batch_b;
   int rc = kOk;
   if (batch_a == 0 || batch_b == 0 || M == 0 || N == 0) return kOk;
+  // three factors below 2^31 each can pass 2^63: bound every operand's element count before forming it
+  const int64_t max_elems = int64_t(1) << 40;
+  TFHIP_CHECK_ARG(product_below(max_elems, {batch_a, M, K > 0 ? K : 1}) && product_below(max_elems, {batch_b, K > 0 ? K : 1, N}) &&
+                      product_below(max_elems, {batch, M, N}),
+                  "%s: an operand exceeds 2^40 elements", who);
   auto live = [&](const void *ptr, int64_t elems, const char *name) {
     if (ptr != nullptr && range_is_live(ptr, (size_t)elems * 4)) return (int)kOk;
     return fail(kOutOfRange, "%s: operand '%s' (%lld elements of 4 bytes at %p) is not inside a live device buffer",

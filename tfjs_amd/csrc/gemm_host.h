@@ -106,15 +106,25 @@ inline int launch_gemm(GemmParams &p) {
       }
     }
     const int forced = tuning(kTuneSplitK);   // tuning / test override
-    if (forced > 0 && forced <= 64 && forced <= k_tiles) best = forced;
-    if (best > 1) {
-      const size_t bytes = (size_t)best * p.batch * p.M * p.N * sizeof(float);
-      float *ws = bytes <= (size_t(1) << 30) ? static_cast<float *>(workspace(bytes)) : nullptr;
-      if (!ws && workspace_is_fixed())
+    const bool was_forced = forced > 0 && forced <= 64 && forced <= k_tiles;
+    if (was_forced) best = forced;
+    const size_t slice_bytes = (size_t)p.batch * p.M * p.N * sizeof(float);
+    if (best > 1 && workspace_is_fixed() && (size_t)best * slice_bytes > fixed_workspace_bytes()) {
+      // a caller's fixed scratch: a slice count the caller forced is refused, the library's own choice
+      // comes down to what fits (one slice needs no scratch at all). The library's own choice keeps
+      // slices x tiles within the compute units and a tile within 128 x 128, so on 256 units it never
+      // asks for more than 16 MiB; this is for a device with more of them.
+      if (was_forced)
         return fail(kBadArgument,
                     "gemm: %d K slices of a %d x %d x %d output need %zu bytes of scratch; the static array of the "
                     "entry point that allocates nothing holds %zu",
-                    best, p.batch, p.M, p.N, bytes, fixed_workspace_bytes());
+                    best, p.batch, p.M, p.N, (size_t)best * slice_bytes, fixed_workspace_bytes());
+      best = (int)(fixed_workspace_bytes() / slice_bytes);
+      if (best < 2) best = 1;
+    }
+    if (best > 1) {
+      const size_t bytes = (size_t)best * slice_bytes;
+      float *ws = bytes <= (size_t(1) << 30) ? static_cast<float *>(workspace(bytes)) : nullptr;
       if (ws) {
         p.splits = best;
         p.k_per_split = ((k_tiles + best - 1) / best) * BK;
@@ -122,6 +132,7 @@ inline int launch_gemm(GemmParams &p) {
       }
     }
   }
+  note_splits(p.splits);
   const long long grid = tiles * p.splits;
   {
     // ids resident together on one XCD: its share of the grid, at most two

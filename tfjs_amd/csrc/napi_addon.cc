@@ -248,6 +248,18 @@ napi_value MemoryInfo(napi_env env, napi_callback_info) {
   return obj;
 }
 
+napi_value WorkspaceInfo(napi_env env, napi_callback_info) {
+  size_t bytes = 0, allocations = 0;
+  int splits = 0;
+  HIP_OK(tfhip_workspace_info(&bytes, &allocations, &splits));
+  napi_value obj;
+  NAPI_OK(napi_create_object(env, &obj));
+  napi_set_named_property(env, obj, "bytes", make_number(env, (double)bytes));
+  napi_set_named_property(env, obj, "allocations", make_number(env, (double)allocations));
+  napi_set_named_property(env, obj, "lastSplits", make_number(env, (double)splits));
+  return obj;
+}
+
 napi_value EventRecord(napi_env env, napi_callback_info info) {
   Args a(env, info, 1, "eventRecord");
   const int slot = a.i32(0);
@@ -644,6 +656,7 @@ napi_value Register(napi_env env, napi_value exports) {
       FN("download", Download),
       FN("sync", Sync),
       FN("memoryInfo", MemoryInfo),
+      FN("workspaceInfo", WorkspaceInfo),
       FN("eventRecord", EventRecord),
       FN("eventElapsed", EventElapsed),
       FN("setLaunchRepeat", SetLaunchRepeat),

@@ -1,6 +1,7 @@
 // Library lifetime, the single stream, the pooled device allocator with its
 // live-block registry, host<->device copies through pinned staging, event
 // timing, and recording of a sequence of launches into a HIP graph.
+#include <ctype.h>
 #include <string.h>
 
 #include <map>
@@ -116,20 +117,29 @@ void note_kernel(const char *fmt, ...) {
 int launch_repeat() { return g_repeat; }
 
 int g_init_count = 0;
-int g_tuning[kTuneCount] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
-const char *const kTuningNames[kTuneCount] = {"tile", "splitk", "dw_rows", "dw_halo", "no_skinny", "dw_flat", "skinny_regs", "small_k", "fuse_pw_dw", "pw_dw_tile", "tile_slice", "tile_chunks", "block_rows", "fuse_block", "k_groups", "pw_dw_stream", "stream_rows", "stream_blocks", "skinny_stage"};
-int tuning(int key) { return g_tuning[key]; }
+const char *const kTuningNames[kTuneCount] = {
+#define TFHIP_TUNING_NAME(id, name) name,
+    TFHIP_TUNING_KNOBS(TFHIP_TUNING_NAME)
+#undef TFHIP_TUNING_NAME
+};
+// Every knob starts unset, whatever their number.
+struct TuningTable {
+  int value[kTuneCount];
+  TuningTable() {
+    for (int &v : value) v = -1;
+  }
+};
+TuningTable g_tuning;
+int tuning(int key) { return g_tuning.value[key]; }
 
 void read_tuning_from_environment() {
-  static const char *const env_names[kTuneCount] = {"TFHIP_TILE", "TFHIP_SPLITK", "TFHIP_DW_ROWS", "TFHIP_DW_HALO",
-                                                    "TFHIP_NO_SKINNY", "TFHIP_DW_FLAT", "TFHIP_SKINNY_REGS",
-                                                    "TFHIP_SMALL_K", "TFHIP_FUSE_PW_DW", "TFHIP_PW_DW_TILE",
-                                                    "TFHIP_TILE_SLICE", "TFHIP_TILE_CHUNKS", "TFHIP_BLOCK_ROWS",
-                                                    "TFHIP_FUSE_BLOCK", "TFHIP_K_GROUPS", "TFHIP_PW_DW_STREAM",
-                                                    "TFHIP_STREAM_ROWS", "TFHIP_STREAM_BLOCKS", "TFHIP_SKINNY_STAGE"};
   for (int i = 0; i < kTuneCount; ++i) {
-    const char *e = getenv(env_names[i]);
-    g_tuning[i] = e ? atoi(e) : -1;
+    char env_name[64] = "TFHIP_";
+    size_t at = strlen(env_name);
+    for (const char *c = kTuningNames[i]; *c && at + 1 < sizeof env_name; ++c) env_name[at++] = (char)toupper((unsigned char)*c);
+    env_name[at] = 0;
+    const char *e = getenv(env_name);
+    g_tuning.value[i] = e ? atoi(e) : -1;
   }
 }
 
@@ -142,9 +152,14 @@ int num_cus() { return g.prop.multiProcessorCount; }
 // Scratch for kernels that need device memory beyond their operands (split-K
 // partial sums). One block that only grows; work on the single stream is
 // ordered, so consecutive launches may share it.
-void *g_fixed_ws = nullptr;
-size_t g_fixed_ws_bytes = 0;
-bool g_ws_fixed = false;
+// The fixed block belongs to the calling thread (the entry point that allocates
+// nothing sets it for the length of its call): another thread's launches keep
+// the library's own block.
+thread_local void *g_fixed_ws = nullptr;
+thread_local size_t g_fixed_ws_bytes = 0;
+thread_local bool g_ws_fixed = false;
+size_t g_workspace_allocations = 0;   // hipMalloc calls made by workspace() since tfhip_init
+int g_last_splits = 0;                // K slices of the last GEMM launch
 
 FixedWorkspace::FixedWorkspace(void *ptr, size_t bytes) {
   g_fixed_ws = ptr;
@@ -178,8 +193,11 @@ void *workspace(size_t bytes) {
     return nullptr;
   }
   g.workspace_bytes = want;
+  ++g_workspace_allocations;
   return g.workspace;
 }
+
+void note_splits(int splits) { g_last_splits = splits; }
 
 bool range_is_live(const void *p, size_t bytes) {
   std::lock_guard<std::mutex> lock(g_mutex);
@@ -287,6 +305,8 @@ int tfhip_shutdown(void) {
   if (g.workspace) (void)hipFree(g.workspace);
   g.workspace = nullptr;
   g.workspace_bytes = 0;
+  g_workspace_allocations = 0;
+  g_last_splits = 0;
   (void)hipStreamDestroy(g.stream);
   g.stream = nullptr;
   g.ready = false;
@@ -398,6 +418,14 @@ int tfhip_memory_info(size_t *live, size_t *live_bytes, size_t *pooled_bytes) {
   return kOk;
 }
 
+int tfhip_workspace_info(size_t *bytes, size_t *allocations, int *last_splits) {
+  TFHIP_REQUIRE_INIT();
+  if (bytes) *bytes = g.workspace_bytes;
+  if (allocations) *allocations = g_workspace_allocations;
+  if (last_splits) *last_splits = g_last_splits;
+  return kOk;
+}
+
 int tfhip_upload(void *dst, size_t dst_offset, const void *host, size_t bytes) {
   TFHIP_REQUIRE_INIT();
   TFHIP_REFUSE_WHILE_RECORDING();
@@ -459,7 +487,7 @@ int tfhip_download(void *host, const void *src, size_t src_offset, size_t bytes)
 int tfhip_set_tuning(const char *name, int value) {
   for (int i = 0; name && i < kTuneCount; ++i) {
     if (strcmp(name, kTuningNames[i]) == 0) {
-      g_tuning[i] = value < 0 ? -1 : value;
+      g_tuning.value[i] = value < 0 ? -1 : value;
       return kOk;
     }
   }

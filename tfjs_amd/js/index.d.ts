@@ -111,6 +111,7 @@ export interface HipBinding {
   download(ptr: DevicePtr, offset: number, out: ArrayBufferView): ArrayBufferView;
   sync(): void;
   memoryInfo(): {live: number, liveBytes: number, pooledBytes: number};
+  workspaceInfo(): {bytes: number, allocations: number, lastSplits: number};
   eventRecord(slot: number): void;
   eventElapsed(startSlot: number, endSlot: number): number;
   setLaunchRepeat(n: number): void;

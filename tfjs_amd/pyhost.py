@@ -50,6 +50,14 @@ def memory_info():
     return dict(live=live.value, live_bytes=live_bytes.value, pooled_bytes=pooled.value)
 
 
+def workspace_info():
+    """The library's scratch block (split-K partial sums): its size, the hipMalloc calls made for it
+    since init, and the K slices of the last GEMM launch."""
+    size, allocations, splits = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_int()
+    check(load_library().tfhip_workspace_info(ctypes.byref(size), ctypes.byref(allocations), ctypes.byref(splits)))
+    return dict(bytes=size.value, allocations=allocations.value, last_splits=splits.value)
+
+
 def _f32(a):
     return np.ascontiguousarray(a, dtype=np.float32)
 
