@@ -1,9 +1,11 @@
 'use strict';
 /**
- * Offline stand-in for tfjs-converter's GraphModel, restricted to the ops of the
- * fused inference path: it loads a converter-format graph model (model.json with
- * modelTopology, signature and weightsManifest, plus the weight shards) and
- * executes it through the public tfjs ops, whatever backend is active.
+ * The reference's half of the boundary, for an image without @tensorflow/tfjs-converter:
+ * a GraphModel restricted to the ops of the fused inference path. It loads a
+ * converter-format graph model (model.json with modelTopology, signature and
+ * weightsManifest, plus the weight shards) and executes it node by node through the
+ * public tfjs ops, whatever backend is active. Not part of the tfjs-backend-hip
+ * package.
  *
  * It follows the reference's behaviour for this path:
  *   GraphModel / loadGraphModel   tfjs-converter/src/executor/graph_model.ts:88-181, :410-516, :630-708
@@ -16,38 +18,18 @@
  *                                 transformation_executor.ts (Reshape, Squeeze, Cast, Transpose),
  *                                 graph_executor.ts (Identity ...)
  * The third constructor argument is the io module whose decodeWeights turns the
- * weight bytes into tensors (graph_model.ts:104-107, used at :177): pass
- * {decodeWeights: require('tfjs-backend-hip').decodeWeights} to have quantized
- * weights uploaded as bytes and dequantized on the GPU.
+ * weight bytes into tensors (graph_model.ts:104-107, used at :177); there is no
+ * default here, the caller names one.
  *
- * One thing it does that the reference's executor does not: when the active
- * backend registers a 'FusedConv2DAdd' kernel, a _FusedConv2D node whose only
- * reader is an Add / AddV2 node (a projection convolution and the skip connection
- * of a residual block) is executed together with that Add as one kernel. The
- * result has the bits of the two separate kernels; {fuseResidualAdd: false} in
- * the load options turns it off. Likewise, with a 'FusedPointwiseDepthwiseConv2D'
- * kernel, a 1x1 _FusedConv2D (or one over at most 4 input channels: a stem) whose only
- * reader is a 3x3 FusedDepthwiseConv2dNative with the same relu / relu6 activation
- * (the expansion and the depthwise stage of an inverted-residual block) is one step, and the kernel decides per shape
- * whether one launch or the two are faster; {fusePointwiseDepthwise: false} turns
- * that off.
- *
- * And with {recordLaunches: true} in the load options, on a backend that can
- * record (beginRecording / endRecording / replay, as the hip backend has), the
- * kernels of one execution are recorded into a device-side graph the second time
- * the model runs with inputs of a given shape, and every later execution with
- * that shape replays the graph: one native call instead of one per node, which is
- * what a small batch is bound by. The inputs are copied into buffers the recording
- * owns (skipped while the same tensor is passed again), the results are copied
- * out of them, so tensors keep their value semantics. A graph whose execution
- * reads tensor values on the host cannot be recorded and keeps running node by node.
- *
- * Where @tensorflow/tfjs-converter is installed, use its GraphModel instead; the
- * backend and the injected decodeWeights are the same.
+ * One hook the reference's executor does not have: `loadOptions.planner`, an object
+ * with planFusions(view, loadOptions), wantsRecording(loadOptions), runRecorded(...)
+ * and disposeRecordings(map). A backend package passes its own (tfjs-backend-hip
+ * passes tfjs_amd/js/graph_plan.js) to run groups of nodes as one kernel and to
+ * replay recorded launch sequences. Without a planner every node runs on its own.
  */
 const fs = require('fs');
 const path = require('path');
-const tf = require('../core');
+const tf = require('./index');
 
 // ---- attribute decoding (operation_mapper.ts:437-610) ---------------------------
 function parseStringParam(s, keepCase) {
@@ -174,79 +156,6 @@ function fusedConvParams(node) {
     preluActivationWeights: isBiasAdd ? inputs[3] : inputs[2],
     leakyreluAlpha: fixed.leakyreluAlpha
   });
-}
-
-/**
- * _FusedConv2D node + the Add that reads it -> function(inputs) => Tensor, where
- * inputs are the convolution's own inputs followed by the Add's other operand.
- */
-function compileConvAdd(convNode) {
-  const params = fusedConvParams(convNode);
-  const convInputs = (convNode.input || []).filter(i => i[0] !== '^').length;
-  return inputs => {
-    const p = params(inputs);
-    let x = p.x, residual = inputs[convInputs];
-    const batched = x.shape.length === 4;
-    if (!batched) {
-      // as tf.fused.conv2d does for rank 3: a batch of one going in, rank 3 coming out
-      x = tf.reshape(x, [1, x.shape[0], x.shape[1], x.shape[2]]);
-      if (residual.shape.length === 3) {
-        residual = tf.reshape(residual, [1, residual.shape[0], residual.shape[1], residual.shape[2]]);
-      }
-    }
-    const out = tf.engine().runKernel(
-        'FusedConv2DAdd',
-        {x, filter: p.filter, bias: p.bias, preluActivationWeights: p.preluActivationWeights, residual},
-        {strides: p.strides, pad: p.pad, dataFormat: p.dataFormat, dilations: p.dilations,
-         dimRoundingMode: undefined, activation: p.activation, leakyreluAlpha: p.leakyreluAlpha});
-    if (batched) {
-      return out;
-    }
-    const squeezed = tf.reshape(out, [out.shape[1], out.shape[2], out.shape[3]]);
-    tf.dispose([x, out]);
-    if (residual !== inputs[convInputs]) {
-      residual.dispose();
-    }
-    return squeezed;
-  };
-}
-
-/**
- * _FusedConv2D (1x1, or over few input channels) + the FusedDepthwiseConv2dNative that reads it -> function(inputs) => Tensor,
- * inputs = [x, filter, bias, dwFilter, dwBias]; null when the pair is not of the form the
- * FusedPointwiseDepthwiseConv2D kernel covers (checked on the attributes; shapes are checked by
- * the kernel, which runs the two convolutions itself where it must).
- */
-function compilePointwiseDepthwise(convNode, dwNode, weightMap) {
-  let conv, dw;
-  try {
-    conv = fusedConvParams(convNode)([null, null, null]);
-    dw = fusedConvParams(dwNode)([null, null, null]);
-  } catch (e) {
-    return null;   // a malformed node throws when it is executed on its own, as in the reference
-  }
-  const dataInputs = node => (node.input || []).filter(i => i[0] !== '^');
-  const fusedOps = node => getStringArrayParam(node.attr || {}, 'fused_ops', []);
-  const act = conv.activation;
-  const filter = weightMap[parseNodeName(dataInputs(convNode)[1] || '')[0]];
-  const dwFilter = weightMap[parseNodeName(dataInputs(dwNode)[1] || '')[0]];
-  const ok = dataInputs(convNode).length === 3 && dataInputs(dwNode).length === 3 &&
-      fusedOps(convNode)[0] === 'biasadd' && fusedOps(dwNode)[0] === 'biasadd' &&
-      (act === 'relu' || act === 'relu6') && dw.activation === act &&
-      conv.dataFormat === 'NHWC' && dw.dataFormat === 'NHWC' &&
-      conv.dilations[0] === 1 && conv.dilations[1] === 1 && dw.dilations[0] === 1 && dw.dilations[1] === 1 &&
-      filter != null && filter.shape.length === 4 &&
-      ((filter.shape[0] === 1 && filter.shape[1] === 1 && conv.strides[0] === 1 && conv.strides[1] === 1) ||
-       (filter.shape[2] <= 4 && filter.shape[0] * filter.shape[1] * filter.shape[2] <= 36)) &&
-      dwFilter != null && dwFilter.shape.length === 4 && dwFilter.shape[0] === 3 && dwFilter.shape[1] === 3;
-  if (!ok) {
-    return null;
-  }
-  const attrs = {strides: dw.strides, pad: dw.pad, dimRoundingMode: undefined, activation: act,
-                 convStrides: conv.strides, convPad: conv.pad};
-  return inputs => tf.engine().runKernel(
-      'FusedPointwiseDepthwiseConv2D',
-      {x: inputs[0], filter: inputs[1], bias: inputs[2], dwFilter: inputs[3], dwBias: inputs[4]}, attrs);
 }
 
 /**
@@ -389,7 +298,11 @@ class GraphModel {
   constructor(handler, loadOptions, tfio) {
     this.handler = typeof handler === 'string' ? fileSystem(handler) : handler;
     this.loadOptions = loadOptions || {};
-    this.io = tfio || {decodeWeights: require('../io/decode_weights').decodeWeights};
+    if (tfio == null || typeof tfio.decodeWeights !== 'function') {
+      throw new Error('GraphModel: pass the io module whose decodeWeights decodes the weight bytes as the third argument');
+    }
+    this.io = tfio;
+    this.planner = this.loadOptions.planner || null;
     this.version = 'n/a';
     this.weightMap = null;
   }
@@ -582,8 +495,9 @@ class GraphModel {
       compiled = this.makePlan(feeds, fetches);
       this.plans.set(planKey, compiled);
     }
-    if (this.loadOptions.recordLaunches === true && typeof tf.backend().beginRecording === 'function') {
-      return this.executeRecorded(planKey, compiled, feeds);
+    if (this.planner != null && this.planner.wantsRecording(this.loadOptions)) {
+      return this.planner.runRecorded(this.recordings, planKey, feeds, compiled.outputs.length === 1,
+                                      staged => this.runPlan(compiled, staged));
     }
     return this.runPlan(compiled, feeds);
   }
@@ -610,17 +524,12 @@ class GraphModel {
           for (let i = 0; i < args.length; i++) {
             args[i] = values[step.sources[i]];
           }
-          const key = step.conv != null ? name + '<-' + step.conv : (step.pointwise != null ? name + '<=' + step.pointwise : name);
-          let run = this.compiled[key];
+          let run = step.run;
           if (run === undefined) {
-            if (step.conv != null) {
-              run = compileConvAdd(this.nodes[step.conv]);
-            } else if (step.pointwise != null) {
-              run = step.run;
-            } else {
-              run = compileNode(this.nodes[name]);
+            run = this.compiled[name];
+            if (run === undefined) {
+              run = this.compiled[name] = compileNode(this.nodes[name]);
             }
-            this.compiled[key] = run;
           }
           const out = values[name] = run(args);
           if (this.afterNode != null) {
@@ -639,65 +548,6 @@ class GraphModel {
       const result = outNames.map(n => values[n]);
       return result.length > 1 ? result : result[0];
     });
-  }
-
-  /**
-   * Execution through a recorded launch sequence: node by node the first time a
-   * combination of input shapes is seen (that run also fills the caches a
-   * recording must not touch), recorded and replayed the second time, replayed
-   * from then on.
-   */
-  executeRecorded(planKey, compiled, feeds) {
-    const backend = tf.backend();
-    const names = Object.keys(feeds);
-    const key = planKey + '|' + names.map(n => `${feeds[n].dtype}[${feeds[n].shape}]`).join(';');
-    let rec = this.recordings.get(key);
-    if (rec === undefined) {
-      this.recordings.set(key, {state: 'seen'});
-      return this.runPlan(compiled, feeds);
-    }
-    if (rec.state === 'unrecordable') {
-      return this.runPlan(compiled, feeds);
-    }
-    if (rec.state === 'seen') {
-      const staged = {}, stagedFrom = {};
-      names.forEach(n => {
-        staged[n] = tf.keep(tf.engine().runKernel('HipCopy', {x: feeds[n]}));
-        stagedFrom[n] = feeds[n].dataId;
-      });
-      let outputs = null, graph = null;
-      backend.beginRecording();
-      try {
-        outputs = this.runPlan(compiled, staged);
-        graph = backend.endRecording(true);
-      } catch (e) {
-        if (backend.recording) {
-          backend.endRecording(false);
-        }
-        tf.dispose(staged);
-        if (outputs != null) {
-          tf.dispose(outputs);
-        }
-        rec.state = 'unrecordable';
-        rec.reason = e.message;
-        return this.runPlan(compiled, feeds);
-      }
-      outputs = Array.isArray(outputs) ? outputs : [outputs];
-      outputs.forEach(t => tf.keep(t));
-      rec = {state: 'ready', id: graph.id, nodes: graph.nodes, staged, stagedFrom, outputs,
-             single: compiled.outputs.length === 1};
-      this.recordings.set(key, rec);
-    }
-    names.forEach(n => {
-      // a tensor's values never change: the same dataId again needs no copy
-      if (feeds[n].dataId !== rec.stagedFrom[n]) {
-        backend.copyData(rec.staged[n].dataId, feeds[n].dataId);
-        rec.stagedFrom[n] = feeds[n].dataId;
-      }
-    });
-    backend.replay(rec.id);
-    const results = rec.outputs.map(t => tf.engine().runKernel('HipCopy', {x: t}));
-    return rec.single ? results[0] : results;
   }
 
   /**
@@ -734,8 +584,7 @@ class GraphModel {
       return src;
     });
 
-    // _FusedConv2D read by one Add only -> one step at the convolution's place
-    // that yields the Add's value (the other operand must exist by then).
+    // a backend's planner may run groups of nodes as one step
     const position = {}, readers = {};
     order.forEach((n, idx) => {
       position[n] = idx;
@@ -746,76 +595,38 @@ class GraphModel {
         });
       }
     });
-    const fuse = this.loadOptions.fuseResidualAdd !== false && tf.getKernel != null &&
-        tf.getKernel('FusedConv2DAdd', tf.getBackend()) != null;
-    const convOf = {}, addOf = {};   // Add name -> conv name and back
-    if (fuse) {
-      order.forEach(n => {
-        const node = this.nodes[n];
-        if (!isOp(n) || (node.op !== 'Add' && node.op !== 'AddV2') || (node.input || []).length !== 2) {
-          return;
-        }
-        const src = dataSources(n);
-        if (src.length !== 2 || src[0] === src[1]) {
-          return;
-        }
-        const candidates = [0, 1].filter(k => {
-          const c = src[k], other = src[1 - k];
-          return isOp(c) && this.nodes[c].op === '_FusedConv2D' && readers[c] === 1 && !fetchSet.has(c) &&
-              addOf[c] == null && position[other] < position[c];
-        });
-        if (candidates.length > 0) {
-          const c = src[candidates[candidates.length - 1]];
-          convOf[n] = c;
-          addOf[c] = n;
-        }
-      });
-    }
-
-    // 1x1 _FusedConv2D read by one 3x3 FusedDepthwiseConv2dNative only -> one step at the depthwise node's place
-    const pointwiseOf = {}, depthwiseOf = {}, pairRun = {};
-    const fusePair = this.loadOptions.fusePointwiseDepthwise !== false && tf.getKernel != null &&
-        tf.getKernel('FusedPointwiseDepthwiseConv2D', tf.getBackend()) != null;
-    if (fusePair) {
-      order.forEach(n => {
-        const node = this.nodes[n];
-        if (!isOp(n) || node.op !== 'FusedDepthwiseConv2dNative') {
-          return;
-        }
-        const c = dataSources(n)[0];
-        if (c == null || !isOp(c) || this.nodes[c].op !== '_FusedConv2D' || readers[c] !== 1 || fetchSet.has(c) ||
-            addOf[c] != null) {
-          return;
-        }
-        const run = compilePointwiseDepthwise(this.nodes[c], node, this.weightMap);
-        if (run != null) {
-          pointwiseOf[n] = c;
-          depthwiseOf[c] = n;
-          pairRun[n] = run;
-        }
+    const placed = {}, dropped = new Set();
+    if (this.planner != null) {
+      const view = {
+        order,
+        op: n => this.nodes[n].op,
+        isOp: n => this.nodes[n] != null && isOp(n),
+        sources: dataSources,
+        readers: n => readers[n] || 0,
+        position: n => position[n],
+        isFetched: n => fetchSet.has(n),
+        convParams: n => fusedConvParams(this.nodes[n]),
+        fusedOps: n => getStringArrayParam(this.nodes[n].attr || {}, 'fused_ops', []),
+        weight: n => n == null ? undefined : this.weightMap[n]
+      };
+      this.planner.planFusions(view, this.loadOptions).forEach(f => {
+        placed[f.place] = f;
+        f.drops.forEach(d => dropped.add(d));
       });
     }
 
     const steps = [];
     order.forEach(name => {
-      if (depthwiseOf[name] != null) {
-        return;   // runs inside the step of the depthwise node that reads it
-      }
-      if (pointwiseOf[name] != null) {
-        const conv = pointwiseOf[name];
-        steps.push({name, kind: 'op', pointwise: conv, run: pairRun[name],
-                    sources: dataSources(conv).concat(dataSources(name).slice(1))});
-        return;
-      }
-      if (feeds[name] != null) {
+      const fusion = placed[name];
+      if (fusion != null) {
+        steps.push(Object.assign({name: fusion.yields, kind: 'op', sources: fusion.sources, run: fusion.run}, fusion.tags));
+      } else if (dropped.has(name)) {
+        return;   // runs inside another node's step
+      } else if (feeds[name] != null) {
         steps.push({name, kind: 'feed'});
       } else if (this.nodes[name].op === 'Const') {
         steps.push({name, kind: 'const'});
-      } else if (addOf[name] != null) {
-        const add = addOf[name];
-        const other = dataSources(add).filter(srcName => srcName !== name)[0];
-        steps.push({name: add, kind: 'op', conv: name, sources: dataSources(name).concat([other])});
-      } else if (convOf[name] == null) {
+      } else {
         steps.push({name, kind: 'op', sources: dataSources(name)});
       }
     });
@@ -832,15 +643,8 @@ class GraphModel {
   }
 
   dispose() {
-    if (this.recordings != null) {
-      this.recordings.forEach(rec => {
-        if (rec.state === 'ready') {
-          tf.backend().deleteRecording(rec.id);
-          tf.dispose(rec.staged);
-          tf.dispose(rec.outputs);
-        }
-      });
-      this.recordings.clear();
+    if (this.recordings != null && this.planner != null) {
+      this.planner.disposeRecordings(this.recordings);
     }
     if (this.weightMap != null) {
       Object.keys(this.weightMap).forEach(k => this.weightMap[k].dispose());

@@ -241,6 +241,42 @@ function matMul(a, b, transposeA, transposeB) {
   });
 }
 
+/**
+ * tfjs-core/src/ops/dot.ts:44-84: vectors and matrices only; each form is a matMul of the operands
+ * seen as matrices (a vector on the left is a row, on the right a column), and the result loses
+ * the axes that came from a vector.
+ */
+function dot(t1, t2) {
+  const $t1 = convertToTensor(t1, 't1', 'dot'), $t2 = convertToTensor(t2, 't2', 'dot');
+  const ranksOk = r => r === 1 || r === 2;
+  util.assert(
+      ranksOk($t1.rank) && ranksOk($t2.rank),
+      () => `Error in dot: inputs must all be rank 1 or 2, but got ranks ${$t1.rank} and ${$t2.rank}.`);
+  const inner1 = $t1.rank === 1 ? $t1.size : $t1.shape[1];
+  const inner2 = $t2.rank === 1 ? $t2.size : $t2.shape[0];
+  util.assert(
+      inner1 === inner2,
+      () => `Error in dot: inner dimensions of inputs must match, but got ${inner1} and ${inner2}.`);
+  return ENGINE.tidy(() => {
+    const left = $t1.rank === 1 ? reshape($t1, [1, inner1]) : $t1;
+    const right = $t2.rank === 1 ? reshape($t2, [inner2, 1]) : $t2;
+    const product = matMul(left, right);
+    if ($t1.rank === 2 && $t2.rank === 2) {
+      return product;
+    }
+    return reshape(product, $t1.rank === 1 && $t2.rank === 1 ? [] : [product.size]);
+  });
+}
+
+/** tfjs-core/src/ops/outer_product.ts:42-55: column vector times row vector. */
+function outerProduct(v1, v2) {
+  const $v1 = convertToTensor(v1, 'v1', 'outerProduct'), $v2 = convertToTensor(v2, 'v2', 'outerProduct');
+  util.assert(
+      $v1.rank === 1 && $v2.rank === 1,
+      () => `Error in outerProduct: inputs must be rank 1, but got ranks ${$v1.rank} and ${$v2.rank}.`);
+  return ENGINE.tidy(() => matMul(reshape($v1, [$v1.size, 1]), reshape($v2, [1, $v2.size])));
+}
+
 /** tfjs-core/src/ops/fused/mat_mul.ts:58-211 */
 function fusedMatMul(args) {
   const transposeA = !!args.transposeA, transposeB = !!args.transposeB;
@@ -463,7 +499,7 @@ function chain(method, op) {
 [['reshape', reshape], ['add', add], ['sub', binaryOp('Sub', 'sub')], ['mul', binaryOp('Multiply', 'mul')],
  ['relu', unaryOp('Relu', 'relu')], ['relu6', unaryOp('Relu6', 'relu6')], ['elu', unaryOp('Elu', 'elu')],
  ['sigmoid', unaryOp('Sigmoid', 'sigmoid')], ['leakyRelu', leakyRelu], ['cast', cast], ['avgPool', avgPool],
- ['squeeze', squeeze], ['transpose', transpose], ['mean', mean], ['matMul', matMul], ['conv2d', conv2d],
+ ['squeeze', squeeze], ['transpose', transpose], ['mean', mean], ['matMul', matMul], ['dot', dot], ['conv2d', conv2d],
  ['depthwiseConv2d', depthwiseConv2d]].forEach(([method, op]) => chain(method, op));
 
 module.exports = {
@@ -494,6 +530,8 @@ module.exports = {
   transpose,
   mean,
   matMul,
+  dot,
+  outerProduct,
   conv2d,
   depthwiseConv2d,
   fused: {matMul: fusedMatMul, conv2d: fusedConv2d, depthwiseConv2d: fusedDepthwiseConv2d}

@@ -9,7 +9,8 @@ Classes:
   hand-js      a spec about the form of a call, transcribed into tests/js/hand_specs.js
   error-path   a spec that expects a throw, transcribed into tests/js/error_specs.js
   gradient     tf.grad / tf.grads / tf.valueAndGrad specs: the path is inference, there is no tape
-  other-op     tf.dot and tf.outerProduct specs that live in mat_mul_test.ts: ops outside the path
+(The tf.dot and tf.outerProduct specs of mat_mul_test.ts are compositions that end in BatchMatMul; their
+value specs are in hand_specs.js and their throwing ones in error_specs.js, like the matMul specs'.)
 
 Run:  python tests/golden/make_spec_manifest.py        (needs /root/reference to read the test files)
 """
@@ -33,7 +34,6 @@ TEST_FILES = {
 SPEC = re.compile(r"^\s*(?:it|fit|xit)\(\s*$|^\s*(?:it|fit|xit)\(\s*['`\"]")
 SUITE = re.compile(r"^\s*describe\w*\(\s*['`\"]([^'`\"]*)")
 GRADIENT_CALL = re.compile(r"\btf\.(grad|grads|valueAndGrad|valueAndGrads)\b")
-OTHER_OP_CALL = re.compile(r"\b(tf\.dot|tf\.outerProduct|\w+\.dot)\(")
 
 
 def read_specs(rel_path):
@@ -125,8 +125,6 @@ def build():
                 entry.update({"class": "hand-values", "covered_by": "tests/golden/hand_transcribed.json"})
             elif GRADIENT_CALL.search(body) or "gradient" in suite.lower():
                 entry.update({"class": "gradient", "covered_by": None})
-            elif OTHER_OP_CALL.search(body):
-                entry.update({"class": "other-op", "covered_by": None})
             else:
                 entry.update({"class": "unaccounted", "covered_by": None})
             manifest.append(entry)

@@ -117,6 +117,60 @@ h.test('engine: async backend factory resolves through setBackend', async () => 
   useBackend('cpu');
 });
 
+h.test('flags: HIP_* flags are registered with the Environment and reach the native library (flags_wasm.ts is the model)', () => {
+  const fake = require('./fake_addon');
+  const flags = hip.flags;
+  // every knob of the native library has a flag, unset (-1) by default
+  const header = require('fs').readFileSync(require('path').join(__dirname, '..', '..', 'tfjs_amd', 'csrc', 'common.h'), 'utf8');
+  const native = [];
+  header.replace(/X\((\w+), "(\w+)"\)/g, (_, id, name) => native.push(name));
+  h.assertEqual(flags.TUNING_KNOBS, native);
+  flags.TUNING_KNOBS.forEach(knob => h.assertEqual(tf.env().get(flags.flagOf(knob)), -1));
+  h.assertEqual(flags.flagOf('fuse_pw_dw'), 'HIP_FUSE_PW_DW');
+  // set: the hook calls tfhip_set_tuning at once; a negative value restores the heuristic
+  let mark = fake.calls.length;
+  tf.env().set('HIP_TILE', 12);
+  h.assertEqual(fake.calls.slice(mark), ['setTuning']);
+  h.assertEqual(fake.lastArgs.setTuning, ['tile', 12]);
+  tf.env().set('HIP_DW_ROWS', 6);
+  // a backend that starts later hands the library every flag that is set (it read its environment at init)
+  mark = fake.calls.length;
+  flags.applyTuningFlags();
+  h.assertEqual(fake.calls.slice(mark), ['setTuning', 'setTuning']);
+  tf.env().set('HIP_TILE', -1);
+  h.assertEqual(fake.lastArgs.setTuning, ['tile', -1]);
+  tf.env().set('HIP_DW_ROWS', -5);
+  h.assertEqual(fake.lastArgs.setTuning, ['dw_rows', -1]);
+  mark = fake.calls.length;
+  flags.applyTuningFlags();
+  h.assertEqual(fake.calls.slice(mark), []);
+  // the planner's defaults
+  h.assertEqual([tf.env().getBool('HIP_FUSE_RESIDUAL_ADD'), tf.env().getBool('HIP_FUSE_POINTWISE_DEPTHWISE'),
+                 tf.env().getBool('HIP_RECORD_LAUNCHES')], [true, true, false]);
+});
+
+h.test('flags: HIP_FUSE_RESIDUAL_ADD is the default of the load option of the same meaning', () => {
+  useBackend('hip');
+  const io = {decodeWeights: hip.decodeWeights};
+  const opNames = model => Array.from(model.plans.values())[0].steps.filter(s => s.kind === 'op').map(s => s.name);
+  const x = tf.tensor(new Float32Array(64), [1, 4, 4, 4]);
+  tf.env().set('HIP_FUSE_RESIDUAL_ADD', false);
+  try {
+    const off = hip.loadGraphModel({load: () => residualGraphArtifacts()}, {}, io);
+    off.predict(x).dispose();
+    h.assertEqual(opNames(off), ['e', 'p', 'sum', 'twice', 'out']);
+    off.dispose();
+    // the load option, when given, wins
+    const on = hip.loadGraphModel({load: () => residualGraphArtifacts()}, {fuseResidualAdd: true}, io);
+    on.predict(x).dispose();
+    h.assertEqual(opNames(on), ['e', 'sum', 'twice', 'out']);
+    on.dispose();
+  } finally {
+    tf.env().set('HIP_FUSE_RESIDUAL_ADD', true);
+  }
+  x.dispose();
+});
+
 h.test('engine: IS_TEST leak check flags a kernel that leaks a data id', () => {
   useBackend('cpu');
   tf.env().set('IS_TEST', true);

@@ -4,7 +4,6 @@
  * hand: each entry names its spec (file:line of the `it(`) and gives the call and, where the spec
  * checks one, the message pattern. They run through the op layer in front of whatever backend is
  * active: these errors are thrown before (or, for shape mismatches inside the kernel, by) the backend.
- *   (tf.dot / tf.outerProduct specs are not here: those ops are not on the path.)
  */
 const O = 'tfjs-core/src/ops/';
 
@@ -47,6 +46,14 @@ function specs(tf) {
     {at: O + 'mat_mul_test.ts:663', fn: () => tf.matMul(tf.tensor([2], [1, 1]), {}), message: /Argument 'b' passed to 'matMul' must be a Tensor/},
     {at: O + 'mat_mul_test.ts:709', fn: () => tf.matMul([['a']], [['b']]), message: /Argument 'a' passed to 'matMul' must be numeric tensor/},
     {at: O + 'mat_mul_test.ts:906', fn: () => tf.matMul(ramp(24, [4, 3, 2]), ramp(30, [5, 2, 3]), false, false)},
+    // ---- tf.dot (ops/dot.ts: thrown by the op before BatchMatMul is reached)
+    {at: O + 'mat_mul_test.ts:423', fn: () => tf.dot(ramp(8, [2, 2, 2]), tf.tensor([2, 3]))},
+    {at: O + 'mat_mul_test.ts:447', fn: () => tf.dot(tf.tensor([2, 3, 3]), tf.tensor([2, 1]))},
+    {at: O + 'mat_mul_test.ts:447', fn: () => tf.dot(tf.tensor([2, 1]), tf.tensor([2, 3, 3]))},
+    {at: O + 'mat_mul_test.ts:1279', fn: () => tf.dot(tf.tensor([[1, 2, 3], [4, 5, 6]], [2, 3]), tf.tensor([1, 2, 1, 2], [2, 1, 2]))},
+    {at: O + 'mat_mul_test.ts:1283', fn: () => tf.dot(tf.tensor([1, 2]), tf.tensor([1, 2], [1, 1, 2]))},
+    {at: O + 'mat_mul_test.ts:1283', fn: () => tf.dot(tf.tensor([1, 2]), tf.scalar(1))},
+    {at: O + 'mat_mul_test.ts:1295', fn: () => tf.dot('a', 'b'), message: /Argument 't1' passed to 'dot' must be numeric tensor/},
     // ---- conv2d
     {at: O + 'conv2d_test.ts:603', fn: () => tf.conv2d(tf.tensor([1, 2, 3, 4], [2, 2]), tf.tensor([3, 1, 5, 0], [2, 2, 1, 1]), 1, 0)},
     {at: O + 'conv2d_test.ts:618', fn: () => tf.conv2d(x3(), tf.tensor([3, 1, 5, 0], [2, 2, 1]), 1, 0)},

@@ -59,7 +59,7 @@ module.exports = {
   eventElapsed() { return 0; },
   setLaunchRepeat() {},
   lastKernel() { return 'fake'; },
-  setTuning() {},
+  setTuning() { record('setTuning', arguments); },
   fusedMatMul() { record('fusedMatMul', arguments); },
   fusedConv2D() { record('fusedConv2D', arguments); },
   fusedDepthwiseConv2D() { record('fusedDepthwiseConv2D', arguments); },

@@ -53,6 +53,53 @@ function specs(tf, h) {
       h.assertEqual(c.dtype, 'int32');
       close(c, [5, 6, 11, 15]);
     }},
+    // ---- tf.dot / tf.outerProduct (compositions that end in BatchMatMul: ops/dot.ts, outer_product.ts)
+    {at: O + 'mat_mul_test.ts:227', fn: () => close(tf.dot(tf.tensor1d([2, 3]), tf.tensor2d([1, 2, 3, 4], [2, 2])), [11, 16])},
+    {at: O + 'mat_mul_test.ts:236', fn: () => close(tf.dot(tf.tensor1d([2, 3]), tf.tensor2d([1, 2, 3, 4], [2, 2])), [11, 16])},
+    {at: O + 'mat_mul_test.ts:246', fn: () => close(tf.dot(tf.tensor2d([1, 2, 3, 4], [2, 2]), tf.tensor1d([2, 3])), [8, 18])},
+    {at: O + 'mat_mul_test.ts:432', fn: () => close(tf.dot(tf.tensor1d([2, 3]), tf.tensor1d([2, 1])), [7])},
+    {at: O + 'mat_mul_test.ts:455', fn: () => {
+      const result = tf.outerProduct(tf.tensor1d([2, 3]), tf.tensor1d([2, 1]));
+      h.assertEqual(result.shape, [2, 2]);
+      close(result, [4, 2, 6, 3]);
+    }},
+    {at: O + 'mat_mul_test.ts:465', fn: () => {
+      const result = tf.outerProduct([2, 3], [2, 1]);
+      h.assertEqual(result.shape, [2, 2]);
+      close(result, [4, 2, 6, 3]);
+    }},
+    {at: O + 'mat_mul_test.ts:1227', fn: () => {
+      const a = tf.tensor1d([1, 2]);
+      const aa = tf.dot(a, a);
+      close(aa, [5]);
+      h.assertEqual(aa.shape, []);
+    }},
+    {at: O + 'mat_mul_test.ts:1233', fn: () => {
+      const a = tf.tensor1d([1, 2]);
+      const ab = tf.dot(a, tf.tensor2d([[1, 2], [3, 4]])), ac = tf.dot(a, tf.tensor2d([[1, 2, 3], [4, 5, 6]]));
+      h.assertEqual(ab.shape, [2]);
+      h.assertEqual(ac.shape, [3]);
+      close(ab, [7, 10]);
+      close(ac, [9, 12, 15]);
+    }},
+    {at: O + 'mat_mul_test.ts:1242', fn: () => {
+      const ba = tf.tensor2d([[1, 2], [3, 4]]).dot(tf.tensor1d([1, 2]));
+      h.assertEqual(ba.shape, [2]);
+      close(ba, [5, 11]);
+    }},
+    {at: O + 'mat_mul_test.ts:1248', fn: () => {
+      const b = tf.tensor2d([[1, 2], [3, 4]]), c = tf.tensor2d([[1, 2, 3], [4, 5, 6]]);
+      const bb = tf.dot(b, b), bc = tf.dot(b, c);
+      h.assertEqual(bb.shape, [2, 2]);
+      h.assertEqual(bc.shape, [2, 3]);
+      close(bb, [7, 10, 15, 22]);
+      close(bc, [9, 12, 15, 19, 26, 33]);
+    }},
+    {at: O + 'mat_mul_test.ts:1288', fn: () => {
+      const res = tf.dot([1, 2, 3], [1, 2, 3]);
+      close(res, [14]);
+      h.assertEqual(res.shape, []);
+    }},
     {at: O + 'mat_mul_test.ts:677', fn: () => {
       const c = tf.tensor([[1, 2, 3], [4, 5, 6]], [2, 3]).matMul([[0, 1], [-3, 2], [2, 1]]);
       h.assertEqual(c.shape, [2, 2]);

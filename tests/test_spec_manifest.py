@@ -1,7 +1,6 @@
 """Every spec of the reference's six op test files for this path is accounted for: carried by a
 fixture or a transcribed JavaScript spec that the suites here run, or classed out of scope with a
-reason (gradients: no tape on an inference path; tf.dot / tf.outerProduct: other ops that share
-mat_mul_test.ts). The manifest is data written by tests/golden/make_spec_manifest.py."""
+reason (gradients only: no tape on an inference path). The manifest is data written by tests/golden/make_spec_manifest.py."""
 import importlib.util
 import json
 import os
@@ -13,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 GOLDEN = os.path.join(HERE, "golden")
 REFERENCE = os.environ.get("TFJS_REFERENCE", "/root/reference")
 CARRIED = {"golden", "hand-values", "hand-js", "error-path"}
-OUT_OF_SCOPE = {"gradient", "other-op"}
+OUT_OF_SCOPE = {"gradient"}
 EXPECTED_TOTALS = {  # `it(` specs per file of the reference at the surveyed commit
     "tfjs-core/src/ops/fused/fused_mat_mul_test.ts": 21,
     "tfjs-core/src/ops/fused/fused_conv2d_test.ts": 54,
@@ -45,8 +44,9 @@ def test_no_spec_is_unaccounted_and_every_file_is_complete():
         per_file[e["file"]] = per_file.get(e["file"], 0) + 1
     assert per_file == EXPECTED_TOTALS
     carried = sum(1 for e in specs if e["class"] in CARRIED)
-    # every forward, shape and error spec of the six files: all but the gradient and tf.dot ones
-    assert carried == len(specs) - sum(1 for e in specs if e["class"] in OUT_OF_SCOPE) == 191
+    # every forward, shape and error spec of the six files, tf.dot / tf.outerProduct included: all but the gradient ones
+    assert carried == len(specs) - sum(1 for e in specs if e["class"] in OUT_OF_SCOPE) == 207
+    assert not [e for e in specs if e["class"] == "other-op"]
 
 
 def test_every_carried_spec_points_at_something_the_suites_run():

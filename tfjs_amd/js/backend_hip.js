@@ -55,6 +55,7 @@ class HipBackend extends tf.KernelBackend {
   constructor(device) {
     super();
     addon.init(device == null ? 0 : device);
+    require('./flags_hip').applyTuningFlags();   // HIP_* flags set before the native library read its environment
     this.deviceInfo = addon.deviceInfo();
     this.data = new tf.DataStorage(this, tf.engine());
     this.nextEventSlot = 0;

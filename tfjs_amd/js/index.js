@@ -15,7 +15,40 @@ const {decodeWeights} = require('./io/decode_weights');
 const matmul = require('./kernels/matmul');
 const conv = require('./kernels/conv');
 const glue = require('./kernels/glue');
-const graphModel = require('./standin/graph_model');
+const flags = require('./flags_hip');
+const graphPlan = require('./graph_plan');
+
+/**
+ * The graph-model executor: @tensorflow/tfjs-converter when it is installed, else
+ * the stand-in for it that the repository keeps outside the package
+ * (reference_standin/graph_model.js). Either way the weights are decoded by this
+ * package's decodeWeights unless the caller names another io module; the
+ * stand-in also takes this package's planner (fusions across nodes, recorded
+ * launch sequences), which the converter's own executor has no hook for.
+ */
+function resolveGraphModel() {
+  if (!tf.usingStandin) {
+    try {
+      return require('@tensorflow/tfjs-converter');
+    } catch (e) {
+      // fall through: core without converter
+    }
+  }
+  try {
+    return require('../../reference_standin/graph_model');
+  } catch (e) {
+    return null;
+  }
+}
+const graphModel = resolveGraphModel();
+const withPlanner = options => Object.assign({planner: graphPlan}, options);
+
+function loadGraphModel(modelUrl, options, tfio) {
+  if (graphModel == null) {
+    throw new Error('loadGraphModel needs @tensorflow/tfjs-converter; it is not installed');
+  }
+  return graphModel.loadGraphModel(modelUrl, withPlanner(options), tfio || {decodeWeights});
+}
 
 const kernelConfigs = [
   matmul.fusedMatMulConfig, matmul.batchMatMulConfig, conv.fusedConv2DConfig,
@@ -34,9 +67,10 @@ module.exports = {
   HipBackend,
   decodeWeights,
   kernelConfigs,
-  // graph-model loader for where @tensorflow/tfjs-converter is not installed
-  GraphModel: graphModel.GraphModel,
-  loadGraphModel: graphModel.loadGraphModel,
-  fileSystem: graphModel.fileSystem,
+  graphPlan,
+  flags,
+  GraphModel: graphModel ? graphModel.GraphModel : undefined,
+  loadGraphModel,
+  fileSystem: graphModel ? graphModel.fileSystem : undefined,
   version: '0.1.0'
 };
