@@ -75,6 +75,18 @@ int tfhip_memory_info(size_t *live, size_t *live_bytes, size_t *pooled_bytes);
  * number of K slices of the last matmul / convolution launched as a GEMM. For
  * tests and diagnosis; no counterpart in the reference. */
 int tfhip_workspace_info(size_t *bytes, size_t *allocations, int *last_splits);
+/* *finite = 0 when the `elems` floats at `filter` hold an Inf or a NaN, else 1.
+ * The reference skips filter taps that fall outside the image
+ * (tfjs-backend-cpu/src/kernels/Conv2D.ts:72-84, DepthwiseConv2dNative.ts:72-86);
+ * the matrix-core kernels read a zero there and multiply it, which is the same
+ * number unless the filter value is not finite. The convolution entry points
+ * look for themselves and give such a filter to kernels that skip the taps; the
+ * fused pair and block entry points refuse it, and this tells a caller
+ * beforehand to run the separate convolutions instead. The answer is remembered
+ * per filter (address, length, allocation), so asking costs one small kernel and
+ * one wait for the stream the first time and a table look-up afterwards; the
+ * first question about a filter cannot be asked while recording. */
+int tfhip_filter_is_finite(const float *filter, int64_t elems, int *finite);
 /* Lets kernels accept device memory the caller allocated elsewhere. */
 int tfhip_register_external(void *dptr, size_t bytes);
 int tfhip_unregister_external(void *dptr);

@@ -529,14 +529,8 @@ def main():
         f.write("Specs of the reference's test files that make_fixtures.py's parser did not read, with the "
                 "parser's reason (line = start of the match, which may sit a blank line above the `it(`). "
                 "Where each of them is carried instead (hand_transcribed.json, tests/js/hand_specs.js, "
-                "tests/js/error_specs.js) or why it is out of scope (gradient, other-op) is in spec_manifest.json.\n")
+                "tests/js/error_specs.js) or why it is out of scope (gradient) is in spec_manifest.json.\n")
         f.write("\n".join(skipped) + "\n")
-        f.write("\nKnown divergence outside every spec above: a tap of a convolution window that lies in the padding is "
-                "skipped by tfjs-backend-cpu (Conv2D.ts:64-100, DepthwiseConv2dNative.ts:62-95) and read as zero times the "
-                "weight by the GEMM-shaped and row-pipeline kernels of the hip backend. An Inf or NaN filter weight therefore "
-                "gives NaN at border outputs there, and the reference's value here in the oracle. Finite weights (every spec, "
-                "every model) are unaffected.\n")
-
 
 if __name__ == "__main__":
     main()

@@ -49,6 +49,7 @@ module.exports = {
     return out;
   },
   sync() {},
+  filterIsFinite() { return true; },
   workspaceInfo() { return {bytes: 0, allocations: 0, lastSplits: 1}; },
   memoryInfo() {
     let bytes = 0;

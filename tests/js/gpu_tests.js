@@ -308,6 +308,53 @@ h.test('FusedConv2DAdd: one launch with the bits of FusedConv2D followed by Add;
   h.assertEqual(tf.backend().numDataIds(), before);
 });
 
+h.test('FusedPointwiseDepthwiseConv2D: a depthwise filter with an Inf or NaN takes the separate convolutions, which skip taps outside the image like the reference', () => {
+  let seed = 29;
+  const rnd = n => Float32Array.from({length: n}, () => ((seed = (Math.imul(seed, 1664525) + 1013904223) >>> 0) / 2 ** 32) + 0.25);
+  const addon = require('../../tfjs_amd/js/binding').addon;
+  const [n, size, cin, mid] = [32, 56, 24, 144];
+  const xv = rnd(n * size * size * cin), wv = rnd(cin * mid).map(v => v - 0.6), bv = rnd(mid), dbv = rnd(mid);
+  [Infinity, NaN].forEach(bad => {
+    const dwv = rnd(9 * mid).map(v => v - 0.7);
+    dwv[0 * mid + 5] = bad;             // tap (0, 0) of channel 5: outside the image for the first row and column
+    dwv[8 * mid + 77] = bad;            // tap (2, 2) of channel 77
+    const run = backendName => {
+      h.assert(tf.engine().setBackend(backendName) === true);
+      const x = tf.tensor(xv, [n, size, size, cin]), filter = tf.tensor(wv, [1, 1, cin, mid]), bias = tf.tensor(bv, [mid]);
+      const dwFilter = tf.tensor(dwv, [3, 3, mid, 1]), dwBias = tf.tensor(dbv, [mid]);
+      let y;
+      if (backendName === 'hip') {
+        y = tf.engine().runKernel('FusedPointwiseDepthwiseConv2D', {x, filter, bias, dwFilter, dwBias},
+                                  {strides: [1, 1], pad: 'same', activation: 'relu6'});
+        h.assertEqual(addon.lastKernel(), 'depthwise_generic');   // not the pair kernel this shape takes with a finite filter
+      } else {
+        const e = tf.fused.conv2d({x, filter, strides: [1, 1], pad: 'valid', dataFormat: 'NHWC', dilations: [1, 1], bias, activation: 'relu6'});
+        y = tf.fused.depthwiseConv2d({x: e, filter: dwFilter, strides: [1, 1], pad: 'same', dataFormat: 'NHWC', dilations: [1, 1],
+                                      bias: dwBias, activation: 'relu6'});
+        e.dispose();
+      }
+      const values = y.dataSync();
+      tf.dispose([x, filter, bias, dwFilter, dwBias, y]);
+      return values;
+    };
+    const want = run('cpu'), got = run('hip');
+    let nans = 0, worst = 0;
+    for (let i = 0; i < want.length; i++) {
+      if (Number.isNaN(want[i]) !== Number.isNaN(got[i])) {
+        throw new Error(`element ${i}: got ${got[i]}, the reference has ${want[i]}`);
+      }
+      if (Number.isNaN(want[i])) {
+        nans++;
+      } else {
+        worst = Math.max(worst, Math.abs(got[i] - want[i]) / Math.max(1, Math.abs(want[i])));
+      }
+    }
+    h.assert(worst <= 1e-3, `max scaled error ${worst}`);
+    h.assert(Number.isNaN(bad) ? nans > 0 && nans < want.length : true);
+  });
+  h.assert(tf.engine().setBackend('hip') === true);
+});
+
 h.test('FusedPointwiseDepthwiseConv2D: expansion + depthwise stage in one launch, the bits of the two kernels; used by the graph model at batch 32', () => {
   h.assert(tf.engine().setBackend('hip') === true);
   const before = tf.backend().numDataIds();

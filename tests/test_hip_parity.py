@@ -1011,6 +1011,188 @@ def test_pointwise_depthwise_stream_kernel_non_finite(hip, orc, tuning, stride, 
     np.testing.assert_array_equal(got[ok].view(np.uint32), two[ok].view(np.uint32))
 
 
+def _same_non_finite_pattern(got, want):
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+    np.testing.assert_array_equal(np.isposinf(got), np.isposinf(want))
+    np.testing.assert_array_equal(np.isneginf(got), np.isneginf(want))
+    finite = np.isfinite(want)
+    assert finite.any()
+    assert_parity(got[finite], want[finite])
+
+
+def _last_kernel():
+    from tfjs_amd import capi
+    name = ctypes.create_string_buffer(256)
+    capi.load_library().tfhip_last_kernel(name, 256)
+    return name.value.decode()
+
+
+NON_FINITE_CONV_CASES = [
+    # name, x shape, filter shape, strides, pad, data format, with bias / activation / residual, kernel a finite filter takes
+    ("implicit gemm 3x3", (2, 9, 11, 16), (3, 3, 16, 32), 1, "same", "NHWC", True, "gemm_kernel"),
+    ("implicit gemm 3x3 stride 2", (2, 10, 10, 8), (3, 3, 8, 16), 2, "same", "NHWC", True, "gemm_kernel"),
+    ("implicit gemm 5x5 explicit pad", (1, 8, 8, 4), (5, 5, 4, 12), 1, [[0, 0], [2, 1], [0, 3], [0, 0]], "NHWC", False, ""),
+    ("stem on the matrix cores", (2, 16, 16, 3), (3, 3, 3, 32), 2, "same", "NHWC", True, "conv_few_taps"),
+    ("stem, lane per pixel", (1, 12, 12, 3), (5, 5, 3, 8), 1, "same", "NHWC", True, "conv_few_channels"),
+    ("scalar loaders, odd channels", (1, 7, 6, 5), (3, 3, 5, 7), 1, "same", "NHWC", False, "gemm_kernel"),
+    ("channels first", (1, 4, 9, 8), (3, 3, 4, 8), 1, "same", "NCHW", False, "gemm_kernel"),
+]
+
+
+@pytest.mark.parametrize("case", NON_FINITE_CONV_CASES, ids=[c[0] for c in NON_FINITE_CONV_CASES])
+@pytest.mark.parametrize("bad", [np.inf, np.nan], ids=["inf", "nan"])
+def test_conv2d_with_a_non_finite_filter_value_skips_taps_outside_the_image(hip, orc, case, bad):
+    """The reference skips filter taps that fall outside the image (Conv2D.ts:72-84): an Inf or NaN filter
+    value reaches only the outputs whose window holds the tap INSIDE the image. The matrix-core kernels read
+    a zero for an outside tap and would multiply it (0 x Inf = NaN at every border output); a padded
+    convolution whose filter is not finite therefore runs on the tap-skipping kernel, whatever kernel the
+    same shape takes with a finite filter."""
+    _, x_shape, w_shape, strides, pad, fmt, fused, finite_kernel = case
+    rng = np.random.default_rng(len(case[0]) * 31 + w_shape[3])
+    x = rng.uniform(0.5, 1.5, x_shape).astype(np.float32)
+    w = rng.normal(0, 0.3, w_shape).astype(np.float32)
+    out_c = w_shape[3]
+    kw = {}
+    if fused:
+        kw = dict(bias=rng.uniform(-1, 1, (out_c,)).astype(np.float32), activation="relu6")
+    got = hip.fused_conv2d(x, w, strides=strides, pad=pad, data_format=fmt, **kw)
+    if finite_kernel:
+        assert _last_kernel().startswith(finite_kernel), _last_kernel()
+    assert_parity(got, orc.fused_conv2d(x, w, strides=strides, pad=pad, data_format=fmt, **kw))
+    w[0, 0, 0, 1] = bad                      # the top-left tap: outside the image for the first row and column
+    w[w_shape[0] - 1, w_shape[1] - 1, w_shape[2] - 1, out_c - 1] = -bad if np.isinf(bad) else bad   # and the bottom-right one
+    want = orc.fused_conv2d(x, w, strides=strides, pad=pad, data_format=fmt, **kw)
+    # (a border output whose window holds the bad tap outside the image stays a number: multiplying the
+    # padding's zero by the tap would have made it NaN)
+    assert not np.isnan(want).all()
+    got = hip.fused_conv2d(x, w, strides=strides, pad=pad, data_format=fmt, **kw)
+    assert _last_kernel() == "conv_skip_taps"
+    _same_non_finite_pattern(got, want)
+    if fused and fmt == "NHWC":
+        res = rng.uniform(-2, 2, want.shape).astype(np.float32)
+        got = hip.fused_conv2d(x, w, strides=strides, pad=pad, residual=res, **kw)
+        _same_non_finite_pattern(got, orc.add(want, res))
+
+
+def test_conv2d_without_padding_keeps_its_kernel_for_a_non_finite_filter(hip, orc):
+    """No window reaches outside the image: nothing to skip, the filter is not even looked at."""
+    rng = np.random.default_rng(5)
+    x = rng.uniform(0.5, 1.5, (2, 6, 6, 16)).astype(np.float32)
+    for w_shape, pad in [((1, 1, 16, 32), "same"), ((3, 3, 16, 32), "valid")]:
+        w = rng.normal(0, 0.3, w_shape).astype(np.float32)
+        w[0, 0, 2, 3] = np.inf
+        w[0, 0, 5, 7] = np.nan
+        got = hip.fused_conv2d(x, w, pad=pad)
+        assert _last_kernel().startswith("gemm_kernel")
+        _same_non_finite_pattern(got, orc.fused_conv2d(x, w, pad=pad))
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("flat", [0, 1], ids=["rows", "flat"])
+@pytest.mark.parametrize("bad", [np.inf, np.nan], ids=["inf", "nan"])
+def test_depthwise_with_a_non_finite_filter_value_skips_taps_outside_the_image(hip, orc, tuning, stride, flat, bad):
+    """DepthwiseConv2dNative.ts:72-86 skips taps outside the image as well: the 3x3 row kernels, which read
+    zeros there, hand a filter that is not finite to the general kernel."""
+    tuning("dw_flat", flat)
+    rng = np.random.default_rng(17 + stride)
+    x = rng.uniform(0.5, 1.5, (2, 13, 10, 8)).astype(np.float32)
+    w = rng.normal(0, 0.4, (3, 3, 8, 1)).astype(np.float32)
+    b = rng.uniform(-1, 1, (8,)).astype(np.float32)
+    got = hip.fused_depthwise_conv2d(x, w, strides=stride, pad="same", bias=b, activation="relu6")
+    assert _last_kernel().startswith("depthwise_3x3_flat" if flat else "depthwise_3x3_rows"), _last_kernel()
+    w[0, 0, 1, 0] = bad
+    w[2, 2, 6, 0] = bad
+    want = orc.fused_depthwise_conv2d(x, w, strides=stride, pad="same", bias=b, activation="relu6")
+    if stride == 1:
+        assert not np.isnan(want[0, 0, 0, 1])    # the corner's window holds the bad tap outside the image: skipped
+    got = hip.fused_depthwise_conv2d(x, w, strides=stride, pad="same", bias=b, activation="relu6")
+    assert _last_kernel() == "depthwise_generic"
+    _same_non_finite_pattern(got, want)
+    # 'valid': no window leaves the image, the row kernels keep the filter
+    got = hip.fused_depthwise_conv2d(x, w, strides=stride, pad="valid", bias=b, activation="relu6")
+    assert _last_kernel().startswith("depthwise_3x3_")
+    _same_non_finite_pattern(got, orc.fused_depthwise_conv2d(x, w, strides=stride, pad="valid", bias=b, activation="relu6"))
+
+
+def test_pair_and_block_kernels_refuse_a_non_finite_filter(hip, orc):
+    """The fused pair kernels and the block kernel pad the expanded tensor with zeros and multiply them by
+    the depthwise filter: with an Inf or NaN in it they refuse, tfhip_filter_is_finite says so beforehand,
+    and the separate convolutions (which then skip the taps) match the reference. What the library
+    remembers about a filter goes when its buffer is written again."""
+    from tfjs_amd import capi
+    from tfjs_amd.capi import DeviceBuffer, HipBackendError, check
+    lib = capi.load_library()
+    rng = np.random.default_rng(23)
+    n, h, w_, cin, mid, cout = 2, 14, 14, 64, 128, 64
+    x = rng.uniform(-1, 1, (n, h, w_, cin)).astype(np.float32)
+    w1 = rng.normal(0, 0.2, (1, 1, cin, mid)).astype(np.float32)
+    b1 = rng.uniform(0, 1, (mid,)).astype(np.float32)
+    w2 = rng.normal(0, 0.4, (3, 3, mid, 1)).astype(np.float32)
+    b2 = rng.uniform(-1, 1, (mid,)).astype(np.float32)
+    w3 = rng.normal(0, 0.1, (1, 1, mid, cout)).astype(np.float32)
+    stem_x = rng.uniform(-1, 1, (2, 32, 32, 3)).astype(np.float32)
+    stem_w = rng.normal(0, 0.3, (3, 3, 3, 32)).astype(np.float32)
+    stem_dw = rng.normal(0, 0.4, (3, 3, 32, 1)).astype(np.float32)
+    stem_b = rng.uniform(0, 1, (32,)).astype(np.float32)
+    # finite filters: all three take the shapes
+    hip.fused_pointwise_depthwise(x, w1, w2, pw_bias=b1, pw_activation="relu6", dw_bias=b2, dw_activation="relu6")
+    hip.fused_inverted_residual(x, w1, w2, w3, pw_bias=b1, dw_bias=b2)
+    hip.fused_conv2d_depthwise(stem_x, stem_w, stem_dw, strides=2, bias=stem_b, dw_bias=stem_b)
+    w2[0, 1, 5, 0] = np.inf
+    with pytest.raises(HipBackendError, match="Inf or NaN"):
+        hip.fused_pointwise_depthwise(x, w1, w2, pw_bias=b1, pw_activation="relu6", dw_bias=b2, dw_activation="relu6")
+    with pytest.raises(HipBackendError, match="Inf or NaN"):
+        hip.fused_inverted_residual(x, w1, w2, w3, pw_bias=b1, dw_bias=b2)
+    bad_dw = stem_dw.copy()
+    bad_dw[2, 2, 0, 0] = np.nan
+    with pytest.raises(HipBackendError, match="Inf or NaN"):
+        hip.fused_conv2d_depthwise(stem_x, stem_w, bad_dw, strides=2, bias=stem_b, dw_bias=stem_b)
+    bad_w = stem_w.copy()
+    bad_w[0, 0, 1, 4] = -np.inf
+    with pytest.raises(HipBackendError, match="Inf or NaN"):
+        hip.fused_conv2d_depthwise(stem_x, bad_w, stem_dw, strides=2, bias=stem_b, dw_bias=stem_b)
+    # the separate convolutions instead: the reference's values
+    e = hip.fused_conv2d(x, w1, bias=b1, activation="relu6")
+    got = hip.fused_depthwise_conv2d(e, w2, pad="same", bias=b2, activation="relu6")
+    want = orc.fused_depthwise_conv2d(orc.fused_conv2d(x, w1, bias=b1, activation="relu6"), w2, pad="same", bias=b2,
+                                      activation="relu6")
+    _same_non_finite_pattern(got, want)
+    got = hip.fused_depthwise_conv2d(hip.fused_conv2d(stem_x, bad_w, strides=2, pad="same", bias=stem_b, activation="relu6"),
+                                     stem_dw, pad="same", bias=stem_b, activation="relu6")
+    want = orc.fused_depthwise_conv2d(orc.fused_conv2d(stem_x, bad_w, strides=2, pad="same", bias=stem_b, activation="relu6"),
+                                      stem_dw, pad="same", bias=stem_b, activation="relu6")
+    _same_non_finite_pattern(got, want)
+    # the question itself, and its memory: an upload into the buffer makes the library look again
+    buf = DeviceBuffer.from_numpy(w2)
+    finite = ctypes.c_int(-1)
+    try:
+        check(lib.tfhip_filter_is_finite(buf.ptr, w2.size, ctypes.byref(finite)))
+        assert finite.value == 0
+        w2[0, 1, 5, 0] = 0.25
+        buf.upload(w2)
+        check(lib.tfhip_filter_is_finite(buf.ptr, w2.size, ctypes.byref(finite)))
+        assert finite.value == 1
+        # a kernel's result written into it counts as well
+        src = DeviceBuffer.from_numpy(np.full(w2.size, np.nan, np.float32))
+        check(lib.tfhip_copy(buf.ptr, src.ptr, w2.size * 4))
+        check(lib.tfhip_filter_is_finite(buf.ptr, w2.size, ctypes.byref(finite)))
+        assert finite.value == 0
+        src.free()
+        # a first question cannot be asked while recording (it waits for the stream)
+        fresh = DeviceBuffer.from_numpy(w2)
+        check(lib.tfhip_capture_begin())
+        try:
+            assert lib.tfhip_filter_is_finite(fresh.ptr, w2.size, ctypes.byref(finite)) != 0
+            assert b"recording" in lib.tfhip_last_error()
+            check(lib.tfhip_filter_is_finite(buf.ptr, w2.size, ctypes.byref(finite)))   # a remembered one can
+            assert finite.value == 0
+        finally:
+            check(lib.tfhip_capture_end(None, None))
+        fresh.free()
+    finally:
+        buf.free()
+
+
 BLOCK_CASES = [
     # batch, h, w, in_c, mid_c, out_c, stride, pad, activation, residual, block_rows knob
     (2, 14, 14, 64, 384, 64, 1, "same", "relu6", True, None),       # MobileNetV2 b7-b9: two waves per pixel block
@@ -1258,7 +1440,38 @@ def test_recorded_graph_replays(hip, orc):
 
 # ------------------------------------------------------------- MobileNetV2 graph
 
-def test_config4_mobilenet_v2_batch1_vs_oracle(hip, orc, tmp_path):
+def test_config4_mobilenet_v2_batch1_fused_plan_vs_oracle(hip, orc, tmp_path):
+    """Batch 1, the reference's own benchmark setting and what the bench line's `b1` runs: the fused plan
+    (17 expansion pairs, 10 conv + Add pairs) with the kernels that batch selects - the one-row depthwise
+    kernel everywhere, 16-channel stem slices, the pair kernels at every size - against the oracle run
+    layer by layer, and against the unfused plan."""
+    from tfjs_amd import workloads
+    weights = workloads.mobilenet_v2_weights(seed=3)
+    workloads.write_model(str(tmp_path), weights, np.uint8)
+    buf, specs = workloads.read_model(str(tmp_path))
+    decoded = orc.decode_weights(buf, specs)
+    x = workloads.mobilenet_v2_input(1)
+    ops, _ = workloads.mobilenet_v2_graph()
+    want = workloads.run_graph(orc, ops, decoded, x)
+    outs = {}
+    for fused in (True, False):
+        model = workloads.DeviceMobileNetV2(str(tmp_path), 1, fuse_residual_add=fused, fuse_expand_depthwise=fused)
+        try:
+            kinds = [op["kind"] for op, _ in model.plan]
+            assert sum(k in ("pwdw", "cvdw") for k in kinds) == (17 if fused else 0)
+            assert sum("residual" in op for op, _ in model.plan) == (10 if fused else 0)
+            model.set_input(x)
+            outs[fused] = model.predict()
+            np.testing.assert_array_equal(outs[fused], model.predict())
+        finally:
+            model.close()
+    assert want.shape == (1, 1000)
+    assert_parity(outs[True], want)
+    assert_parity(outs[False], want)
+    assert_parity(outs[True], outs[False], 1e-4)
+
+
+def test_config4_mobilenet_v2_batch2_and_batch32_vs_oracle(hip, orc, tmp_path):
     """The whole graph, uint8-quantized weights dequantized on load, device
     resident, against the oracle run layer by layer on the same decoded weights."""
     from tfjs_amd import workloads

@@ -107,7 +107,7 @@ def test_c_abi_library_exports_every_declared_symbol():
 def test_addon_loads_and_exports_every_entry_point():
     proc = subprocess.run([NODE, "-e", """
       const a = require('%s/tfjs_amd/lib/tfjs_hip.node');
-      const want = ['init','shutdown','deviceInfo','alloc','free','upload','download','sync','memoryInfo','workspaceInfo','eventRecord',
+      const want = ['init','shutdown','deviceInfo','alloc','free','upload','download','sync','memoryInfo','workspaceInfo','filterIsFinite','eventRecord',
                     'eventElapsed','setLaunchRepeat','lastKernel','fusedMatMul','fusedConv2D','fusedDepthwiseConv2D',
                     'dequantAffine','dequantF16','add','meanHW','binary','unary','avgPool','cast','transpose2d',
                     'fusedInvertedResidual','invertedResidualPays','fusedMatMulNoAlloc','fusedPointwiseDepthwise',
@@ -132,9 +132,13 @@ def test_node_gpu_tier(tmp_path):
 
 @pytest.mark.gpu
 @needs_node
-def test_graph_model_predict_batch32_matches_the_c_oracle(tmp_path):
+@pytest.mark.parametrize("batch", [32, 1], ids=["batch32", "batch1"])
+def test_graph_model_predict_matches_the_c_oracle(tmp_path, batch):
     """The headline's own path, end to end: a converter-format MobileNetV2 (uint8 weights, dequantized on
-    the GPU at load) through loadGraphModel + GraphModel.predict in Node at batch 32, against the C oracle
+    the GPU at load) through loadGraphModel + GraphModel.predict in Node, at batch 32 (the headline) and at
+    batch 1 (the reference's own benchmark setting, e2e/benchmarks/benchmark_util.js:246-286, where the
+    library selects other kernels: the one-row depthwise kernel everywhere, 16-channel stem slices), node by
+    node and as a replayed recording (what the bench line's `b1` measures), against the C oracle
     run layer by layer on the same decoded weights and the same input. Tolerance: the float32 bound of the
     build, |got - want| <= 1e-3 * max(1, |want|) on every logit (tfjs's float32 test epsilon); the
     observed error is about 2e-5."""
@@ -145,7 +149,7 @@ def test_graph_model_predict_batch32_matches_the_c_oracle(tmp_path):
     workloads.write_graph_model(str(model_dir), workloads.mobilenet_v2_weights(seed=3), np.uint8)
     buf, specs = workloads.read_model(str(model_dir))
     decoded = orc.decode_weights(buf, specs)
-    x = workloads.mobilenet_v2_input(32)
+    x = workloads.mobilenet_v2_input(batch)
     ops, _ = workloads.mobilenet_v2_graph()
     want = workloads.run_graph(orc, ops, decoded, x)
     x.astype("<f4").tofile(str(tmp_path / "x.bin"))
@@ -156,7 +160,7 @@ def test_graph_model_predict_batch32_matches_the_c_oracle(tmp_path):
       (async () => {
         await tf.setBackend('hip');
         const raw = fs.readFileSync(process.argv[3]);
-        const x = tf.tensor(new Float32Array(raw.buffer, raw.byteOffset, raw.length / 4), [32, 224, 224, 3]);
+        const x = tf.tensor(new Float32Array(raw.buffer, raw.byteOffset, raw.length / 4), [%d, 224, 224, 3]);
         const out = {};
         for (const record of [false, true]) {
           const model = hip.loadGraphModel(process.argv[2], {recordLaunches: record}, {decodeWeights: hip.decodeWeights});
@@ -167,12 +171,15 @@ def test_graph_model_predict_batch32_matches_the_c_oracle(tmp_path):
           }
           out[record ? 'recorded' : 'plain'] = Array.from(y.dataSync());
           out.shape = y.shape;
+          if (record) {
+            out.recordings = Array.from(model.recordings.values()).map(r => r.state);
+          }
           y.dispose();
           model.dispose();
         }
         fs.writeFileSync(process.argv[4], JSON.stringify(out));
       })().catch(e => { console.error(e.stack); process.exit(1); });
-    """ % ROOT
+    """ % (ROOT, batch)
     (tmp_path / "run.js").write_text(script)
     proc = subprocess.run([NODE, str(tmp_path / "run.js"), str(model_dir), str(tmp_path / "x.bin"), str(tmp_path / "out.json")],
                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
@@ -183,4 +190,5 @@ def test_graph_model_predict_batch32_matches_the_c_oracle(tmp_path):
     err = np.abs(plain.astype(np.float64) - want) / np.maximum(1.0, np.abs(want))
     assert err.max() <= 1e-3, err.max()
     # a replay runs the recorded kernels on the same operands: the same bits
+    assert got["recordings"] == ["ready"], got["recordings"]
     np.testing.assert_array_equal(np.array(got["recorded"], dtype=np.float32).reshape(want.shape), plain)

@@ -33,6 +33,7 @@ SIGNATURES = {
     "tfhip_copy": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t],
     "tfhip_set_tuning": [ctypes.c_char_p, ctypes.c_int],
     "tfhip_memory_info": [ctypes.POINTER(ctypes.c_size_t)] * 3,
+    "tfhip_filter_is_finite": [c_f32p, c_i64, ctypes.POINTER(ctypes.c_int)],
     "tfhip_workspace_info": [ctypes.POINTER(ctypes.c_size_t)] * 2 + [ctypes.POINTER(ctypes.c_int)],
     "tfhip_register_external": [ctypes.c_void_p, ctypes.c_size_t],
     "tfhip_unregister_external": [ctypes.c_void_p],

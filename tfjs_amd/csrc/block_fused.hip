@@ -457,10 +457,16 @@ extern "C" int tfhip_fused_inverted_residual(const float *x, const float *pw_fil
   if (pw_bias) TFHIP_CHECK_RANGE(pw_bias, mid_c, 4, "pw_bias");
   if (dw_bias) TFHIP_CHECK_RANGE(dw_bias, mid_c, 4, "dw_bias");
   if (proj_bias) TFHIP_CHECK_RANGE(proj_bias, out_c, 4, "proj_bias");
-  TFHIP_CHECK_RANGE(y, batch * out_h * out_w * out_c, 4, "y");
+  TFHIP_CHECK_OUTPUT(y, batch * out_h * out_w * out_c, 4, "y");
   if (residual) {
     TFHIP_CHECK_RANGE(residual, batch * out_h * out_w * out_c, 4, "residual");
     TFHIP_CHECK_ARG(residual != y, "tfhip_fused_inverted_residual: residual and y are the same buffer");
+  }
+  if (window_can_miss(in_h, out_h, stride, pad_top, 3, 1) || window_can_miss(in_w, out_w, stride, pad_left, 3, 1)) {
+    bool refuse = false;
+    const int rc = refuse_nonfinite_filter(dw_filter, 9 * mid_c, "tfhip_fused_inverted_residual", &refuse);
+    if (rc != kOk) return rc;
+    if (refuse) return fail(kBadArgument, "tfhip_fused_inverted_residual: %s", kNonfiniteFilterMessage);
   }
   const float *ptrs[] = {x, pw_filter_t, pw_bias, dw_filter, dw_bias, proj_filter_t, proj_bias, residual, y};
   bool aligned = true;

@@ -60,6 +60,29 @@ inline bool product_below(int64_t limit, std::initializer_list<int64_t> factors)
   }
   return p < limit;
 }
+// Whether the `elems` floats at `w` hold an Inf or a NaN. The answer is remembered per (address,
+// length, allocation generation of the block), so a filter costs one small kernel and one wait for
+// the stream, once; a call for a filter not seen yet fails while a recording is open. `who` names
+// the entry point in error messages.
+int scan_filter(const float *w, int64_t elems, const char *who, bool *nonfinite);
+// Drops what scan_filter remembers about the block that holds p (the block is being written).
+void forget_filter_scans(const void *p);
+// True when a filter window of `f` taps (dilation `dil`) can reach outside an axis of `in` positions:
+// `out` windows, `stride` apart, the first one starting `pad` positions before the axis.
+inline bool window_can_miss(int64_t in, int64_t out, int64_t stride, int64_t pad, int64_t f, int64_t dil) {
+  return pad > 0 || (out - 1) * stride - pad + (f - 1) * dil >= in;
+}
+// For the fused kernels that pad with zeros and multiply them by the filter: kOk with *refuse = true when
+// the `elems` values of the filter at `w` are not all finite (the reference skips taps outside the image,
+// so an Inf or NaN filter value must not meet the padding: the caller runs the separate kernels, which
+// route such a filter to their tap-skipping form).
+constexpr const char *kNonfiniteFilterMessage =
+    "a filter holds Inf or NaN and its windows reach outside the image: the fused kernel multiplies the padding's "
+    "zeros by it where the reference skips the tap; run the separate convolutions (tfhip_filter_is_finite tells "
+    "beforehand)";
+inline int refuse_nonfinite_filter(const float *w, int64_t elems, const char *who, bool *refuse) {
+  return scan_filter(w, elems, who, refuse);
+}
 // True between tfhip_capture_begin and tfhip_capture_end.
 bool capturing();
 
@@ -100,6 +123,14 @@ bool capturing();
                            "is not inside a live device buffer",               \
                            __func__, name, (long long)(elems), (int)(esize),   \
                            (const void *)(ptr));                               \
+  } while (0)
+
+// Operand `name` is about to be written: it must be live, and what the library remembered about its
+// block's contents (filters searched for Inf / NaN) no longer holds.
+#define TFHIP_CHECK_OUTPUT(ptr, elems, esize, name)       \
+  do {                                                    \
+    TFHIP_CHECK_RANGE(ptr, elems, esize, name);           \
+    ::tfhip::forget_filter_scans(ptr);                    \
   } while (0)
 
 // Checks the launch that was just enqueued.

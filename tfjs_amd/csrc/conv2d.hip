@@ -251,6 +251,65 @@ int launch_few_channels(const GemmParams &p, int f_h) {
   return kOk;
 }
 
+// The reference's own loop, one output element per lane: taps outside the image are SKIPPED, not
+// read as zero (tfjs-backend-cpu/src/kernels/Conv2D.ts:72-84). For a finite filter the two are the
+// same number; a filter that holds Inf or NaN gives NaN at every border output when a zero is
+// multiplied by it, and leaves those outputs alone in the reference. The MFMA kernels cannot skip
+// a tap per output pixel, so a padded convolution whose filter is not finite runs here: any layout,
+// stride, dilation, epilogue and residual, sums in the reference's order (filter row, filter
+// column, input channel) with one float32 rounding per multiply-add.
+struct SkipTapsArgs {
+  const float *x, *w;
+  float *y;
+  int in_h, in_w, in_c, f_h, f_w, out_c;
+  int stride_h, stride_w, dil_h, dil_w, pad_top, pad_left, out_h, out_w;
+  long long xs_n, xs_h, xs_w, xs_c;
+};
+
+__global__ __launch_bounds__(256) void conv_skip_taps(SkipTapsArgs g, Epilogue e, long long total) {
+  const long long stride = (long long)gridDim.x * 256;
+  for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += stride) {
+    const int oc = (int)(idx % g.out_c);
+    long long t = idx / g.out_c;
+    const int ow = (int)(t % g.out_w);
+    t /= g.out_w;
+    const int oh = (int)(t % g.out_h);
+    const long long n = t / g.out_h;
+    float acc = 0.f;
+    for (int r = 0; r < g.f_h; ++r) {
+      const int ih = oh * g.stride_h - g.pad_top + r * g.dil_h;
+      if (ih < 0 || ih >= g.in_h) continue;
+      for (int c = 0; c < g.f_w; ++c) {
+        const int iw = ow * g.stride_w - g.pad_left + c * g.dil_w;
+        if (iw < 0 || iw >= g.in_w) continue;
+        const float *xp = g.x + n * g.xs_n + ih * g.xs_h + iw * g.xs_w;
+        const float *wp = g.w + ((long long)(r * g.f_w + c) * g.in_c) * g.out_c + oc;
+        for (int d = 0; d < g.in_c; ++d) acc = fmaf(xp[d * g.xs_c], wp[(long long)d * g.out_c], acc);
+      }
+    }
+    float v = finish(e, acc, 0, n * g.out_h * g.out_w + (long long)oh * g.out_w + ow, oc, n, oh, ow);
+    const long long at = n * e.y_s[0] + oh * e.y_s[1] + ow * e.y_s[2] + oc * e.y_s[3];
+    if (e.residual) v = v + e.residual[at];
+    g.y[at] = v;
+  }
+}
+
+int launch_skip_taps(const GemmParams &p, int f_h, long long batch) {
+  SkipTapsArgs g;
+  const ConvGeom &c = p.conv;
+  g.x = p.a; g.w = p.b; g.y = p.c;
+  g.in_h = c.in_h; g.in_w = c.in_w; g.in_c = c.in_c; g.f_h = f_h; g.f_w = c.f_w; g.out_c = p.N;
+  g.stride_h = c.stride_h; g.stride_w = c.stride_w; g.dil_h = c.dil_h; g.dil_w = c.dil_w;
+  g.pad_top = c.pad_top; g.pad_left = c.pad_left; g.out_h = c.out_h; g.out_w = c.out_w;
+  g.xs_n = c.xs_n; g.xs_h = c.xs_h; g.xs_w = c.xs_w; g.xs_c = c.xs_c;
+  const long long total = (long long)p.M * p.N;
+  long long blocks = (total + 255) / 256;
+  const long long cap = (long long)num_cus() * 32;
+  note_kernel("conv_skip_taps");
+  TFHIP_LAUNCH((conv_skip_taps<<<dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(256), 0, stream()>>>(g, p.epi, total)));
+  return kOk;
+}
+
 // y += residual for the kernels whose tail does not take a residual itself.
 __global__ __launch_bounds__(256) void add_residual(float *__restrict__ y, const float *__restrict__ residual,
                                                     long long total) {
@@ -287,7 +346,7 @@ int fused_conv2d(const float *x, const float *filter, float *y, int64_t batch, i
   if (M == 0) return kOk;
   TFHIP_CHECK_RANGE(x, batch * in_h * in_w * in_c, 4, "x");
   TFHIP_CHECK_RANGE(filter, K * out_c, 4, "filter");
-  TFHIP_CHECK_RANGE(y, M * out_c, 4, "y");
+  TFHIP_CHECK_OUTPUT(y, M * out_c, 4, "y");
   if (residual) TFHIP_CHECK_RANGE(residual, M * out_c, 4, "residual");
 
   GemmParams p = {};
@@ -334,6 +393,16 @@ int fused_conv2d(const float *x, const float *filter, float *y, int64_t batch, i
   const bool x16 = reinterpret_cast<uintptr_t>(x) % 16 == 0 && p.a_bytes != 0,
              w16 = reinterpret_cast<uintptr_t>(filter) % 16 == 0 && p.b_bytes != 0;
   const bool vec = !nchw && x16 && w16 && in_c % 4 == 0 && out_c % 4 == 0;
+  // A window can reach outside the image: the reference skips such taps, the kernels below read
+  // zeros for them, which differs only under a filter value that is not finite.
+  const bool taps_can_miss = pad_top > 0 || pad_left > 0 ||
+                             (out_h - 1) * stride_h - pad_top + (f_h - 1) * dilation_h >= in_h ||
+                             (out_w - 1) * stride_w - pad_left + (f_w - 1) * dilation_w >= in_w;
+  if (taps_can_miss) {
+    bool nonfinite = false;
+    if ((rc = scan_filter(filter, K * out_c, "tfhip_fused_conv2d", &nonfinite)) != kOk) return rc;
+    if (nonfinite) return launch_skip_taps(p, (int)f_h, batch);
+  }
   const bool pointwise = !nchw && f_h == 1 && f_w == 1 && stride_h == 1 && stride_w == 1 && pad_top == 0 &&
                          pad_left == 0 && out_h == in_h && out_w == in_w;
   if (pointwise) {

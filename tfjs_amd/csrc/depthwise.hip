@@ -501,7 +501,7 @@ extern "C" int tfhip_fused_depthwise_conv2d(
   if (total == 0) return kOk;
   TFHIP_CHECK_RANGE(x, batch * in_h * in_w * in_c, 4, "x");
   TFHIP_CHECK_RANGE(filter, f_h * f_w * in_c * ch_mul, 4, "filter");
-  TFHIP_CHECK_RANGE(y, total, 4, "y");
+  TFHIP_CHECK_OUTPUT(y, total, 4, "y");
   const int64_t dims[4] = {batch, out_h, out_w, out_c};
 
   Epilogue e = {};
@@ -542,9 +542,20 @@ extern "C" int tfhip_fused_depthwise_conv2d(
 
   const bool aligned16 = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(filter) % 16 == 0 &&
                          reinterpret_cast<uintptr_t>(y) % 16 == 0;
+  // The 3x3 kernels read a zero for a tap outside the image and multiply it by the filter value; the
+  // reference skips the tap (DepthwiseConv2dNative.ts:72-86), which differs under a value that is not
+  // finite: such a filter, where a window can reach outside, takes the general kernel, which skips.
+  const bool taps_can_miss = pad_top > 0 || pad_left > 0 ||
+                             (out_h - 1) * stride_h - pad_top + (f_h - 1) * dilation_h >= in_h ||
+                             (out_w - 1) * stride_w - pad_left + (f_w - 1) * dilation_w >= in_w;
+  bool nonfinite = false;
+  if (taps_can_miss) {
+    const int rc = scan_filter(filter, f_h * f_w * in_c * ch_mul, "tfhip_fused_depthwise_conv2d", &nonfinite);
+    if (rc != kOk) return rc;
+  }
   const bool fast = f_h == 3 && f_w == 3 && ch_mul == 1 && dilation_h == 1 && dilation_w == 1 &&
                     stride_h == stride_w && (stride_h == 1 || stride_h == 2) && in_c % 4 == 0 && aligned16 &&
-                    batch <= 65535;
+                    batch <= 65535 && !nonfinite;
   // the row pipeline addresses both tensors with 32-bit byte offsets
   const bool fits32 = batch * in_h * in_w * in_c * 4 <= 0xfffffff0LL && total * 4 <= 0xfffffff0LL;
   if (fast && fits32 && tuning(kTuneDwHalo) <= 0) {

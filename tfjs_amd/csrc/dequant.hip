@@ -221,7 +221,7 @@ int tfhip_dequant_affine(const void *q, int bits, int64_t n, double scale, doubl
   TFHIP_CHECK_ARG(n >= 0, "tfhip_dequant_affine: negative element count");
   if (n == 0) return kOk;
   TFHIP_CHECK_RANGE(q, n, bits / 8, "q");
-  TFHIP_CHECK_RANGE(out, n, 4, "out");
+  TFHIP_CHECK_OUTPUT(out, n, 4, "out");
   TFHIP_CHECK_ARG(reinterpret_cast<uintptr_t>(out) % 4 == 0, "tfhip_dequant_affine: out is not 4-byte aligned");
   return launch(q, bits / 8, n, scale, min, out, to_int32 ? 1 : 0);
 }
@@ -231,7 +231,7 @@ int tfhip_dequant_f16(const void *q, int64_t n, float *out) {
   TFHIP_CHECK_ARG(n >= 0, "tfhip_dequant_f16: negative element count");
   if (n == 0) return kOk;
   TFHIP_CHECK_RANGE(q, n, 2, "q");
-  TFHIP_CHECK_RANGE(out, n, 4, "out");
+  TFHIP_CHECK_OUTPUT(out, n, 4, "out");
   TFHIP_CHECK_ARG(reinterpret_cast<uintptr_t>(out) % 4 == 0, "tfhip_dequant_f16: out is not 4-byte aligned");
   return launch(q, 2, n, 0.0, 0.0, out, 2);
 }

@@ -405,7 +405,13 @@ extern "C" int tfhip_fused_pointwise_depthwise(const float *x, const float *pw_f
   TFHIP_CHECK_RANGE(dw_filter, 9 * mid_c, 4, "dw_filter");
   if (pw_bias) TFHIP_CHECK_RANGE(pw_bias, mid_c, 4, "pw_bias");
   if (dw_bias) TFHIP_CHECK_RANGE(dw_bias, mid_c, 4, "dw_bias");
-  TFHIP_CHECK_RANGE(y, batch * out_h * out_w * mid_c, 4, "y");
+  TFHIP_CHECK_OUTPUT(y, batch * out_h * out_w * mid_c, 4, "y");
+  if (window_can_miss(in_h, out_h, stride, pad_top, 3, 1) || window_can_miss(in_w, out_w, stride, pad_left, 3, 1)) {
+    bool refuse = false;
+    const int rc = refuse_nonfinite_filter(dw_filter, 9 * mid_c, "tfhip_fused_pointwise_depthwise", &refuse);
+    if (rc != kOk) return rc;
+    if (refuse) return fail(kBadArgument, "tfhip_fused_pointwise_depthwise: %s", kNonfiniteFilterMessage);
+  }
 
   const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(pw_filter) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(dw_filter) % 16 == 0 &&
@@ -554,7 +560,18 @@ extern "C" int tfhip_fused_conv2d_depthwise(const float *x, const float *filter,
   TFHIP_CHECK_RANGE(dw_filter, 9 * mid_c, 4, "dw_filter");
   if (bias) TFHIP_CHECK_RANGE(bias, mid_c, 4, "bias");
   if (dw_bias) TFHIP_CHECK_RANGE(dw_bias, mid_c, 4, "dw_bias");
-  TFHIP_CHECK_RANGE(y, batch * out_h * out_w * mid_c, 4, "y");
+  TFHIP_CHECK_OUTPUT(y, batch * out_h * out_w * mid_c, 4, "y");
+  {
+    bool refuse = false;
+    int rc = kOk;
+    if (window_can_miss(mid_h, out_h, dw_stride, dw_pad_top, 3, 1) || window_can_miss(mid_w, out_w, dw_stride, dw_pad_left, 3, 1))
+      rc = refuse_nonfinite_filter(dw_filter, 9 * mid_c, "tfhip_fused_conv2d_depthwise", &refuse);
+    if (rc == kOk && !refuse &&
+        (window_can_miss(in_h, mid_h, stride, pad_top, f_h, 1) || window_can_miss(in_w, mid_w, stride, pad_left, f_w, 1)))
+      rc = refuse_nonfinite_filter(filter, K * mid_c, "tfhip_fused_conv2d_depthwise", &refuse);
+    if (rc != kOk) return rc;
+    if (refuse) return fail(kBadArgument, "tfhip_fused_conv2d_depthwise: %s", kNonfiniteFilterMessage);
+  }
 
   ExpandDwArgs g = {};
   g.x = x; g.w1 = filter; g.b1 = bias; g.w2 = dw_filter; g.b2 = dw_bias; g.y = y;

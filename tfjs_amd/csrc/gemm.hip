@@ -117,6 +117,7 @@ static int fused_matmul_impl(const char *who, const float *a, const float *b, fl
     if ((rc = live(b, batch_b * K * N, "b")) != kOk) return rc;
   }
   if ((rc = live(out, batch * M * N, "out")) != kOk) return rc;
+  forget_filter_scans(out);
 
   GemmParams p = {};
   p.a = a; p.b = b; p.c = out;

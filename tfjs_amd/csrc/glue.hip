@@ -279,7 +279,7 @@ int tfhip_transpose2d(const float *x, float *y, int64_t rows, int64_t cols) {
   if (rows * cols == 0) return kOk;
   TFHIP_CHECK_ARG((rows + 31) / 32 <= 65535, "tfhip_transpose2d: more than 2 097 120 rows");
   TFHIP_CHECK_RANGE(x, rows * cols, 4, "x");
-  TFHIP_CHECK_RANGE(y, rows * cols, 4, "y");
+  TFHIP_CHECK_OUTPUT(y, rows * cols, 4, "y");
   TFHIP_CHECK_ARG(x != y, "tfhip_transpose2d: x and y are the same buffer");
   note_kernel("transpose2d");
   const dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32));
@@ -308,7 +308,7 @@ int tfhip_add(const float *a, const int64_t *a_strides, const float *b, const in
   if (total == 0) return kOk;
   TFHIP_CHECK_RANGE(a, strided_extent(out_shape, a_strides, rank), 4, "a");
   TFHIP_CHECK_RANGE(b, strided_extent(out_shape, b_strides, rank), 4, "b");
-  TFHIP_CHECK_RANGE(out, total, 4, "out");
+  TFHIP_CHECK_OUTPUT(out, total, 4, "out");
   const bool aligned = reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(out) % 16 == 0;
   if (dense && aligned && total % 4 == 0) {
@@ -345,7 +345,7 @@ int tfhip_binary(int op, const float *a, const int64_t *a_strides, const float *
   if (total == 0) return kOk;
   TFHIP_CHECK_RANGE(a, strided_extent(out_shape, a_strides, rank), 4, "a");
   TFHIP_CHECK_RANGE(b, strided_extent(out_shape, b_strides, rank), 4, "b");
-  TFHIP_CHECK_RANGE(out, total, 4, "out");
+  TFHIP_CHECK_OUTPUT(out, total, 4, "out");
   const bool aligned = reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(out) % 16 == 0;
   if (dense && aligned && total % 4 == 0) {
@@ -376,7 +376,7 @@ int tfhip_unary(int activation, const float *x, float *y, int64_t n, double leak
   TFHIP_CHECK_ARG(n >= 0, "tfhip_unary: negative size");
   if (n == 0) return kOk;
   TFHIP_CHECK_RANGE(x, n, 4, "x");
-  TFHIP_CHECK_RANGE(y, n, 4, "y");
+  TFHIP_CHECK_OUTPUT(y, n, 4, "y");
   note_kernel("unary_activation");
   TFHIP_LAUNCH((unary_activation<<<grid_for(n), 256, 0, stream()>>>(x, y, n, activation, leakyrelu_alpha)));
   return kOk;
@@ -398,7 +398,7 @@ int tfhip_avg_pool(const float *x, float *y, int64_t batch, int64_t in_h, int64_
   TFHIP_CHECK_ARG(out_w == 0 || (out_w - 1) * stride_w - pad_left < in_w, "tfhip_avg_pool: out_w does not fit the input");
   if (batch * out_h * out_w * c == 0) return kOk;
   TFHIP_CHECK_RANGE(x, batch * in_h * in_w * c, 4, "x");
-  TFHIP_CHECK_RANGE(y, batch * out_h * out_w * c, 4, "y");
+  TFHIP_CHECK_OUTPUT(y, batch * out_h * out_w * c, 4, "y");
   PoolParams p = {x, y, (int)batch, (int)in_h, (int)in_w, (int)c, (int)f_h, (int)f_w, (int)stride_h, (int)stride_w,
                   (int)pad_top, (int)pad_left, (int)out_h, (int)out_w};
   note_kernel("avg_pool");
@@ -413,7 +413,7 @@ int tfhip_cast(const void *x, int from_dtype, void *y, int to_dtype, int64_t n) 
   TFHIP_CHECK_ARG(n >= 0, "tfhip_cast: negative size");
   if (n == 0) return kOk;
   TFHIP_CHECK_RANGE(x, n, from_dtype == 2 ? 1 : 4, "x");
-  TFHIP_CHECK_RANGE(y, n, to_dtype == 2 ? 1 : 4, "y");
+  TFHIP_CHECK_OUTPUT(y, n, to_dtype == 2 ? 1 : 4, "y");
   note_kernel("cast_elements");
   TFHIP_LAUNCH((cast_elements<<<grid_for(n), 256, 0, stream()>>>(x, y, n, from_dtype, to_dtype)));
   return kOk;
@@ -424,7 +424,7 @@ int tfhip_mean_hw(const float *x, float *y, int64_t batch, int64_t h, int64_t w,
   TFHIP_CHECK_ARG(batch >= 0 && h > 0 && w > 0 && c >= 0, "tfhip_mean_hw: bad dimensions");
   if (batch * c == 0) return kOk;
   TFHIP_CHECK_RANGE(x, batch * h * w * c, 4, "x");
-  TFHIP_CHECK_RANGE(y, batch * c, 4, "y");
+  TFHIP_CHECK_OUTPUT(y, batch * c, 4, "y");
   if (c % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
     long long blocks = (batch * (c / 4) + 31) / 32;
     const long long cap = (long long)num_cus() * 32;
@@ -444,7 +444,7 @@ int tfhip_copy(void *dst, const void *src, size_t bytes) {
                       reinterpret_cast<uintptr_t>(src) % 16 == 0,
                   "tfhip_copy: pointers and size must be multiples of 16 bytes");
   TFHIP_CHECK_RANGE(src, bytes, 1, "src");
-  TFHIP_CHECK_RANGE(dst, bytes, 1, "dst");
+  TFHIP_CHECK_OUTPUT(dst, bytes, 1, "dst");
   note_kernel("copy_f4");
   TFHIP_LAUNCH((copy_f4<<<grid_for(bytes / 16), 256, 0, stream()>>>((const float4 *)src, (float4 *)dst,
                                                                       (long long)(bytes / 16))));

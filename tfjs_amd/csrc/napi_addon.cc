@@ -529,6 +529,19 @@ napi_value InvertedResidualPays(napi_env env, napi_callback_info info) {
   return out;
 }
 
+// filterIsFinite(filter, elems): boolean
+napi_value FilterIsFinite(napi_env env, napi_callback_info info) {
+  Args a(env, info, 2, "filterIsFinite");
+  const float *filter = (const float *)a.ptr(0);
+  const int64_t elems = a.i64(1);
+  if (!a.ok) return nullptr;
+  int finite = 1;
+  HIP_OK(tfhip_filter_is_finite(filter, elems, &finite));
+  napi_value out;
+  NAPI_OK(napi_get_boolean(env, finite == 1, &out));
+  return out;
+}
+
 // meanHW(x, y, batch, h, w, c)
 napi_value MeanHW(napi_env env, napi_callback_info info) {
   Args a(env, info, 6, "meanHW");
@@ -657,6 +670,7 @@ napi_value Register(napi_env env, napi_value exports) {
       FN("sync", Sync),
       FN("memoryInfo", MemoryInfo),
       FN("workspaceInfo", WorkspaceInfo),
+      FN("filterIsFinite", FilterIsFinite),
       FN("eventRecord", EventRecord),
       FN("eventElapsed", EventElapsed),
       FN("setLaunchRepeat", SetLaunchRepeat),

@@ -64,6 +64,18 @@ struct Runtime {
   std::map<int, RecordedGraph> graphs;
   int next_graph = 1;
   std::vector<void *> retired_workspaces;  // outgrown while a graph might still name them
+  // Filters that were searched for Inf / NaN: block base -> scans of ranges inside that block.
+  // An entry holds the generation of the block it was made for, and leaves when the block is
+  // written through this library (uploads, kernel results) or freed.
+  struct FilterScan {
+    uintptr_t ptr;
+    size_t elems;
+    uint64_t generation;
+    bool nonfinite;
+  };
+  std::unordered_map<uintptr_t, std::vector<FilterScan>> filter_scans;
+  int *scan_flag = nullptr;   // pinned host word the scan kernel's verdict is copied to
+  int *scan_flag_dev = nullptr;
 };
 
 
@@ -212,6 +224,73 @@ bool range_is_live(const void *p, size_t bytes) {
 
 bool capturing() { return g.capturing; }
 
+__global__ void clear_word(int *word) { *word = 0; }
+
+// 1 in *flag when any of the n values has an all-ones exponent (Inf or NaN)
+__global__ __launch_bounds__(256) void find_nonfinite(const unsigned *__restrict__ bits, long long n, int *flag) {
+  const long long stride = (long long)gridDim.x * 256;
+  bool hit = false;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) hit |= (bits[i] & 0x7f800000u) == 0x7f800000u;
+  if (hit) *flag = 1;   // (every writer writes the same value)
+}
+
+void forget_filter_scans(const void *p) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (g.filter_scans.empty()) return;
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+  auto it = g.live.upper_bound(a);
+  if (it == g.live.begin()) return;
+  --it;
+  if (a < it->first + it->second) g.filter_scans.erase(it->first);
+}
+
+int scan_filter(const float *w, int64_t elems, const char *who, bool *nonfinite) {
+  *nonfinite = false;
+  if (elems <= 0) return kOk;
+  const uintptr_t a = reinterpret_cast<uintptr_t>(w);
+  uintptr_t base = 0;
+  uint64_t generation = 0;
+  {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    auto it = g.live.upper_bound(a);
+    if (it == g.live.begin()) return fail(kOutOfRange, "%s: the filter is not inside a live device buffer", who);
+    --it;
+    if (a + (size_t)elems * 4 > it->first + it->second)
+      return fail(kOutOfRange, "%s: the filter is not inside a live device buffer", who);
+    base = it->first;
+    generation = g.generation[base];
+    auto found = g.filter_scans.find(base);
+    if (found != g.filter_scans.end()) {
+      for (const Runtime::FilterScan &f : found->second) {
+        if (f.ptr == a && f.elems == (size_t)elems && f.generation == generation) {
+          *nonfinite = f.nonfinite;
+          return kOk;
+        }
+      }
+    }
+  }
+  // not known yet: one small kernel and a wait for its verdict, once per filter
+  if (g.capturing)
+    return fail(kBadArgument,
+                "%s: this filter has not been searched for Inf / NaN yet, which needs a wait for the stream; run the "
+                "call once outside the recording",
+                who);
+  *g.scan_flag = 0;
+  clear_word<<<dim3(1), dim3(1), 0, g.stream>>>(g.scan_flag_dev);
+  long long blocks = (elems + 255) / 256;
+  if (blocks > 1024) blocks = 1024;
+  find_nonfinite<<<dim3((unsigned)blocks), dim3(256), 0, g.stream>>>(reinterpret_cast<const unsigned *>(w), elems,
+                                                                     g.scan_flag_dev);
+  TFHIP_CHECK_HIP(hipGetLastError());
+  TFHIP_CHECK_HIP(hipMemcpyAsync(g.scan_flag, g.scan_flag_dev, sizeof(int), hipMemcpyDeviceToHost, g.stream));
+  TFHIP_CHECK_HIP(hipStreamSynchronize(g.stream));
+  *nonfinite = *g.scan_flag != 0;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  // (the block may have gone while the lock was open: the entry would then never match)
+  g.filter_scans[base].push_back({a, (size_t)elems, generation, *nonfinite});
+  return kOk;
+}
+
 // Copies a small result straight into pinned host memory: a kernel starts within
 // a few microseconds, the copy engine needs 10-15 for a transfer of any size.
 __global__ __launch_bounds__(256) void copy_to_host(const float4 *__restrict__ src, float4 *__restrict__ dst, int n4) {
@@ -253,6 +332,8 @@ int tfhip_init(int device) {
     TFHIP_CHECK_HIP(hipEventCreateWithFlags(&g.staging_done[i], hipEventDisableTiming));
     g.staging_busy[i] = false;
   }
+  TFHIP_CHECK_HIP(hipHostMalloc(reinterpret_cast<void **>(&g.scan_flag), sizeof(int), hipHostMallocDefault));
+  TFHIP_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&g.scan_flag_dev), sizeof(int)));
   g.device = device;
   ++g_init_count;
   read_tuning_from_environment();
@@ -289,6 +370,11 @@ int tfhip_shutdown(void) {
   g.live.clear();
   g.owned.clear();
   g.generation.clear();
+  g.filter_scans.clear();
+  if (g.scan_flag) (void)hipHostFree(g.scan_flag);
+  if (g.scan_flag_dev) (void)hipFree(g.scan_flag_dev);
+  g.scan_flag = nullptr;
+  g.scan_flag_dev = nullptr;
   g.live_bytes = 0;
   release_pool_locked();
   for (int i = 0; i < kStagingBuffers; ++i) {
@@ -374,6 +460,7 @@ int tfhip_free(void *dptr) {
   g.live.erase(it);
   g.owned.erase(a);
   g.generation.erase(a);
+  g.filter_scans.erase(a);
   g.live_bytes -= cls;
   if (g.capturing) {
     g.capture_free[cls].push_back(dptr);   // the graph being recorded names it: the graph keeps it
@@ -404,6 +491,7 @@ int tfhip_unregister_external(void *dptr) {
   g.live.erase(it);
   g.owned.erase(a);
   g.generation.erase(a);
+  g.filter_scans.erase(a);
   return kOk;
 }
 
@@ -426,13 +514,23 @@ int tfhip_workspace_info(size_t *bytes, size_t *allocations, int *last_splits) {
   return kOk;
 }
 
+int tfhip_filter_is_finite(const float *filter, int64_t elems, int *finite) {
+  TFHIP_REQUIRE_INIT();
+  TFHIP_CHECK_ARG(finite != nullptr && elems >= 0, "tfhip_filter_is_finite: bad argument");
+  bool nonfinite = false;
+  const int rc = scan_filter(filter, elems, "tfhip_filter_is_finite", &nonfinite);
+  if (rc != kOk) return rc;
+  *finite = nonfinite ? 0 : 1;
+  return kOk;
+}
+
 int tfhip_upload(void *dst, size_t dst_offset, const void *host, size_t bytes) {
   TFHIP_REQUIRE_INIT();
   TFHIP_REFUSE_WHILE_RECORDING();
   if (bytes == 0) return kOk;
   TFHIP_CHECK_ARG(host != nullptr, "tfhip_upload: host pointer is NULL");
   char *d = static_cast<char *>(dst) + dst_offset;
-  TFHIP_CHECK_RANGE(d, bytes, 1, "dst");
+  TFHIP_CHECK_OUTPUT(d, bytes, 1, "dst");
   const char *h = static_cast<const char *>(host);
   size_t done = 0;
   while (done < bytes) {

@@ -112,6 +112,7 @@ export interface HipBinding {
   sync(): void;
   memoryInfo(): {live: number, liveBytes: number, pooledBytes: number};
   workspaceInfo(): {bytes: number, allocations: number, lastSplits: number};
+  filterIsFinite(filter: number, elems: number): boolean;
   eventRecord(slot: number): void;
   eventElapsed(startSlot: number, endSlot: number): number;
   setLaunchRepeat(n: number): void;

@@ -145,6 +145,22 @@ const cvdwGeom = new Float64Array(17);
  * does not take the shape), the two kernels run one after the other here; the
  * result is the same either way.
  */
+/**
+ * Whether a filter tensor is free of Inf / NaN, asked of the native library once per tensor (a
+ * tensor's values never change). The fused pair kernels pad the expanded tensor with zeros and
+ * multiply them by the filter, where the reference skips taps outside the image: with a filter
+ * value that is not finite the two differ, so such a filter takes the separate convolutions.
+ */
+const finiteFilters = new WeakMap();   // dataId -> boolean
+function filterIsFinite(backend, filter) {
+  let finite = finiteFilters.get(filter.dataId);
+  if (finite === undefined) {
+    finite = addon.filterIsFinite(backend.ptr(filter.dataId), tf.util.sizeFromShape(filter.shape));
+    finiteFilters.set(filter.dataId, finite);
+  }
+  return finite;
+}
+
 function fusedPointwiseDepthwise(args) {
   const {x, filter, bias, dwFilter, dwBias} = args.inputs;
   const {strides, pad, dimRoundingMode, activation} = args.attrs;
@@ -170,7 +186,8 @@ function fusedPointwiseDepthwise(args) {
     const square = info.strideHeight === info.strideWidth && first.strideHeight === first.strideWidth &&
         tf.util.sizeFromShape(info.outShape) > 0;
     const code = activationCode(activation, opName);
-    if (square && pointwise &&
+    const finite = filterIsFinite(backend, dwFilter) && (pointwise || filterIsFinite(backend, filter));
+    if (finite && square && pointwise &&
         addon.pointwiseDepthwisePays(
             info.batchSize, x.shape[3], midC, info.strideHeight, info.outHeight, info.outWidth)) {
       const out = backend.makeOutput(info.outShape, 'float32');
@@ -189,7 +206,7 @@ function fusedPointwiseDepthwise(args) {
           backend.ptr(dwFilter.dataId), backend.ptr(dwBias.dataId), code, backend.ptr(out.dataId), pwdwGeom);
       return out;
     }
-    if (square && !pointwise &&
+    if (finite && square && !pointwise &&
         addon.conv2dDepthwisePays(
             info.batchSize, x.shape[3], first.filterHeight, first.filterWidth, midC, first.outHeight, first.outWidth,
             info.strideHeight, info.outHeight, info.outWidth)) {
