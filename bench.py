@@ -304,8 +304,9 @@ def bench_model_node(model_dir, steps, warmup, prime, batch=BATCH, record=False,
     return json.loads(proc.stdout.strip().splitlines()[-1])
 
 
-def bench_kernels(cold=True):
-    """One line per benchmark configuration: its kernel at its shape."""
+def bench_kernels(cold=True, only=None):
+    """One line per benchmark configuration: its kernel at its shape. `only`: a substring the
+    configuration's name must hold (for a look at one kernel)."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import synth
     from tfjs_amd import pyhost, workloads
@@ -379,22 +380,47 @@ def bench_kernels(cold=True):
         q.free()
         o.free()
 
-    c = synth.config1()
-    matmul("cfg1 _FusedMatMul 256x512x512 +bias relu", **c)
-    c = synth.config2a()
-    conv("cfg2a FusedConv2D stem [1,224,224,3] 3x3/2 ->32 relu6", c["x"], c["w"], c["bias"], 2, "same", "relu6")
-    c = synth.config2b()
-    conv("cfg2b FusedConv2D 1x1 [8,56,56,144]->24", c["x"], c["w"], c["bias"], 1, "same", "linear")
+    def copy(name, nbytes_each):
+        """The yardstick of the memory-bound rows: a plain copy kernel (copy_f4) that reads and writes as
+        many bytes as configuration 3's depthwise convolution, in the same cold rotation."""
+        nbytes = 2.0 * nbytes_each
+        sets = sets_for(nbytes)
+        src, dst = Slab(nbytes_each, sets), Slab(nbytes_each, sets)
+        launch = lambda i: check(lib.tfhip_copy(dst[i].ptr, src[i].ptr, nbytes_each))
+        warm = time_launches(lib, check, ev, lambda: launch(0))
+        row(name, 0.0, nbytes, warm, time_launches_cold(lib, check, ev, launch, sets) if cold else warm)
+        out[-1]["kernel"] = "copy_f4"
+        src.free()
+        dst.free()
+
+    wanted = lambda name: only is None or only in name
+    if wanted("cfg1"):
+        c = synth.config1()
+        matmul("cfg1 _FusedMatMul 256x512x512 +bias relu", **c)
+    if wanted("cfg2a"):
+        c = synth.config2a()
+        conv("cfg2a FusedConv2D stem [1,224,224,3] 3x3/2 ->32 relu6", c["x"], c["w"], c["bias"], 2, "same", "relu6")
+    if wanted("cfg2b"):
+        c = synth.config2b()
+        conv("cfg2b FusedConv2D 1x1 [8,56,56,144]->24", c["x"], c["w"], c["bias"], 1, "same", "linear")
     for s in (1, 2):
-        c = synth.config3(s)
-        conv("cfg3 FusedDepthwiseConv2D [8,112,112,96] 3x3 s%d relu6" % s, c["x"], c["w"], c["bias"], s, "same",
-             "relu6", depthwise=True)
+        if wanted("cfg3 FusedDepthwiseConv2D [8,112,112,96] 3x3 s%d" % s):
+            c = synth.config3(s)
+            conv("cfg3 FusedDepthwiseConv2D [8,112,112,96] 3x3 s%d relu6" % s, c["x"], c["w"], c["bias"], s, "same",
+                 "relu6", depthwise=True)
+    if wanted("cfg3 copy yardstick"):
+        copy("cfg3 copy yardstick: 38.5 MB in, 38.5 MB out (the stride-1 depthwise row's traffic)", 8 * 112 * 112 * 96 * 4)
     for name, *_ in synth.BERT_MATMULS:
-        matmul("cfg5 %s" % name, **synth.config5(name))
-    dequant("cfg4 dequant uint8 3469760 weights", 3469760, "uint8")
-    dequant("cfg5 dequant float16 7077888 weights", 7077888, "float16")
-    dequant("dequant uint8 268435456 weights", 1 << 28, "uint8")
-    dequant("dequant float16 134217728 weights", 1 << 27, "float16")
+        if wanted("cfg5 %s" % name):
+            matmul("cfg5 %s" % name, **synth.config5(name))
+    if wanted("cfg4 dequant"):
+        dequant("cfg4 dequant uint8 3469760 weights", 3469760, "uint8")
+    if wanted("cfg5 dequant"):
+        dequant("cfg5 dequant float16 7077888 weights", 7077888, "float16")
+    if wanted("dequant uint8 268435456"):
+        dequant("dequant uint8 268435456 weights", 1 << 28, "uint8")
+    if wanted("dequant float16 134217728"):
+        dequant("dequant float16 134217728 weights", 1 << 27, "float16")
     return out
 
 
@@ -472,6 +498,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--kernels-only", action="store_true")
     ap.add_argument("--no-kernels", action="store_true")
+    ap.add_argument("--only", metavar="TEXT", help="kernel rows: only the configurations whose name holds TEXT")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the batch-1 and unfused-plan legs (three more Node processes); for profiler runs, which "
@@ -506,7 +533,7 @@ def main():
                          "(the path shards by batch with no exchange step)\n" % args.gpus)
         sys.exit(2)
     if args.kernels_only:
-        kernels = bench_kernels(not args.no_cold)
+        kernels = bench_kernels(not args.no_cold, args.only)
         print(json.dumps(dict(kernels=kernels, copy_yardstick_gbs=copy_yardstick(args.copy_yardstick) if args.copy_yardstick else None)))
         return
 
@@ -543,7 +570,7 @@ def main():
     if args.per_op:
         with open(args.per_op, "w") as f:
             json.dump(m["ops"], f, indent=0)
-    kernels = None if args.no_kernels else bench_kernels(not args.no_cold)
+    kernels = None if args.no_kernels else bench_kernels(not args.no_cold, args.only)
     copy_gbs = copy_yardstick(args.copy_yardstick) if args.copy_yardstick else None
     ms_per_step = js["ms_per_step"] if js else m["ms_per_step"]
     host = ("node %s, %s -> tfjs API -> KernelBackend 'hip' -> N-API addon -> C ABI (tfjs-core: %s)"

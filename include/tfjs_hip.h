@@ -136,9 +136,9 @@ int tfhip_graph_destroy(int graph_id);
  *   scaled by.
  * tfhip_set_tuning(name, value): overrides a kernel-selection heuristic; value < 0
  *   restores it. Knobs: "tile" (GEMM tile shape index), "splitk" (K slices),
- *   "dw_rows" (depthwise rows per lane), "dw_halo" (1: LDS halo depthwise kernel),
- *   "no_skinny" (1: tiled GEMM also for tall products), "dw_flat" (1: the
- *   one-row-per-lane depthwise kernel always, 0: never), "skinny_regs" (0: the
+ *   "dw_rows" (output rows per chunk of the 3x3 depthwise kernel), "dw_halo" (1: the
+ *   LDS halo depthwise kernel), "no_skinny" (1: tiled GEMM also for tall products),
+ *   "skinny_regs" (0: the
  *   streaming GEMM always stages B in LDS), "small_k" (32 / 64: the one-shot GEMM for
  *   K <= 64 with that many rows per tile; unset or 0: never), "fuse_pw_dw"
  *   (tfhip_pointwise_depthwise_pays: 1: yes for every shape the fused kernel

@@ -311,9 +311,9 @@ def test_conv2d_epilogue_forms(hip, orc, act, bias_shape, prelu_shape):
     ((1, 11, 10, 6), (5, 3, 6, 3), (2, 1), 1, "same"), ((1, 11, 10, 8), (3, 3, 8, 1), 1, 2, "same"),
     ((1, 8, 8, 8), (3, 3, 8, 1), 1, 1, 1), ((1, 6, 6, 8), (3, 3, 8, 1), 1, 1, [[0, 0], [2, 0], [1, 3], [0, 0]]),
 ])
-@pytest.mark.parametrize("flat", [0, 1])
-def test_depthwise_shapes(hip, orc, tuning, xs, fs, stride, dil, pad, flat):
-    tuning("dw_flat", flat)   # 3x3 with four-channel groups: one row per lane, or the row pipeline
+@pytest.mark.parametrize("halo", [0, 1], ids=["cols", "halo"])
+def test_depthwise_shapes(hip, orc, tuning, xs, fs, stride, dil, pad, halo):
+    tuning("dw_halo", halo)   # 3x3 with four-channel groups: the column kernel, or the LDS halo kernel of oversized tensors
     rng = np.random.default_rng(sum(xs) + sum(fs) * 3)
     x = rng.uniform(0, 1, xs).astype(np.float32)
     w = rng.normal(0, 0.5, fs).astype(np.float32)
@@ -325,10 +325,10 @@ def test_depthwise_shapes(hip, orc, tuning, xs, fs, stride, dil, pad, flat):
 @pytest.mark.parametrize("stride", [1, 2])
 @pytest.mark.parametrize("act", ["linear", "relu", "elu", "sigmoid", "leakyrelu", "prelu"])
 @pytest.mark.parametrize("bias_shape,prelu_shape", [((8,), (8,)), ((), (1, 1, 8)), ((5, 8), (6, 5, 1)), ((2, 6, 5, 8), (1,))])
-@pytest.mark.parametrize("flat", [0, 1])
-def test_depthwise_epilogue_forms(hip, orc, tuning, act, bias_shape, prelu_shape, stride, flat):
-    # 3x3 with four-channel groups: the row-pipeline kernel and the one-row-per-lane kernel, both epilogue variants
-    tuning("dw_flat", flat)
+@pytest.mark.parametrize("rows", [-1, 1], ids=["chunks", "one row"])
+def test_depthwise_epilogue_forms(hip, orc, tuning, act, bias_shape, prelu_shape, stride, rows):
+    # 3x3 with four-channel groups: the column kernel, both epilogue variants, row chunks and a single row per lane
+    tuning("dw_rows", rows)
     rng = np.random.default_rng(29)
     x = rng.uniform(-1, 1, (2, 6 * stride, 5 * stride, 8)).astype(np.float32)
     w = rng.normal(0, 0.5, (3, 3, 8, 1)).astype(np.float32)
@@ -341,7 +341,8 @@ def test_depthwise_epilogue_forms(hip, orc, tuning, act, bias_shape, prelu_shape
 @pytest.mark.parametrize("rows", [1, 2, 3, 5, 7, 16])
 @pytest.mark.parametrize("stride,pad", [(1, "same"), (2, "same"), (1, "valid"), (2, "valid")])
 def test_depthwise_row_chunks(hip, orc, tuning, rows, stride, pad):
-    # every chunk length of the row pipeline, ragged last chunk and ragged last column strip
+    # every chunk length of the column kernel's row ring (its period is 4 rows at stride 1, 5 at stride 2), ragged
+    # last chunk, and a row of 39 float4 that ends inside a wavefront
     tuning("dw_rows", rows)
     rng = np.random.default_rng(31 + rows)
     x = rng.uniform(-1, 1, (2, 23, 13, 12)).astype(np.float32)
@@ -362,14 +363,14 @@ def test_depthwise_large_result_is_streamed(hip, orc, stride):
     got = hip.fused_depthwise_conv2d(x, w, **kw)
     name = ctypes.create_string_buffer(256)
     load_library().tfhip_last_kernel(name, 256)
-    assert name.value.decode() == "depthwise_3x3_rows<%d, false, true>" % stride, name.value
+    assert name.value.decode() == "depthwise_3x3_cols<%d, false, true>" % stride, name.value
     assert_parity(got, orc.fused_depthwise_conv2d(x, w, **kw))
     # the top 64 output rows of the first image on their own (4 MB): cached stores, and the same
     # bits wherever the cut does not change the padding
     small = hip.fused_depthwise_conv2d(x[:1, :64 * stride], w, **kw)
     load_library().tfhip_last_kernel(name, 256)
-    label = name.value.decode()   # (the row pipeline, or the one-row-per-lane kernel: neither streams)
-    assert label.startswith("depthwise_3x3_") and not label.endswith("true>"), label
+    label = name.value.decode()
+    assert label.startswith("depthwise_3x3_cols<") and not label.endswith("true>"), label
     assert np.array_equal(small[:, :62], got[:1, :62])
 
 
@@ -1088,18 +1089,18 @@ def test_conv2d_without_padding_keeps_its_kernel_for_a_non_finite_filter(hip, or
 
 
 @pytest.mark.parametrize("stride", [1, 2])
-@pytest.mark.parametrize("flat", [0, 1], ids=["rows", "flat"])
+@pytest.mark.parametrize("halo", [0, 1], ids=["cols", "halo"])
 @pytest.mark.parametrize("bad", [np.inf, np.nan], ids=["inf", "nan"])
-def test_depthwise_with_a_non_finite_filter_value_skips_taps_outside_the_image(hip, orc, tuning, stride, flat, bad):
-    """DepthwiseConv2dNative.ts:72-86 skips taps outside the image as well: the 3x3 row kernels, which read
+def test_depthwise_with_a_non_finite_filter_value_skips_taps_outside_the_image(hip, orc, tuning, stride, halo, bad):
+    """DepthwiseConv2dNative.ts:72-86 skips taps outside the image as well: the 3x3 kernels, which read
     zeros there, hand a filter that is not finite to the general kernel."""
-    tuning("dw_flat", flat)
+    tuning("dw_halo", halo)
     rng = np.random.default_rng(17 + stride)
     x = rng.uniform(0.5, 1.5, (2, 13, 10, 8)).astype(np.float32)
     w = rng.normal(0, 0.4, (3, 3, 8, 1)).astype(np.float32)
     b = rng.uniform(-1, 1, (8,)).astype(np.float32)
     got = hip.fused_depthwise_conv2d(x, w, strides=stride, pad="same", bias=b, activation="relu6")
-    assert _last_kernel().startswith("depthwise_3x3_flat" if flat else "depthwise_3x3_rows"), _last_kernel()
+    assert _last_kernel().startswith("depthwise_3x3_halo" if halo else "depthwise_3x3_cols"), _last_kernel()
     w[0, 0, 1, 0] = bad
     w[2, 2, 6, 0] = bad
     want = orc.fused_depthwise_conv2d(x, w, strides=stride, pad="same", bias=b, activation="relu6")

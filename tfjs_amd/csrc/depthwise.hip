@@ -1,10 +1,10 @@
 // FusedDepthwiseConv2D, NHWC float32.
 //
 // Bandwidth-bound (about 2 flops per byte), so no matrix cores. Three kernels:
-//  * depthwise_3x3_rows: 3x3, stride 1 or 2, channel multiplier 1 (every
-//    MobileNet layer). A register row pipeline: each input row is fetched once
-//    per lane as float4 over the contiguous channel axis and scattered into
-//    rotating accumulators; no LDS, no barriers.
+//  * depthwise_3x3_cols: 3x3, stride 1 or 2, channel multiplier 1 (every
+//    MobileNet layer). Lanes lie along an output row in memory order, one float4
+//    of one column each, and walk down a chunk of rows with the input rows in a
+//    register ring; no LDS, no barriers.
 //  * depthwise_3x3_halo: the same shapes when a tensor is too large for 32-bit
 //    buffer offsets; stages an input halo tile of 32 channels in LDS.
 //  * depthwise_generic: any filter, stride, dilation, channel multiplier.
@@ -130,24 +130,10 @@ __global__ __launch_bounds__(256) void depthwise_3x3_halo(DwParams p, Epilogue e
 }
 
 
-// ---- 3x3, channel multiplier 1, dilation 1, stride S: register row pipeline ----
-// Each lane owns four channels (one float4) of a strip of 4 output columns and
-// walks down `rows` output rows. Every input row it needs is fetched exactly
-// once by that lane (4*S + 2 float4 loads: the 8 lanes that share a pixel read
-// one contiguous 128-byte line, the column overlap with the neighbouring strip
-// is served by the vector cache) and is scattered at once into the accumulators
-// of the up to three output rows it contributes to, which live in registers and
-// rotate as rows complete. The loads of input row i+1 are issued before the
-// arithmetic of row i. No barriers, no LDS: the only traffic besides the
-// compulsory reads and writes is the halo rows of vertically adjacent chunks.
-//
-// All accesses are buffer loads/stores over the whole tensor with 32-bit byte
-// offsets: padding taps and ragged edges use an offset outside the descriptor,
-// which reads as zero and drops stores, so the row pipeline has no branches.
-constexpr int kRowsPW = 4;   // output columns per lane
-#ifndef DW_WAVES
-#define DW_WAVES 1
-#endif
+// ---- shared by the 3x3 kernels ------------------------------------------------------
+// All accesses are buffer loads / stores over the whole tensor with 32-bit byte offsets: padding
+// taps and ragged edges use an offset outside the descriptor, which reads as zero and drops
+// stores, so the row loops have no branches.
 constexpr unsigned kDwNoOffset = 0xffffffffu;
 // Results of at least this many bytes are stored non-temporally: an L2 holds 4 MB,
 // so such a result cannot wait there for its reader (measured with operands from
@@ -155,29 +141,6 @@ constexpr unsigned kDwNoOffset = 0xffffffffu;
 // instead, 21.6 and 13.6 us).
 constexpr long long kDwStreamBytes = 8LL << 20;
 typedef unsigned int dw_uint4 __attribute__((ext_vector_type(4)));
-
-struct DwRowsArgs {
-  int strips_w;      // column strips per output row
-  int chunks_h;      // row chunks per image
-  int rows;          // output rows per chunk
-  int c4_total;
-  long long strips;  // batch * chunks_h * strips_w
-  unsigned x_bytes, y_bytes;
-};
-
-template <int S>
-struct DwRowsState {
-  static constexpr int NIN = (kRowsPW - 1) * S + 3;   // input columns a strip needs
-  static constexpr int NSLOT = S == 1 ? 3 : 2;          // output rows in flight
-  float4 acc[NSLOT][kRowsPW];
-  float4 w[9];
-  float4 bias4;               // per-channel bias of this lane (channel addressing)
-  unsigned x_col[NIN];        // byte offset of input column j (+ channel group) within a row, or kDwNoOffset
-  unsigned y_col[kRowsPW];    // same for the output columns
-  unsigned x_img, y_img;      // byte offset of the image
-  unsigned x_row, y_row;      // bytes per row
-  int in_h, out_h, ih0, oh0, ow0, rows, rows_in, c, n;
-};
 
 __device__ __forceinline__ float4 dw_load4(__amdgpu_buffer_rsrc_t r, unsigned off) {
 #ifndef TFHIP_DW_LOAD_AUX
@@ -227,249 +190,117 @@ __device__ __forceinline__ float4 dw_finish4(const Epilogue &e, float4 a, float4
   return dw_finish4_general(e, a, c, n, oh, ow);
 }
 
-// Issues the loads of input row i of the chunk (relative to its first input row).
-template <int S>
-__device__ __forceinline__ void dw_load_row(const DwRowsState<S> &st, __amdgpu_buffer_rsrc_t rx, int i,
-                                            float4 (&in)[DwRowsState<S>::NIN]) {
-  const int ih = st.ih0 + i;
-  const bool row_ok = ih >= 0 && ih < st.in_h && i < st.rows_in;
-  const unsigned row_off = st.x_img + (unsigned)ih * st.x_row;
-#pragma unroll
-  for (int j = 0; j < DwRowsState<S>::NIN; ++j) {
-    const unsigned off = (row_ok && st.x_col[j] != kDwNoOffset) ? row_off + st.x_col[j] : kDwNoOffset;
-    in[j] = dw_load4(rx, off);
-  }
-}
+// ---- 3x3, channel multiplier 1, dilation 1, stride S: one output column per lane ----
+// The lanes of a launch lie along an output row in MEMORY order: lane f of a row chunk owns
+// float4 f of the row ([column][channel quad], the NHWC order), so a wavefront's store covers
+// one contiguous kilobyte and its three loads per input row (the columns left of, at and right
+// of its own) cover contiguous kilobytes too, each element asked for by three lanes and served
+// to two of them by the vector cache. A lane walks down `rows` output rows with the input rows
+// in a register ring (the three a window needs plus S fetched ahead), so a row is fetched once
+// per lane; with three float4 per input row a lane is light on registers, and a launch has
+// thousands of wavefronts: the bytes in flight that a memory-bound kernel needs come from
+// occupancy. Taps accumulate from zero by filter row, then column, one fused multiply-add each
+// (the reference's order: DepthwiseConv2dNative.ts:62-95).
+// Measured on [8,112,112,96] with operands from memory, against a kernel that gave a lane a strip of
+// four columns (six loads per input row, 252 workgroups, one wavefront per SIMD): 20.3 -> 18.7 us at
+// stride 1, 12.7 -> 11.6 at stride 2; a plain copy of the same bytes takes 16.1 us there. What is
+// left is not latency (two to four rows fetched ahead change nothing), not the rows two chunks
+// both read (chunks walking towards each other, so that those rows are read at the same time:
+// no change) and not arithmetic (a third of the multiply-adds: no change): reads alone take
+// 9.7 us (12.7 with the two neighbour loads), stores the rest, and the two do not overlap better
+// than in the copy.
+constexpr int kColsThreads = 64;
+struct DwColsArgs {
+  int c4_total;        // channel quads per pixel
+  int row_quads;       // out_w * c4_total: float4 per output row
+  int blocks_per_row;  // workgroups along a row
+  int chunks_h, rows;  // row chunks per image, output rows per chunk
+  int xcd_run;         // > 0: workgroup ids are dealt to the XCDs in contiguous runs of this many
+  unsigned x_bytes, y_bytes;
+};
 
-// Scatters input row i into the output rows it is a tap row of; PHASE is i
-// modulo the rotation period of the accumulators, so slots are compile-time.
-template <int S, int PHASE, bool GENERAL, bool STREAM>
-__device__ __forceinline__ void dw_compute_row(DwRowsState<S> &st, const Epilogue &e, __amdgpu_buffer_rsrc_t ry,
-                                               int i, const float4 (&in)[DwRowsState<S>::NIN]) {
-  using St = DwRowsState<S>;
-  constexpr int PERIOD = S * St::NSLOT;
-  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-  for (int wr = 0; wr < 3; ++wr) {
-    constexpr int kBig = 4 * PERIOD;
-    if ((PHASE - wr + kBig) % S != 0) continue;          // this input row is not tap row `wr` of any output row
-    const int o = (i - wr) / S;                            // output row (relative to the chunk) it feeds
-    if (i - wr < 0 || o >= st.rows) continue;
-    const int slot = ((PHASE - wr + kBig) / S) % St::NSLOT;
-#pragma unroll
-    for (int x = 0; x < kRowsPW; ++x) {
-      float4 a = wr == 0 ? zero : st.acc[slot][x];
-#pragma unroll
-      for (int wc = 0; wc < 3; ++wc) {
-        const float4 xv = in[x * S + wc];
-        const float4 wv = st.w[wr * 3 + wc];
-        a.x = fmaf(xv.x, wv.x, a.x);
-        a.y = fmaf(xv.y, wv.y, a.y);
-        a.z = fmaf(xv.z, wv.z, a.z);
-        a.w = fmaf(xv.w, wv.w, a.w);
-      }
-      st.acc[slot][x] = a;
-    }
-    if (wr == 2) {
-      // the row is complete: bias + activation, one float4 store per column
-      const int oh = st.oh0 + o;
-      const bool row_ok = oh < st.out_h;
-      const unsigned row_off = st.y_img + (unsigned)oh * st.y_row;
-#pragma unroll
-      for (int x = 0; x < kRowsPW; ++x) {
-        const unsigned off = (row_ok && st.y_col[x] != kDwNoOffset) ? row_off + st.y_col[x] : kDwNoOffset;
-        dw_store4<STREAM>(ry, off, dw_finish4<GENERAL>(e, st.acc[slot][x], st.bias4, st.c, st.n, oh, st.ow0 + x));
-      }
-    }
-  }
-}
-
-// One pipeline step: `a` holds input row i0+K, `b` receives row i0+K+1.
-template <int S, int K, bool GENERAL, bool STREAM>
-__device__ __forceinline__ void dw_step(DwRowsState<S> &st, const Epilogue &e, __amdgpu_buffer_rsrc_t rx,
-                                        __amdgpu_buffer_rsrc_t ry, int i0, const float4 (&a)[DwRowsState<S>::NIN],
-                                        float4 (&b)[DwRowsState<S>::NIN]) {
-  constexpr int PERIOD = S * DwRowsState<S>::NSLOT;
-  if (i0 + K >= st.rows_in) return;
-  dw_load_row<S>(st, rx, i0 + K + 1, b);
-  dw_compute_row<S, K % PERIOD, GENERAL, STREAM>(st, e, ry, i0 + K, a);
-}
-
-// GENERAL = false: per-channel bias and a relu-family activation, all inline.
 template <int S, bool GENERAL, bool STREAM>
-__global__ __launch_bounds__(256, DW_WAVES) void depthwise_3x3_rows(DwParams p, Epilogue e, DwRowsArgs g) {
-  using St = DwRowsState<S>;
-  const int c4 = blockIdx.y * kCQ + (threadIdx.x % kCQ);
-  const long long strip = (long long)blockIdx.x * kSlots + threadIdx.x / kCQ;
-  if (c4 >= g.c4_total || strip >= g.strips) return;
-  const int sw = (int)(strip % g.strips_w);
-  const long long t = strip / g.strips_w;
-  const int ch = (int)(t % g.chunks_h);
-  const int n = (int)(t / g.chunks_h);
+__global__ __launch_bounds__(kColsThreads) void depthwise_3x3_cols(DwParams p, Epilogue e, DwColsArgs g) {
+  constexpr int A = S;        // input rows in flight beyond the window in use: one output row ahead (two, three and
+                              // four rows ahead measured the same: the launch is not short of loads in flight)
+  constexpr int NB = 3 + A;   // ring of input rows
+  // workgroup ids i, i + 8, ... share an XCD: each XCD takes a contiguous run, so that the columns
+  // two neighbouring workgroups both read come from one L2
+  const unsigned wg = g.xcd_run ? (blockIdx.x % 8) * (unsigned)g.xcd_run + blockIdx.x / 8 : blockIdx.x;
+  const int bx = (int)(wg % (unsigned)g.blocks_per_row);
+  const unsigned t = wg / (unsigned)g.blocks_per_row;
+  const int chunk = (int)(t % (unsigned)g.chunks_h), n = (int)(t / (unsigned)g.chunks_h);
+  const int f = bx * kColsThreads + (int)threadIdx.x;
+  if (f >= g.row_quads) return;
+  const int ow = f / g.c4_total, q = f - ow * g.c4_total;
   const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, (int)g.x_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc((void *)p.y, 0, (int)g.y_bytes, 0x00020000);
-
-  St st;
-  st.in_h = p.in_h; st.out_h = p.out_h;
-  st.oh0 = ch * g.rows;
-  st.ow0 = sw * kRowsPW;
-  st.ih0 = st.oh0 * S - p.pad_top;
-  st.rows = g.rows;
-  st.rows_in = (g.rows - 1) * S + 3;
-  st.c = c4 * 4;
-  st.n = n;
   const unsigned pix = (unsigned)g.c4_total * 16u;   // bytes per pixel
-  st.x_row = (unsigned)p.in_w * pix;
-  st.y_row = (unsigned)p.out_w * pix;
-  st.x_img = (unsigned)n * (unsigned)p.in_h * st.x_row;
-  st.y_img = (unsigned)n * (unsigned)p.out_h * st.y_row;
-  const int iw0 = st.ow0 * S - p.pad_left;
+  const unsigned x_row = (unsigned)p.in_w * pix, y_row = (unsigned)p.out_w * pix;
+  const unsigned x_img = (unsigned)n * (unsigned)p.in_h * x_row, y_img = (unsigned)n * (unsigned)p.out_h * y_row;
+  const int oh0 = chunk * g.rows;
+  const int rows = oh0 + g.rows <= p.out_h ? g.rows : p.out_h - oh0;
+  const int rows_in = (rows - 1) * S + 3;
+  const int ih0 = oh0 * S - p.pad_top;
+  unsigned x_col[3];
 #pragma unroll
-  for (int j = 0; j < St::NIN; ++j) {
-    const int iw = iw0 + j;
-    st.x_col[j] = (iw >= 0 && iw < p.in_w) ? (unsigned)iw * pix + (unsigned)c4 * 16u : kDwNoOffset;
+  for (int wc = 0; wc < 3; ++wc) {
+    const int iw = ow * S - p.pad_left + wc;
+    x_col[wc] = (iw >= 0 && iw < p.in_w) ? (unsigned)iw * pix + (unsigned)q * 16u : kDwNoOffset;
   }
+  const unsigned y_col = (unsigned)f * 16u;
+  float4 ring[NB][3];
+  auto fetch = [&](float4 (&row)[3], int i) __attribute__((always_inline)) {
+    const int ih = ih0 + i;
+    const bool row_ok = ih >= 0 && ih < p.in_h && i < rows_in;
+    const unsigned row_off = x_img + (unsigned)ih * x_row;
 #pragma unroll
-  for (int x = 0; x < kRowsPW; ++x) {
-    const int ow = st.ow0 + x;
-    st.y_col[x] = ow < p.out_w ? (unsigned)ow * pix + (unsigned)c4 * 16u : kDwNoOffset;
-  }
-  const float4 *w4 = reinterpret_cast<const float4 *>(p.w) + c4;
+    for (int wc = 0; wc < 3; ++wc) row[wc] = dw_load4(rx, (row_ok && x_col[wc] != kDwNoOffset) ? row_off + x_col[wc] : kDwNoOffset);
+  };
+  // the first window's rows, then this lane's filter taps and bias: one round trip for all of them
 #pragma unroll
-  for (int k = 0; k < 9; ++k) st.w[k] = w4[(long long)k * g.c4_total];
-  st.bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int i = 0; i < 3 + A - S; ++i) fetch(ring[i], i);
+  float4 w[9];
+  const float4 *w4 = reinterpret_cast<const float4 *>(p.w) + q;
+#pragma unroll
+  for (int k = 0; k < 9; ++k) w[k] = w4[(long long)k * g.c4_total];
+  float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  const int c = q * 4;
   if (!GENERAL && e.bias) {
     const long long bs = e.bias_s[3];
-    st.bias4 = make_float4(e.bias[(st.c + 0) * bs], e.bias[(st.c + 1) * bs], e.bias[(st.c + 2) * bs],
-                           e.bias[(st.c + 3) * bs]);
+    bias4 = make_float4(e.bias[(c + 0) * bs], e.bias[(c + 1) * bs], e.bias[(c + 2) * bs], e.bias[(c + 3) * bs]);
   }
-
-  // The two row buffers swap roles every step, so the loop is unrolled by an
-  // even multiple of the accumulator rotation period.
-  constexpr int PERIOD = S * St::NSLOT;
-  constexpr int UNROLL = PERIOD % 2 == 0 ? PERIOD : 2 * PERIOD;
-  float4 cur[St::NIN], nxt[St::NIN];
-  dw_load_row<S>(st, rx, 0, cur);
-  for (int i0 = 0; i0 < st.rows_in; i0 += UNROLL) {
-    dw_step<S, 0, GENERAL, STREAM>(st, e, rx, ry, i0, cur, nxt);
-    dw_step<S, 1, GENERAL, STREAM>(st, e, rx, ry, i0, nxt, cur);
-    dw_step<S, 2, GENERAL, STREAM>(st, e, rx, ry, i0, cur, nxt);
-    dw_step<S, 3, GENERAL, STREAM>(st, e, rx, ry, i0, nxt, cur);
-    if (UNROLL > 4) {
-      dw_step<S, 4, GENERAL, STREAM>(st, e, rx, ry, i0, cur, nxt);
-      dw_step<S, 5, GENERAL, STREAM>(st, e, rx, ry, i0, nxt, cur);
+  for (int o0 = 0; o0 < rows; o0 += NB) {
+#pragma unroll
+    for (int k = 0; k < NB; ++k) {
+      const int o = o0 + k;
+      if (o < rows) {
+        // input row r of the chunk lives in ring[r % NB]; o0 is a multiple of NB
+#pragma unroll
+        for (int j = 0; j < S; ++j) fetch(ring[(S * k + 3 + A - S + j) % NB], S * o + 3 + A - S + j);
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int wr = 0; wr < 3; ++wr) {
+#pragma unroll
+          for (int wc = 0; wc < 3; ++wc) {
+            const float4 xv = ring[(S * k + wr) % NB][wc];
+            const float4 wv = w[wr * 3 + wc];
+            a.x = fmaf(xv.x, wv.x, a.x);
+            a.y = fmaf(xv.y, wv.y, a.y);
+            a.z = fmaf(xv.z, wv.z, a.z);
+            a.w = fmaf(xv.w, wv.w, a.w);
+          }
+        }
+        const int oh = oh0 + o;
+        dw_store4<STREAM>(ry, y_img + (unsigned)oh * y_row + y_col, dw_finish4<GENERAL>(e, a, bias4, c, n, oh, ow));
+      }
     }
   }
-}
-
-// The same strip of four output columns, but a single output row per lane with
-// its three input rows fetched at once: one memory round trip instead of a
-// chain of them. For feature maps so small that the whole launch is a wave or
-// two of lanes, where the row pipeline above never fills.
-template <int S, bool GENERAL>
-__global__ __launch_bounds__(256) void depthwise_3x3_flat(DwParams p, Epilogue e, DwRowsArgs g) {
-  using St = DwRowsState<S>;
-  const int c4 = blockIdx.y * kCQ + (threadIdx.x % kCQ);
-  const long long strip = (long long)blockIdx.x * kSlots + threadIdx.x / kCQ;
-  if (c4 >= g.c4_total || strip >= g.strips) return;
-  const int sw = (int)(strip % g.strips_w);
-  const long long t = strip / g.strips_w;
-  const int oh = (int)(t % p.out_h);
-  const int n = (int)(t / p.out_h);
-  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, (int)g.x_bytes, 0x00020000);
-  const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc((void *)p.y, 0, (int)g.y_bytes, 0x00020000);
-
-  St st;
-  st.in_h = p.in_h; st.out_h = p.out_h;
-  st.oh0 = oh;
-  st.ow0 = sw * kRowsPW;
-  st.ih0 = oh * S - p.pad_top;
-  st.rows = 1;
-  st.rows_in = 3;
-  st.c = c4 * 4;
-  st.n = n;
-  const unsigned pix = (unsigned)g.c4_total * 16u;   // bytes per pixel
-  st.x_row = (unsigned)p.in_w * pix;
-  st.y_row = (unsigned)p.out_w * pix;
-  st.x_img = (unsigned)n * (unsigned)p.in_h * st.x_row;
-  st.y_img = (unsigned)n * (unsigned)p.out_h * st.y_row;
-  const int iw0 = st.ow0 * S - p.pad_left;
-#pragma unroll
-  for (int j = 0; j < St::NIN; ++j) {
-    const int iw = iw0 + j;
-    st.x_col[j] = (iw >= 0 && iw < p.in_w) ? (unsigned)iw * pix + (unsigned)c4 * 16u : kDwNoOffset;
-  }
-#pragma unroll
-  for (int x = 0; x < kRowsPW; ++x) {
-    const int ow = st.ow0 + x;
-    st.y_col[x] = ow < p.out_w ? (unsigned)ow * pix + (unsigned)c4 * 16u : kDwNoOffset;
-  }
-  float4 r0[St::NIN], r1[St::NIN], r2[St::NIN];
-  dw_load_row<S>(st, rx, 0, r0);
-  dw_load_row<S>(st, rx, 1, r1);
-  dw_load_row<S>(st, rx, 2, r2);
-  const float4 *w4 = reinterpret_cast<const float4 *>(p.w) + c4;
-#pragma unroll
-  for (int k = 0; k < 9; ++k) st.w[k] = w4[(long long)k * g.c4_total];
-  st.bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (!GENERAL && e.bias) {
-    const long long bs = e.bias_s[3];
-    st.bias4 = make_float4(e.bias[(st.c + 0) * bs], e.bias[(st.c + 1) * bs], e.bias[(st.c + 2) * bs],
-                           e.bias[(st.c + 3) * bs]);
-  }
-  dw_compute_row<S, 0, GENERAL, false>(st, e, ry, 0, r0);
-  dw_compute_row<S, 1, GENERAL, false>(st, e, ry, 1, r1);
-  dw_compute_row<S, 2, GENERAL, false>(st, e, ry, 2, r2);
 }
 
 int balanced_tile(int extent, int max_tile) {
   const int tiles = (extent + max_tile - 1) / max_tile;
   return (extent + tiles - 1) / tiles;
-}
-
-// Output rows per lane for the row pipeline. A lane that walks more rows
-// re-reads fewer halo rows (each chunk of r output rows fetches (r-1)*S+3 input
-// rows) but is a longer serial chain of row fetches, and fewer, longer chains
-// may not keep enough loads in flight. The estimate below is
-// max(latency chain, traffic / bandwidth) with constants fitted to sweeps over
-// r on MI355X (one row fetch per lane is about 0.8 us of memory latency, one
-// wavefront sustains about 7.5 GB/s, the chip about 6.5 TB/s; halo rows of a
-// working set that fits the 256 MB memory-side cache mostly hit it).
-int choose_rows(int batch, int in_h, int in_w, int in_c, int out_h, int out_w, int S, int cus) {
-  const double in_bytes = 4.0 * batch * in_h * in_w * in_c;
-  const double out_bytes = 4.0 * batch * out_h * out_w * in_c;
-  const int strips_w = (out_w + kRowsPW - 1) / kRowsPW;
-  const int c_blocks = (in_c / 4 + kCQ - 1) / kCQ;
-  const long long slots = (long long)cus * 8;   // resident wavefronts: two per SIMD at this kernel's register count
-  const bool cached = in_bytes + out_bytes <= 250e6;
-  int best = 1;
-  double best_t = 1e30;
-  for (int r = 1; r <= 24 && r <= out_h; ++r) {
-    const int chunks = (out_h + r - 1) / r;
-    const int rb = (out_h + chunks - 1) / chunks;
-    if (rb != r) continue;   // the balanced tile is what runs: only score those
-    const int rows_in = (rb - 1) * S + 3;
-    const long long wgs = (((long long)batch * chunks * strips_w + kSlots - 1) / kSlots) * c_blocks;
-    const long long waves = wgs * 4;
-    const long long rounds = (waves + slots - 1) / slots;
-    const double halo = (double)chunks * rows_in / in_h;
-    const double traffic = in_bytes * (cached ? 1.0 + (halo - 1.0) * 0.3 : halo) + out_bytes;
-    const double wave_bw = 7500.0 * (S == 2 ? 1.5 : 1.0);   // bytes per us
-    const double conc = (double)(waves < slots ? waves : slots);
-    const double bw = conc * wave_bw < 6.5e6 ? conc * wave_bw : 6.5e6;
-    // workgroups that do not fill the compute units evenly leave some idle at the
-    // end (measured at stride 1: 294 workgroups on 256 units run 8% longer than 252;
-    // at stride 2 the effect is not seen)
-    // (a last channel block that is partly empty counts by its share of lanes)
-    const double full_wgs = (double)(wgs / c_blocks) * (in_c / 4) / kCQ;
-    const double per_cu = ceil(full_wgs / cus);
-    const double balance = S == 1 ? full_wgs / (per_cu * cus) : 1.0;
-    const double t_bw = traffic / bw / (0.85 + 0.15 * balance);
-    const double t_lat = rounds * (1.5 + rows_in * 0.8);
-    const double t = t_lat > t_bw ? t_lat : t_bw;
-    if (t < best_t) { best_t = t; best = r; }
-  }
-  return best;
 }
 
 }  // namespace
@@ -560,67 +391,46 @@ extern "C" int tfhip_fused_depthwise_conv2d(
   const bool fits32 = batch * in_h * in_w * in_c * 4 <= 0xfffffff0LL && total * 4 <= 0xfffffff0LL;
   if (fast && fits32 && tuning(kTuneDwHalo) <= 0) {
     const int S = (int)stride_h;
-    DwRowsArgs g;
+    DwColsArgs g;
     g.c4_total = (int)(in_c / 4);
-    g.strips_w = ((int)out_w + kRowsPW - 1) / kRowsPW;
-    {
-      // one output row per lane when all its wavefronts are resident at once and the
-      // input is small enough for its rows, each fetched by up to three output rows,
-      // to come from cache (measured against the row pipeline: 5-15% faster up to
-      // about 3000 wavefronts and 24 MB, slower beyond either)
-      const long long flat_strips = (long long)batch * out_h * g.strips_w;
-      const long long flat_blocks = (flat_strips + kSlots - 1) / kSlots;
-      const long long flat_waves = flat_blocks * ((g.c4_total + kCQ - 1) / kCQ) * 4;
-      const int forced = tuning(kTuneDwFlat);
-      const bool flat = forced >= 0 ? forced > 0 : (tuning(kTuneDwRows) <= 0 && flat_waves <= (long long)num_cus() * 12 &&
-                                              batch * in_h * in_w * in_c * 4 <= 24000000);
-      if (flat && flat_blocks <= 0x7fffffffLL) {
-        g.rows = 1;
-        g.chunks_h = (int)out_h;
-        g.strips = flat_strips;
-        g.x_bytes = (unsigned)(batch * in_h * in_w * in_c * 4);
-        g.y_bytes = (unsigned)(total * 4);
-        dim3 grid((unsigned)flat_blocks, (g.c4_total + kCQ - 1) / kCQ, 1);
-        const bool general = !(e.addressing == kChannel && activation <= TFHIP_RELU6);
-        note_kernel("depthwise_3x3_flat<%d, %s>", S, general ? "true" : "false");
-        if (S == 1 && !general)
-          TFHIP_LAUNCH((depthwise_3x3_flat<1, false><<<grid, 256, 0, stream()>>>(p, e, g)));
-        else if (S == 1)
-          TFHIP_LAUNCH((depthwise_3x3_flat<1, true><<<grid, 256, 0, stream()>>>(p, e, g)));
-        else if (!general)
-          TFHIP_LAUNCH((depthwise_3x3_flat<2, false><<<grid, 256, 0, stream()>>>(p, e, g)));
-        else
-          TFHIP_LAUNCH((depthwise_3x3_flat<2, true><<<grid, 256, 0, stream()>>>(p, e, g)));
-        return kOk;
-      }
+    g.row_quads = (int)out_w * g.c4_total;
+    g.blocks_per_row = (g.row_quads + kColsThreads - 1) / kColsThreads;
+    // Rows per chunk: a chunk of r output rows fetches (r - 1) S + 3 input rows, so longer chunks re-read
+    // fewer rows, and shorter ones make more wavefronts. 14 rows (8 at stride 2) measured best on
+    // [8,112,112,96] with operands from memory (stride 1: 18.7 us at 14 rows, 19.2 at 8, 20.5 at 4, 22.2 at 28;
+    // stride 2: 11.6 at 8, 13.5 at 14); smaller launches take shorter chunks until there are two
+    // wavefronts for every SIMD of the chip.
+    int rows = S == 1 ? 14 : 8;
+    if (tuning(kTuneDwRows) > 0) {
+      rows = tuning(kTuneDwRows);
+    } else {
+      const long long want = 8LL * num_cus();
+      while (rows > 1 && (long long)g.blocks_per_row * ((out_h + rows - 1) / rows) * batch < want) rows = (rows + 1) / 2;
     }
-    int rows = choose_rows((int)batch, (int)in_h, (int)in_w, (int)in_c, (int)out_h, (int)out_w, S, num_cus());
-    if (tuning(kTuneDwRows) > 0) rows = tuning(kTuneDwRows);   // tuning override
-    rows = rows < 1 ? 1 : (rows > 32 ? 32 : rows);
-    if (rows > out_h) rows = (int)out_h;
+    rows = rows > out_h ? (int)out_h : rows;
     g.rows = balanced_tile((int)out_h, rows);
     g.chunks_h = ((int)out_h + g.rows - 1) / g.rows;
-    g.strips = (long long)batch * g.chunks_h * g.strips_w;
     g.x_bytes = (unsigned)(batch * in_h * in_w * in_c * 4);
     g.y_bytes = (unsigned)(total * 4);
-    const long long blocks_x = (g.strips + kSlots - 1) / kSlots;
-    if (blocks_x <= 0x7fffffffLL) {
-      dim3 grid((unsigned)blocks_x, (g.c4_total + kCQ - 1) / kCQ, 1);
+    const long long wgs = (long long)g.blocks_per_row * g.chunks_h * batch;
+    if (wgs <= 0x7fffffffLL) {
+      g.xcd_run = wgs % 8 == 0 ? (int)(wgs / 8) : 0;
       const bool general = !(e.addressing == kChannel && activation <= TFHIP_RELU6);
       const bool streamed = !general && total * 4 >= kDwStreamBytes;
-      note_kernel("depthwise_3x3_rows<%d, %s, %s>", S, general ? "true" : "false", streamed ? "true" : "false");
+      note_kernel("depthwise_3x3_cols<%d, %s, %s>", S, general ? "true" : "false", streamed ? "true" : "false");
+      const dim3 grid((unsigned)wgs), block(kColsThreads);
       if (S == 1 && streamed)
-        TFHIP_LAUNCH((depthwise_3x3_rows<1, false, true><<<grid, 256, 0, stream()>>>(p, e, g)));
+        TFHIP_LAUNCH((depthwise_3x3_cols<1, false, true><<<grid, block, 0, stream()>>>(p, e, g)));
       else if (S == 1 && !general)
-        TFHIP_LAUNCH((depthwise_3x3_rows<1, false, false><<<grid, 256, 0, stream()>>>(p, e, g)));
+        TFHIP_LAUNCH((depthwise_3x3_cols<1, false, false><<<grid, block, 0, stream()>>>(p, e, g)));
       else if (S == 1)
-        TFHIP_LAUNCH((depthwise_3x3_rows<1, true, false><<<grid, 256, 0, stream()>>>(p, e, g)));
+        TFHIP_LAUNCH((depthwise_3x3_cols<1, true, false><<<grid, block, 0, stream()>>>(p, e, g)));
       else if (streamed)
-        TFHIP_LAUNCH((depthwise_3x3_rows<2, false, true><<<grid, 256, 0, stream()>>>(p, e, g)));
+        TFHIP_LAUNCH((depthwise_3x3_cols<2, false, true><<<grid, block, 0, stream()>>>(p, e, g)));
       else if (!general)
-        TFHIP_LAUNCH((depthwise_3x3_rows<2, false, false><<<grid, 256, 0, stream()>>>(p, e, g)));
+        TFHIP_LAUNCH((depthwise_3x3_cols<2, false, false><<<grid, block, 0, stream()>>>(p, e, g)));
       else
-        TFHIP_LAUNCH((depthwise_3x3_rows<2, true, false><<<grid, 256, 0, stream()>>>(p, e, g)));
+        TFHIP_LAUNCH((depthwise_3x3_cols<2, true, false><<<grid, block, 0, stream()>>>(p, e, g)));
       return kOk;
     }
   }
