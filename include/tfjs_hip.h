@@ -138,9 +138,7 @@ int tfhip_graph_destroy(int graph_id);
  *   restores it. Knobs: "tile" (GEMM tile shape index), "splitk" (K slices),
  *   "dw_rows" (output rows per chunk of the 3x3 depthwise kernel), "dw_halo" (1: the
  *   LDS halo depthwise kernel), "no_skinny" (1: tiled GEMM also for tall products),
- *   "skinny_regs" (0: the
- *   streaming GEMM always stages B in LDS), "small_k" (32 / 64: the one-shot GEMM for
- *   K <= 64 with that many rows per tile; unset or 0: never), "fuse_pw_dw"
+ *   "skinny_regs" (0: the streaming GEMM always stages B in LDS), "fuse_pw_dw"
  *   (tfhip_pointwise_depthwise_pays: 1: yes for every shape the fused kernel
  *   takes, 0: never), "pw_dw_tile" (1 / 0: the channel-sliced / the row-ring
  *   pointwise + depthwise kernel where both take a shape), "tile_slice" (32 / 48 /

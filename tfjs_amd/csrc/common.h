@@ -147,7 +147,7 @@ int launch_repeat();
 // name tfhip_set_tuning takes, and (in capitals behind TFHIP_) its environment variable.
 #define TFHIP_TUNING_KNOBS(X)                                                                              \
   X(Tile, "tile") X(SplitK, "splitk") X(DwRows, "dw_rows") X(DwHalo, "dw_halo") X(NoSkinny, "no_skinny")    \
-  X(SkinnyRegs, "skinny_regs") X(SmallK, "small_k") X(FusePwDw, "fuse_pw_dw")          \
+  X(SkinnyRegs, "skinny_regs") X(FusePwDw, "fuse_pw_dw")          \
   X(PwDwTile, "pw_dw_tile") X(TileSlice, "tile_slice") X(TileChunks, "tile_chunks")                         \
   X(FuseBlock, "fuse_block") X(KGroups, "k_groups") X(PwDwStream, "pw_dw_stream")                           \
   X(StreamRows, "stream_rows") X(StreamBlocks, "stream_blocks") X(SkinnyStage, "skinny_stage")              \

@@ -2,16 +2,11 @@
 // loaders the memory layout allows and a tile shape, and launches gemm_kernel.
 #include "gemm_host.h"
 #include "skinny_gemm.h"
-#include "small_k_gemm.h"
 
 using namespace tfhip;
 
 int tfhip::launch_plain_gemm(GemmParams &p, bool transpose_a, bool transpose_b, bool vec) {
   if (skinny_applies(p, transpose_a, transpose_b, vec) && tuning(kTuneNoSkinny) <= 0) return launch_skinny(p);
-  // (off unless asked for: back to back it beats the tiled kernel, but inside a network, where
-  // its operands come from memory rather than from the cache a repeated launch leaves them in, it
-  // loses more often than it wins)
-  if (small_k_applies(p, transpose_a, transpose_b, vec) && tuning(kTuneSmallK) > 0) return launch_small_k(p);
   if (vec) {
     const int shape = choose_tile_shape(p.M, p.N, p.K, p.batch, num_cus());
     if (!transpose_a && !transpose_b) return launch_gemm_shape<kLoadKVec, kLoadXVec>(shape, p);

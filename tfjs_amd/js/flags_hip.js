@@ -19,7 +19,7 @@ const {addon} = require('./binding');
 
 /** The native library's knobs (tfhip_set_tuning), in its own order. */
 const TUNING_KNOBS = [
-  'tile', 'splitk', 'dw_rows', 'dw_halo', 'no_skinny', 'skinny_regs', 'small_k', 'fuse_pw_dw',
+  'tile', 'splitk', 'dw_rows', 'dw_halo', 'no_skinny', 'skinny_regs', 'fuse_pw_dw',
   'pw_dw_tile', 'tile_slice', 'tile_chunks', 'fuse_block', 'k_groups', 'pw_dw_stream', 'stream_rows',
   'stream_blocks', 'skinny_stage', 'block_rows'
 ];
