@@ -52,17 +52,22 @@ def symbol(kernel_name):
     return head.split("::")[-1] + tail.replace("tfhip::", "").replace("(anonymous namespace)::", "")
 
 
-def read_counter(path, counter, by_grid=False):
+def read_counter(path, counter, by_grid=False, copy_bytes=None):
     """{symbol: [value per dispatch]} for one counter; the values of one dispatch (one row per
     XCD or shader engine in some rocprofv3 versions) are summed. by_grid: a symbol's launches are
-    told apart by their grid size (one template serves several shapes)."""
+    told apart by their grid size (one template serves several shapes). copy_bytes: only the
+    copy_f4 launches of that size (one float4 per lane) keep the plain name `copy_f4`, the unit
+    of the scaling; other copies (a benchmark row of their own) are named with their grid."""
     per_dispatch = {}
     with open(path, newline="") as f:
         for row in csv.DictReader(f):
             if row["Counter_Name"] != counter:
                 continue
             name = symbol(row["Kernel_Name"])
-            if by_grid and name != "copy_f4":
+            if name == "copy_f4":
+                if copy_bytes is not None and int(row["Grid_Size"]) != copy_bytes // 16:
+                    name += " grid " + row["Grid_Size"]
+            elif by_grid:
                 name += " grid " + row["Grid_Size"]
             key = (row["Dispatch_Id"], name)
             per_dispatch[key] = per_dispatch.get(key, 0.0) + float(row["Counter_Value"])
@@ -73,7 +78,8 @@ def read_counter(path, counter, by_grid=False):
 
 
 def summarise(fetch_csv, write_csv, copy_bytes, by_grid=False):
-    fetch, write = read_counter(fetch_csv, "FETCH_SIZE", by_grid), read_counter(write_csv, "WRITE_SIZE", by_grid)
+    fetch = read_counter(fetch_csv, "FETCH_SIZE", by_grid, copy_bytes)
+    write = read_counter(write_csv, "WRITE_SIZE", by_grid, copy_bytes)
     if "copy_f4" not in fetch or "copy_f4" not in write:
         raise SystemExit("the profiled command launched no copy_f4 kernel: nothing to scale the counters by")
     mean = lambda v: sum(v) / len(v)
