@@ -381,8 +381,8 @@ def bench_kernels(cold=True, only=None):
         o.free()
 
     def copy(name, nbytes_each):
-        """The yardstick of the memory-bound rows: a plain copy kernel (copy_f4) that reads and writes as
-        many bytes as configuration 3's depthwise convolution, in the same cold rotation."""
+        """The yardstick of a memory-bound row: a plain copy kernel (copy_f4) that moves as many bytes as
+        the row it stands beside (half of them read, half written), in the same cold rotation."""
         nbytes = 2.0 * nbytes_each
         sets = sets_for(nbytes)
         src, dst = Slab(nbytes_each, sets), Slab(nbytes_each, sets)
@@ -410,9 +410,13 @@ def bench_kernels(cold=True, only=None):
                  "relu6", depthwise=True)
     if wanted("cfg3 copy yardstick"):
         copy("cfg3 copy yardstick: 38.5 MB in, 38.5 MB out (the stride-1 depthwise row's traffic)", 8 * 112 * 112 * 96 * 4)
+    if wanted("cfg2b copy yardstick"):
+        copy("cfg2b copy yardstick: 8.4 MB in, 8.4 MB out (the pointwise row's 16.9 MB)", 8 * 56 * 56 * (144 + 24) * 2)
     for name, *_ in synth.BERT_MATMULS:
         if wanted("cfg5 %s" % name):
             matmul("cfg5 %s" % name, **synth.config5(name))
+    if wanted("cfg5 scores copy yardstick"):
+        copy("cfg5 scores copy yardstick: 6.3 MB in, 6.3 MB out (the 12.6 MB of scores and of context)", 96 * 128 * 128 * 4)
     if wanted("cfg4 dequant"):
         dequant("cfg4 dequant uint8 3469760 weights", 3469760, "uint8")
     if wanted("cfg5 dequant"):
