@@ -1188,6 +1188,25 @@ def test_pair_and_block_kernels_refuse_a_non_finite_filter(hip, orc):
         finally:
             check(lib.tfhip_capture_end(None, None))
         fresh.free()
+        # a replay writes the buffer again, with whatever its source holds by then
+        w2[0, 1, 5, 0] = 0.5
+        buf.upload(w2)
+        src = DeviceBuffer.from_numpy(w2)
+        check(lib.tfhip_capture_begin())
+        try:
+            check(lib.tfhip_copy(buf.ptr, src.ptr, w2.size * 4))
+        finally:
+            gid, nodes = ctypes.c_int(), ctypes.c_int()
+            check(lib.tfhip_capture_end(ctypes.byref(gid), ctypes.byref(nodes)))
+        check(lib.tfhip_filter_is_finite(buf.ptr, w2.size, ctypes.byref(finite)))
+        assert finite.value == 1
+        w2[2, 0, 9, 0] = -np.inf
+        src.upload(w2)
+        check(lib.tfhip_graph_launch(gid.value))
+        check(lib.tfhip_filter_is_finite(buf.ptr, w2.size, ctypes.byref(finite)))
+        assert finite.value == 0
+        check(lib.tfhip_graph_destroy(gid.value))
+        src.free()
     finally:
         buf.free()
 

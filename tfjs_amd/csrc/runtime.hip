@@ -28,6 +28,7 @@ struct RecordedGraph {
     uint64_t generation;
   };
   std::vector<Ref> refs;   // blocks a recorded kernel names and that were live when the recording ended
+  std::vector<uintptr_t> writes;   // of those, the blocks a recorded call writes: a replay changes their contents
 };
 
 struct Runtime {
@@ -61,6 +62,7 @@ struct Runtime {
   bool capturing = false;
   std::unordered_map<size_t, std::vector<void *>> capture_free;
   std::set<uintptr_t> capture_refs;
+  std::set<uintptr_t> capture_writes;   // of those, the blocks some recorded call writes
   std::map<int, RecordedGraph> graphs;
   int next_graph = 1;
   std::vector<void *> retired_workspaces;  // outgrown while a graph might still name them
@@ -236,12 +238,15 @@ __global__ __launch_bounds__(256) void find_nonfinite(const unsigned *__restrict
 
 void forget_filter_scans(const void *p) {
   std::lock_guard<std::mutex> lock(g_mutex);
-  if (g.filter_scans.empty()) return;
+  if (g.filter_scans.empty() && !g.capturing) return;
   const uintptr_t a = reinterpret_cast<uintptr_t>(p);
   auto it = g.live.upper_bound(a);
   if (it == g.live.begin()) return;
   --it;
-  if (a < it->first + it->second) g.filter_scans.erase(it->first);
+  if (a >= it->first + it->second) return;
+  g.filter_scans.erase(it->first);
+  // a replay writes the block again, with whatever its inputs hold then
+  if (g.capturing) g.capture_writes.insert(it->first);
 }
 
 int scan_filter(const float *w, int64_t elems, const char *who, bool *nonfinite) {
@@ -362,6 +367,7 @@ int tfhip_shutdown(void) {
   }
   g.capture_free.clear();
   g.capture_refs.clear();
+  g.capture_writes.clear();
   for (void *p : g.retired_workspaces) (void)hipFree(p);
   g.retired_workspaces.clear();
   for (auto &kv : g.live) {
@@ -641,6 +647,7 @@ int tfhip_capture_begin(void) {
   TFHIP_CHECK_HIP(hipStreamBeginCapture(g.stream, hipStreamCaptureModeRelaxed));
   g.capturing = true;
   g.capture_refs.clear();
+  g.capture_writes.clear();
   return kOk;
 }
 
@@ -665,6 +672,7 @@ int tfhip_capture_end(int *graph_id, int *nodes) {
     }
     g.capture_free.clear();
     g.capture_refs.clear();
+    g.capture_writes.clear();
     if (e != hipSuccess) return fail(kHipError, "tfhip_capture_end: %s", hipGetErrorString(e));
     if (nodes) *nodes = (int)rec.nodes;
     return kOk;
@@ -678,9 +686,13 @@ int tfhip_capture_end(int *graph_id, int *nodes) {
   g.capture_free.clear();
   for (uintptr_t base : g.capture_refs) {
     auto it = g.live.find(base);
-    if (it != g.live.end()) rec.refs.push_back({base, it->second, g.generation[base]});
+    if (it != g.live.end()) {
+      rec.refs.push_back({base, it->second, g.generation[base]});
+      if (g.capture_writes.count(base)) rec.writes.push_back(base);
+    }
   }
   g.capture_refs.clear();
+  g.capture_writes.clear();
   const int id = g.next_graph++;
   if (nodes) *nodes = (int)rec.nodes;
   g.graphs[id] = std::move(rec);
@@ -705,6 +717,8 @@ int tfhip_graph_launch(int graph_id) {
                   graph_id, reinterpret_cast<void *>(r.base), r.size);
     }
   }
+  // what the library remembered about the old contents of the blocks this replay writes
+  for (uintptr_t base : it->second.writes) g.filter_scans.erase(base);
   for (int r = g_repeat; r > 0; --r) TFHIP_CHECK_HIP(hipGraphLaunch(it->second.exec, g.stream));
   return kOk;
 }
