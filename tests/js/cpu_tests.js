@@ -232,6 +232,28 @@ h.test('hip storage: write/read round trip, refCounts, disposeData', () => {
   h.assertEqual(backend.disposeData({}), true, 'unknown dataId is reported as released');
 });
 
+h.test('hip kernels: a call that throws releases the output it had allocated; a filter larger than the padded input throws as the reference does', () => {
+  useBackend('hip');
+  const backend = tf.backend(), fake = require('./fake_addon');
+  const x = tf.tensor(new Float32Array(2 * 4 * 4 * 3), [2, 4, 4, 3]);
+  const filter = tf.tensor(new Float32Array(3 * 3 * 3 * 8), [3, 3, 3, 8]);
+  const ids0 = backend.numDataIds(), live0 = backend.memory().numDeviceBuffers;
+  const real = fake.fusedConv2D;
+  fake.fusedConv2D = () => { throw new Error('tfhip_fused_conv2d: refused'); };
+  try {
+    h.assertThrows(() => tf.conv2d(x, filter, 1, 'same'), /refused/);
+  } finally {
+    fake.fusedConv2D = real;
+  }
+  h.assertEqual(backend.numDataIds(), ids0, 'no data id left behind');
+  h.assertEqual(backend.memory().numDeviceBuffers, live0, 'no device buffer left behind');
+  // new TensorBuffer(outShape) of the reference's kernels: new Float32Array(-64)
+  const big = tf.tensor(new Float32Array(7 * 3 * 3 * 8), [7, 3, 3, 8]);
+  h.assertThrows(() => tf.conv2d(x, big, 1, 'valid'), /Invalid typed array length: -64/);
+  h.assertEqual(backend.numDataIds(), ids0 + 1);
+  tf.dispose([x, filter, big]);
+});
+
 h.test('hip storage: tensors move between backends with their refCount (engine.moveData)', () => {
   useBackend('cpu');
   const cpuBackend = tf.backend();

@@ -65,6 +65,7 @@ class HipBackend extends tf.KernelBackend {
     this.poolLimitBytes = this.deviceInfo.hbmBytes / 4;
     this.recording = false;
     this.liveRecordings = 0;
+    this.outputsInFlight = [];   // outputs of the kernel call that is running (guarded)
   }
 
   /** Kernels enqueued from now on are recorded, not run. */
@@ -243,7 +244,25 @@ class HipBackend extends tf.KernelBackend {
   /** Registers a result buffer for a kernel: TensorInfo with a fresh dataId. */
   makeOutput(shape, dtype) {
     const dataId = this.allocate(shape, dtype || 'float32');
-    return {dataId, shape, dtype: dtype || 'float32'};
+    const info = {dataId, shape, dtype: dtype || 'float32'};
+    this.outputsInFlight.push(info);
+    return info;
+  }
+
+  /**
+   * Runs one kernel function; when it throws, the outputs it had allocated by then (makeOutput)
+   * are released before the error goes on, so a refused call leaves no device buffer behind.
+   */
+  guarded(kernelFunc, args) {
+    const mark = this.outputsInFlight.length;
+    try {
+      const result = kernelFunc(args);
+      this.outputsInFlight.length = mark;
+      return result;
+    } catch (e) {
+      this.outputsInFlight.splice(mark).forEach(info => this.disposeIntermediateTensorInfo(info));
+      throw e;
+    }
   }
 
   ptr(dataId) {

@@ -60,13 +60,18 @@ const kernelConfigs = [
 ];
 
 tf.registerBackend('hip', () => new HipBackend(), 3 /* priority */);
-kernelConfigs.forEach(config => tf.registerKernel(config));
+// Every kernel function runs guarded: a call that throws (a shape the native library refuses)
+// releases the outputs it had allocated by then.
+const guardedConfigs = kernelConfigs.map(config => Object.assign({}, config, {
+  kernelFunc: args => args.backend.guarded(config.kernelFunc, args)
+}));
+guardedConfigs.forEach(config => tf.registerKernel(config));
 
 module.exports = {
   tf,
   HipBackend,
   decodeWeights,
-  kernelConfigs,
+  kernelConfigs: guardedConfigs,
   graphPlan,
   flags,
   GraphModel: graphModel ? graphModel.GraphModel : undefined,

@@ -90,8 +90,19 @@ function convImpl(args, depthwise, fused, opName, residual) {
     backend.disposeIntermediateTensorInfo(y);
     return sum;
   }
+  const outSize = tf.util.sizeFromShape(info.outShape);
+  if (outSize < 0) {
+    // A filter that does not fit the padded input. The reference's kernels allocate the result first
+    // (`new TensorBuffer(convInfo.outShape)`: tfjs-backend-cpu/src/kernels/Conv2D.ts:46,
+    // DepthwiseConv2dNative.ts:57), which is `new Float32Array(outSize)`: V8's RangeError.
+    throw new RangeError(`Invalid typed array length: ${outSize}`);
+  }
+  if (outSize > 0 && info.outShape.some(d => d < 0)) {
+    // (two negative extents: the reference goes on with a buffer of their product and loops that never run)
+    throw new Error(`${opName}: the filter does not fit the padded input (output shape [${info.outShape}])`);
+  }
   const out = backend.makeOutput(info.outShape, 'float32');
-  if (tf.util.sizeFromShape(info.outShape) === 0) {
+  if (outSize === 0) {
     return out;
   }
   geom[0] = info.batchSize;
