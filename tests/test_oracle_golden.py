@@ -525,3 +525,24 @@ def test_oracle_avg_pool_against_brute_force():
                 cols = [j for j in range(c - left, c - left + 2) if 0 <= j < 6]
                 window = x[n][np.ix_(rows, cols)].astype(np.float64)
                 np.testing.assert_allclose(got[n, r, c], window.mean(axis=(0, 1)), rtol=1e-6)
+
+
+def test_oracle_avg_pool_of_a_window_outside_the_image_is_nan():
+    """pool_utils.ts:45-84 divides the sum of the taps inside the image by their count: a window with
+    none (a one-row filter on a padded border row; the output columns a numeric pad derives from the
+    row stride, conv_util.ts:350-365) gives 0 / 0."""
+    x = np.arange(40, dtype=np.float32).reshape(1, 4, 10, 1)
+    got = orc.avg_pool(x, (1, 3), 1, 1)
+    assert got.shape == (1, 6, 12, 1)
+    for r in range(6):
+        for c in range(12):
+            rows = [i for i in range(r - 1, r) if 0 <= i < 4]
+            cols = [j for j in range(c - 1, c + 2) if 0 <= j < 10]
+            if not rows or not cols:
+                assert np.isnan(got[0, r, c, 0])
+            else:
+                np.testing.assert_allclose(got[0, r, c, 0], x[0][np.ix_(rows, cols)].mean(), rtol=1e-6)
+    # strides (1, 2) with pad 0: the width comes out as for stride 1, and the windows from column 6 on start beyond the image
+    got = orc.avg_pool(np.ones((2, 8, 11, 3), np.float32), 3, (1, 2), 0)
+    assert got.shape == (2, 6, 9, 3)
+    assert not np.isnan(got[:, :, :6]).any() and np.isnan(got[:, :, 6:]).all()

@@ -393,9 +393,11 @@ int tfhip_avg_pool(const float *x, float *y, int64_t batch, int64_t in_h, int64_
   TFHIP_CHECK_ARG(batch < lim && in_h < lim && in_w < lim && c < lim && f_h < lim && f_w < lim && stride_h < lim &&
                       stride_w < lim && pad_top < lim && pad_left < lim && out_h < lim && out_w < lim,
                   "tfhip_avg_pool: dimension exceeds 2^31-1");
-  // every window starts at or before the last row / column of the image
-  TFHIP_CHECK_ARG(out_h == 0 || (out_h - 1) * stride_h - pad_top < in_h, "tfhip_avg_pool: out_h does not fit the input");
-  TFHIP_CHECK_ARG(out_w == 0 || (out_w - 1) * stride_w - pad_left < in_w, "tfhip_avg_pool: out_w does not fit the input");
+  // (a window may lie outside the image altogether - the reference's output extent for a numeric pad is worked
+  // out from the filter height and the row stride alone, computeOutputShape2D in conv_util.ts:350-365 - and
+  // averages nothing: 0 / 0, NaN, as pool_utils.ts:81 leaves it)
+  TFHIP_CHECK_ARG(out_h * stride_h + f_h < lim && out_w * stride_w + f_w < lim,
+                  "tfhip_avg_pool: window positions exceed 2^31-1");
   if (batch * out_h * out_w * c == 0) return kOk;
   TFHIP_CHECK_RANGE(x, batch * in_h * in_w * c, 4, "x");
   TFHIP_CHECK_OUTPUT(y, batch * out_h * out_w * c, 4, "y");

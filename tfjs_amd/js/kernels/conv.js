@@ -17,7 +17,7 @@
  * two kernels here.
  */
 const tf = require('../core');
-const {activationCode, broadcastStrides, requireFloat32, addon} = require('./fused_util');
+const {activationCode, broadcastStrides, outputSize, requireFloat32, addon} = require('./fused_util');
 const glue = require('./glue');
 
 // Scratch that carries the geometry and the epilogue strides to the addon.
@@ -90,17 +90,7 @@ function convImpl(args, depthwise, fused, opName, residual) {
     backend.disposeIntermediateTensorInfo(y);
     return sum;
   }
-  const outSize = tf.util.sizeFromShape(info.outShape);
-  if (outSize < 0) {
-    // A filter that does not fit the padded input. The reference's kernels allocate the result first
-    // (`new TensorBuffer(convInfo.outShape)`: tfjs-backend-cpu/src/kernels/Conv2D.ts:46,
-    // DepthwiseConv2dNative.ts:57), which is `new Float32Array(outSize)`: V8's RangeError.
-    throw new RangeError(`Invalid typed array length: ${outSize}`);
-  }
-  if (outSize > 0 && info.outShape.some(d => d < 0)) {
-    // (two negative extents: the reference goes on with a buffer of their product and loops that never run)
-    throw new Error(`${opName}: the filter does not fit the padded input (output shape [${info.outShape}])`);
-  }
+  const outSize = outputSize(info.outShape, opName);
   const out = backend.makeOutput(info.outShape, 'float32');
   if (outSize === 0) {
     return out;

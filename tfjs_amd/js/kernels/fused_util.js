@@ -7,6 +7,7 @@
  * the kernel configs reuse from call to call: every addon call is synchronous
  * and has read its arguments when it returns.
  */
+const tf = require('../core');
 const {addon, FusableActivation} = require('../binding');
 
 function activationCode(activation, opName) {
@@ -68,4 +69,23 @@ function requireFloat32(tensors, opName) {
   }
 }
 
-module.exports = {activationCode, broadcastStrides, requireFloat32, addon};
+/**
+ * The element count of a result about to be allocated. A window larger than its padded input makes
+ * conv_util's output extents negative; the reference's kernels allocate the result first
+ * (`new TensorBuffer(outShape)` / `buffer(outShape)`: tfjs-backend-cpu/src/kernels/Conv2D.ts:46,
+ * DepthwiseConv2dNative.ts:57, utils/pool_utils.ts:37), which is `new Float32Array(size)` with a
+ * negative size: V8's RangeError, thrown here with the same text. Two negative extents multiply to
+ * a positive size, which the reference goes on with (loops that never run): refused here.
+ */
+function outputSize(outShape, opName) {
+  const size = tf.util.sizeFromShape(outShape);
+  if (size < 0) {
+    throw new RangeError(`Invalid typed array length: ${size}`);
+  }
+  if (size > 0 && outShape.some(d => d < 0)) {
+    throw new Error(`${opName}: the window does not fit the padded input (output shape [${outShape}])`);
+  }
+  return size;
+}
+
+module.exports = {outputSize, activationCode, broadcastStrides, requireFloat32, addon};

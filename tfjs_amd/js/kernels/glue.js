@@ -13,7 +13,7 @@
  * launch sequence.
  */
 const tf = require('../core');
-const {broadcastStrides, requireFloat32, addon} = require('./fused_util');
+const {broadcastStrides, outputSize, requireFloat32, addon} = require('./fused_util');
 const {FusableActivation} = require('../binding');
 
 const aStrides = new Float64Array(6);
@@ -82,8 +82,9 @@ function avgPool(args) {
   if (info.filterWidth === 1 && info.filterHeight === 1 && tf.util.arraysEqual(info.inShape, info.outShape)) {
     return identity({inputs: {x}, backend});
   }
+  const outSize = outputSize(info.outShape, 'AvgPool');
   const out = backend.makeOutput(info.outShape, 'float32');
-  if (tf.util.sizeFromShape(info.outShape) > 0) {
+  if (outSize > 0) {
     const g = poolGeom;
     g[0] = info.batchSize; g[1] = info.inHeight; g[2] = info.inWidth; g[3] = info.inChannels;
     g[4] = info.effectiveFilterHeight; g[5] = info.effectiveFilterWidth; g[6] = info.strideHeight;
