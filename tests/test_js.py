@@ -20,8 +20,8 @@ NODE = shutil.which("node")
 needs_node = pytest.mark.skipif(NODE is None, reason="node is not installed")
 
 
-def run_node(script, env=None, timeout=900):
-    proc = subprocess.run([NODE, os.path.join(ROOT, script)], cwd=ROOT, env=dict(os.environ, **(env or {})),
+def run_node(script, *args, env=None, timeout=900):
+    proc = subprocess.run([NODE, os.path.join(ROOT, script)] + list(args), cwd=ROOT, env=dict(os.environ, **(env or {})),
                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=timeout)
     sys.stdout.write(proc.stdout[-6000:])
     return proc
@@ -126,6 +126,17 @@ def test_node_gpu_tier(tmp_path):
     from tfjs_amd import workloads
     workloads.write_graph_model(str(tmp_path), workloads.mobilenet_v2_weights(seed=3), np.uint8)
     proc = run_node("tests/js/gpu_tests.js", env={"TFJS_HIP_TEST_MODEL_DIR": str(tmp_path)})
+    assert proc.returncode == 0, proc.stdout[-4000:]
+    assert " 0 failed" in proc.stdout
+
+
+@pytest.mark.gpu
+@needs_node
+@pytest.mark.parametrize("seed", [1, 2])
+def test_node_random_ops_match_the_js_oracle(seed):
+    """Seeded random calls of the op wrappers on the hip backend against the JavaScript oracle backend
+    (tests/js/random_ops.js): values, shapes, dtypes, and the message of every call both refuse."""
+    proc = run_node("tests/js/random_ops.js", str(seed), "1200")
     assert proc.returncode == 0, proc.stdout[-4000:]
     assert " 0 failed" in proc.stdout
 
