@@ -50,17 +50,58 @@ export declare class HipBackend extends KernelBackend {
   readonly recording: boolean;
 }
 
-/** Load options of the stand-in graph model beyond the reference's. */
+/** Load options of a graph model beyond the reference's; one left out takes the flag named. */
 export interface HipGraphModelOptions {
-  /** default true: a _FusedConv2D read by one Add/AddV2 only runs with it as one FusedConv2DAdd kernel */
+  /** flag HIP_FUSE_RESIDUAL_ADD (true): a _FusedConv2D read by one Add/AddV2 only runs with it as one FusedConv2DAdd kernel */
   fuseResidualAdd?: boolean;
-  /** default true: a 1x1 _FusedConv2D read by one 3x3 FusedDepthwiseConv2dNative only is one FusedPointwiseDepthwiseConv2D step */
+  /** flag HIP_FUSE_POINTWISE_DEPTHWISE (true): a 1x1 _FusedConv2D read by one 3x3 FusedDepthwiseConv2dNative only is one FusedPointwiseDepthwiseConv2D step */
   fusePointwiseDepthwise?: boolean;
-  /** default false: record the kernels of an execution into a HIP graph and replay it for the same input shapes */
+  /** flag HIP_RECORD_LAUNCHES (false): record the kernels of an execution into a HIP graph and replay it for the same input shapes */
   recordLaunches?: boolean;
+  /** what plans the fusions and runs the recordings: loadGraphModel of this package passes its `graphPlan` */
+  planner?: GraphPlanner;
   /** default true: DepthwiseConv2dNative -> BiasAdd -> Relu | Relu6 | Elu chains run as one FusedDepthwiseConv2dNative step */
   fuseDepthwiseBiasActivation?: boolean;
 }
+
+/** The executor's view of the nodes it is about to run, as graph_plan.js reads it. */
+export interface PlanView {
+  order: string[];
+  op(name: string): string;
+  isOp(name: string): boolean;
+  sources(name: string): string[];
+  readers(name: string): number;
+  position(name: string): number;
+  isFetched(name: string): boolean;
+  convParams(name: string): (inputs: Array<Tensor|null>) => object;
+  fusedOps(name: string): string[];
+  weight(name: string): Tensor|undefined;
+}
+/** One step that replaces graph nodes: run `run` on the values of `sources` at `place`, store it as `yields`, skip `drops`. */
+export interface PlannedFusion {
+  place: string;
+  yields: string;
+  drops: string[];
+  sources: string[];
+  run(inputs: Tensor[]): Tensor;
+  tags: {conv?: string, pointwise?: string};
+}
+export interface GraphPlanner {
+  planFusions(view: PlanView, options?: HipGraphModelOptions): PlannedFusion[];
+  wantsRecording(options?: HipGraphModelOptions): boolean;
+  runRecorded(recordings: Map<string, object>, key: string, feeds: {[name: string]: Tensor}, single: boolean,
+              runPlan: (feeds: {[name: string]: Tensor}) => Tensor|Tensor[]): Tensor|Tensor[];
+  disposeRecordings(recordings: Map<string, object>): void;
+}
+/** Plan-time fusion and launch recording for a graph-model executor (graph_plan.js). */
+export declare const graphPlan: GraphPlanner;
+/** The HIP_* flags registered on tf.env() (flags_hip.js): the plan options and one flag per tuning knob of the native library. */
+export declare const flags: {
+  TUNING_KNOBS: string[];
+  PLAN_FLAGS: {[flag: string]: boolean};
+  flagOf(knob: string): string;
+  applyTuningFlags(): void;
+};
 
 /** decodeWeights with the dequantize step on the GPU; inject as GraphModel's tfio. */
 export declare function decodeWeights(
