@@ -1370,6 +1370,43 @@ def test_fused_pairs_refuse_sizes_that_overflow(hip):
         assert rc != 0 and "supported range" in lib.tfhip_last_error().decode()
 
 
+def test_every_entry_point_refuses_sizes_that_overflow(hip):
+    """Extents whose products wrap 64 bits (or only exceed any memory) are refused before a size is formed
+    from them: an error return, never a launch with truncated dimensions."""
+    from tfjs_amd import capi
+    lib = capi.load_library()
+    big, huge = 1 << 40, 1 << 62
+    z3, z4, z6 = capi.i64_array([0] * 3), capi.i64_array([0] * 4), capi.i64_array([0] * 6)
+    with capi.DeviceBuffer(64) as buf:
+        p = buf.ptr
+        calls = {
+            "conv2d": lambda: lib.tfhip_fused_conv2d(p, p, p, big, big, big, 3, 3, 3, 8, 1, 1, 1, 1, 0, 0, big, big, 0, None, z4, 0,
+                                                     None, z4, 0.2, None),
+            "conv2d, wrapping channel count": lambda: lib.tfhip_fused_conv2d(p, p, p, 1, 4, 4, huge, 2, 2, 8, 1, 1, 1, 1, 0, 0, 3, 3,
+                                                                             0, None, z4, 0, None, z4, 0.2, None),
+            "depthwise": lambda: lib.tfhip_fused_depthwise_conv2d(p, p, p, (1 << 31) - 2, (1 << 31) - 2, (1 << 31) - 2, 8, 3, 3, 1, 1, 1,
+                                                                  1, 1, 1, 1, (1 << 31) - 2, (1 << 31) - 2, None, z4, 0, None, z4, 0.2),
+            "depthwise, wrapping multiplier": lambda: lib.tfhip_fused_depthwise_conv2d(p, p, p, 1, 4, 4, big, 3, 3, big, 1, 1, 1, 1, 1, 1,
+                                                                                       4, 4, None, z4, 0, None, z4, 0.2),
+            "avg_pool": lambda: lib.tfhip_avg_pool(p, p, (1 << 31) - 2, (1 << 31) - 2, (1 << 31) - 2, 8, 2, 2, 1, 1, 0, 0,
+                                                   (1 << 31) - 3, (1 << 31) - 3),
+            "mean_hw": lambda: lib.tfhip_mean_hw(p, p, big, big, big, 4),
+            "add": lambda: lib.tfhip_add(p, z6, p, z6, p, capi.i64_array([big] * 6), 6),
+            "binary": lambda: lib.tfhip_binary(2, p, z6, p, z6, p, capi.i64_array([big] * 6), 6),
+            "add, wrapping stride": lambda: lib.tfhip_add(p, capi.i64_array([huge, 1]), p, capi.i64_array([0, 1]), p,
+                                                          capi.i64_array([5, 2]), 2),
+            "unary": lambda: lib.tfhip_unary(1, p, p, huge, 0.2),
+            "cast": lambda: lib.tfhip_cast(p, 0, p, 1, huge),
+            "dequant_affine": lambda: lib.tfhip_dequant_affine(p, 16, huge, 1.0, 0.0, p, 0),
+            "dequant_f16": lambda: lib.tfhip_dequant_f16(p, huge, p),
+            "matmul": lambda: lib.tfhip_fused_matmul(p, p, p, big, big, big, big, big, 0, 0, None, z3, 0, None, z3, 0.2),
+        }
+        for name, call in calls.items():
+            assert call() != 0, name
+            message = lib.tfhip_last_error().decode()
+            assert "supported range" in message or "not inside a live device buffer" in message or "exceed" in message, (name, message)
+
+
 # -------------------------------------------------- recorded launch sequences
 
 def test_recorded_graph_replays(hip, orc):

@@ -48,6 +48,10 @@ int setup_static_scratch(int device);
 
 // True when [p, p + bytes) lies inside one live block (own or external).
 bool range_is_live(const void *p, size_t bytes);
+// No operand has more elements than this (2^40: four times the bytes of the largest memory this
+// library runs on): element counts beyond it are refused before anything is multiplied by them.
+constexpr long long kMaxElems = 1LL << 40;
+
 // True when the product of the non-negative factors is below `limit`, decided
 // without forming a product that could overflow 64 bits.
 inline bool product_below(int64_t limit, std::initializer_list<int64_t> factors) {
@@ -117,7 +121,8 @@ bool capturing();
 // Operand `name` of `elems` float-sized (`esize` bytes) elements must be live.
 #define TFHIP_CHECK_RANGE(ptr, elems, esize, name)                             \
   do {                                                                         \
-    if ((ptr) == nullptr || !::tfhip::range_is_live((ptr), (size_t)(elems) * (esize))) \
+    if ((ptr) == nullptr || (long long)(elems) < 0 || (long long)(elems) > ::tfhip::kMaxElems || \
+        !::tfhip::range_is_live((ptr), (size_t)(elems) * (esize)))             \
       return ::tfhip::fail(::tfhip::kOutOfRange,                               \
                            "%s: operand '%s' (%lld elements of %d bytes at %p) " \
                            "is not inside a live device buffer",               \
@@ -174,7 +179,10 @@ inline int64_t strided_extent(const int64_t *dims, const int64_t *strides, int r
   int64_t last = 0;
   for (int i = 0; i < rank; ++i) {
     if (dims[i] <= 0) return 0;
+    // (an extent beyond kMaxElems is no operand: say so without forming a product that could wrap)
+    if (strides[i] < 0 || (dims[i] > 1 && strides[i] > kMaxElems / (dims[i] - 1))) return kMaxElems + 1;
     last += (dims[i] - 1) * strides[i];
+    if (last > kMaxElems) return kMaxElems + 1;
   }
   return last + 1;
 }

@@ -338,9 +338,10 @@ int fused_conv2d(const float *x, const float *filter, float *y, int64_t batch, i
                   "tfhip_fused_conv2d: non-positive dimension");
   TFHIP_CHECK_ARG(pad_top >= 0 && pad_left >= 0, "tfhip_fused_conv2d: negative padding");
   const int64_t lim = 0x7fffffff;
-  const int64_t M = batch * out_h * out_w, K = f_h * f_w * in_c;
-  TFHIP_CHECK_ARG(M < lim && K < lim && out_c < lim && in_h < lim && in_w < lim && batch * in_h * in_w * in_c < (lim << 8),
+  TFHIP_CHECK_ARG(product_below(lim, {batch, out_h, out_w}) && product_below(lim, {f_h, f_w, in_c}) && out_c < lim &&
+                      in_h < lim && in_w < lim && product_below(lim << 8, {batch, in_h, in_w, in_c}),
                   "tfhip_fused_conv2d: dimension exceeds the supported range");
+  const int64_t M = batch * out_h * out_w, K = f_h * f_w * in_c;
   TFHIP_CHECK_ARG(batch * in_h * in_w * in_c * 4 <= 0xfffffffeLL,
                   "tfhip_fused_conv2d: an input above 4 GiB is not supported");
   if (M == 0) return kOk;

@@ -326,9 +326,12 @@ extern "C" int tfhip_fused_depthwise_conv2d(
   TFHIP_CHECK_ARG(activation != TFHIP_PRELU || prelu_weights != nullptr,
                   "tfhip_fused_depthwise_conv2d: prelu activation without weights");
   const int64_t lim = 0x7fffffff;
-  TFHIP_CHECK_ARG(batch < lim && in_h < lim && in_w < lim && in_c * ch_mul < lim && out_h < lim && out_w < lim,
+  TFHIP_CHECK_ARG(batch < lim && in_h < lim && in_w < lim && product_below(lim, {in_c, ch_mul}) && out_h < lim && out_w < lim,
                   "tfhip_fused_depthwise_conv2d: dimension exceeds 2^31-1");
   TFHIP_CHECK_ARG(pad_top >= 0 && pad_left >= 0, "tfhip_fused_depthwise_conv2d: negative padding");
+  TFHIP_CHECK_ARG(product_below(kMaxElems, {batch, in_h, in_w, in_c}) && product_below(kMaxElems, {batch, out_h, out_w, in_c, ch_mul}) &&
+                      product_below(lim, {f_h, f_w, in_c, ch_mul}),
+                  "tfhip_fused_depthwise_conv2d: tensor exceeds the supported range");
   const int64_t out_c = in_c * ch_mul;
   const int64_t total = batch * out_h * out_w * out_c;
   if (total == 0) return kOk;

@@ -298,6 +298,7 @@ int tfhip_add(const float *a, const int64_t *a_strides, const float *b, const in
   bool dense = true;
   for (int d = rank - 1; d >= 0; --d) {
     TFHIP_CHECK_ARG(out_shape[d] >= 0 && a_strides[d] >= 0 && b_strides[d] >= 0, "tfhip_add: negative extent or stride");
+    TFHIP_CHECK_ARG(out_shape[d] == 0 || total <= kMaxElems / out_shape[d], "tfhip_add: tensor exceeds the supported range");
     if (out_shape[d] > 1 && (a_strides[d] != total || b_strides[d] != total)) dense = false;
     p.shape[d] = out_shape[d];
     p.a_s[d] = a_strides[d];
@@ -335,6 +336,7 @@ int tfhip_binary(int op, const float *a, const int64_t *a_strides, const float *
   bool dense = true;
   for (int d = rank - 1; d >= 0; --d) {
     TFHIP_CHECK_ARG(out_shape[d] >= 0 && a_strides[d] >= 0 && b_strides[d] >= 0, "tfhip_binary: negative extent or stride");
+    TFHIP_CHECK_ARG(out_shape[d] == 0 || total <= kMaxElems / out_shape[d], "tfhip_binary: tensor exceeds the supported range");
     if (out_shape[d] > 1 && (a_strides[d] != total || b_strides[d] != total)) dense = false;
     p.shape[d] = out_shape[d];
     p.a_s[d] = a_strides[d];
@@ -398,6 +400,8 @@ int tfhip_avg_pool(const float *x, float *y, int64_t batch, int64_t in_h, int64_
   // averages nothing: 0 / 0, NaN, as pool_utils.ts:81 leaves it)
   TFHIP_CHECK_ARG(out_h * stride_h + f_h < lim && out_w * stride_w + f_w < lim,
                   "tfhip_avg_pool: window positions exceed 2^31-1");
+  TFHIP_CHECK_ARG(product_below(kMaxElems, {batch, in_h, in_w, c}) && product_below(kMaxElems, {batch, out_h, out_w, c}),
+                  "tfhip_avg_pool: tensor exceeds the supported range");
   if (batch * out_h * out_w * c == 0) return kOk;
   TFHIP_CHECK_RANGE(x, batch * in_h * in_w * c, 4, "x");
   TFHIP_CHECK_OUTPUT(y, batch * out_h * out_w * c, 4, "y");
@@ -424,6 +428,7 @@ int tfhip_cast(const void *x, int from_dtype, void *y, int to_dtype, int64_t n) 
 int tfhip_mean_hw(const float *x, float *y, int64_t batch, int64_t h, int64_t w, int64_t c) {
   TFHIP_REQUIRE_INIT();
   TFHIP_CHECK_ARG(batch >= 0 && h > 0 && w > 0 && c >= 0, "tfhip_mean_hw: bad dimensions");
+  TFHIP_CHECK_ARG(product_below(kMaxElems, {batch, h, w, c}), "tfhip_mean_hw: tensor exceeds the supported range");
   if (batch * c == 0) return kOk;
   TFHIP_CHECK_RANGE(x, batch * h * w * c, 4, "x");
   TFHIP_CHECK_OUTPUT(y, batch * c, 4, "y");
